@@ -1,0 +1,182 @@
+"""TEST INFRASTRUCTURE — not product code.
+
+ctypes/numpy front end of the C restatement in ``qmm_oracle.c`` (the CPU oracle of the
+quantized-matmul path).  Only ``tests/``, ``__graft_entry__.smoke()`` and ``bench.py``'s
+``cpu_baseline`` leg may import this package; the product path never does.
+
+Arrays are numpy; 16-bit floats travel as their uint16 bit patterns and float8 as uint8
+codes, so nothing here depends on torch.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+F32, F16, BF16, E4M3, E5M2 = 0, 1, 2, 3, 4
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+_lib = None
+
+
+def build(force=False):
+    """Compiles qmm_oracle.c with gcc (see Makefile)."""
+    src = os.path.join(_HERE, "qmm_oracle.c")
+    if force or not os.path.exists(_LIB_PATH) or os.path.getmtime(_LIB_PATH) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "liboracle.so"], stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        L = _lib
+        L.orc_f32_to_bf16.restype = ctypes.c_uint16
+        L.orc_f32_to_bf16.argtypes = [ctypes.c_float]
+        L.orc_f32_to_f16.restype = ctypes.c_uint16
+        L.orc_f32_to_f16.argtypes = [ctypes.c_float]
+        L.orc_f32_to_fp8.restype = ctypes.c_uint8
+        L.orc_f32_to_fp8.argtypes = [ctypes.c_float, ctypes.c_int]
+        L.orc_fp8_to_f32.restype = ctypes.c_float
+        L.orc_fp8_to_f32.argtypes = [ctypes.c_uint8, ctypes.c_int]
+        L.orc_f16_to_f32.restype = ctypes.c_float
+        L.orc_f16_to_f32.argtypes = [ctypes.c_uint16]
+        L.orc_q4_pack.restype = ctypes.c_int64
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _c(a, dtype=None):
+    a = np.ascontiguousarray(a)
+    return a if dtype is None else a.astype(dtype, copy=False)
+
+
+_NP = {F32: np.float32, F16: np.uint16, BF16: np.uint16, E4M3: np.uint8, E5M2: np.uint8}
+I64 = ctypes.c_int64
+
+
+# ------------------------------------------------------------------ casts (vectorised loops in Python: small inputs only)
+def f32_to_bf16(x):
+    x = np.asarray(x, np.float32)
+    u = x.view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    return np.where(np.isnan(x), np.uint16(0x7FC0), r)
+
+
+def bf16_to_f32(h):
+    return (np.asarray(h, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def f32_to_f16(x):
+    L = lib()
+    x = np.asarray(x, np.float32)
+    return np.array([L.orc_f32_to_f16(float(v)) for v in x.ravel()], np.uint16).reshape(x.shape)
+
+
+def f32_to_fp8(x, fmt):
+    L = lib()
+    x = np.asarray(x, np.float32)
+    return np.array([L.orc_f32_to_fp8(ctypes.c_float(v), fmt) for v in x.ravel()], np.uint8).reshape(x.shape)
+
+
+def fp8_table(fmt):
+    L = lib()
+    return np.array([L.orc_fp8_to_f32(i, fmt) for i in range(256)], np.float32)
+
+
+def to_f32(a, dtype):
+    if dtype == F32:
+        return np.asarray(a, np.float32)
+    if dtype == BF16:
+        return bf16_to_f32(a)
+    if dtype == F16:
+        return np.asarray(a, np.uint16).view(np.float16).astype(np.float32)
+    return fp8_table(dtype)[np.asarray(a, np.uint8)]
+
+
+# ------------------------------------------------------------------ ops
+def qmm8(a, dtype, b, scales, want_f64=False):
+    """_weight_int8pack_mm.  a: [M,K] storage array of `dtype`, unit stride along K, any
+    row stride (a numpy view such as base[::2] is read in place); b int8 [N,K]; scales [N]
+    storage array of `dtype`.  Returns c (storage array [M,N]) or (c, c64, mag)."""
+    a = np.asarray(a, _NP[dtype])
+    b = _c(b, np.int8)
+    scales = _c(scales, _NP[dtype])
+    N, K = b.shape
+    M = a.shape[0]
+    if M > 1 and K > 1 and a.strides[1] != a.itemsize:
+        a = np.ascontiguousarray(a)
+    a_sm = a.strides[0] // a.itemsize if M > 1 else K
+    c = np.empty((M, N), _NP[dtype])
+    c64 = np.empty((M, N), np.float64)
+    mag = np.empty((M, N), np.float64)
+    lib().orc_qmm8(_p(a), dtype, I64(a_sm), _p(b), _p(scales), _p(c), _p(c64), _p(mag), I64(M), I64(N), I64(K))
+    return (c, c64, mag) if want_f64 else c
+
+
+def qmm8_f32order(a, dtype, b, scales):
+    a = _c(a, _NP[dtype])
+    b = _c(b, np.int8)
+    scales = _c(scales, _NP[dtype])
+    (M, K), N = a.shape, b.shape[0]
+    c = np.empty((M, N), _NP[dtype])
+    lib().orc_qmm8_f32order(_p(a), dtype, I64(K), _p(b), _p(scales), _p(c), I64(M), I64(N), I64(K))
+    return c
+
+
+def q4_pack(w, scales, scales_dtype, bias):
+    """_dyn_quant_pack_4bit_weight: float32 vector [bytes | scales | bias]."""
+    w = _c(w, np.uint8)
+    scales = _c(scales, _NP[scales_dtype])
+    nb = 0 if bias is None else bias.size
+    bias = None if bias is None else _c(bias, np.float32)
+    out = np.empty(w.size + scales.size + nb, np.float32)
+    n = lib().orc_q4_pack(_p(w), I64(w.size), _p(scales), scales_dtype, I64(scales.size), _p(bias), I64(nb), _p(out))
+    assert n == out.size
+    return out
+
+
+def q4_rowquant(x, dtype, groupwise):
+    x = _c(x, _NP[dtype])
+    M, K = x.shape
+    q = np.empty((M, K), np.int32)
+    recip = np.empty(M, np.float32)
+    nzp = np.empty(M, np.int32)
+    lib().orc_q4_rowquant(_p(x), dtype, I64(M), I64(K), int(bool(groupwise)), _p(q), _p(recip), _p(nzp))
+    return q, recip, nzp
+
+
+def q4_matmul(x, dtype, packed, bs, K, N, want_iacc=False):
+    """_dyn_quant_matmul_4bit.  Returns out [M,N] (storage array) or (out, iacc[M,N,nblocks])."""
+    x = _c(x, _NP[dtype])
+    packed = _c(packed, np.float32)
+    M = x.shape[0]
+    out = np.empty((M, N), _NP[dtype])
+    nblocks = (K + bs - 1) // bs
+    iacc = np.empty((M, N, nblocks), np.int32) if want_iacc else None
+    lib().orc_q4_matmul(_p(x), dtype, _p(packed), I64(packed.size), I64(M), I64(K), I64(N), I64(bs), _p(out), _p(iacc))
+    return (out, iacc) if want_iacc else out
+
+
+def scaled_mm(a, fmt_a, bt, fmt_b, sa, sb, rowwise, bias=None, bias_dtype=F32, scale_result=None, out_dtype=BF16,
+              want_mag=False):
+    """_scaled_mm.  a: uint8 codes [M,K]; bt: uint8 codes [N,K] (mat2 column-major);
+    sa/sb float32 ([1] or [M]/[N])."""
+    a = _c(a, np.uint8)
+    bt = _c(bt, np.uint8)
+    (M, K), N = a.shape, bt.shape[0]
+    sa = _c(np.asarray(sa, np.float32).reshape(-1))
+    sb = _c(np.asarray(sb, np.float32).reshape(-1))
+    bias = None if bias is None else _c(bias, _NP[bias_dtype])
+    sr = None if scale_result is None else np.asarray([scale_result], np.float32)
+    out = np.empty((M, N), _NP[out_dtype])
+    mag = np.empty((M, N), np.float64) if want_mag else None
+    lib().orc_scaled_mm(_p(a), fmt_a, _p(bt), fmt_b, _p(sa), _p(sb), int(bool(rowwise)), _p(bias), bias_dtype, _p(sr),
+                        _p(out), out_dtype, _p(mag), I64(M), I64(N), I64(K))
+    return (out, mag) if want_mag else out
