@@ -1,0 +1,150 @@
+/*
+ * C ABI of the MI355X (gfx950) runtime for torch-vulkan's quantized-matmul path.
+ *
+ * The first block reproduces, name for name and argument for argument, the C ABI the
+ * reference's C++ backend binds (reference crates/pyvk/csrc/vk.h:49-69, implemented in
+ * Rust at crates/pyvk/src/ffi.rs:42-206).  A backend built against those declarations
+ * links against this library unchanged.  Conventions (ffi.rs:1-28): every fallible
+ * function returns 0 on success and -1 on failure; the message of the last failure on
+ * the calling thread is returned by vkt_last_error().
+ *
+ * Differences that follow from HIP (device memory is not host-mapped):
+ *   - VktAlloc.host is always NULL; VktAlloc.address is the device pointer.
+ *   - host <-> device transfers go through vkt_copy_* (second block).
+ *   - vkt_dispatch takes the grid for signature compatibility; for the kernels of this
+ *     path the launch geometry is planned by the library from the parameter block
+ *     (a grid of 0 workgroups in any dimension is still an error, as in the reference).
+ *
+ * The parameter blocks ("push constants", at most 128 bytes, copied at call time) are
+ * declared at the end; Q8Params and Q4Params keep the reference's layouts
+ * (crates/pyvk/csrc/quant.cpp:31-43).
+ */
+#ifndef VKT_H
+#define VKT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---------------------------------------------------------------- reference C ABI */
+
+/* vk.h:50-55 / ffi.rs:31-40 */
+typedef struct VktAlloc {
+  void* handle;     /* opaque, pass to vkt_free */
+  uint8_t* host;    /* NULL: HBM is not host-mapped */
+  uint64_t address; /* device address of the first byte (256-byte aligned) */
+  uint64_t size;    /* usable bytes (>= the request) */
+} VktAlloc;
+
+const char* vkt_last_error(void);                                  /* vk.h:56, ffi.rs:42-45 */
+int vkt_alloc(uint64_t nbytes, VktAlloc* out);                     /* vk.h:57, ffi.rs:47-60 */
+void vkt_free(void* handle);                                       /* vk.h:58, ffi.rs:62-72 (no-op after shutdown) */
+int vkt_synchronize(void);                                         /* vk.h:59, ffi.rs:74-80 */
+int vkt_empty_cache(void);                                         /* vk.h:60, ffi.rs:82-95 */
+void vkt_memory_stats(uint64_t* allocated, uint64_t* reserved);    /* vk.h:61, ffi.rs:97-110 */
+/* vk.h:62-63, ffi.rs:112-142: queue kernel `name` specialised with spec[0..nspec),
+ * parameters push[0..npush), asynchronously and in order with all earlier work. */
+int vkt_dispatch(const char* name, const uint32_t* spec, size_t nspec, const uint8_t* push, size_t npush, uint32_t gx,
+                 uint32_t gy, uint32_t gz);
+int vkt_grid_1d(uint64_t n, uint32_t* groups, uint32_t* stride);   /* vk.h:64, ffi.rs:150-162 */
+int vkt_has_float64(void);                                         /* vk.h:65, ffi.rs:164-168 */
+uint32_t vkt_vendor_id(void);                                      /* vk.h:66, ffi.rs:170-174 (0x1002) */
+uint32_t vkt_capabilities(void);                                   /* vk.h:67, ffi.rs:190-206 (Feature bits, vk.h:92-101) */
+uint32_t vkt_kernel_subgroup_size(const char* name);               /* vk.h:68, ffi.rs:176-188 (64 for this path's kernels) */
+
+/* ---------------------------------------------------------------- HIP additions */
+
+/* Blocking transfers, ordered after all queued work (the reference memcpy()s through
+ * VktAlloc.host after vkt_synchronize(): backend.cpp:692-699,781-788). */
+int vkt_copy_to_device(uint64_t dst_address, const void* src, uint64_t nbytes);
+int vkt_copy_to_host(void* dst, uint64_t src_address, uint64_t nbytes);
+/* Queued (asynchronous, in order) device copy and byte fill. */
+int vkt_copy_on_device(uint64_t dst_address, uint64_t src_address, uint64_t nbytes);
+int vkt_fill(uint64_t dst_address, uint8_t value, uint64_t nbytes);
+
+/* Device facts for rooflines and planning. */
+typedef struct VktDeviceInfo {
+  char name[64];      /* gcnArchName, e.g. "gfx950:sramecc+:xnack-" */
+  uint32_t compute_units;
+  uint32_t clock_khz; /* maximum engine clock */
+  uint32_t mem_clock_khz;
+  uint32_t mem_bus_bits;
+  uint64_t hbm_bytes;
+  uint32_t lds_bytes_per_block;
+  uint32_t l2_bytes;
+} VktDeviceInfo;
+int vkt_device_info(VktDeviceInfo* out);
+
+/* Timing on the stream the kernels run on (HIP events). */
+int vkt_event_create(void** event);
+int vkt_event_record(void* event);
+int vkt_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop` */
+void vkt_event_destroy(void* event);
+
+uint64_t vkt_dispatch_count(void); /* kernels queued so far (reference pyvk/src/lib.rs:112-116) */
+void vkt_shutdown(void);           /* releases the device; later vkt_free calls are no-ops */
+
+/* Bytes of the compact int4 side-car that "qmm4c_pack" writes for an [N,K] weight with
+ * blocks of `bs` (0 if the shape has no compact form). */
+uint64_t vkt_qmm4c_bytes(uint32_t n, uint32_t k, uint32_t bs);
+/* Bytes of the activation scratch (`q` of Q4CParams) for m rows of k values. */
+uint64_t vkt_qmm4c_q_bytes(uint32_t m, uint32_t k);
+
+/* ---------------------------------------------------------------- parameter blocks */
+
+/* "qmm8_f32" | "qmm8_f16" | "qmm8_bf16", spec {ROWS}: C = A @ (B * scales).T
+ * (quant.cpp:31-37, qmm8.slang:21-33).  56 bytes. */
+typedef struct Q8Params {
+  uint64_t a, b, scales, c; /* A [m,k] (row stride a_sm, a_sk must be 1), B int8 [n,k], scales [n], C [m,n] */
+  uint32_t m, n, k;
+  int32_t a_sm, a_sk; /* in elements */
+  uint32_t pad;
+} Q8Params;
+
+/* "qmm4_f32" | "qmm4_bf16", spec {PHASE, GROUPWISE} (quant.cpp:39-43, qmm4.slang:34-47).
+ * PHASE 0 quantises the rows of inp into q (int32 [m,k]) and rows ([m,2]: bits of
+ * 1/scale, -zero_point); PHASE 1 multiplies with the float32-expanded packed weights.
+ * 64 bytes. */
+typedef struct Q4Params {
+  uint64_t inp, q, rows, packed, out;
+  uint32_t m, n, k, bs, has_bias, pad;
+} Q4Params;
+
+/* "qmm4c_pack", spec {}: packed float32 vector -> compact side-car (nibbles, scales,
+ * bias, per-block nibble sums) laid out for the streaming kernels. */
+typedef struct Q4PackParams {
+  uint64_t packed, compact;
+  uint32_t n, k, bs, has_bias;
+} Q4PackParams;
+
+/* "qmm4c_f32" | "qmm4c_bf16", spec {PHASE, GROUPWISE}: as qmm4 but PHASE 0 writes int8
+ * activations (+ per-block sums) into q (vkt_qmm4c_q_bytes) and PHASE 1 streams the
+ * compact side-car.  Results are bit-identical to qmm4. */
+typedef struct Q4CParams {
+  uint64_t inp, q, rows, compact, out;
+  uint32_t m, n, k, bs, has_bias, pad;
+} Q4CParams;
+
+/* "fp8mm", spec {}: out = cast((f32(A)*sa) @ (f32(B)*sb) + bias) [* 1/scale_result]
+ * (quant.cpp:279-300 fused into one kernel).  A: fp8 [m,k] row-major (lda bytes);
+ * B: fp8, column-major, i.e. [n,k] rows ldb bytes apart.  104 bytes. */
+typedef struct F8Params {
+  uint64_t a, b, scale_a, scale_b, bias, scale_result, out; /* bias / scale_result may be 0 */
+  uint32_t m, n, k;
+  uint32_t lda, ldb, ldo;  /* row strides in elements */
+  uint32_t fmt_a, fmt_b;   /* VKT_E4M3 | VKT_E5M2 */
+  uint32_t out_dtype;      /* VKT_F32 | VKT_F16 | VKT_BF16 | VKT_E4M3 | VKT_E5M2 */
+  uint32_t bias_dtype;     /* VKT_F32 | VKT_F16 | VKT_BF16 */
+  uint32_t rowwise;        /* 0: one scale each; 1: scale_a [m], scale_b [n] */
+  uint32_t pad;
+} F8Params;
+
+enum { VKT_F32 = 0, VKT_F16 = 1, VKT_BF16 = 2, VKT_E4M3 = 3, VKT_E5M2 = 4 };
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VKT_H */

@@ -1,0 +1,113 @@
+"""Runs the quantized-matmul kernels through the C ABI (vkt_alloc / vkt_copy_* /
+vkt_dispatch) on numpy storage arrays, the way the reference's C++ op layer drives its
+runtime (crates/pyvk/csrc/quant.cpp).  GPU tests only."""
+import numpy as np
+
+import oracle
+from torch_vulkan_amd import abi
+
+_NP = {oracle.F32: np.float32, oracle.F16: np.uint16, oracle.BF16: np.uint16, oracle.E4M3: np.uint8,
+       oracle.E5M2: np.uint8}
+
+
+def qmm8(a, odt, b, s, variant=0, row_step=1):
+    """_weight_int8pack_mm.  a: storage array [M_total,K]; rows taken every `row_step`
+    (a strided A as in a[::2]); returns the storage array [M,N]."""
+    a = np.ascontiguousarray(a)
+    b = np.ascontiguousarray(b, dtype=np.int8)
+    s = np.ascontiguousarray(s)
+    k, n = a.shape[1], b.shape[0]
+    m = (a.shape[0] + row_step - 1) // row_step
+    da, db, ds = abi.Buffer.from_numpy(a), abi.Buffer.from_numpy(b), abi.Buffer.from_numpy(s)
+    dc = abi.Buffer(max(m * n * a.itemsize, 1))
+    p = abi.Q8Params(a=da.address, b=db.address, scales=ds.address, c=dc.address, m=m, n=n, k=k, a_sm=k * row_step,
+                     a_sk=1)
+    # the reference's launch: ROWS = M for M <= 8, else the tile grid (quant.cpp:86-118)
+    spec = [m if m <= 8 else 0, variant]
+    grid = ((n + 7) // 8,) if m <= 8 else ((n + 63) // 64, (m + 63) // 64)
+    if m and n:
+        abi.dispatch("qmm8_" + abi.SUFFIX[odt], spec, p, grid)
+    return dc.to_numpy(_NP[odt], (m, n))
+
+
+def q4_reference_layout(x, odt, packed, bs, k, n, want_intermediates=False):
+    """_dyn_quant_matmul_4bit through the reference's own parameter block and buffers
+    ("qmm4_*": int32 q, float32-expanded packed vector; quant.cpp:178-202)."""
+    x = np.ascontiguousarray(x)
+    packed = np.ascontiguousarray(packed, dtype=np.float32)
+    m = x.shape[0]
+    dx, dp = abi.Buffer.from_numpy(x), abi.Buffer.from_numpy(packed)
+    dq, dr = abi.Buffer(max(m * k * 4, 1)), abi.Buffer(max(m * 8, 1))
+    do = abi.Buffer(max(m * n * x.itemsize, 1))
+    wcount, nscale = n * k // 2, n * (k // bs)
+    has_bias = int(packed.size - (wcount + nscale) != 0)
+    p = abi.Q4Params(inp=dx.address, q=dq.address, rows=dr.address, packed=dp.address, out=do.address, m=m, n=n, k=k,
+                     bs=bs, has_bias=has_bias)
+    g = int(bs != k)
+    name = "qmm4_" + abi.SUFFIX[odt]
+    if m and n:
+        abi.dispatch(name, [0, g], p, (m,))
+        abi.dispatch(name, [1, g], p, ((n + 31) // 32, (m + 7) // 8))
+    out = do.to_numpy(_NP[odt], (m, n))
+    if want_intermediates:
+        rows = dr.to_numpy(np.uint32, (m, 2))
+        return out, dq.to_numpy(np.int32, (m, k)), rows[:, 0].view(np.float32), rows[:, 1].view(np.int32)
+    return out
+
+
+class CompactWeights:
+    """The compact side-car of a packed float32 vector ("qmm4c_pack"), built once."""
+
+    def __init__(self, packed, bs, k, n):
+        packed = np.ascontiguousarray(packed, dtype=np.float32)
+        nbytes = abi.lib().vkt_qmm4c_bytes(n, k, bs)
+        assert nbytes, "no compact form"
+        self.n, self.k, self.bs = n, k, bs
+        self.has_bias = int(packed.size - (n * k // 2 + n * (k // bs)) != 0)
+        dp = abi.Buffer.from_numpy(packed)
+        self.buf = abi.Buffer(nbytes)
+        p = abi.Q4PackParams(packed=dp.address, compact=self.buf.address, n=n, k=k, bs=bs, has_bias=self.has_bias)
+        abi.dispatch("qmm4c_pack", [], p)
+        abi.synchronize()
+        dp.free()
+
+
+def q4_compact(x, odt, cw, variant=0):
+    """_dyn_quant_matmul_4bit through the streaming path ("qmm4c_*")."""
+    x = np.ascontiguousarray(x)
+    m, n, k, bs = x.shape[0], cw.n, cw.k, cw.bs
+    dx = abi.Buffer.from_numpy(x)
+    dq = abi.Buffer(max(abi.lib().vkt_qmm4c_q_bytes(m, k), 1))
+    dr = abi.Buffer(max(m * 8, 1))
+    do = abi.Buffer(max(m * n * x.itemsize, 1))
+    p = abi.Q4CParams(inp=dx.address, q=dq.address, rows=dr.address, compact=cw.buf.address, out=do.address, m=m, n=n,
+                      k=k, bs=bs, has_bias=cw.has_bias)
+    g = int(bs != k)
+    name = "qmm4c_" + abi.SUFFIX[odt]
+    if m and n:
+        abi.dispatch(name, [0, g, variant], p, (m,))
+        abi.dispatch(name, [1, g, variant], p, ((n + 31) // 32, (m + 7) // 8))
+    return do.to_numpy(_NP[odt], (m, n))
+
+
+def scaled_mm(a, fmt_a, bt, fmt_b, sa, sb, rowwise, bias=None, bias_dtype=oracle.F32, scale_result=None,
+              out_dtype=oracle.BF16, variant=0):
+    """_scaled_mm ("fp8mm").  a: uint8 codes [M,K]; bt: uint8 codes [N,K] (mat2 column-major)."""
+    a = np.ascontiguousarray(a, dtype=np.uint8)
+    bt = np.ascontiguousarray(bt, dtype=np.uint8)
+    (m, k), n = a.shape, bt.shape[0]
+    sa = np.ascontiguousarray(np.asarray(sa, np.float32).reshape(-1))
+    sb = np.ascontiguousarray(np.asarray(sb, np.float32).reshape(-1))
+    da, db = abi.Buffer.from_numpy(a), abi.Buffer.from_numpy(bt)
+    dsa, dsb = abi.Buffer.from_numpy(sa), abi.Buffer.from_numpy(sb)
+    dbias = None if bias is None else abi.Buffer.from_numpy(np.ascontiguousarray(bias))
+    dsr = None if scale_result is None else abi.Buffer.from_numpy(np.asarray([scale_result], np.float32))
+    item = np.dtype(_NP[out_dtype]).itemsize
+    do = abi.Buffer(max(m * n * item, 1))
+    p = abi.F8Params(a=da.address, b=db.address, scale_a=dsa.address, scale_b=dsb.address,
+                     bias=dbias.address if dbias else 0, scale_result=dsr.address if dsr else 0, out=do.address, m=m,
+                     n=n, k=k, lda=k, ldb=k, ldo=n, fmt_a=fmt_a, fmt_b=fmt_b, out_dtype=out_dtype,
+                     bias_dtype=bias_dtype, rowwise=int(bool(rowwise)))
+    if m and n:
+        abi.dispatch("fp8mm", [variant], p)
+    return do.to_numpy(_NP[out_dtype], (m, n))

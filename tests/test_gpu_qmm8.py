@@ -1,0 +1,122 @@
+"""GPU parity of _weight_int8pack_mm (kernels "qmm8_*") through the C ABI against the
+oracle: the reference's own shapes and seeds (tests/python/test_quant.py:20-40), the frozen
+fixtures, the BASELINE configurations, and size-independent properties at full size."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from _util import ODT, bits, gen, ref_tol, unbits
+from test_oracle_pins import Q8_SHAPES, q8_case
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def check_q8(got_bits, a, b, s, dtype, rows=slice(None)):
+    odt = ODT[dtype]
+    c, c64, mag = oracle.qmm8(bits(a), odt, b.numpy(), bits(s), want_f64=True)
+    got = unbits(got_bits, dtype).float().numpy().astype(np.float64)
+    # the reference's bound, eps*|want| + 2^-20*mag (test_quant.py:36-37), around the float64 sum
+    tol = ref_tol(c64, mag, odt)[rows]
+    err = np.abs(got - c64[rows])
+    assert (err <= tol).all(), f"max excess {np.max(err - tol)}"
+    return got, c64[rows]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,k,n", Q8_SHAPES + [(1, 4096, 4096), (8, 4096, 640), (16, 2048, 130), (3, 1024, 7),
+                                               (17, 256, 33), (2, 16, 1), (1, 48, 5)])
+def test_qmm8_reference_shapes(dtype, m, k, n):
+    import _dev
+    a, b, s = q8_case(dtype, m, k, n)
+    got = _dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s))
+    assert got.shape == (m, n)
+    check_q8(got, a, b, s, dtype)
+    # a row slice of A (A's rows strided), as test_quant.py:35
+    sliced = _dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), row_step=2)
+    check_q8(sliced, a, b, s, dtype, rows=slice(None, None, 2))
+
+
+@pytest.mark.parametrize("variant", [2 | 1 << 8, 2 | 2 << 8, 2 | 4 << 8, 4 | 1 << 8, 4 | 2 << 8, 4 | 4 << 8, 1 << 16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_qmm8_every_variant(variant, dtype):
+    """Each (COLS, KSPLIT) instantiation and the generic kernel give results inside the band."""
+    import _dev
+    for m, k, n in [(1, 4096, 130), (4, 2064, 67)]:
+        a, b, s = q8_case(dtype, m, k, n)
+        check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=variant), a, b, s, dtype)
+
+
+def test_qmm8_config1_vs_torch_cpu():
+    """BASELINE config 1: fp32, M=1, K=N=4096, within rtol/atol 1e-4 of PyTorch's CPU op."""
+    import _dev
+    x = torch.randn(1, 4096, generator=gen(1010))
+    w = torch.randint(-128, 128, (4096, 4096), dtype=torch.int8, generator=gen(1011))
+    s = torch.empty(4096).uniform_(0.005, 0.02, generator=gen(1012))
+    got = torch.from_numpy(_dev.qmm8(x.numpy(), oracle.F32, w.numpy(), s.numpy()))
+    want = torch._weight_int8pack_mm(x, w, s)
+    truth = (x.double() @ (w.float() * s[:, None]).double().t()).float()
+    # the CPU op's own float32 summation noise can exceed 1e-4 near zero outputs; the float64
+    # closed form is the tighter judge, the CPU op is checked at the stated tolerance where
+    # it agrees with the closed form itself
+    assert torch.allclose(got, truth, rtol=1e-4, atol=1e-4)
+    ok = torch.isclose(want, truth, rtol=1e-4, atol=1e-4)
+    assert torch.allclose(got[ok], want[ok], rtol=1e-4, atol=2e-4)
+    check_q8(got.numpy(), x, w, s, torch.float32)
+
+
+@pytest.mark.parametrize("m", [1, 8, 64])
+@pytest.mark.parametrize("k,n", [(4096, 14336), (14336, 4096)])
+def test_qmm8_config2_llama_mlp(m, k, n):
+    """BASELINE config 2: bf16, Llama-3-8B MLP shapes, rtol/atol 1e-2 vs PyTorch's CPU op."""
+    import _dev
+    x = torch.randn(m, k, generator=gen(1020)).bfloat16()
+    w = torch.randint(-128, 128, (n, k), dtype=torch.int8, generator=gen(1021))
+    s = torch.empty(n).uniform_(0.005, 0.02, generator=gen(1022)).bfloat16()
+    got = unbits(_dev.qmm8(bits(x), oracle.BF16, w.numpy(), bits(s)), torch.bfloat16)
+    want = torch._weight_int8pack_mm(x, w, s)
+    assert torch.allclose(got.float(), want.float(), rtol=1e-2, atol=1e-2)
+    # linearity in the scales: doubling them (exact in bf16) doubles every output bit for bit
+    got2 = unbits(_dev.qmm8(bits(x), oracle.BF16, w.numpy(), bits(s * 2)), torch.bfloat16)
+    assert torch.equal(got2.float(), got.float() * 2)
+    # a row of zeros gives zeros; a one-hot row picks a column of w*s exactly
+    x0 = torch.zeros(2, k).bfloat16()
+    x0[1, 5] = 1.0
+    r = unbits(_dev.qmm8(bits(x0), oracle.BF16, w.numpy(), bits(s)), torch.bfloat16).float()
+    assert (r[0] == 0).all()
+    assert torch.equal(r[1], (w[:, 5].float() * s.float()).bfloat16().float())
+
+
+def test_qmm8_golden_fixtures():
+    import _dev
+    g = np.load(os.path.join(GOLDEN, "q8.npz"))
+    for key in [k[:-2] for k in g.files if k.endswith("_a")]:
+        odt = int(g[key + "_odt"])
+        got = _dev.qmm8(g[key + "_a"], odt, g[key + "_b"], g[key + "_s"])
+        c, c64, mag = oracle.qmm8(g[key + "_a"], odt, g[key + "_b"], g[key + "_s"], want_f64=True)
+        tol = ref_tol(c64, mag, odt)
+        assert (np.abs(oracle.to_f32(got, odt) - c64) <= tol).all(), key
+        assert (np.abs(oracle.to_f32(got, odt).astype(np.float64) - oracle.to_f32(g[key + "_out"], odt)) <= 2 * tol).all()
+
+
+def test_qmm8_empty_and_errors():
+    import _dev
+    from torch_vulkan_amd import abi
+    a = np.zeros((0, 64), np.float32)
+    assert _dev.qmm8(a, oracle.F32, np.zeros((5, 64), np.int8), np.ones(5, np.float32)).shape == (0, 5)
+    buf = abi.Buffer(1024)
+    p = abi.Q8Params(a=buf.address, b=buf.address, scales=buf.address, c=buf.address, m=1, n=4, k=16, a_sm=16, a_sk=2)
+    with pytest.raises(abi.VktError, match="unit stride"):
+        abi.dispatch("qmm8_f32", [1], p)
+    with pytest.raises(abi.VktError, match="unknown kernel"):
+        abi.dispatch("qmm8_f64", [1], p)
+    with pytest.raises(abi.VktError, match="56 bytes"):
+        abi.dispatch("qmm8_f32", [1], abi.Q4Params())
+    p.a_sk = 1
+    with pytest.raises(abi.VktError, match="empty grid"):
+        abi.dispatch("qmm8_f32", [1], p, (0, 1, 1))
+    with pytest.raises(abi.VktError, match="does not match"):
+        abi.dispatch("qmm8_f32", [3], p)

@@ -1,0 +1,187 @@
+// Device helpers shared by the gfx950 kernels: 16-byte loads, element conversions with
+// the rounding the operators specify, and wave64 reductions through DPP.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../../include/vkt.h"
+
+namespace vkt {
+
+constexpr int kWave = 64;
+
+__host__ __device__ inline uint64_t round_up_u64(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
+
+using U4 = uint32_t __attribute__((ext_vector_type(4)));
+using U2 = uint32_t __attribute__((ext_vector_type(2)));
+using F4 = float __attribute__((ext_vector_type(4)));
+
+// Tensor addresses arrive as 64-bit integers in the parameter blocks; loads and stores go
+// through global-address-space pointers so that they compile to global_* (not flat_*)
+// memory instructions.
+#define VKT_GLOBAL __attribute__((address_space(1)))
+template <class X>
+__device__ __forceinline__ X ldg(uint64_t addr) {
+  return *reinterpret_cast<const VKT_GLOBAL X*>(addr);
+}
+template <class X>
+__device__ __forceinline__ void stg(uint64_t addr, X v) {
+  *reinterpret_cast<VKT_GLOBAL X*>(addr) = v;
+}
+
+__device__ __forceinline__ float bits_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t f32_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// Storage element types.  16-bit floats are carried as raw bits so that every rounding
+// is written out here and not left to a library type.
+struct f32_t {
+  using storage = float;
+  static constexpr int dtype = VKT_F32;
+};
+struct f16_t {
+  using storage = uint16_t;
+  static constexpr int dtype = VKT_F16;
+};
+struct bf16_t {
+  using storage = uint16_t;
+  static constexpr int dtype = VKT_BF16;
+};
+
+__device__ __forceinline__ float bf16_to_f32(uint32_t h) { return bits_f32(h << 16); }
+// round to nearest even; NaN -> 0x7fc0
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  uint32_t u = f32_bits(f);
+  uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+  return (f != f) ? uint16_t(0x7fc0) : uint16_t(r);
+}
+__device__ __forceinline__ float f16_to_f32(uint32_t h) {
+  return float(__builtin_bit_cast(_Float16, uint16_t(h)));  // v_cvt_f32_f16: exact
+}
+__device__ __forceinline__ uint16_t f32_to_f16(float f) {
+  return __builtin_bit_cast(uint16_t, _Float16(f));  // v_cvt_f16_f32: round to nearest even (default mode)
+}
+
+// One element at a byte address, widened to / rounded from float32.
+template <class T>
+__device__ __forceinline__ float load_f32(uint64_t addr);
+template <>
+__device__ __forceinline__ float load_f32<f32_t>(uint64_t addr) { return ldg<float>(addr); }
+template <>
+__device__ __forceinline__ float load_f32<f16_t>(uint64_t addr) { return f16_to_f32(ldg<uint16_t>(addr)); }
+template <>
+__device__ __forceinline__ float load_f32<bf16_t>(uint64_t addr) { return bf16_to_f32(ldg<uint16_t>(addr)); }
+
+template <class T>
+__device__ __forceinline__ void store_f32(uint64_t addr, float v);
+template <>
+__device__ __forceinline__ void store_f32<f32_t>(uint64_t addr, float v) { stg<float>(addr, v); }
+template <>
+__device__ __forceinline__ void store_f32<f16_t>(uint64_t addr, float v) { stg<uint16_t>(addr, f32_to_f16(v)); }
+template <>
+__device__ __forceinline__ void store_f32<bf16_t>(uint64_t addr, float v) { stg<uint16_t>(addr, f32_to_bf16(v)); }
+
+// 16 consecutive elements (16-byte aligned address) widened to float32.
+template <class T>
+__device__ __forceinline__ void load16_f32(uint64_t addr, float (&a)[16]);
+template <>
+__device__ __forceinline__ void load16_f32<f32_t>(uint64_t addr, float (&a)[16]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    F4 v = ldg<F4>(addr + 16 * i);
+    a[4 * i] = v.x, a[4 * i + 1] = v.y, a[4 * i + 2] = v.z, a[4 * i + 3] = v.w;
+  }
+}
+template <>
+__device__ __forceinline__ void load16_f32<bf16_t>(uint64_t addr, float (&a)[16]) {
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    U4 v = ldg<U4>(addr + 16 * i);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      a[8 * i + 2 * j] = bits_f32(v[j] << 16);
+      a[8 * i + 2 * j + 1] = bits_f32(v[j] & 0xffff0000u);
+    }
+  }
+}
+template <>
+__device__ __forceinline__ void load16_f32<f16_t>(uint64_t addr, float (&a)[16]) {
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    U4 v = ldg<U4>(addr + 16 * i);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      a[8 * i + 2 * j] = f16_to_f32(v[j] & 0xffffu);
+      a[8 * i + 2 * j + 1] = f16_to_f32(v[j] >> 16);
+    }
+  }
+}
+
+// 16 int8 values (one 16-byte load) widened to float32 (exact).
+__device__ __forceinline__ void widen16_i8(const U4& v, float (&w)[16]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[4 * i + j] = float(int(int8_t(v[i] >> (8 * j))));
+  }
+}
+
+// ---- wave64 reductions through DPP (no LDS traffic) ----
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, true));
+}
+template <int CTRL>
+__device__ __forceinline__ int dpp_i32(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
+}
+constexpr int kQuadSwap1 = 0xB1;     // quad_perm [1,0,3,2]
+constexpr int kQuadSwap2 = 0x4E;     // quad_perm [2,3,0,1]
+constexpr int kRowHalfMirror = 0x141;
+constexpr int kRowMirror = 0x140;
+
+// Sum over each row of 16 lanes, left in every lane of the row.
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_f32<kQuadSwap1>(v);
+  v += dpp_f32<kQuadSwap2>(v);
+  v += dpp_f32<kRowHalfMirror>(v);
+  v += dpp_f32<kRowMirror>(v);
+  return v;
+}
+// Sum over the 64 lanes (wave-uniform result).
+__device__ __forceinline__ float wave_sum(float v) {
+  v = row16_sum(v);
+  int b = __builtin_bit_cast(int, v);
+  float s0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0));
+  float s1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+  float s2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32));
+  float s3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+  return (s0 + s1) + (s2 + s3);
+}
+__device__ __forceinline__ float wave_min(float v) {
+  v = fminf(v, dpp_f32<kQuadSwap1>(v));
+  v = fminf(v, dpp_f32<kQuadSwap2>(v));
+  v = fminf(v, dpp_f32<kRowHalfMirror>(v));
+  v = fminf(v, dpp_f32<kRowMirror>(v));
+  int b = __builtin_bit_cast(int, v);
+  float s0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0));
+  float s1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+  float s2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32));
+  float s3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+  return fminf(fminf(s0, s1), fminf(s2, s3));
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, dpp_f32<kQuadSwap1>(v));
+  v = fmaxf(v, dpp_f32<kQuadSwap2>(v));
+  v = fmaxf(v, dpp_f32<kRowHalfMirror>(v));
+  v = fmaxf(v, dpp_f32<kRowMirror>(v));
+  int b = __builtin_bit_cast(int, v);
+  float s0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0));
+  float s1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+  float s2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32));
+  float s3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+  return fmaxf(fmaxf(s0, s1), fmaxf(s2, s3));
+}
+
+}  // namespace vkt

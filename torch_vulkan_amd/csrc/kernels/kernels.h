@@ -1,0 +1,33 @@
+// Launchers of the gfx950 kernels.  Each validates what its kernels assume about
+// shapes, strides and alignment before launching (a wrong launch is a GPU fault, not an
+// error code), queues its kernels on `stream` and returns 0, or sets *err and returns -1.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <string>
+
+#include "../../../include/vkt.h"
+
+namespace vkt {
+
+struct Machine {
+  int compute_units = 256;
+};
+
+// spec[1] of the qmm8 kernels: 0 = planned by the library; otherwise an explicit
+// variant id (COLS | KSPLIT << 8 | FORCE_GENERIC << 16) used by tuning sweeps.
+int launch_qmm8(const Q8Params& p, int dtype, uint32_t variant, const Machine& mc, hipStream_t stream,
+                std::string* err);
+int launch_qmm4(const Q4Params& p, int dtype, uint32_t phase, uint32_t groupwise, const Machine& mc,
+                hipStream_t stream, std::string* err);
+int launch_qmm4c_pack(const Q4PackParams& p, const Machine& mc, hipStream_t stream, std::string* err);
+int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwise, uint32_t variant,
+                 const Machine& mc, hipStream_t stream, std::string* err);
+int launch_fp8mm(const F8Params& p, uint32_t variant, const Machine& mc, hipStream_t stream, std::string* err);
+int launch_fill(uint64_t dst, uint8_t value, uint64_t nbytes, hipStream_t stream, std::string* err);
+
+uint64_t qmm4c_bytes(uint32_t n, uint32_t k, uint32_t bs);
+uint64_t qmm4c_q_bytes(uint32_t m, uint32_t k);
+
+}  // namespace vkt

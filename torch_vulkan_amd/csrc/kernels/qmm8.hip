@@ -1,0 +1,247 @@
+// aten::_weight_int8pack_mm on gfx950:  C[m,n] = round_T( scale[n] * sum_k A[m,k] * B[n,k] )
+// for A [M,K] float32/float16/bfloat16 (unit stride along K), B int8 [N,K] contiguous,
+// per-output-channel scales [N] in A's dtype, C [M,N] in A's dtype.
+// Replaces the reference's crates/vkcore/shaders/qmm8.slang (GEMV :78-111, tiles :113-173)
+// behind the same parameter block (crates/pyvk/csrc/quant.cpp:31-37).
+//
+// The op is a stream over the N*K weight bytes (HBM-bound up to M in the tens), so the
+// kernels are built around that stream:
+//   qmm8_gemv    M <= 16.  A wave owns COLS weight rows and walks K with one 16-byte
+//                load per lane per row (1 KiB contiguous per wave per load, several in
+//                flight), widens int8 -> float32 in registers (exact), accumulates every
+//                row of A against it in float32 and reduces across the wave with DPP.
+//                KSPLIT waves of a workgroup share a column group when N alone would
+//                leave the machine's 1024 SIMDs short of work.  The per-channel scale is
+//                applied once to the finished sum (the reference scales each weight; the
+//                two differ by one float32 rounding, inside its test's tolerance).
+//   qmm8_generic any shape, stride or alignment (K not a multiple of 16, unaligned rows):
+//                a wave per output column, byte loads.
+// Rows beyond 16 are served by the launcher in chunks (the weight stream is then re-read
+// per chunk) until the MFMA tile kernel takes them.
+#include "common.h"
+#include "kernels.h"
+
+namespace vkt {
+namespace {
+
+template <class T, int ROWS, int COLS, int KSPLIT>
+__global__ __launch_bounds__(256) void qmm8_gemv(Q8Params p) {
+  constexpr int WAVES = 4, GROUPS = WAVES / KSPLIT;
+  constexpr uint64_t item = sizeof(typename T::storage);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int grp = wave / KSPLIT, ks = wave % KSPLIT;
+  const uint32_t n0 = (blockIdx.x * GROUPS + grp) * COLS;
+
+  float acc[ROWS][COLS];
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) acc[r][c] = 0.0f;
+
+  // rows of B this wave reads (clamped: the tail group re-reads the last row, masked at the store)
+  uint64_t brow[COLS];
+#pragma unroll
+  for (int c = 0; c < COLS; ++c) {
+    uint32_t n = n0 + c < p.n ? n0 + c : p.n - 1;
+    brow[c] = p.b + uint64_t(n) * p.k;
+  }
+  uint64_t arow[ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) {
+    uint32_t m = uint32_t(r) < p.m ? uint32_t(r) : p.m - 1;
+    arow[r] = p.a + uint64_t(int64_t(m) * p.a_sm * int64_t(item));
+  }
+
+  for (uint32_t k = (ks * 64 + lane) * 16; k < p.k; k += 1024 * KSPLIT) {
+    U4 wv[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) wv[c] = ldg<U4>(brow[c] + k);
+    float w[COLS][16];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) widen16_i8(wv[c], w[c]);
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      float a[16];
+      load16_f32<T>(arow[r] + k * item, a);
+#pragma unroll
+      for (int c = 0; c < COLS; ++c)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[r][c] = fmaf(a[i], w[c][i], acc[r][c]);
+    }
+  }
+
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) acc[r][c] = wave_sum(acc[r][c]);
+
+  __shared__ float part[WAVES][ROWS * COLS];
+  if constexpr (KSPLIT > 1) {
+    if (lane == 0) {
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) part[wave][r * COLS + c] = acc[r][c];
+    }
+    __syncthreads();
+    if (ks != 0) return;
+  }
+  // lane (r, c) of the group's first wave finishes output (r, n0 + c)
+  if (lane < ROWS * COLS) {
+    const int r = lane / COLS, c = lane % COLS;
+    float sum = 0.0f;
+    // select acc[r][c] without dynamic register indexing
+#pragma unroll
+    for (int rr = 0; rr < ROWS; ++rr)
+#pragma unroll
+      for (int cc = 0; cc < COLS; ++cc)
+        if (rr == r && cc == c) sum = acc[rr][cc];
+    if constexpr (KSPLIT > 1) {
+      sum = part[wave][lane];
+#pragma unroll
+      for (int s = 1; s < KSPLIT; ++s) sum += part[wave + s][lane];
+    }
+    const uint32_t n = n0 + c;
+    if (uint32_t(r) < p.m && n < p.n) {
+      const float scale = load_f32<T>(p.scales + n * item);
+      store_f32<T>(p.c + (uint64_t(r) * p.n + n) * item, sum * scale);
+    }
+  }
+}
+
+// Any shape: a wave per output column, lanes strided along k with element loads, rows of
+// A in chunks of 8.
+template <class T>
+__global__ __launch_bounds__(256) void qmm8_generic(Q8Params p) {
+  constexpr uint64_t item = sizeof(typename T::storage);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t n = blockIdx.x * 4 + wave;
+  if (n >= p.n) return;
+  const uint64_t brow = p.b + uint64_t(n) * p.k;
+  const float scale = load_f32<T>(p.scales + n * item);
+  for (uint32_t m0 = blockIdx.y * 8; m0 < p.m; m0 += gridDim.y * 8) {
+    float acc[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) acc[r] = 0.0f;
+    for (uint32_t k = lane; k < p.k; k += 64) {
+      const float w = float(int(ldg<int8_t>(brow + k)));
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        const uint32_t m = m0 + r < p.m ? m0 + r : p.m - 1;
+        acc[r] = fmaf(load_f32<T>(p.a + uint64_t((int64_t(m) * p.a_sm + k) * int64_t(item))), w, acc[r]);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const float sum = wave_sum(acc[r]);
+      if (lane == 0 && m0 + r < p.m) store_f32<T>(p.c + (uint64_t(m0 + r) * p.n + n) * item, sum * scale);
+    }
+  }
+}
+
+template <class T, int ROWS, int COLS, int KSPLIT>
+void launch_gemv(const Q8Params& p, hipStream_t stream) {
+  constexpr int per_wg = COLS * (4 / KSPLIT);
+  const uint32_t grid = (p.n + per_wg - 1) / per_wg;
+  hipLaunchKernelGGL((qmm8_gemv<T, ROWS, COLS, KSPLIT>), dim3(grid), dim3(256), 0, stream, p);
+}
+
+template <class T, int ROWS, int COLS>
+bool launch_gemv_ks(const Q8Params& p, int ksplit, hipStream_t stream) {
+  switch (ksplit) {
+    case 1: launch_gemv<T, ROWS, COLS, 1>(p, stream); return true;
+    case 2: launch_gemv<T, ROWS, COLS, 2>(p, stream); return true;
+    case 4: launch_gemv<T, ROWS, COLS, 4>(p, stream); return true;
+  }
+  return false;
+}
+
+template <class T, int ROWS, int CA, int CB>
+bool launch_gemv_cols(const Q8Params& p, int cols, int ksplit, hipStream_t stream) {
+  if (cols == CA) return launch_gemv_ks<T, ROWS, CA>(p, ksplit, stream);
+  if (cols == CB) return launch_gemv_ks<T, ROWS, CB>(p, ksplit, stream);
+  return false;
+}
+
+// Picks COLS and KSPLIT so that the grid puts at least ~2 waves on each of the machine's
+// SIMDs while each wave keeps several 16-byte loads in flight.
+void plan_gemv(const Q8Params& p, int rows, const Machine& mc, int* cols, int* ksplit) {
+  const int64_t simds = int64_t(mc.compute_units) * 4;
+  const int wide = rows <= 4 ? 4 : 2, narrow = rows <= 4 ? 2 : 1;
+  *cols = (int64_t(p.n) / wide >= 2 * simds) ? wide : narrow;
+  int ks = 1;
+  while (ks < 4 && int64_t(p.n) / *cols * ks < 2 * simds && p.k >= 2048u * ks) ks *= 2;
+  *ksplit = ks;
+}
+
+template <class T>
+int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipStream_t stream, std::string* err) {
+  const size_t item = sizeof(typename T::storage);
+  const bool vector_ok = p0.k % 16 == 0 && p0.a % 16 == 0 && p0.b % 16 == 0 &&
+                         (p0.m == 1 || (int64_t(p0.a_sm) * int64_t(item)) % 16 == 0) && !((variant >> 16) & 1);
+  if (!vector_ok) {
+    const uint32_t gy = p0.m <= 8 ? 1 : (p0.m + 7) / 8 < 64 ? (p0.m + 7) / 8 : 64;
+    hipLaunchKernelGGL((qmm8_generic<T>), dim3((p0.n + 3) / 4, gy), dim3(256), 0, stream, p0);
+    return 0;
+  }
+  for (uint32_t r0 = 0; r0 < p0.m; r0 += 16) {
+    Q8Params p = p0;
+    p.m = p0.m - r0 < 16 ? p0.m - r0 : 16;
+    p.a = p0.a + uint64_t(int64_t(r0) * p0.a_sm * int64_t(item));
+    p.c = p0.c + uint64_t(r0) * p0.n * item;
+    const int rows = p.m <= 1 ? 1 : p.m <= 2 ? 2 : p.m <= 4 ? 4 : p.m <= 8 ? 8 : 16;
+    int cols, ksplit;
+    plan_gemv(p, rows, mc, &cols, &ksplit);
+    if (variant & 0xffff) {
+      cols = variant & 0xff;
+      ksplit = (variant >> 8) & 0xff;
+    }
+    bool ok = false;
+    switch (rows) {
+      case 1: ok = launch_gemv_cols<T, 1, 2, 4>(p, cols, ksplit, stream); break;
+      case 2: ok = launch_gemv_cols<T, 2, 2, 4>(p, cols, ksplit, stream); break;
+      case 4: ok = launch_gemv_cols<T, 4, 2, 4>(p, cols, ksplit, stream); break;
+      case 8: ok = launch_gemv_cols<T, 8, 1, 2>(p, cols, ksplit, stream); break;
+      case 16: ok = launch_gemv_cols<T, 16, 1, 2>(p, cols, ksplit, stream); break;
+    }
+    if (!ok) {
+      *err = "qmm8: no kernel variant COLS=" + std::to_string(cols) + " KSPLIT=" + std::to_string(ksplit) +
+             " for " + std::to_string(rows) + " rows";
+      return -1;
+    }
+  }
+  return 0;
+}
+
+}  // namespace
+
+int launch_qmm8(const Q8Params& p, int dtype, uint32_t variant, const Machine& mc, hipStream_t stream,
+                std::string* err) {
+  if (p.a_sk != 1) {
+    *err = "qmm8: A must have unit stride along k (a_sk == 1)";
+    return -1;
+  }
+  if (p.m == 0 || p.n == 0) return 0;
+  if (p.a == 0 || p.b == 0 || p.scales == 0 || p.c == 0) {
+    *err = "qmm8: null tensor address";
+    return -1;
+  }
+  if (uint64_t(p.n) * p.k >= (1ull << 32) || uint64_t(p.m) * p.n >= (1ull << 32)) {
+    *err = "qmm8: weights or output too large for 32-bit indexing";
+    return -1;
+  }
+  int rc;
+  switch (dtype) {
+    case VKT_F32: rc = launch_qmm8_t<f32_t>(p, variant, mc, stream, err); break;
+    case VKT_F16: rc = launch_qmm8_t<f16_t>(p, variant, mc, stream, err); break;
+    case VKT_BF16: rc = launch_qmm8_t<bf16_t>(p, variant, mc, stream, err); break;
+    default: *err = "qmm8: unsupported dtype"; return -1;
+  }
+  if (rc == 0 && hipGetLastError() != hipSuccess) {
+    *err = "qmm8: kernel launch failed";
+    return -1;
+  }
+  return rc;
+}
+
+}  // namespace vkt
