@@ -1,0 +1,168 @@
+"""GPU parity of _scaled_mm (kernel "fp8mm") through the C ABI against the oracle and
+PyTorch's CPU op: the reference's parametrisation (tests/python/test_quant.py:101-128: every
+mix of e4m3fn / e5m2 operands, five output dtypes, tensor-wise and row-wise scales, bias,
+scale_result), the frozen fixtures, tile-edge shapes, and the BASELINE shapes through
+properties that do not need a full-size CPU product."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from _util import ODT, bits, gen, ref_tol, unbits
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+FLOAT8 = [torch.float8_e4m3fn, torch.float8_e5m2]
+
+
+# The fp8 matrix core adds the 128 products of one instruction in a fixed-point window
+# ~14 bits below the largest product (a hardware property, measured: ~2^-15.3 of sum|a||b| on
+# random data); bfloat16 / float8 outputs take that path, float32 / float16 outputs do not.
+HW_WINDOW = 2.0**-13
+
+
+def on_matrix_cores(odt, variant, k):
+    if variant == 255 or k % 16:
+        return False
+    return variant in (1, 2, 3) or odt in (oracle.BF16, oracle.E4M3, oracle.E5M2)
+
+
+def run_case(m, k, n, fa, fb, out_dtype, rowwise, bias_dtype=None, scale_result=None, variant=0, seed=1, scale=1.0):
+    import _dev
+    a = (torch.randn(m, k, generator=gen(seed)) * scale).to(fa)
+    bt = (torch.randn(n, k, generator=gen(seed + 1)) * scale).to(fb)
+    sa = torch.rand(m, 1, generator=gen(seed + 2)) + 0.5 if rowwise else torch.tensor(1.25)
+    sb = torch.rand(1, n, generator=gen(seed + 3)) + 0.5 if rowwise else torch.tensor(0.75)
+    bias = None if bias_dtype is None else torch.randn(n, generator=gen(seed + 4)).to(bias_dtype)
+    res = out_dtype or fa
+    kw = dict(bias=None if bias is None else bits(bias), bias_dtype=ODT[bias_dtype] if bias is not None else 0,
+              scale_result=scale_result, out_dtype=ODT[res])
+    want, mag = oracle.scaled_mm(bits(a), ODT[fa], bits(bt), ODT[fb], sa.numpy(), sb.numpy(), rowwise, want_mag=True,
+                                 **kw)
+    got = _dev.scaled_mm(bits(a), ODT[fa], bits(bt), ODT[fb], sa.numpy(), sb.numpy(), rowwise, variant=variant, **kw)
+    want_f, got_f = oracle.to_f32(want, ODT[res]).astype(np.float64), oracle.to_f32(got, ODT[res]).astype(np.float64)
+    if scale_result is not None:
+        mag = mag / scale_result
+    tol = ref_tol(want_f, mag, ODT[res])  # eps*|want| + 2^-20*mag, test_quant.py:124-126
+    if on_matrix_cores(ODT[res], variant, k):
+        tol = tol + HW_WINDOW * mag
+    finite = np.isfinite(want_f)
+    assert np.array_equal(np.isfinite(got_f), finite)
+    assert (np.abs(got_f - want_f)[finite] <= tol[finite]).all(), float(np.max((np.abs(got_f - want_f) - tol)[finite]))
+    return a, bt, sa, sb, bias, got_f
+
+
+@pytest.mark.parametrize("fa,fb", [(FLOAT8[0], FLOAT8[0]), (FLOAT8[1], FLOAT8[0]), (FLOAT8[0], FLOAT8[1]),
+                                   (FLOAT8[1], FLOAT8[1])])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32, torch.float16, torch.float8_e4m3fn, None])
+@pytest.mark.parametrize("rowwise", [False, True])
+def test_scaled_mm_reference_cases(fa, fb, out_dtype, rowwise):
+    bias_dtype = torch.bfloat16 if out_dtype == torch.bfloat16 else None
+    sr = 2.0 if out_dtype == torch.float8_e4m3fn else None
+    a, bt, sa, sb, bias, got = run_case(16, 32, 48, fa, fb, out_dtype, rowwise, bias_dtype, sr)
+    if not rowwise:  # torch 2.10's CPU kernel takes per-tensor scales only
+        want = torch._scaled_mm(a, bt.t(), sa, sb, bias=bias, out_dtype=out_dtype,
+                                scale_result=None if sr is None else torch.tensor(sr)).float().numpy()
+        res = ODT[out_dtype or fa]
+        mag = ((a.float() * sa).abs() @ (bt.float() * sb).abs().t()).numpy() / (sr or 1.0)
+        tol = ref_tol(want, mag, res) + (HW_WINDOW * mag if on_matrix_cores(res, 0, 32) else 0)
+        assert (np.abs(got - want) <= tol).all()
+        if res == oracle.BF16:  # the stated bar for bfloat16 outputs
+            assert np.allclose(got, want, rtol=1e-2, atol=1e-2)
+        if res == oracle.F32:
+            assert np.allclose(got, want, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("m,k,n", [(1, 16, 1), (130, 256, 70), (257, 384, 129), (64, 1040, 300), (300, 128, 520),
+                                   (5, 100, 7), (33, 48, 17)])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 255])
+@pytest.mark.parametrize("rowwise", [False, True])
+def test_scaled_mm_tile_edges(m, k, n, variant, rowwise):
+    """Shapes that are not multiples of any tile, K tails (K % 128 != 0, K % 16 != 0 -> the
+    unaligned kernel), every tile variant and the one-thread-per-output kernel (255)."""
+    run_case(m, k, n, FLOAT8[0], FLOAT8[0], torch.bfloat16, rowwise, torch.float32, variant=variant, seed=20)
+    run_case(m, k, n, FLOAT8[1], FLOAT8[0], torch.float32, rowwise, variant=variant, seed=30)
+
+
+def test_scaled_mm_fp8_output_saturation_and_nan():
+    # large products: e4m3fn output overflows to NaN (c10 does not saturate), e5m2 to inf
+    run_case(32, 256, 32, FLOAT8[0], FLOAT8[0], torch.float8_e4m3fn, False, scale=8.0)
+    run_case(32, 256, 32, FLOAT8[0], FLOAT8[0], torch.float8_e5m2, False, scale=30.0, scale_result=0.01)
+
+
+def test_scaled_mm_golden_fixtures():
+    import _dev
+    g = np.load(os.path.join(GOLDEN, "f8.npz"))
+    for key in [k[:-2] for k in g.files if k.endswith("_a")]:
+        fa, fb, odt = (int(v) for v in g[key + "_fmt"])
+        kw = dict(bias=g[key + "_bias"] if key + "_bias" in g else None, bias_dtype=oracle.BF16,
+                  scale_result=float(g[key + "_sr"]) if key + "_sr" in g else None, out_dtype=odt)
+        got = _dev.scaled_mm(g[key + "_a"], fa, g[key + "_bt"], fb, g[key + "_sa"], g[key + "_sb"], False, **kw)
+        _, mag = oracle.scaled_mm(g[key + "_a"], fa, g[key + "_bt"], fb, g[key + "_sa"], g[key + "_sb"], False,
+                                  want_mag=True, **kw)
+        want = oracle.to_f32(g[key + "_out"], odt).astype(np.float64)
+        if key + "_sr" in g:
+            mag = mag / float(g[key + "_sr"])
+        tol = ref_tol(want, mag, odt) + (HW_WINDOW * mag if on_matrix_cores(odt, 0, 32) else 0)
+        assert (np.abs(oracle.to_f32(got, odt) - want) <= tol).all(), key
+
+
+def _sampled_check(a, bt, sa, sb, got, rows, cols, rowwise):
+    """Float64 closed form on a sample of output rows and columns."""
+    af = oracle.fp8_table(oracle.E4M3)[a[rows]].astype(np.float64)
+    bf = oracle.fp8_table(oracle.E4M3)[bt[cols]].astype(np.float64)
+    sa_ = sa.reshape(-1)[rows][:, None] if rowwise else float(sa)
+    sb_ = sb.reshape(-1)[cols][None, :] if rowwise else float(sb)
+    truth = (af @ bf.T) * sa_ * sb_
+    mag = (np.abs(af) @ np.abs(bf).T) * sa_ * sb_
+    sub = oracle.bf16_to_f32(got[np.ix_(rows, cols)]).astype(np.float64)
+    assert (np.abs(sub - truth) <= ref_tol(truth, mag, oracle.BF16) + HW_WINDOW * mag).all()
+    assert np.allclose(sub, truth, rtol=1e-2, atol=1e-2)  # the stated bar for bfloat16 outputs
+
+
+def test_scaled_mm_config4_8192_cubed():
+    """BASELINE config 4: e4m3fn 8192^3, per-tensor scales 0.5 / 0.5, bf16 out.  A full CPU
+    product takes an hour, so: sampled rows/columns against the float64 closed form, and
+    exactness properties (scaling an operand by 2 doubles every output bit for bit)."""
+    import _dev
+    m = n = k = 8192
+    a = torch.randn(m, k, generator=gen(1040)).clamp(-448, 448).to(torch.float8_e4m3fn)
+    bt = torch.randn(n, k, generator=gen(1041)).clamp(-448, 448).to(torch.float8_e4m3fn)
+    got = _dev.scaled_mm(bits(a), oracle.E4M3, bits(bt), oracle.E4M3, [0.5], [0.5], False, out_dtype=oracle.BF16)
+    rows = np.array([0, 1, 17, 255, 256, 4095, 4096, 8191])
+    cols = np.array([0, 3, 64, 127, 128, 5000, 8190, 8191])
+    _sampled_check(bits(a), bits(bt), np.float32(0.5), np.float32(0.5), got, rows, cols, False)
+    got2 = _dev.scaled_mm(bits(a), oracle.E4M3, bits(bt), oracle.E4M3, [1.0], [0.5], False, out_dtype=oracle.BF16)
+    assert np.array_equal(oracle.bf16_to_f32(got2), oracle.bf16_to_f32(got) * 2)
+
+
+def test_scaled_mm_config5_rowwise_70b():
+    """BASELINE config 5: rowwise scales, M=4096, K=8192, N=28672, bf16 out."""
+    import _dev
+    m, k, n = 4096, 8192, 28672
+    a = torch.randn(m, k, generator=gen(1050)).to(torch.float8_e4m3fn)
+    bt = torch.randn(n, k, generator=gen(1051)).to(torch.float8_e4m3fn)
+    sa = torch.empty(m, 1).uniform_(0.5, 2, generator=gen(1052)).numpy()
+    sb = torch.empty(1, n).uniform_(0.5, 2, generator=gen(1053)).numpy()
+    got = _dev.scaled_mm(bits(a), oracle.E4M3, bits(bt), oracle.E4M3, sa, sb, True, out_dtype=oracle.BF16)
+    rows = np.array([0, 255, 256, 2047, 4095])
+    cols = np.array([0, 127, 128, 14336, 28671, 28670])
+    _sampled_check(bits(a), bits(bt), sa, sb, got, rows, cols, True)
+
+
+def test_scaled_mm_errors():
+    from torch_vulkan_amd import abi
+    buf = abi.Buffer(4096)
+    p = abi.F8Params(a=buf.address, b=buf.address, scale_a=buf.address, scale_b=buf.address, out=buf.address, m=4, n=4,
+                     k=16, lda=16, ldb=16, ldo=4, fmt_a=abi.E4M3, fmt_b=abi.F32, out_dtype=abi.BF16)
+    with pytest.raises(abi.VktError, match="e4m3fn or e5m2"):
+        abi.dispatch("fp8mm", [0], p)
+    p.fmt_b = abi.E5M2
+    p.lda = 8
+    with pytest.raises(abi.VktError, match="strides"):
+        abi.dispatch("fp8mm", [0], p)
+    p.lda = 16
+    with pytest.raises(abi.VktError, match="unknown variant"):
+        abi.dispatch("fp8mm", [9], p)
