@@ -1,0 +1,316 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-matmul path on one MI355X, through the C ABI.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--no-cpu]
+
+A "step" is one pass of the hot path over one batch of seeded synthetic input: one
+`_weight_int8pack_mm` / `_dyn_quant_matmul_4bit` / `_scaled_mm` call's kernels, queued through
+vkt_dispatch with every input already resident in HBM.  The headline workload is the
+configuration the metric is quoted on: M=1 bf16 int8-weight GEMV at the Llama-3-8B gate/up
+shape (K=4096, N=14336).  GEMV workloads rotate through more than 512 MiB of distinct weight
+copies so that the figure is HBM bandwidth and not the 256 MB last-level cache.
+
+Prints ONE JSON line.  `value` is algorithmic bytes (or flops) per step / wall time per step
+over exactly K timed steps bracketed by device synchronisation; `roofline.achieved` is the
+same work / the kernel's average duration from HIP events recorded on the stream the
+kernels run on; `cpu_baseline` times the CPU oracle (a scalar C port of the reference's
+arithmetic, one core) on a bounded sample of the same workload, and `cpu_torch` PyTorch's own
+CPU kernel for the op on all host cores.  `extra` carries the other BASELINE configurations.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
+FP8_PEAK_TFLOPS = 5000.0    # MI355X dense fp8 MFMA, published
+
+
+def _abi():
+    from torch_vulkan_amd import abi
+    return abi
+
+
+class Launch:
+    """One prebuilt vkt_dispatch call (no per-call Python allocation in the timed loop)."""
+
+    def __init__(self, abi, name, spec, params):
+        self.fn = abi.lib().vkt_dispatch
+        self.name = name.encode()
+        self.spec = (abi.u32 * max(len(spec), 1))(*spec)
+        self.nspec = len(spec)
+        self.params = params
+        self.ref = ctypes.byref(params)
+        self.size = ctypes.sizeof(params)
+        self.abi = abi
+
+    def __call__(self):
+        if self.fn(self.name, self.spec, self.nspec, self.ref, self.size, 1, 1, 1) != 0:
+            self.abi.check(-1)
+
+
+def time_steps(abi, step_fns, steps, warmup):
+    """Runs step_fns[i % len] for `warmup` untimed and `steps` timed steps.
+    Returns (wall ms per step, event ms per step)."""
+    n = len(step_fns)
+    for i in range(warmup):
+        step_fns[i % n]()
+    abi.synchronize()
+    e0, e1 = abi.Event(), abi.Event()
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        step_fns[i % n]()
+    e1.record()
+    abi.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) * 1e3 / steps, e0.elapsed_ms(e1) / steps
+
+
+def rotation(nbytes, floor_mib=512):
+    return max(2, int(floor_mib * (1 << 20) // max(nbytes, 1)) + 1)
+
+
+# ------------------------------------------------------------------ workloads
+def wl_q8(abi, m, k, n, dtype, steps, warmup, seed=1020):
+    """_weight_int8pack_mm: x ~N(0,1) [m,k]; w int8 uniform [n,k]; scales ~U(0.005,0.02) [n]."""
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    tdt = {abi.F32: torch.float32, abi.BF16: torch.bfloat16, abi.F16: torch.float16}[dtype]
+    x = torch.randn(m, k, generator=g).to(tdt)
+    w = torch.randint(-128, 128, (n, k), dtype=torch.int8, generator=g)
+    s = torch.empty(n).uniform_(0.005, 0.02, generator=g).to(tdt)
+    item = x.element_size()
+    as_np = (lambda t: t.numpy()) if dtype == abi.F32 else (lambda t: t.view(torch.int16).numpy())
+    dx, ds = abi.Buffer.from_numpy(as_np(x)), abi.Buffer.from_numpy(as_np(s))
+    copies = [abi.Buffer.from_numpy(w.numpy())]
+    for _ in range(rotation(n * k) - 1):
+        b = abi.Buffer(n * k)
+        abi.check(abi.lib().vkt_copy_on_device(b.address, copies[0].address, n * k))
+        copies.append(b)
+    out = abi.Buffer(m * n * item)
+    fns = [Launch(abi, "qmm8_" + abi.SUFFIX[dtype], [0],
+                  abi.Q8Params(a=dx.address, b=c.address, scales=ds.address, c=out.address, m=m, n=n, k=k, a_sm=k,
+                               a_sk=1)) for c in copies]
+    wall, ev = time_steps(abi, fns, steps, warmup)
+    work = n * k + item * (m * k + n + m * n)  # weights once + activations + scales + output
+    keep = (x, w, s)
+    return dict(kind="hbm", work=work, wall_ms=wall, event_ms=ev, flops=2 * m * n * k, inputs=keep,
+                name=f"_weight_int8pack_mm {abi.SUFFIX[dtype]} M={m} K={k} N={n}", copies=len(copies))
+
+
+def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030):
+    """_dyn_quant_matmul_4bit on the compact side-car: both phases per step."""
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    w4 = torch.randint(0, 16, (n, k), dtype=torch.uint8, generator=g)
+    wbytes = (w4[:, 0::2] + 16 * w4[:, 1::2]).contiguous()
+    sc = torch.empty(n, k // bs).uniform_(0.01, 0.05, generator=g)
+    bias = torch.randn(n, generator=g) * 0.1
+    x = torch.randn(m, k, generator=g)
+    packed = torch._dyn_quant_pack_4bit_weight(wbytes, sc, bias, bs, k, n)
+    L = abi.lib()
+    cbytes = L.vkt_qmm4c_bytes(n, k, bs)
+    dp = abi.Buffer.from_numpy(packed.numpy())
+    first = abi.Buffer(cbytes)
+    abi.dispatch("qmm4c_pack", [], abi.Q4PackParams(packed=dp.address, compact=first.address, n=n, k=k, bs=bs,
+                                                    has_bias=1))
+    abi.synchronize()
+    dp.free()
+    copies = [first]
+    for _ in range(rotation(cbytes) - 1):
+        b = abi.Buffer(cbytes)
+        abi.check(L.vkt_copy_on_device(b.address, first.address, cbytes))
+        copies.append(b)
+    dx = abi.Buffer.from_numpy(x.numpy())
+    dq, dr = abi.Buffer(L.vkt_qmm4c_q_bytes(m, k)), abi.Buffer(m * 8)
+    out = abi.Buffer(m * n * 4)
+    fns = []
+    for c in copies:
+        p = abi.Q4CParams(inp=dx.address, q=dq.address, rows=dr.address, compact=c.address, out=out.address, m=m, n=n,
+                          k=k, bs=bs, has_bias=1)
+        a, b = Launch(abi, "qmm4c_f32", [0, 1], p), Launch(abi, "qmm4c_f32", [1, 1], p)
+        fns.append(lambda a=a, b=b: (a(), b()))
+    wall, ev = time_steps(abi, fns, steps, warmup)
+    work = n * k // 2 + 4 * n * (k // bs) + 4 * n + 4 * m * k + 4 * m * n
+    return dict(kind="hbm", work=work, wall_ms=wall, event_ms=ev, flops=2 * m * n * k, inputs=(x, packed),
+                name=f"_dyn_quant_matmul_4bit f32 M={m} K={k} N={n} bs={bs} (compact side-car)", copies=len(copies),
+                reference_layout_bytes=int(packed.numel()) * 4 + 4 * m * k + 4 * m * n)
+
+
+def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040):
+    """_scaled_mm e4m3fn x e4m3fn -> bf16; A row-major, B column-major."""
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(m, k, generator=g).clamp(-448, 448).to(torch.float8_e4m3fn)
+    bt = torch.randn(n, k, generator=g).clamp(-448, 448).to(torch.float8_e4m3fn)
+    if rowwise:
+        sa = torch.empty(m).uniform_(0.5, 2, generator=g)
+        sb = torch.empty(n).uniform_(0.5, 2, generator=g)
+    else:
+        sa, sb = torch.tensor([0.5]), torch.tensor([0.5])
+    da, db = abi.Buffer.from_numpy(a.view(torch.uint8).numpy()), abi.Buffer.from_numpy(bt.view(torch.uint8).numpy())
+    dsa, dsb = abi.Buffer.from_numpy(sa.numpy()), abi.Buffer.from_numpy(sb.numpy())
+    out = abi.Buffer(m * n * 2)
+    p = abi.F8Params(a=da.address, b=db.address, scale_a=dsa.address, scale_b=dsb.address, out=out.address, m=m, n=n,
+                     k=k, lda=k, ldb=k, ldo=n, fmt_a=abi.E4M3, fmt_b=abi.E4M3, out_dtype=abi.BF16, rowwise=int(rowwise))
+    fns = [Launch(abi, "fp8mm", [0], p)]
+    wall, ev = time_steps(abi, fns, steps, warmup)
+    return dict(kind="mfma", work=2 * m * n * k, wall_ms=wall, event_ms=ev, bytes=m * k + n * k + 2 * m * n,
+                inputs=(a, bt, sa, sb), copies=1,
+                name=f"_scaled_mm e4m3fn {'rowwise' if rowwise else 'per-tensor'} M={m} K={k} N={n} -> bf16")
+
+
+def wl_copy(abi, nbytes, steps, warmup):
+    """A plain device-to-device copy of known size (calibrates the HBM traffic counters)."""
+    src, dst = abi.Buffer(nbytes), abi.Buffer(nbytes)
+    abi.check(abi.lib().vkt_fill(src.address, 1, nbytes))
+    L = abi.lib()
+
+    def step():
+        abi.check(L.vkt_copy_on_device(dst.address, src.address, nbytes))
+    wall, ev = time_steps(abi, [step], steps, warmup)
+    return dict(kind="hbm", work=2 * nbytes, wall_ms=wall, event_ms=ev, flops=0, inputs=None, copies=1,
+                name=f"device copy of {nbytes >> 20} MiB (read + write)")
+
+
+WORKLOADS = {
+    # BASELINE.json configs[1]: the configuration the metric is quoted on
+    "c2_m1_k4096_n14336": lambda abi, s, w: wl_q8(abi, 1, 4096, 14336, abi.BF16, s, w),
+    "c2_m1_k14336_n4096": lambda abi, s, w: wl_q8(abi, 1, 14336, 4096, abi.BF16, s, w),
+    "c2_m8_k4096_n14336": lambda abi, s, w: wl_q8(abi, 8, 4096, 14336, abi.BF16, s, w),
+    "c2_m8_k14336_n4096": lambda abi, s, w: wl_q8(abi, 8, 14336, 4096, abi.BF16, s, w),
+    "c2_m64_k4096_n14336": lambda abi, s, w: wl_q8(abi, 64, 4096, 14336, abi.BF16, s, w),
+    "c2_m64_k14336_n4096": lambda abi, s, w: wl_q8(abi, 64, 14336, 4096, abi.BF16, s, w),
+    "c1_f32_m1_k4096_n4096": lambda abi, s, w: wl_q8(abi, 1, 4096, 4096, abi.F32, s, w, seed=1010),
+    "c3_int4_m1": lambda abi, s, w: wl_q4(abi, 1, 4096, 11008, 32, s, w),
+    "c3_int4_m32": lambda abi, s, w: wl_q4(abi, 32, 4096, 11008, 32, max(s // 4, 5), w),
+    "c4_fp8_8192": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 10, 5), max(w // 4, 3)),
+    "c5_fp8_rowwise_70b": lambda abi, s, w: wl_fp8(abi, 4096, 8192, 28672, True, max(s // 10, 5), max(w // 4, 3),
+                                                   seed=1050),
+}
+# not a BASELINE configuration: selected by name only (counter calibration)
+CALIBRATION = {"copy_256mib": lambda abi, s, w: wl_copy(abi, 256 << 20, max(s // 4, 5), w)}
+HEADLINE = "c2_m1_k4096_n14336"
+
+
+def summarise(r):
+    """Throughput and roofline of one workload result."""
+    if r["kind"] == "hbm":
+        value, unit, peak = r["work"] / r["wall_ms"] / 1e6, "GB/s", HBM_PEAK_GBPS
+        achieved = r["work"] / r["event_ms"] / 1e6
+    else:
+        value, unit, peak = r["work"] / r["wall_ms"] / 1e9, "TFLOP/s", FP8_PEAK_TFLOPS
+        achieved = r["work"] / r["event_ms"] / 1e9
+    return value, unit, dict(bound=r["kind"], achieved=round(achieved, 1), peak=peak, unit=unit,
+                             frac=round(achieved / peak, 4), traffic=None)
+
+
+def cpu_baselines(abi, name, r):
+    """The oracle (scalar C port, one core) on a bounded sample, and PyTorch's CPU op on all cores."""
+    import torch
+    import oracle
+    out = {}
+    if not name.startswith(("c1", "c2")):
+        return out
+    x, w, s = r["inputs"]
+    m, k = x.shape
+    n = w.shape[0]
+    odt = {torch.float32: oracle.F32, torch.bfloat16: oracle.BF16, torch.float16: oracle.F16}[x.dtype]
+    xb = x.numpy() if odt == oracle.F32 else x.view(torch.int16).numpy().view(np.uint16)
+    sb = s.numpy() if odt == oracle.F32 else s.view(torch.int16).numpy().view(np.uint16)
+    oracle.qmm8(xb, odt, w.numpy()[:64], sb[:64])  # load + warm
+    reps, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < 10.0 and reps < 200:
+        oracle.qmm8(xb, odt, w.numpy(), sb)
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    out["cpu_baseline"] = dict(value=round(r["work"] / dt / 1e9, 3), unit="GB/s", cores=1, kind="port",
+                               sample=f"{reps} full passes of the same workload through oracle/qmm_oracle.c "
+                                      f"(scalar C restatement), {dt * 1e3:.1f} ms each")
+    torch._weight_int8pack_mm(x, w, s)
+    ts = []
+    for _ in range(15):
+        t0 = time.perf_counter()
+        torch._weight_int8pack_mm(x, w, s)
+        ts.append(time.perf_counter() - t0)
+    dt = sorted(ts)[len(ts) // 2]
+    out["cpu_torch"] = dict(value=round(r["work"] / dt / 1e9, 3), unit="GB/s", cores=torch.get_num_threads(),
+                            host_cpus=os.cpu_count(), kind="torch CPU kernel of the same op",
+                            sample=f"median of 15 calls of torch._weight_int8pack_mm, {dt * 1e3:.2f} ms")
+    return out
+
+
+def load_traffic():
+    """HBM traffic per launch measured with rocprofv3 --pmc (profiles/traffic.json), if recorded."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f)
+    except (OSError, ValueError):
+        return {}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS) + sorted(CALIBRATION))
+    ap.add_argument("--no-extra", action="store_true", help="only the selected workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build is a one-GPU path (no collectives, no sharding); run with --gpus 1")
+    abi = _abi()
+    info = abi.device_info()
+    traffic = load_traffic()
+
+    r = {**WORKLOADS, **CALIBRATION}[args.workload](abi, args.steps, args.warmup)
+    value, unit, roof = summarise(r)
+    roof["traffic"] = traffic.get(args.workload)
+    line = {
+        "metric": "M=1 int8 GEMV GB/s (% of HBM peak)" if r["kind"] == "hbm" else "fp8 _scaled_mm TFLOP/s (% of MFMA peak)",
+        "value": round(value, 1), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(r["wall_ms"], 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 accumulate (bf16 activations, int8 weights)" if args.workload.startswith("c2") else "see workload",
+        "data": "synthetic (seeded)",
+        "config": {"workload": r["name"], "key": args.workload, "weight_copies_rotated": r["copies"],
+                   "device": info.name.decode(), "compute_units": info.compute_units},
+        "roofline": roof,
+    }
+    if not args.no_cpu:
+        line.update(cpu_baselines(abi, args.workload, r))
+    if "cpu_baseline" not in line:
+        line["cpu_baseline"] = None
+    del r
+    if not args.no_extra:
+        extra = []
+        for name, fn in WORKLOADS.items():
+            if name == args.workload:
+                continue
+            rr = fn(abi, args.steps, args.warmup)
+            v, u, rf = summarise(rr)
+            rf["traffic"] = traffic.get(name)
+            e = {"key": name, "workload": rr["name"], "value": round(v, 1), "unit": u,
+                 "ms_per_step": round(rr["wall_ms"], 5), "kernel_ms": round(rr["event_ms"], 5), "roofline": rf}
+            if rr["kind"] == "hbm":
+                e["tflops"] = round(rr["flops"] / rr["event_ms"] / 1e9, 2)
+            else:
+                e["hbm_gbps_algorithmic"] = round(rr["bytes"] / rr["event_ms"] / 1e6, 1)
+            if "reference_layout_bytes" in rr:
+                e["reference_layout_bytes"] = rr["reference_layout_bytes"]
+            extra.append(e)
+            del rr
+        line["extra"] = extra
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -26,6 +26,7 @@ SOURCES = {
     # every float32 operation of the int4 path is a single IEEE operation
     "kernels/qmm4.hip": ["-ffp-contract=off"],
     "kernels/fp8mm.hip": [],
+    "kernels/util.hip": [],
 }
 
 

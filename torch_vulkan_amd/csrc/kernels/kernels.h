@@ -26,6 +26,7 @@ int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwi
                  const Machine& mc, hipStream_t stream, std::string* err);
 int launch_fp8mm(const F8Params& p, uint32_t variant, const Machine& mc, hipStream_t stream, std::string* err);
 int launch_fill(uint64_t dst, uint8_t value, uint64_t nbytes, hipStream_t stream, std::string* err);
+int launch_copy(uint64_t dst, uint64_t src, uint64_t nbytes, hipStream_t stream, std::string* err);
 
 uint64_t qmm4c_bytes(uint32_t n, uint32_t k, uint32_t bs);
 uint64_t qmm4c_q_bytes(uint32_t m, uint32_t k);

@@ -446,19 +446,6 @@ __global__ __launch_bounds__(256) void qmm4c_gemv_channelwise(Q4CParams p, Compa
   }
 }
 
-__global__ __launch_bounds__(256) void fill_kernel(uint64_t dst, uint32_t value, uint64_t nbytes) {
-  const uint64_t stride = uint64_t(gridDim.x) * 256;
-  const uint64_t head = (16 - (dst & 15)) & 15;  // bytes before the first 16-byte boundary
-  uint64_t i = uint64_t(blockIdx.x) * 256 + threadIdx.x;
-  if (i < head && i < nbytes) stg<uint8_t>(dst + i, uint8_t(value));
-  if (nbytes <= head) return;
-  const uint64_t body = (nbytes - head) / 16, word = value * 0x01010101u;
-  const U4 v = {uint32_t(word), uint32_t(word), uint32_t(word), uint32_t(word)};
-  for (uint64_t j = i; j < body; j += stride) stg<U4>(dst + head + j * 16, v);
-  const uint64_t tail0 = head + body * 16;
-  if (tail0 + i < nbytes && i < 16) stg<uint8_t>(dst + tail0 + i, uint8_t(value));
-}
-
 bool check_q4_shape(uint32_t m, uint32_t n, uint32_t k, uint32_t bs, std::string* err) {
   if (bs == 0 || !(bs == k || (bs % 32 == 0 && k % bs == 0))) {
     *err = "qmm4: block size must equal k or be a multiple of 32 dividing k";
@@ -606,17 +593,6 @@ int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwi
   }
   if (hipGetLastError() != hipSuccess) {
     *err = "qmm4c: kernel launch failed";
-    return -1;
-  }
-  return 0;
-}
-
-int launch_fill(uint64_t dst, uint8_t value, uint64_t nbytes, hipStream_t stream, std::string* err) {
-  const uint64_t want = (nbytes / 16 + 255) / 256 + 1;
-  const uint32_t groups = uint32_t(want < 4096 ? want : 4096);
-  hipLaunchKernelGGL(fill_kernel, dim3(groups), dim3(256), 0, stream, dst, uint32_t(value), nbytes);
-  if (hipGetLastError() != hipSuccess) {
-    *err = "fill: kernel launch failed";
     return -1;
   }
   return 0;

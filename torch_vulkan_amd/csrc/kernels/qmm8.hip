@@ -163,15 +163,13 @@ bool launch_gemv_cols(const Q8Params& p, int cols, int ksplit, hipStream_t strea
   return false;
 }
 
-// Picks COLS and KSPLIT so that the grid puts at least ~2 waves on each of the machine's
-// SIMDs while each wave keeps several 16-byte loads in flight.
-void plan_gemv(const Q8Params& p, int rows, const Machine& mc, int* cols, int* ksplit) {
-  const int64_t simds = int64_t(mc.compute_units) * 4;
-  const int wide = rows <= 4 ? 4 : 2, narrow = rows <= 4 ? 2 : 1;
-  *cols = (int64_t(p.n) / wide >= 2 * simds) ? wide : narrow;
-  int ks = 1;
-  while (ks < 4 && int64_t(p.n) / *cols * ks < 2 * simds && p.k >= 2048u * ks) ks *= 2;
-  *ksplit = ks;
+// Picks COLS and KSPLIT.  Measured on MI355X (M = 1, weights rotated through HBM): many
+// small waves beat few large ones, because the whole weight stream is then in flight at
+// once: 2 columns per wave and K split over the 4 waves of a workgroup while a wave still
+// gets one full 1 KiB load per column; rows beyond 4 leave fewer registers per column.
+void plan_gemv(const Q8Params& p, int rows, const Machine&, int* cols, int* ksplit) {
+  *cols = rows <= 4 ? 2 : (p.n >= 8192 ? 2 : 1);
+  *ksplit = p.k >= 4096 ? (p.k <= 8192 ? 4 : 2) : (p.k >= 2048 ? 2 : 1);
 }
 
 template <class T>
