@@ -107,7 +107,7 @@ def wl_q8(abi, m, k, n, dtype, steps, warmup, seed=1020):
 
 
 def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030):
-    """_dyn_quant_matmul_4bit on the compact side-car: both phases per step."""
+    """_dyn_quant_matmul_4bit on the compact side-car (row quantisation fused into the launch)."""
     import torch
     g = torch.Generator().manual_seed(seed)
     w4 = torch.randint(0, 16, (n, k), dtype=torch.uint8, generator=g)
@@ -136,8 +136,7 @@ def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030):
     for c in copies:
         p = abi.Q4CParams(inp=dx.address, q=dq.address, rows=dr.address, compact=c.address, out=out.address, m=m, n=n,
                           k=k, bs=bs, has_bias=1)
-        a, b = Launch(abi, "qmm4c_f32", [0, 1], p), Launch(abi, "qmm4c_f32", [1, 1], p)
-        fns.append(lambda a=a, b=b: (a(), b()))
+        fns.append(Launch(abi, "qmm4c_f32", [2, 1], p))  # row quantisation + product in one launch
     wall, ev = time_steps(abi, fns, steps, warmup)
     work = n * k // 2 + 4 * n * (k // bs) + 4 * n + 4 * m * k + 4 * m * n
     return dict(kind="hbm", work=work, wall_ms=wall, event_ms=ev, flops=2 * m * n * k, inputs=(x, packed),

@@ -72,8 +72,9 @@ class CompactWeights:
         dp.free()
 
 
-def q4_compact(x, odt, cw, variant=0):
-    """_dyn_quant_matmul_4bit through the streaming path ("qmm4c_*")."""
+def q4_compact(x, odt, cw, fused=True):
+    """_dyn_quant_matmul_4bit through the streaming path ("qmm4c_*"): one fused launch
+    (PHASE 2), or row quantisation (PHASE 0) then the product (PHASE 1)."""
     x = np.ascontiguousarray(x)
     m, n, k, bs = x.shape[0], cw.n, cw.k, cw.bs
     dx = abi.Buffer.from_numpy(x)
@@ -84,9 +85,11 @@ def q4_compact(x, odt, cw, variant=0):
                       k=k, bs=bs, has_bias=cw.has_bias)
     g = int(bs != k)
     name = "qmm4c_" + abi.SUFFIX[odt]
-    if m and n:
-        abi.dispatch(name, [0, g, variant], p, (m,))
-        abi.dispatch(name, [1, g, variant], p, ((n + 31) // 32, (m + 7) // 8))
+    if m and n and fused:
+        abi.dispatch(name, [2, g], p, ((n + 31) // 32, (m + 7) // 8))
+    elif m and n:
+        abi.dispatch(name, [0, g], p, (m,))
+        abi.dispatch(name, [1, g], p, ((n + 31) // 32, (m + 7) // 8))
     return do.to_numpy(_NP[odt], (m, n))
 
 

@@ -13,7 +13,7 @@ from test_oracle_pins import Q4_CASES, pack_case, q4_input
 
 pytestmark = pytest.mark.gpu
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
-EXTRA = [(2, 4096, 300, 32, True), (4, 4096 + 2048, 12, 64, False), (7, 8192, 9, 128, True), (3, 512, 5, 256, False),
+EXTRA = [(2, 4096, 300, 32, True), (3, 14336, 20, 32, True), (9, 28672, 6, 128, False), (4, 4096 + 2048, 12, 64, False), (7, 8192, 9, 128, True), (3, 512, 5, 256, False),
          (6, 4160, 10, 4160, True), (1, 32, 1, 32, False), (5, 8, 3, 8, True)]
 
 
@@ -37,7 +37,8 @@ def test_q4_bit_exact(m, k, n, bs, bias, dtype):
     assert np.array_equal(got, want)
     if abi.lib().vkt_qmm4c_bytes(n, k, bs):
         cw = _dev.CompactWeights(packed.numpy(), bs, k, n)
-        assert np.array_equal(_dev.q4_compact(bits(x), odt, cw), want)
+        assert np.array_equal(_dev.q4_compact(bits(x), odt, cw, fused=True), want)
+        assert np.array_equal(_dev.q4_compact(bits(x), odt, cw, fused=False), want)
 
 
 @pytest.mark.parametrize("m", [1, 32])
@@ -100,6 +101,10 @@ def test_q4_errors():
         abi.dispatch("qmm4_f32", [0, 0], p)
     with pytest.raises(abi.VktError, match="PHASE"):
         abi.dispatch("qmm4_f32", [2, 1], p)
+    c = abi.Q4CParams(inp=buf.address, q=buf.address, rows=buf.address, compact=buf.address, out=buf.address, m=1, n=2,
+                      k=64, bs=32, has_bias=0)
+    with pytest.raises(abi.VktError, match="PHASE"):
+        abi.dispatch("qmm4c_f32", [3, 1], c)
     with pytest.raises(abi.VktError, match="unknown kernel"):
         abi.dispatch("qmm4_f16", [0, 1], p)
     assert abi.lib().vkt_qmm4c_bytes(8, 96, 96) > 0 and abi.lib().vkt_qmm4c_bytes(8, 192, 96) == 0

@@ -60,7 +60,7 @@ def test_compact_sizes():
     total = L.vkt_qmm4c_bytes(n, k, 32)
     assert n * k // 2 + 4 * n * k // 32 + 4 * n <= total <= n * k // 2 + 4 * n * k // 32 + 4 * n + 512
     assert L.vkt_qmm4c_bytes(n, k, 96) == 0 and L.vkt_qmm4c_bytes(n, k, k) > 0
-    assert L.vkt_qmm4c_q_bytes(1, 4096) == 4096 + 4 * 128
+    assert L.vkt_qmm4c_q_bytes(1, 4096) == 4096 and L.vkt_qmm4c_q_bytes(3, 100) == 3 * 4096
 
 
 # ------------------------------------------------------------------ pool policy

@@ -15,18 +15,21 @@
 //   "qmm4_*"   the reference's parameter block and buffers as they are (int32 q, the
 //              float32-expanded packed vector: 4 bytes of traffic per byte of nibbles).
 //   "qmm4c_*"  the streaming path.  "qmm4c_pack" rewrites the packed vector once into a
-//              compact side-car (two nibbles per byte, 16 bytes per lane per load,
-//              laid out so that every load of a wave is 1 KiB contiguous); phase 0 writes
-//              int8 activations in the byte order v_dot4 wants plus per-unit sums;
-//              phase 1 is an HBM stream over the side-car:
-//                - a wave owns 4 output columns, one per DPP row of 16 lanes; the 16 lanes
-//                  of a row split K into runs of 8 units (a unit = 32 values of k = one
-//                  16-byte load);
-//                - nibbles stay unsigned: sum (q+nzp)(nib-8) = dot(q,nib) - 8 sum(q)
-//                  + nzp (sum(nib) - 8*32), all v_dot4_i32_i8 and integer adds;
-//                - the float32 block terms must be added in block order, so the lanes of a
-//                  row pass the running sum along with DPP row rotates: 16 short phases per
-//                  round of 128 units, no LDS, no atomics.
+//              compact side-car (two nibbles per byte, 16 bytes per lane per load, laid out
+//              so that every load instruction of a wave reads 1 KiB contiguous), and the
+//              product is an HBM stream over it:
+//                - a workgroup of 4 waves owns 16 output columns; lane = (column, k-part):
+//                  the 16 k-parts (4 waves x 4 groups of 16 lanes) split K into runs of
+//                  8 units per round (a unit = 32 values of k = one 16-byte load);
+//                - everything integer runs on v_dot8_i32_i4: weights nib-8 are nib^8 read
+//                  as signed nibbles (one xor per 8 weights), activations q = 16 qh + ql are
+//                  kept as two signed-nibble planes qh and ql-8, so
+//                  sum (q+nzp) w = 16 dot8(qh,w) + dot8(ql-8,w) + (8+nzp) dot8(1,w):
+//                  four instructions per 8 weights, no unpacking;
+//                - the float32 block terms must be added in block order: each lane adds its
+//                  8 in order, lane groups hand the running sum on with ds_bpermute and
+//                  waves through LDS.  Starting from -0.0f and padding with -0.0f makes every
+//                  step a plain addition (x + -0 = x, -0 + t = t) with the reference's bits.
 #pragma clang fp contract(off)
 
 #include "common.h"
@@ -37,8 +40,9 @@ namespace {
 
 constexpr int kUnit = 32;          // values of k per 16-byte load of nibbles
 constexpr int kUnitsPerLane = 8;   // units a lane handles per round
-constexpr int kRoundUnits = 128;   // 16 lanes * 8 units
-constexpr int kTileCols = 4;       // output columns per wave
+constexpr int kRoundUnits = 128;   // 16 k-parts * 8 units
+constexpr int kTileCols = 16;      // output columns per workgroup
+constexpr int kFusedGroups = 4;    // groups of 8 activations a thread quantises in the fused kernel
 
 __device__ __forceinline__ float round_away(float x) {  // std::round, qmm4.slang:112-118
   float t = truncf(x);
@@ -88,6 +92,31 @@ __device__ __forceinline__ void row_range(uint64_t row, uint32_t k, float* mn_ou
   __syncthreads();
   *mn_out = fminf(fminf(smin[0], smin[1]), fminf(smin[2], smin[3]));
   *mx_out = fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3]));
+}
+
+// Workgroup-wide min / max of per-thread values (256 threads).
+__device__ __forceinline__ void block_range(float* mn, float* mx) {
+  __shared__ float bmin[4], bmax[4];
+  const float a = wave_min(*mn), b = wave_max(*mx);
+  if ((threadIdx.x & 63) == 0) bmin[threadIdx.x >> 6] = a, bmax[threadIdx.x >> 6] = b;
+  __syncthreads();
+  *mn = fminf(fminf(bmin[0], bmin[1]), fminf(bmin[2], bmin[3]));
+  *mx = fmaxf(fmaxf(bmax[0], bmax[1]), fmaxf(bmax[2], bmax[3]));
+}
+
+// 8 consecutive elements at a 16-byte aligned address (float32: 32-byte aligned pairs).
+template <class T>
+__device__ __forceinline__ void load8_f32(uint64_t addr, float (&x)[8]);
+template <>
+__device__ __forceinline__ void load8_f32<f32_t>(uint64_t addr, float (&x)[8]) {
+  const F4 a = ldg<F4>(addr), b = ldg<F4>(addr + 16);
+  x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w, x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
+}
+template <>
+__device__ __forceinline__ void load8_f32<bf16_t>(uint64_t addr, float (&x)[8]) {
+  const U4 v = ldg<U4>(addr);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) x[2 * j] = bits_f32(v[j] << 16), x[2 * j + 1] = bits_f32(v[j] & 0xffff0000u);
 }
 
 // ------------------------------------------------------------------ reference-layout path
@@ -153,7 +182,7 @@ __global__ __launch_bounds__(256) void qmm4_matmul_expanded(Q4Params p) {
 struct CompactLayout {
   uint32_t nunits, rounds, tiles, upb;  // units per block (0: channelwise)
   uint64_t nib_bytes, scale_off, scale_bytes, bias_off, total;
-  uint32_t kpad;  // values of k per activation row in the scratch (rounds * 4096)
+  uint32_t kpad;  // values of k per activation row in LDS / scratch (rounds * 4096)
 };
 
 __host__ __device__ inline bool compact_layout(uint32_t n, uint32_t k, uint32_t bs, CompactLayout* L) {
@@ -165,27 +194,30 @@ __host__ __device__ inline bool compact_layout(uint32_t n, uint32_t k, uint32_t 
   L->rounds = (L->nunits + kRoundUnits - 1) / kRoundUnits;
   L->tiles = (n + kTileCols - 1) / kTileCols;
   L->upb = channelwise ? 0 : bs / kUnit;
-  L->nib_bytes = uint64_t(L->tiles) * L->rounds * kUnitsPerLane * 64 * 16;
+  // [tile][round][wave 4][unit 8][lane 64] x 16 bytes
+  L->nib_bytes = uint64_t(L->tiles) * L->rounds * 4 * kUnitsPerLane * 64 * 16;
   L->scale_off = L->nib_bytes;
+  // groupwise: [tile][round][wave 4][lane 64][blocks per lane] float32; channelwise: [n]
   L->scale_bytes = channelwise ? round_up_u64(uint64_t(n) * 4, 256)
-                               : uint64_t(L->tiles) * L->rounds * (kUnitsPerLane / L->upb) * 64 * 4;
+                               : uint64_t(L->tiles) * L->rounds * 4 * 64 * (kUnitsPerLane / L->upb) * 4;
   L->bias_off = L->scale_off + L->scale_bytes;
   L->total = L->bias_off + round_up_u64(uint64_t(n) * 4, 256);
   L->kpad = L->rounds * kRoundUnits * kUnit;
   return true;
 }
 
-// One thread per 16-byte unit of the side-car (and, in the same grid, per scale slot).
+// One thread per 16-byte unit of the side-car, then per scale slot, then per bias.
 __global__ __launch_bounds__(256) void qmm4c_pack_kernel(Q4PackParams p, CompactLayout L) {
   const uint32_t rstride = (p.k + 1) / 2, nblocks = (p.k + p.bs - 1) / p.bs;
   const uint64_t wcount = uint64_t(p.n) * p.k / 2;
   const uint64_t slots = L.nib_bytes / 16;
   const uint64_t id = uint64_t(blockIdx.x) * 256 + threadIdx.x;
   if (id < slots) {
-    const uint32_t lane = id & 63, j = (id >> 6) % kUnitsPerLane;
-    const uint64_t tr = id / (64 * kUnitsPerLane);
+    const uint32_t lane = id & 63, j = (id >> 6) & 7, wave = (id >> 9) & 3;
+    const uint64_t tr = id >> 11;
     const uint32_t round = tr % L.rounds, tile = tr / L.rounds;
-    const uint32_t n = tile * kTileCols + (lane >> 4), unit = round * kRoundUnits + (lane & 15) * kUnitsPerLane + j;
+    const uint32_t n = tile * kTileCols + (lane & 15), part = wave * 4 + (lane >> 4);
+    const uint32_t unit = round * kRoundUnits + part * kUnitsPerLane + j;
     U4 out;
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
@@ -211,11 +243,11 @@ __global__ __launch_bounds__(256) void qmm4c_pack_kernel(Q4PackParams p, Compact
     const uint32_t bpl = kUnitsPerLane / L.upb;
     const uint64_t sslots = L.scale_bytes / 4;
     if (sid < sslots) {
-      const uint32_t lane = sid & 63, jb = (sid >> 6) % bpl;
-      const uint64_t tr = sid / (64 * bpl);
+      const uint32_t jb = sid % bpl, lane = (sid / bpl) & 63, wave = (sid / (bpl * 64)) & 3;
+      const uint64_t tr = sid / (bpl * 256);
       const uint32_t round = tr % L.rounds, tile = tr / L.rounds;
-      const uint32_t n = tile * kTileCols + (lane >> 4);
-      const uint32_t blk = (round * kRoundUnits + (lane & 15) * kUnitsPerLane) / L.upb + jb;
+      const uint32_t n = tile * kTileCols + (lane & 15), part = wave * 4 + (lane >> 4);
+      const uint32_t blk = (round * kRoundUnits + part * kUnitsPerLane) / L.upb + jb;
       float s = 0.0f;
       if (n < p.n && blk < nblocks) s = ldg<float>(p.packed + (wcount + uint64_t(n) * nblocks + blk) * 4);
       stg<float>(p.compact + L.scale_off + sid * 4, s);
@@ -235,9 +267,33 @@ __global__ __launch_bounds__(256) void qmm4c_pack_kernel(Q4PackParams p, Compact
   }
 }
 
-// Phase 0 for the streaming path, one workgroup per row: int8 activations in dot order
-// (within each 8 values of k: k0 k2 k4 k6 | k1 k3 k5 k7, matching the low / high nibbles of
-// 4 packed bytes), zero beyond k up to kpad; per-unit sums sq [m][kpad/32] int32 after them.
+// 8 quantised values -> their two signed-nibble planes: hi = q >> 4, lo = (q & 15) - 8,
+// nibble i of each word belonging to the i-th value.
+__device__ __forceinline__ void nibble_planes(const int (&q)[8], uint32_t* hi, uint32_t* lo) {
+  uint32_t h = 0, l = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    h |= (uint32_t(q[i] >> 4) & 15u) << (4 * i);
+    l |= ((uint32_t(q[i]) & 15u) ^ 8u) << (4 * i);
+  }
+  *hi = h, *lo = l;
+}
+
+// Activation rows as the streaming kernel reads them: per unit of 32 values 16 bytes of hi
+// nibbles then 16 bytes of lo nibbles.  In LDS a row carries 16 bytes of padding after every
+// 256 (one lane's run of 8 units), so that the four k-parts a wave reads at once, 256 bytes
+// apart, fall on different banks.
+__host__ __device__ inline uint32_t q_row_bytes(uint32_t kpad) { return kpad + kpad / 256 * 16; }
+__host__ __device__ inline uint32_t q_lds_bytes(uint32_t rows, uint32_t kpad) {
+  return rows * q_row_bytes(kpad) + rows * kTileCols * 4 + 64;
+}
+__device__ __forceinline__ uint32_t q_group_offset(uint32_t g) {  // byte offset of 8 values' hi word
+  const uint32_t unit = g >> 2, d = g & 3;
+  return unit * kUnit + unit / 8 * 16 + d * 4;
+}
+
+// Phase 0 for the two-launch form, one workgroup per row: nibble planes into q
+// ([m][kpad] bytes, no padding), rows[2m] = bits(1/scale), rows[2m+1] = -zero_point.
 template <class T>
 __global__ __launch_bounds__(256) void qmm4c_rowquant(Q4CParams p, uint32_t groupwise, uint32_t kpad) {
   constexpr uint64_t item = sizeof(typename T::storage);
@@ -251,198 +307,215 @@ __global__ __launch_bounds__(256) void qmm4c_rowquant(Q4CParams p, uint32_t grou
     stg<int32_t>(p.rows + 8ull * m + 4, -rq.izp);
   }
   const uint64_t qrow = p.q + uint64_t(m) * kpad;
-  const uint64_t sq = p.q + uint64_t(p.m) * kpad + uint64_t(m) * (kpad / kUnit) * 4;
-  // a thread quantises 8 consecutive values of k (two dot operands); 4 threads make a unit
   for (uint32_t g = threadIdx.x; g < kpad / 8; g += 256) {
-    int q[8], sum = 0;
+    int q[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const uint32_t k = g * 8 + i;
       q[i] = k < p.k ? quantise(load_f32<T>(row + k * item), rq) : 0;
-      sum += q[i];
     }
-    U2 o;
-    o.x = uint32_t(q[0] & 255) | uint32_t(q[2] & 255) << 8 | uint32_t(q[4] & 255) << 16 | uint32_t(q[6] & 255) << 24;
-    o.y = uint32_t(q[1] & 255) | uint32_t(q[3] & 255) << 8 | uint32_t(q[5] & 255) << 16 | uint32_t(q[7] & 255) << 24;
-    stg<U2>(qrow + g * 8ull, o);
-    sum += dpp_i32<kQuadSwap1>(sum);  // the 4 threads of a unit are one quad (256 % 4 == 0)
-    sum += dpp_i32<kQuadSwap2>(sum);
-    if ((g & 3) == 0) stg<int32_t>(sq + (g / 4) * 4ull, sum);
+    uint32_t hi, lo;
+    nibble_planes(q, &hi, &lo);
+    const uint64_t at = qrow + (g >> 2) * kUnit + (g & 3) * 4;
+    stg<uint32_t>(at, hi);
+    stg<uint32_t>(at + 16, lo);
   }
 }
 
-constexpr int kRowRor1 = 0x121;  // DPP row_ror:1: lane i of each row of 16 reads lane i-1 (mod 16)
-
-// Phase 1, groupwise (UPB = units per block: 1, 2, 4 or 8), MR rows of activations per pass.
-template <class T, int MR, int UPB>
-__global__ __launch_bounds__(256) void qmm4c_gemv(Q4CParams p, CompactLayout L, uint32_t m0) {
+// The streaming kernel.  UPB = units per scale block (1, 2, 4, 8), or 0 for channelwise (one
+// block spanning K).  FUSED: the workgroup quantises its MR activation rows itself (phase 0
+// folded in: no second launch, no scratch round trip); otherwise it stages the planes that
+// phase 0 left in global memory.  The inner loop reads activations from LDS and weights
+// straight from HBM.
+template <class T, int MR, int UPB, bool FUSED>
+__global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L, uint32_t m0, uint32_t groupwise) {
   constexpr uint64_t item = sizeof(typename T::storage);
-  constexpr int BPL = kUnitsPerLane / UPB;  // blocks per lane per round
-  const int lane = threadIdx.x & 63, part = lane & 15;
-  const uint32_t tile = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (tile >= L.tiles) return;  // whole waves only: no barrier follows
-  const uint32_t n = tile * kTileCols + (lane >> 4);
-  const uint32_t nblocks = p.k / p.bs;
+  constexpr int BPL = UPB ? kUnitsPerLane / UPB : 1;  // blocks per lane per round
+  constexpr int UN = UPB ? UPB : kUnitsPerLane;       // units of a block within a lane
+  extern __shared__ __attribute__((aligned(16))) uint8_t q_lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, grp = lane >> 4, part = wave * 4 + grp;
+  const uint32_t tile = blockIdx.x, n = tile * kTileCols + col;
+  const uint32_t nblocks = UPB ? p.k / p.bs : 1;
+  const uint32_t qs = q_row_bytes(L.kpad);
+  float* const carry = reinterpret_cast<float*>(q_lds + MR * qs);      // [MR][16]: running sums between waves
+  int* const itotal = reinterpret_cast<int*>(carry);                    // (channelwise: integer totals)
 
-  int nzp[MR];
-  uint64_t qrow[MR], sqrow[MR];
+  // the first round's weights are requested before anything else: they are the long pole
+  U4 w[kUnitsPerLane];
+  {
+    const uint64_t base = (uint64_t(tile) * L.rounds * 4 + wave) * kUnitsPerLane;
+#pragma unroll
+    for (int j = 0; j < kUnitsPerLane; ++j) w[j] = ldg<U4>(p.compact + ((base + j) * 64 + lane) * 16);
+  }
+
+  int nzp8[MR];  // 8 - zero_point
+  float recip[MR];
 #pragma unroll
   for (int r = 0; r < MR; ++r) {
     const uint32_t m = m0 + r < p.m ? m0 + r : p.m - 1;
-    nzp[r] = ldg<int32_t>(p.rows + 8ull * m + 4);
-    qrow[r] = p.q + uint64_t(m) * L.kpad;
-    sqrow[r] = p.q + uint64_t(p.m) * L.kpad + uint64_t(m) * (L.kpad / kUnit) * 4;
-  }
-  float acc[MR];
+    if constexpr (FUSED) {
+      const uint64_t row = p.inp + uint64_t(m) * p.k * item;
+      // A thread owns the groups of 8 values g = tid + 256 i, i < kFusedGroups: all loads are
+      // in flight together, the row's range is reduced from registers and the values are
+      // quantised from registers.  (The launcher fuses only when k is a multiple of 8, rows
+      // are 16-byte aligned and k <= 2048 * kFusedGroups; otherwise it runs phase 0 itself.)
+      const uint32_t groups = p.k / 8;
+      float x[kFusedGroups][8];
+      float mn = 3.40282347e38f, mx = -3.40282347e38f;
 #pragma unroll
-  for (int r = 0; r < MR; ++r) acc[r] = 0.0f;
+      for (int i = 0; i < kFusedGroups; ++i) {
+        const uint32_t g = tid + 256 * i;
+        if (g < groups) load8_f32<T>(row + g * 8 * item, x[i]);
+      }
+#pragma unroll
+      for (int i = 0; i < kFusedGroups; ++i) {
+        if (uint32_t(tid + 256 * i) < groups) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) mn = fminf(mn, x[i][e]), mx = fmaxf(mx, x[i][e]);
+        }
+      }
+      block_range(&mn, &mx);
+      const RowQuant rq = row_quant(mn, mx, groupwise != 0);
+      nzp8[r] = 8 - rq.izp;
+      recip[r] = rq.recip;
+#pragma unroll
+      for (int i = 0; i < kFusedGroups; ++i) {
+        const uint32_t g = tid + 256 * i;
+        if (g < L.kpad / 8) {
+          uint32_t hi = 0, lo = 0x88888888u;  // beyond k: value 0 = planes (0, 0 - 8)
+          if (g < groups) {
+            int q[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) q[e] = quantise(x[i][e], rq);
+            nibble_planes(q, &hi, &lo);
+          }
+          uint8_t* at = q_lds + r * qs + q_group_offset(g);
+          *reinterpret_cast<uint32_t*>(at) = hi;
+          *reinterpret_cast<uint32_t*>(at + 16) = lo;
+        }
+      }
+      __syncthreads();  // (the range scratch is reused by the next row)
+    } else {
+      nzp8[r] = 8 + ldg<int32_t>(p.rows + 8ull * m + 4);
+      recip[r] = bits_f32(ldg<uint32_t>(p.rows + 8ull * m));
+      const uint64_t src = p.q + uint64_t(m) * L.kpad;
+      for (uint32_t c = tid; c < L.kpad / 16; c += 256)
+        *reinterpret_cast<U4*>(q_lds + r * qs + c * 16 + c / 16 * 16) = ldg<U4>(src + c * 16ull);
+    }
+  }
+  if (tid < MR * kTileCols) carry[tid] = UPB ? -0.0f : 0.0f;  // (integer 0 and +0.0f share their bits)
+  __syncthreads();
+
+  float acc[MR];
+  int tot_a[MR], tot_b[MR], tot_c = 0;
+#pragma unroll
+  for (int r = 0; r < MR; ++r) acc[r] = 0.0f, tot_a[r] = 0, tot_b[r] = 0;
 
   for (uint32_t round = 0; round < L.rounds; ++round) {
-    const uint64_t base = (uint64_t(tile) * L.rounds + round);
-    U4 w[kUnitsPerLane];
+    const uint64_t base = (uint64_t(tile) * L.rounds + round) * 4 + wave;
+    if (round != 0) {
 #pragma unroll
-    for (int j = 0; j < kUnitsPerLane; ++j) w[j] = ldg<U4>(p.compact + ((base * kUnitsPerLane + j) * 64 + lane) * 16);
+      for (int j = 0; j < kUnitsPerLane; ++j) w[j] = ldg<U4>(p.compact + ((base * kUnitsPerLane + j) * 64 + lane) * 16);
+    }
     float s[BPL];
+    if constexpr (UPB != 0) {
+      const uint64_t sp = p.compact + L.scale_off + (base * 64 + lane) * BPL * 4;
+      if constexpr (BPL == 8) {
+        const F4 s0 = ldg<F4>(sp), s1 = ldg<F4>(sp + 16);
+        s[0] = s0.x, s[1] = s0.y, s[2] = s0.z, s[3] = s0.w, s[4] = s1.x, s[5] = s1.y, s[6] = s1.z, s[7] = s1.w;
+      } else if constexpr (BPL == 4) {
+        const F4 s0 = ldg<F4>(sp);
+        s[0] = s0.x, s[1] = s0.y, s[2] = s0.z, s[3] = s0.w;
+      } else {
 #pragma unroll
-    for (int jb = 0; jb < BPL; ++jb) s[jb] = ldg<float>(p.compact + L.scale_off + ((base * BPL + jb) * 64 + lane) * 4);
+        for (int jb = 0; jb < BPL; ++jb) s[jb] = ldg<float>(sp + 4 * jb);
+      }
+    }
     const uint32_t unit0 = round * kRoundUnits + part * kUnitsPerLane;
+    const uint8_t* qbase = q_lds + unit0 * kUnit + unit0 / 8 * 16;
 
     float t[MR][BPL];
 #pragma unroll
     for (int jb = 0; jb < BPL; ++jb) {
-      int iacc[MR], ones = 0;
+      int da[MR], db[MR], dc = 0;
 #pragma unroll
-      for (int r = 0; r < MR; ++r) iacc[r] = 0;
+      for (int r = 0; r < MR; ++r) da[r] = 0, db[r] = 0;
 #pragma unroll
-      for (int ju = 0; ju < UPB; ++ju) {
-        const int j = jb * UPB + ju;
-        uint32_t lo[4], hi[4];
+      for (int ju = 0; ju < UN; ++ju) {
+        const int j = jb * UN + ju;
+        uint32_t ws[4];
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-          lo[d] = w[j][d] & 0x0f0f0f0fu;
-          hi[d] = (w[j][d] >> 4) & 0x0f0f0f0fu;
-          ones = __builtin_amdgcn_sdot4(0x01010101, int(lo[d]), ones, false);
-          ones = __builtin_amdgcn_sdot4(0x01010101, int(hi[d]), ones, false);
+          ws[d] = w[j][d] ^ 0x88888888u;  // nib - 8 as signed nibbles
+          dc = __builtin_amdgcn_sdot8(0x11111111, int(ws[d]), dc, false);
         }
 #pragma unroll
         for (int r = 0; r < MR; ++r) {
-          const U4 qa = ldg<U4>(qrow[r] + uint64_t(unit0 + j) * kUnit);
-          const U4 qb = ldg<U4>(qrow[r] + uint64_t(unit0 + j) * kUnit + 16);
-          const uint32_t qq[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
-          int a = iacc[r];
+          const U4 qh = *reinterpret_cast<const U4*>(qbase + r * qs + j * kUnit);
+          const U4 ql = *reinterpret_cast<const U4*>(qbase + r * qs + j * kUnit + 16);
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
-            a = __builtin_amdgcn_sdot4(int(qq[2 * d]), int(lo[d]), a, false);
-            a = __builtin_amdgcn_sdot4(int(qq[2 * d + 1]), int(hi[d]), a, false);
+            da[r] = __builtin_amdgcn_sdot8(int(qh[d]), int(ws[d]), da[r], false);
+            db[r] = __builtin_amdgcn_sdot8(int(ql[d]), int(ws[d]), db[r], false);
           }
-          iacc[r] = a - 8 * ldg<int32_t>(sqrow[r] + uint64_t(unit0 + j) * 4);
         }
       }
+      if constexpr (UPB != 0) {
+        const bool valid = unit0 / UPB + jb < nblocks;
 #pragma unroll
-      for (int r = 0; r < MR; ++r) t[r][jb] = float(iacc[r] + nzp[r] * (ones - 8 * kUnit * UPB)) * s[jb];
+        for (int r = 0; r < MR; ++r) {
+          const int iacc = (da[r] << 4) + db[r] + nzp8[r] * dc;
+          t[r][jb] = valid ? float(iacc) * s[jb] : -0.0f;
+        }
+      } else {
+        tot_c += dc;
+#pragma unroll
+        for (int r = 0; r < MR; ++r) tot_a[r] += da[r], tot_b[r] += db[r];
+      }
     }
 
-    // pass the running float32 sums along each row of 16 lanes, in block order
-    const uint32_t blk0 = unit0 / UPB;
+    if constexpr (UPB != 0) {
+      // the running float32 sums travel through the 16 k-parts in order: wave by wave through
+      // LDS, and inside a wave from one group of 16 lanes to the next
 #pragma unroll 1
-    for (int ph = 0; ph < 16; ++ph) {
+      for (int stage = 0; stage < 4; ++stage) {
+        if (wave == stage) {
 #pragma unroll
-      for (int r = 0; r < MR; ++r) {
-        float a = dpp_f32<kRowRor1>(acc[r]);
-        if (part == ph) {
+          for (int r = 0; r < MR; ++r) {
+            float a = carry[r * kTileCols + col];
 #pragma unroll
-          for (int jb = 0; jb < BPL; ++jb) {
-            const uint32_t blk = blk0 + jb;
-            if (blk < nblocks) a = blk == 0 ? t[r][jb] : a + t[r][jb];
+            for (int gg = 0; gg < 4; ++gg) {
+              if (gg != 0) a = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane - 16) * 4, __builtin_bit_cast(int, acc[r])));
+              if (grp == gg) {
+#pragma unroll
+                for (int jb = 0; jb < BPL; ++jb) a = a + t[r][jb];
+                acc[r] = a;
+              }
+            }
+            if (grp == 3) carry[r * kTileCols + col] = acc[r];
           }
-          acc[r] = a;
         }
+        __syncthreads();
       }
+    }
+  }
+  if constexpr (UPB == 0) {
+    // one block: exact integer totals over the 16 k-parts, then one scaling
+#pragma unroll
+    for (int r = 0; r < MR; ++r) atomicAdd(&itotal[r * kTileCols + col], (tot_a[r] << 4) + tot_b[r] + nzp8[r] * tot_c);
+    __syncthreads();
+    if (part == 15) {
+      const float s = ldg<float>(p.compact + L.scale_off + (n < p.n ? n : p.n - 1) * 4ull);
+#pragma unroll
+      for (int r = 0; r < MR; ++r) acc[r] = float(itotal[r * kTileCols + col]) * s;
     }
   }
   if (part == 15 && n < p.n) {
     const float bias = ldg<float>(p.compact + L.bias_off + n * 4ull);
 #pragma unroll
-    for (int r = 0; r < MR; ++r) {
-      if (m0 + r < p.m) {
-        const float recip = bits_f32(ldg<uint32_t>(p.rows + 8ull * (m0 + r)));
-        finish_store<T>(p.out + (uint64_t(m0 + r) * p.n + n) * item, acc[r], recip, p.has_bias != 0, bias);
-      }
-    }
-  }
-}
-
-// Phase 1, channelwise (one block spanning K): integer partial sums per lane, one integer
-// reduction over the row of 16 lanes, one float32 scaling.
-template <class T, int MR>
-__global__ __launch_bounds__(256) void qmm4c_gemv_channelwise(Q4CParams p, CompactLayout L, uint32_t m0) {
-  constexpr uint64_t item = sizeof(typename T::storage);
-  const int lane = threadIdx.x & 63, part = lane & 15;
-  const uint32_t tile = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (tile >= L.tiles) return;
-  const uint32_t n = tile * kTileCols + (lane >> 4);
-  int nzp[MR], iacc[MR], ones = 0;
-  uint64_t qrow[MR], sqrow[MR];
-#pragma unroll
-  for (int r = 0; r < MR; ++r) {
-    const uint32_t m = m0 + r < p.m ? m0 + r : p.m - 1;
-    nzp[r] = ldg<int32_t>(p.rows + 8ull * m + 4);
-    qrow[r] = p.q + uint64_t(m) * L.kpad;
-    sqrow[r] = p.q + uint64_t(p.m) * L.kpad + uint64_t(m) * (L.kpad / kUnit) * 4;
-    iacc[r] = 0;
-  }
-  for (uint32_t round = 0; round < L.rounds; ++round) {
-    const uint64_t base = (uint64_t(tile) * L.rounds + round);
-    U4 w[kUnitsPerLane];
-#pragma unroll
-    for (int j = 0; j < kUnitsPerLane; ++j) w[j] = ldg<U4>(p.compact + ((base * kUnitsPerLane + j) * 64 + lane) * 16);
-    const uint32_t unit0 = round * kRoundUnits + part * kUnitsPerLane;
-#pragma unroll
-    for (int j = 0; j < kUnitsPerLane; ++j) {
-      uint32_t lo[4], hi[4];
-#pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        lo[d] = w[j][d] & 0x0f0f0f0fu;
-        hi[d] = (w[j][d] >> 4) & 0x0f0f0f0fu;
-        ones = __builtin_amdgcn_sdot4(0x01010101, int(lo[d]), ones, false);
-        ones = __builtin_amdgcn_sdot4(0x01010101, int(hi[d]), ones, false);
-      }
-#pragma unroll
-      for (int r = 0; r < MR; ++r) {
-        const U4 qa = ldg<U4>(qrow[r] + uint64_t(unit0 + j) * kUnit);
-        const U4 qb = ldg<U4>(qrow[r] + uint64_t(unit0 + j) * kUnit + 16);
-        const uint32_t qq[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
-        int a = iacc[r];
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          a = __builtin_amdgcn_sdot4(int(qq[2 * d]), int(lo[d]), a, false);
-          a = __builtin_amdgcn_sdot4(int(qq[2 * d + 1]), int(hi[d]), a, false);
-        }
-        iacc[r] = a - 8 * ldg<int32_t>(sqrow[r] + uint64_t(unit0 + j) * 4);
-      }
-    }
-  }
-  // every unit a lane visited (padding included) holds 32 nibbles; padding nibbles are 8
-  ones -= 8 * kUnit * kUnitsPerLane * int(L.rounds);
-#pragma unroll
-  for (int r = 0; r < MR; ++r) {
-    int v = iacc[r] + nzp[r] * ones;
-    v += dpp_i32<kQuadSwap1>(v);
-    v += dpp_i32<kQuadSwap2>(v);
-    v += dpp_i32<kRowHalfMirror>(v);
-    v += dpp_i32<kRowMirror>(v);
-    iacc[r] = v;
-  }
-  if (part == 15 && n < p.n) {
-    const float s = ldg<float>(p.compact + L.scale_off + n * 4ull);
-    const float bias = ldg<float>(p.compact + L.bias_off + n * 4ull);
-#pragma unroll
-    for (int r = 0; r < MR; ++r) {
-      if (m0 + r < p.m) {
-        const float recip = bits_f32(ldg<uint32_t>(p.rows + 8ull * (m0 + r)));
-        finish_store<T>(p.out + (uint64_t(m0 + r) * p.n + n) * item, float(iacc[r]) * s, recip, p.has_bias != 0, bias);
-      }
-    }
+    for (int r = 0; r < MR; ++r)
+      if (m0 + r < p.m) finish_store<T>(p.out + (uint64_t(m0 + r) * p.n + n) * item, acc[r], recip[r], p.has_bias != 0, bias);
   }
 }
 
@@ -458,27 +531,59 @@ bool check_q4_shape(uint32_t m, uint32_t n, uint32_t k, uint32_t bs, std::string
   return true;
 }
 
-template <class T, int MR>
-void launch_gemv_upb(const Q4CParams& p, const CompactLayout& L, uint32_t m0, hipStream_t stream) {
-  const dim3 grid((L.tiles + 3) / 4), block(256);
-  switch (L.upb) {
-    case 0: hipLaunchKernelGGL((qmm4c_gemv_channelwise<T, MR>), grid, block, 0, stream, p, L, m0); break;
-    case 1: hipLaunchKernelGGL((qmm4c_gemv<T, MR, 1>), grid, block, 0, stream, p, L, m0); break;
-    case 2: hipLaunchKernelGGL((qmm4c_gemv<T, MR, 2>), grid, block, 0, stream, p, L, m0); break;
-    case 4: hipLaunchKernelGGL((qmm4c_gemv<T, MR, 4>), grid, block, 0, stream, p, L, m0); break;
-    case 8: hipLaunchKernelGGL((qmm4c_gemv<T, MR, 8>), grid, block, 0, stream, p, L, m0); break;
+template <class T, int MR, int UPB, bool FUSED>
+int launch_stream_one(const Q4CParams& p, const CompactLayout& L, uint32_t m0, uint32_t groupwise, hipStream_t stream,
+                      std::string* err) {
+  auto kernel = qmm4c_stream<T, MR, UPB, FUSED>;
+  const uint32_t lds = q_lds_bytes(MR, L.kpad);
+  static uint32_t reserved = 48 * 1024;  // guarded by the runtime's stream mutex
+  if (lds > reserved) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds) !=
+        hipSuccess) {
+      (void)hipGetLastError();
+      *err = "qmm4c: cannot reserve " + std::to_string(lds) + " bytes of LDS";
+      return -1;
+    }
+    reserved = lds;
   }
+  hipLaunchKernelGGL(kernel, dim3(L.tiles), dim3(256), lds, stream, p, L, m0, groupwise);
+  return 0;
 }
 
-template <class T>
-void launch_gemv_rows(const Q4CParams& p, const CompactLayout& L, hipStream_t stream) {
-  for (uint32_t m0 = 0; m0 < p.m; m0 += 4) {
-    const uint32_t rows = p.m - m0;
-    if (rows >= 4) launch_gemv_upb<T, 4>(p, L, m0, stream);
-    else if (rows == 3) launch_gemv_upb<T, 3>(p, L, m0, stream);
-    else if (rows == 2) launch_gemv_upb<T, 2>(p, L, m0, stream);
-    else launch_gemv_upb<T, 1>(p, L, m0, stream);
+template <class T, int MR, bool FUSED>
+int launch_stream_upb(const Q4CParams& p, const CompactLayout& L, uint32_t m0, uint32_t groupwise, hipStream_t stream,
+                      std::string* err) {
+  switch (L.upb) {
+    case 0: return launch_stream_one<T, MR, 0, FUSED>(p, L, m0, groupwise, stream, err);
+    case 1: return launch_stream_one<T, MR, 1, FUSED>(p, L, m0, groupwise, stream, err);
+    case 2: return launch_stream_one<T, MR, 2, FUSED>(p, L, m0, groupwise, stream, err);
+    case 4: return launch_stream_one<T, MR, 4, FUSED>(p, L, m0, groupwise, stream, err);
+    case 8: return launch_stream_one<T, MR, 8, FUSED>(p, L, m0, groupwise, stream, err);
   }
+  *err = "qmm4c: bad layout";
+  return -1;
+}
+
+// Rows in groups of at most 4 (fewer when the activations of 4 rows would not fit in LDS).
+template <class T, bool FUSED>
+int launch_stream_rows(const Q4CParams& p, const CompactLayout& L, uint32_t groupwise, hipStream_t stream,
+                       std::string* err) {
+  uint32_t per = 4;
+  while (per > 1 && q_lds_bytes(per, L.kpad) > 144 * 1024) per /= 2;
+  if (q_lds_bytes(per, L.kpad) > 144 * 1024) {
+    *err = "qmm4c: k too large for the streaming kernel";
+    return -1;
+  }
+  for (uint32_t m0 = 0; m0 < p.m; m0 += per) {
+    const uint32_t rows = p.m - m0 < per ? p.m - m0 : per;
+    int rc;
+    if (rows >= 4) rc = launch_stream_upb<T, 4, FUSED>(p, L, m0, groupwise, stream, err);
+    else if (rows == 3) rc = launch_stream_upb<T, 3, FUSED>(p, L, m0, groupwise, stream, err);
+    else if (rows == 2) rc = launch_stream_upb<T, 2, FUSED>(p, L, m0, groupwise, stream, err);
+    else rc = launch_stream_upb<T, 1, FUSED>(p, L, m0, groupwise, stream, err);
+    if (rc != 0) return rc;
+  }
+  return 0;
 }
 
 }  // namespace
@@ -491,8 +596,7 @@ uint64_t qmm4c_bytes(uint32_t n, uint32_t k, uint32_t bs) {
 uint64_t qmm4c_q_bytes(uint32_t m, uint32_t k) {
   if (m == 0 || k == 0) return 0;
   const uint64_t nunits = (k + kUnit - 1) / kUnit, rounds = (nunits + kRoundUnits - 1) / kRoundUnits;
-  const uint64_t kpad = rounds * kRoundUnits * kUnit;
-  return round_up_u64(uint64_t(m) * kpad + uint64_t(m) * (kpad / kUnit) * 4, 256);
+  return round_up_u64(uint64_t(m) * rounds * kRoundUnits * kUnit, 256);
 }
 
 int launch_qmm4(const Q4Params& p, int dtype, uint32_t phase, uint32_t groupwise, const Machine&, hipStream_t stream,
@@ -554,7 +658,7 @@ int launch_qmm4c_pack(const Q4PackParams& p, const Machine&, hipStream_t stream,
   return 0;
 }
 
-int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwise, uint32_t, const Machine&,
+int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwise, uint32_t, const Machine& mc,
                  hipStream_t stream, std::string* err) {
   if (p.m == 0 || p.n == 0) return 0;
   CompactLayout L;
@@ -567,7 +671,7 @@ int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwi
     *err = "qmm4c: GROUPWISE must be 1 exactly when bs != k";
     return -1;
   }
-  if (!p.inp || !p.q || !p.rows || !p.out || (p.q & 15)) {
+  if (!p.inp || !p.out || (phase != 2 && (!p.q || !p.rows || (p.q & 15)))) {
     *err = "qmm4c: null or unaligned tensor address";
     return -1;
   }
@@ -585,10 +689,28 @@ int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwi
       *err = "qmm4c: null or unaligned side-car address";
       return -1;
     }
-    if (dtype == VKT_F32) launch_gemv_rows<f32_t>(p, L, stream);
-    else launch_gemv_rows<bf16_t>(p, L, stream);
+    const int rc = dtype == VKT_F32 ? launch_stream_rows<f32_t, false>(p, L, groupwise, stream, err)
+                                    : launch_stream_rows<bf16_t, false>(p, L, groupwise, stream, err);
+    if (rc != 0) return rc;
+  } else if (phase == 2) {
+    // both phases in one launch per group of rows when the rows can be quantised from
+    // registers (then p.q and p.rows are not touched); otherwise phase 0, then phase 1
+    if (!p.compact || (p.compact & 15)) {
+      *err = "qmm4c: null or unaligned side-car address";
+      return -1;
+    }
+    const uint32_t item = dtype == VKT_F32 ? 4 : 2;
+    const bool fuse = p.k % 8 == 0 && p.k <= 2048u * kFusedGroups && (p.inp & 15) == 0 && (uint64_t(p.k) * item) % 16 == 0;
+    if (!fuse) {
+      int rc = launch_qmm4c(p, dtype, 0, groupwise, 0, mc, stream, err);
+      if (rc == 0) rc = launch_qmm4c(p, dtype, 1, groupwise, 0, mc, stream, err);
+      return rc;
+    }
+    const int rc = dtype == VKT_F32 ? launch_stream_rows<f32_t, true>(p, L, groupwise, stream, err)
+                                    : launch_stream_rows<bf16_t, true>(p, L, groupwise, stream, err);
+    if (rc != 0) return rc;
   } else {
-    *err = "qmm4c: PHASE must be 0 or 1";
+    *err = "qmm4c: PHASE must be 0, 1 or 2";
     return -1;
   }
   if (hipGetLastError() != hipSuccess) {
