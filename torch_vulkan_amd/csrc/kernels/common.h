@@ -25,6 +25,12 @@ template <class X>
 __device__ __forceinline__ X ldg(uint64_t addr) {
   return *reinterpret_cast<const VKT_GLOBAL X*>(addr);
 }
+// A load of data that is read exactly once (the weight stream): non-temporal, so that it
+// does not displace the activations and scales that every wave re-reads from L2.
+template <class X>
+__device__ __forceinline__ X ldg_stream(uint64_t addr) {
+  return __builtin_nontemporal_load(reinterpret_cast<const VKT_GLOBAL X*>(addr));
+}
 template <class X>
 __device__ __forceinline__ void stg(uint64_t addr, X v) {
   *reinterpret_cast<VKT_GLOBAL X*>(addr) = v;

@@ -28,6 +28,8 @@
 //                  The B matrix feeds the MFMA's first operand and A its second, so a lane
 //                  ends up with 4 consecutive output columns of one row (vector stores).
 //   fp8mm_generic  any shape / alignment: one thread per output, float32 FMA.
+#include <type_traits>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -117,7 +119,7 @@ __device__ __forceinline__ uint32_t tile_offset(uint32_t row, uint32_t chunk) {
   return row * BK + ((chunk ^ (row & 7u)) << 4);
 }
 
-template <int WAVES_M, int WAVES_N, int TM, int TN, int FA, int FB>
+template <int WAVES_M, int WAVES_N, int TM, int TN, int FA, int FB, int DBG = 0>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, uint32_t tiles_m, uint32_t tiles_n) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * TM * 16, BN = WAVES_N * TN * 16;
@@ -173,47 +175,112 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, 
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = V4F{0.0f, 0.0f, 0.0f, 0.0f};
 
-  V4I a_reg[A_CHUNKS], b_reg[B_CHUNKS];
+  // Operand staging, software pipelined by hand.  One wave per SIMD means nothing else hides
+  // what this wave does not: every global load and LDS write is issued between two MFMAs,
+  // never in a block of its own.  Per k-step the 16-byte chunks a thread moves form two sets
+  // (A rows, B rows); while the matrix core works through step s the wave, in four quarters,
+  //   writes set A of step s+1 to LDS, loads set A of step s+2 into the same registers,
+  //   writes set B of step s+1,        loads set B of step s+2,
+  // so a load has three quarters of a step to arrive and the registers hold one set each.
+  constexpr int NC = A_CHUNKS + B_CHUNKS;      // chunks per thread per step
+  constexpr int NSIDE = 2 * NC, NMFMA = TM * TN;  // side operations / MFMAs per step
+  V4I reg[NC];
   const V4I zero = {0, 0, 0, 0};
-  auto fetch = [&](uint32_t k0) {
-#pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) a_reg[i] = k0 + a_k[i] < p.k ? ldg<V4I>(a_src[i] + k0) : zero;
-#pragma unroll
-    for (int i = 0; i < B_CHUNKS; ++i) b_reg[i] = k0 + b_k[i] < p.k ? ldg<V4I>(b_src[i] + k0) : zero;
+  const uint32_t steps = (p.k + BK - 1) / BK;
+  // chunk c: A chunks first, then B chunks
+  // A full step's chunk is loaded as is: nothing may touch the register until the LDS write,
+  // or the wave would wait for the load where it was issued.  Only the last step of a k that
+  // is not a multiple of 128 pays for a select (chunks beyond k read as zeros).
+  auto load_chunk = [&](int c, uint32_t k0) {
+    const uint64_t src = c < A_CHUNKS ? a_src[c < A_CHUNKS ? c : 0] : b_src[c < A_CHUNKS ? 0 : c - A_CHUNKS];
+    reg[c] = ldg<V4I>(src + k0);
   };
-  auto stash = [&](uint32_t stage) {
-    uint8_t* base = lds + stage * STAGE;
-#pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) *reinterpret_cast<V4I*>(base + a_dst[i]) = a_reg[i];
-#pragma unroll
-    for (int i = 0; i < B_CHUNKS; ++i) *reinterpret_cast<V4I*>(base + b_dst[i]) = b_reg[i];
+  auto load_chunk_tail = [&](int c, uint32_t k0) {
+    const uint64_t src = c < A_CHUNKS ? a_src[c < A_CHUNKS ? c : 0] : b_src[c < A_CHUNKS ? 0 : c - A_CHUNKS];
+    const uint32_t kc = c < A_CHUNKS ? a_k[c < A_CHUNKS ? c : 0] : b_k[c < A_CHUNKS ? 0 : c - A_CHUNKS];
+    const bool inside = k0 + kc < p.k;
+    const V4I v = ldg<V4I>(src + (inside ? k0 : 0));  // (k >= 16: chunk 0 of the row exists)
+    reg[c] = inside ? v : zero;
+  };
+  const uint32_t full_steps = p.k / BK;  // steps whose 128 bytes all lie inside k
+  auto load_step = [&](int c, uint32_t step) {
+    if (step < full_steps) load_chunk(c, step * BK);
+    else load_chunk_tail(c, step * BK);
+  };
+  auto store_chunk = [&](int c, uint32_t stage) {
+    const uint32_t dst = c < A_CHUNKS ? a_dst[c < A_CHUNKS ? c : 0] : b_dst[c < A_CHUNKS ? 0 : c - A_CHUNKS];
+    *reinterpret_cast<V4I*>(lds + stage * STAGE + dst) = reg[c];
   };
   auto fragment = [&](const uint8_t* tile, uint32_t row) {
     const V4I lo = *reinterpret_cast<const V4I*>(tile + tile_offset(row, 2 * g));
     const V4I hi = *reinterpret_cast<const V4I*>(tile + tile_offset(row, 2 * g + 1));
     return V8I{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
-
-  const uint32_t steps = (p.k + BK - 1) / BK;
-  fetch(0);
-  stash(0);
-  __syncthreads();
-  for (uint32_t s = 0; s < steps; ++s) {
-    if (s + 1 < steps) fetch((s + 1) * BK);
+  // Side operation `op` of step s: [0,AC) write A chunks of step s+1, [AC,2AC) load A chunks
+  // of step s+2, then the same for the B chunks.  STEADY: both steps exist and are full, so
+  // the code is straight-line (a branch here would make the compiler wait for every load
+  // where it is issued).
+  auto side = [&](int op, uint32_t s, auto steady) {
+    constexpr bool kSteady = decltype(steady)::value;
+    constexpr int AC = A_CHUNKS, BC = B_CHUNKS;
+    if (op < AC) {
+      if (kSteady || s + 1 < steps) store_chunk(op, (s + 1) & 1u);
+    } else if (op < 2 * AC) {
+      if (kSteady) load_chunk(op - AC, (s + 2) * BK);
+      else if (s + 2 < steps) load_step(op - AC, s + 2);
+    } else if (op < 2 * AC + BC) {
+      if (kSteady || s + 1 < steps) store_chunk(AC + op - 2 * AC, (s + 1) & 1u);
+    } else {
+      if (kSteady) load_chunk(AC + op - 2 * AC - BC, (s + 2) * BK);
+      else if (s + 2 < steps) load_step(AC + op - 2 * AC - BC, s + 2);
+    }
+  };
+  // One k-step: the wave's TM x TN MFMAs with the side operations and the LDS reads of the
+  // next row fragment spread between them; the scheduling barriers keep the compiler from
+  // moving anything back into blocks.
+  auto step = [&](uint32_t s, auto steady) {
     const uint8_t* ta = lds + (s & 1u) * STAGE;
     const uint8_t* tb = ta + BM * BK;
     V8I bf[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j) bf[j] = fragment(tb, (wn * TN + j) * 16 + l16);
+    V8I af = fragment(ta, (wm * TM) * 16 + l16);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      const V8I af = fragment(ta, (wm * TM + i) * 16 + l16);
+      V8I next = af;
+      if (i + 1 < TM) next = fragment(ta, (wm * TM + i + 1) * 16 + l16);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = mfma_f8<FA, FB>(bf[j], af, acc[i][j]);
+      for (int j = 0; j < TN; ++j) {
+        const int n = i * TN + j;
+        const int lo_op = n * NSIDE / NMFMA, hi_op = (n + 1) * NSIDE / NMFMA;
+#pragma unroll
+        for (int op = lo_op; op < hi_op; ++op) {
+          if (!(DBG & 1)) side(op, s, steady);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        acc[i][j] = mfma_f8<FA, FB>(bf[j], af, acc[i][j]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      af = next;
     }
-    if (s + 1 < steps) stash((s + 1) & 1u);
-    __syncthreads();
+    if (!(DBG & 4)) __syncthreads();
+  };
+
+  // prologue: step 0 into LDS, step 1 into the registers
+#pragma unroll
+  for (int c = 0; c < NC; ++c) load_step(c, 0);
+#pragma unroll
+  for (int c = 0; c < NC; ++c) store_chunk(c, 0);
+  if (steps > 1) {
+#pragma unroll
+    for (int c = 0; c < NC; ++c) load_step(c, 1);
   }
+  __syncthreads();
+
+  uint32_t s = 0;
+  for (; s + 2 < full_steps; ++s) step(s, std::true_type{});
+  for (; s < steps; ++s) step(s, std::false_type{});
 
   // Epilogue.  A lane holds out[m = .. + l16][n = .. + 4 g + r], r = 0..3, for each of its
   // TM x TN tiles.  Each wave transposes its sub-tile through its own slice of LDS (the
@@ -301,13 +368,13 @@ __global__ __launch_bounds__(256) void fp8mm_generic(F8Params p) {
   store_out(p, uint64_t(m) * p.ldo + n, finish(p, acc, sa, sb, n, output_inv(p)));
 }
 
-template <int WAVES_M, int WAVES_N, int TM, int TN, int FA, int FB>
+template <int WAVES_M, int WAVES_N, int TM, int TN, int FA, int FB, int DBG = 0>
 int launch_tile(const F8Params& p, hipStream_t stream, std::string* err) {
   constexpr int BM = WAVES_M * TM * 16, BN = WAVES_N * TN * 16;
   constexpr uint32_t operand_bytes = 2 * (BM + BN) * BK, epilogue_bytes = WAVES_M * WAVES_N * TM * 16 * 256;
   constexpr uint32_t lds_bytes = operand_bytes > epilogue_bytes ? operand_bytes : epilogue_bytes;
   static_assert(TN % 4 == 0, "the epilogue moves 64 columns (4 tiles) per pass");
-  auto kernel = fp8mm_mfma<WAVES_M, WAVES_N, TM, TN, FA, FB>;
+  auto kernel = fp8mm_mfma<WAVES_M, WAVES_N, TM, TN, FA, FB, DBG>;
   static bool configured = false;  // guarded by the runtime's stream mutex
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -339,6 +406,10 @@ int launch_formats(const F8Params& p, uint32_t variant, hipStream_t stream, std:
     case 1: return launch_tile<2, 2, 4, 4, FA, FB>(p, stream, err);
     case 2: return launch_tile<2, 2, 8, 8, FA, FB>(p, stream, err);
     case 3: return launch_tile<2, 2, 8, 4, FA, FB>(p, stream, err);
+    case 101: return launch_tile<2, 2, 8, 8, FA, FB, 1>(p, stream, err);
+    case 102: return launch_tile<2, 2, 8, 8, FA, FB, 2>(p, stream, err);
+    case 103: return launch_tile<2, 2, 8, 8, FA, FB, 3>(p, stream, err);
+    case 107: return launch_tile<2, 2, 8, 8, FA, FB, 7>(p, stream, err);
   }
   *err = "fp8mm: unknown variant " + std::to_string(variant);
   return -1;

@@ -346,7 +346,7 @@ __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L
   {
     const uint64_t base = (uint64_t(tile) * L.rounds * 4 + wave) * kUnitsPerLane;
 #pragma unroll
-    for (int j = 0; j < kUnitsPerLane; ++j) w[j] = ldg<U4>(p.compact + ((base + j) * 64 + lane) * 16);
+    for (int j = 0; j < kUnitsPerLane; ++j) w[j] = ldg_stream<U4>(p.compact + ((base + j) * 64 + lane) * 16);
   }
 
   int nzp8[MR];  // 8 - zero_point
@@ -416,13 +416,13 @@ __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L
     const uint64_t base = (uint64_t(tile) * L.rounds + round) * 4 + wave;
     if (round != 0) {
 #pragma unroll
-      for (int j = 0; j < kUnitsPerLane; ++j) w[j] = ldg<U4>(p.compact + ((base * kUnitsPerLane + j) * 64 + lane) * 16);
+      for (int j = 0; j < kUnitsPerLane; ++j) w[j] = ldg_stream<U4>(p.compact + ((base * kUnitsPerLane + j) * 64 + lane) * 16);
     }
     float s[BPL];
     if constexpr (UPB != 0) {
       const uint64_t sp = p.compact + L.scale_off + (base * 64 + lane) * BPL * 4;
       if constexpr (BPL == 8) {
-        const F4 s0 = ldg<F4>(sp), s1 = ldg<F4>(sp + 16);
+        const F4 s0 = ldg_stream<F4>(sp), s1 = ldg_stream<F4>(sp + 16);
         s[0] = s0.x, s[1] = s0.y, s[2] = s0.z, s[3] = s0.w, s[4] = s1.x, s[5] = s1.y, s[6] = s1.z, s[7] = s1.w;
       } else if constexpr (BPL == 4) {
         const F4 s0 = ldg<F4>(sp);

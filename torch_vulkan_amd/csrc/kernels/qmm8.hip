@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) void qmm8_gemv(Q8Params p) {
   for (uint32_t k = (ks * 64 + lane) * 16; k < p.k; k += 1024 * KSPLIT) {
     U4 wv[COLS];
 #pragma unroll
-    for (int c = 0; c < COLS; ++c) wv[c] = ldg<U4>(brow[c] + k);
+    for (int c = 0; c < COLS; ++c) wv[c] = ldg_stream<U4>(brow[c] + k);
     float w[COLS][16];
 #pragma unroll
     for (int c = 0; c < COLS; ++c) widen16_i8(wv[c], w[c]);
