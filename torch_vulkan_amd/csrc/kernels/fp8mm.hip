@@ -19,11 +19,11 @@
 // The scales multiply once per output instead of once per operand element (one rounding
 // less than the reference, inside the same bound).
 //
-//   fp8mm_mfma     V_MFMA_F32_16X16X128_F8F6F4 (8192 flop/clk/CU: the only fp8 rate that
-//                  reaches the 5 PFLOP/s peak; the 16x16x32 fp8 instruction runs at half).
+//   fp8mm_mfma     V_MFMA_F32_32X32X64_F8F6F4 / 16X16X128 (8192 flop/clk/CU: the only fp8 rate
+//                  that reaches the 5 PFLOP/s peak; the 16x16x32 fp8 instruction runs at half).
 //                  A workgroup computes a BM x BN tile, K in steps of 128 bytes; both
 //                  operand tiles are staged in LDS (double buffered, 16-byte chunks XOR-
-//                  swizzled by row so that the 32-byte-per-lane fragment reads are
+//                  swizzled by row pair so that the 32-byte-per-lane fragment reads are
 //                  conflict free), each wave owns a (TM*16) x (TN*16) sub-tile in registers.
 //                  The B matrix feeds the MFMA's first operand and A its second, so a lane
 //                  ends up with 4 consecutive output columns of one row (vector stores).
@@ -114,12 +114,23 @@ __device__ __forceinline__ V4F mfma_f8(const V8I& first, const V8I& second, cons
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(first, second, acc, FB, FA, 0, 0, 0, 0);
 }
 
-// LDS tile: rows of 128 bytes; 16-byte chunk c of row r sits at chunk c ^ (r & 7).
-__device__ __forceinline__ uint32_t tile_offset(uint32_t row, uint32_t chunk) {
-  return row * BK + ((chunk ^ (row & 7u)) << 4);
+using V16F = float __attribute__((ext_vector_type(16)));
+template <int FA, int FB>
+__device__ __forceinline__ V16F mfma_f8_32(const V8I& first, const V8I& second, const V16F& acc) {
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(first, second, acc, FB, FA, 0, 0, 0, 0);
 }
 
-template <int WAVES_M, int WAVES_N, int TM, int TN, int FA, int FB, int DBG = 0>
+// LDS tile: rows of 128 bytes; 16-byte chunk c of row r sits at chunk c ^ ((r >> 1) & 7).
+// The LDS serves 16 lanes of a 128-bit read per clock from 64 banks (256 bytes), and the 16
+// lanes of a fragment read hold 16 consecutive rows at one logical chunk: two rows share a
+// 256-byte line, and the key changes every two rows, so the 16 lanes land on 16 different
+// 16-byte slots of the line (keying on r & 7 made rows r and r + 8 collide: measured as 4
+// conflict cycles on every read).
+__device__ __forceinline__ uint32_t tile_offset(uint32_t row, uint32_t chunk) {
+  return row * BK + ((chunk ^ ((row >> 1) & 7u)) << 4);
+}
+
+template <int WAVES_M, int WAVES_N, int TM, int TN, int FA, int FB, bool MF32 = false, bool DIRECT = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, uint32_t tiles_m, uint32_t tiles_n) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * TM * 16, BN = WAVES_N * TN * 16;
@@ -154,7 +165,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, 
   uint32_t a_dst[A_CHUNKS], b_dst[B_CHUNKS], a_k[A_CHUNKS], b_k[B_CHUNKS];
 #pragma unroll
   for (int i = 0; i < A_CHUNKS; ++i) {
-    const uint32_t id = tid + NT * i, row = id >> 3, c = id & 7u;
+    // DIRECT: the load lands at LDS slot id (lane order), so the lane fetches the logical
+    // chunk that the swizzle keeps in that slot
+    const uint32_t id = tid + NT * i, row = id >> 3, c = DIRECT ? (id & 7u) ^ ((row >> 1) & 7u) : id & 7u;
     const uint32_t m = m0 + row < p.m ? m0 + row : p.m - 1;
     a_src[i] = p.a + uint64_t(m) * p.lda + c * 16;
     a_dst[i] = tile_offset(row, c);
@@ -162,28 +175,40 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, 
   }
 #pragma unroll
   for (int i = 0; i < B_CHUNKS; ++i) {
-    const uint32_t id = tid + NT * i, row = id >> 3, c = id & 7u;
+    const uint32_t id = tid + NT * i, row = id >> 3, c = DIRECT ? (id & 7u) ^ ((row >> 1) & 7u) : id & 7u;
     const uint32_t n = n0 + row < p.n ? n0 + row : p.n - 1;
     b_src[i] = p.b + uint64_t(n) * p.ldb + c * 16;
     b_dst[i] = BM * BK + tile_offset(row, c);
     b_k[i] = c * 16;
   }
 
-  V4F acc[TM][TN];
+  // MF32: the wave's sub-tile as (TM/2) x (TN/2) tiles of 32x32 (V_MFMA_F32_32X32X64_F8F6F4,
+  // two per k-step along k); otherwise TM x TN tiles of 16x16 (one 16X16X128 per k-step).
+  // Both leave a lane with groups of 4 consecutive output columns of one row.
+  constexpr int TM2 = MF32 ? TM / 2 : 1, TN2 = MF32 ? TN / 2 : 1;
+  V4F acc[MF32 ? 1 : TM][MF32 ? 1 : TN];
+  V16F acc32[TM2][TN2];
+  if constexpr (MF32) {
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM2; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j) acc[i][j] = V4F{0.0f, 0.0f, 0.0f, 0.0f};
+      for (int j = 0; j < TN2; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc32[i][j][r] = 0.0f;
+  } else {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = V4F{0.0f, 0.0f, 0.0f, 0.0f};
+  }
 
   // Operand staging, software pipelined by hand.  One wave per SIMD means nothing else hides
   // what this wave does not: every global load and LDS write is issued between two MFMAs,
-  // never in a block of its own.  Per k-step the 16-byte chunks a thread moves form two sets
-  // (A rows, B rows); while the matrix core works through step s the wave, in four quarters,
-  //   writes set A of step s+1 to LDS, loads set A of step s+2 into the same registers,
-  //   writes set B of step s+1,        loads set B of step s+2,
-  // so a load has three quarters of a step to arrive and the registers hold one set each.
+  // never in a block of its own.  While the matrix core works through step s the wave writes
+  // the chunks of step s+1 from registers to LDS (first half of the step) and loads the
+  // chunks of step s+2 into the same registers (second half).
   constexpr int NC = A_CHUNKS + B_CHUNKS;      // chunks per thread per step
-  constexpr int NSIDE = 2 * NC, NMFMA = TM * TN;  // side operations / MFMAs per step
+  constexpr int NSIDE = DIRECT ? NC : 2 * NC, NMFMA = MF32 ? TM * TN / 2 : TM * TN;  // side operations / MFMAs per step
   V4I reg[NC];
   const V4I zero = {0, 0, 0, 0};
   const uint32_t steps = (p.k + BK - 1) / BK;
@@ -216,23 +241,31 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, 
     const V4I hi = *reinterpret_cast<const V4I*>(tile + tile_offset(row, 2 * g + 1));
     return V8I{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
-  // Side operation `op` of step s: [0,AC) write A chunks of step s+1, [AC,2AC) load A chunks
-  // of step s+2, then the same for the B chunks.  STEADY: both steps exist and are full, so
-  // the code is straight-line (a branch here would make the compiler wait for every load
-  // where it is issued).
+  // Side operation `op` of step s: [0,NC) write the chunks of step s+1 to LDS, [NC,2NC) load
+  // the chunks of step s+2 into the same registers (all writes first: when the next step's
+  // writes begin, every load is at least half a step old).  STEADY: both steps exist and are
+  // full, so the code is straight-line (a branch here would make the compiler wait for
+  // every load where it is issued).
+  // DIRECT (k a multiple of 128): global_load_lds_dwordx4 moves a chunk from global memory
+  // straight into LDS (a wave's 64 lanes fill 1 KiB at a wave-uniform base, in lane order):
+  // no staging registers, no LDS write instructions.  The chunks of step s+1 go into the
+  // stage that step s-1 read, while step s computes.
+  auto direct_chunk = [&](int c, uint32_t step) {
+    const uint64_t src = c < A_CHUNKS ? a_src[c < A_CHUNKS ? c : 0] : b_src[c < A_CHUNKS ? 0 : c - A_CHUNKS];
+    const uint32_t tile_base = c < A_CHUNKS ? uint32_t(c) * NT * 16 : BM * BK + uint32_t(c - A_CHUNKS) * NT * 16;
+    uint8_t* dst = lds + (step & 1u) * STAGE + tile_base + uint32_t(wave) * 1024;
+    __builtin_amdgcn_global_load_lds(reinterpret_cast<const VKT_GLOBAL void*>(src + uint64_t(step) * BK),
+                                     (__attribute__((address_space(3))) void*)(dst), 16, 0, 0);
+  };
   auto side = [&](int op, uint32_t s, auto steady) {
     constexpr bool kSteady = decltype(steady)::value;
-    constexpr int AC = A_CHUNKS, BC = B_CHUNKS;
-    if (op < AC) {
+    if constexpr (DIRECT) {
+      if (kSteady || s + 1 < steps) direct_chunk(op, s + 1);
+    } else if (op < NC) {
       if (kSteady || s + 1 < steps) store_chunk(op, (s + 1) & 1u);
-    } else if (op < 2 * AC) {
-      if (kSteady) load_chunk(op - AC, (s + 2) * BK);
-      else if (s + 2 < steps) load_step(op - AC, s + 2);
-    } else if (op < 2 * AC + BC) {
-      if (kSteady || s + 1 < steps) store_chunk(AC + op - 2 * AC, (s + 1) & 1u);
     } else {
-      if (kSteady) load_chunk(AC + op - 2 * AC - BC, (s + 2) * BK);
-      else if (s + 2 < steps) load_step(AC + op - 2 * AC - BC, s + 2);
+      if (kSteady) load_chunk(op - NC, (s + 2) * BK);
+      else if (s + 2 < steps) load_step(op - NC, s + 2);
     }
   };
   // One k-step: the wave's TM x TN MFMAs with the side operations and the LDS reads of the
@@ -241,46 +274,91 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, 
   auto step = [&](uint32_t s, auto steady) {
     const uint8_t* ta = lds + (s & 1u) * STAGE;
     const uint8_t* tb = ta + BM * BK;
-    V8I bf[TN];
+    if constexpr (MF32) {
+      // lane: row lane % 32 of a 32-row tile, 32 bytes of k at chunk pair 4 kk + 2 (lane / 32)
+      const int l32 = lane & 31, h = lane >> 5;
+      auto frag32 = [&](const uint8_t* tile, uint32_t row, int kk) {
+        const V4I lo = *reinterpret_cast<const V4I*>(tile + tile_offset(row, 4 * kk + 2 * h));
+        const V4I hi = *reinterpret_cast<const V4I*>(tile + tile_offset(row, 4 * kk + 2 * h + 1));
+        return V8I{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      };
+      V8I bf[2][TN2];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) bf[j] = fragment(tb, (wn * TN + j) * 16 + l16);
-    V8I af = fragment(ta, (wm * TM) * 16 + l16);
+      for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      V8I next = af;
-      if (i + 1 < TM) next = fragment(ta, (wm * TM + i + 1) * 16 + l16);
-      __builtin_amdgcn_sched_barrier(0);
+        for (int j = 0; j < TN2; ++j) bf[kk][j] = frag32(tb, (wn * TN2 + j) * 32 + l32, kk);
+      V8I af = frag32(ta, (wm * TM2) * 32 + l32, 0);
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int n = i * TN + j;
-        const int lo_op = n * NSIDE / NMFMA, hi_op = (n + 1) * NSIDE / NMFMA;
+      for (int gi = 0; gi < 2 * TM2; ++gi) {
+        const int kk = gi / TM2, i = gi % TM2;
+        V8I next = af;
+        if (gi + 1 < 2 * TM2) next = frag32(ta, (wm * TM2 + (gi + 1) % TM2) * 32 + l32, (gi + 1) / TM2);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int op = lo_op; op < hi_op; ++op) {
-          if (!(DBG & 1)) side(op, s, steady);
-          __builtin_amdgcn_sched_barrier(0);
+        for (int j = 0; j < TN2; ++j) {
+          const int n = gi * TN2 + j;
+          const int lo_op = n * NSIDE / NMFMA, hi_op = (n + 1) * NSIDE / NMFMA;
+#pragma unroll
+          for (int op = lo_op; op < hi_op; ++op) {
+            side(op, s, steady);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          acc32[i][j] = mfma_f8_32<FA, FB>(bf[kk][j], af, acc32[i][j]);
         }
-        acc[i][j] = mfma_f8<FA, FB>(bf[j], af, acc[i][j]);
+        __builtin_amdgcn_sched_barrier(0);
+        af = next;
       }
-      __builtin_amdgcn_sched_barrier(0);
-      af = next;
+    } else {
+      V8I bf[TN];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) bf[j] = fragment(tb, (wn * TN + j) * 16 + l16);
+      V8I af = fragment(ta, (wm * TM) * 16 + l16);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        V8I next = af;
+        if (i + 1 < TM) next = fragment(ta, (wm * TM + i + 1) * 16 + l16);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int n = i * TN + j;
+          const int lo_op = n * NSIDE / NMFMA, hi_op = (n + 1) * NSIDE / NMFMA;
+#pragma unroll
+          for (int op = lo_op; op < hi_op; ++op) {
+            side(op, s, steady);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          acc[i][j] = mfma_f8<FA, FB>(bf[j], af, acc[i][j]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        af = next;
+      }
     }
-    if (!(DBG & 4)) __syncthreads();
+    if constexpr (DIRECT) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this step's LDS-direct loads have landed
+    __syncthreads();
   };
 
-  // prologue: step 0 into LDS, step 1 into the registers
-#pragma unroll
-  for (int c = 0; c < NC; ++c) load_step(c, 0);
-#pragma unroll
-  for (int c = 0; c < NC; ++c) store_chunk(c, 0);
-  if (steps > 1) {
-#pragma unroll
-    for (int c = 0; c < NC; ++c) load_step(c, 1);
-  }
-  __syncthreads();
-
   uint32_t s = 0;
-  for (; s + 2 < full_steps; ++s) step(s, std::true_type{});
-  for (; s < steps; ++s) step(s, std::false_type{});
+  if constexpr (DIRECT) {
+#pragma unroll
+    for (int c = 0; c < NC; ++c) direct_chunk(c, 0);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    for (; s + 1 < steps; ++s) step(s, std::true_type{});
+    for (; s < steps; ++s) step(s, std::false_type{});
+  } else {
+    // prologue: step 0 into LDS, step 1 into the registers
+#pragma unroll
+    for (int c = 0; c < NC; ++c) load_step(c, 0);
+#pragma unroll
+    for (int c = 0; c < NC; ++c) store_chunk(c, 0);
+    if (steps > 1) {
+#pragma unroll
+      for (int c = 0; c < NC; ++c) load_step(c, 1);
+    }
+    __syncthreads();
+    for (; s + 2 < full_steps; ++s) step(s, std::true_type{});
+    for (; s < steps; ++s) step(s, std::false_type{});
+  }
 
   // Epilogue.  A lane holds out[m = .. + l16][n = .. + 4 g + r], r = 0..3, for each of its
   // TM x TN tiles.  Each wave transposes its sub-tile through its own slice of LDS (the
@@ -299,14 +377,29 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, 
     // (the first pass may start only when every wave is done reading operands; later ones
     // when this wave's previous pass has been read back)
     __syncthreads();
+    if constexpr (MF32) {
+      // a 32x32 tile leaves lane l with row l % 32 and, for q = 0..3, columns 8 q + 4 (l / 32) .. + 3
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < TM2; ++i)
 #pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const uint32_t row = i * 16 + l16, chunk = jj * 4 + g;
-        *reinterpret_cast<V4F*>(reinterpret_cast<uint8_t*>(ep) + row * EP_ROW + ((chunk ^ (row & 7u)) << 4)) =
-            acc[i][pass * 4 + jj];
-      }
+        for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const uint32_t row = i * 32 + (lane & 31), chunk = jj * 8 + 2 * q + (lane >> 5);
+            const V16F& t = acc32[i][pass * 2 + jj];
+            *reinterpret_cast<V4F*>(reinterpret_cast<uint8_t*>(ep) + row * EP_ROW + ((chunk ^ (row & 15u)) << 4)) =
+                V4F{t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
+          }
+    } else {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          const uint32_t row = i * 16 + l16, chunk = jj * 4 + g;
+          *reinterpret_cast<V4F*>(reinterpret_cast<uint8_t*>(ep) + row * EP_ROW + ((chunk ^ (row & 15u)) << 4)) =
+              acc[i][pass * 4 + jj];
+        }
+    }
     __syncthreads();
     // lane -> (row offset lane / 16, chunk lane % 16): 4 consecutive columns, fixed over the loop
     const uint32_t chunk = lane & 15, n = wn0 + pass * 64 + chunk * 4;
@@ -322,7 +415,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, 
     for (uint32_t it = 0; it < TM * 4; ++it) {
       const uint32_t row = it * 4 + (lane >> 4), m = wm0 + row;
       const V4F t = *reinterpret_cast<const V4F*>(reinterpret_cast<const uint8_t*>(ep) + row * EP_ROW +
-                                                   ((chunk ^ (row & 7u)) << 4));
+                                                   ((chunk ^ (row & 15u)) << 4));
       if (m >= p.m || n >= p.n) continue;
       const float sa = p.rowwise ? ldg<float>(p.scale_a + 4ull * m) : sa_all;
       float v[4];
@@ -368,13 +461,13 @@ __global__ __launch_bounds__(256) void fp8mm_generic(F8Params p) {
   store_out(p, uint64_t(m) * p.ldo + n, finish(p, acc, sa, sb, n, output_inv(p)));
 }
 
-template <int WAVES_M, int WAVES_N, int TM, int TN, int FA, int FB, int DBG = 0>
+template <int WAVES_M, int WAVES_N, int TM, int TN, int FA, int FB, bool MF32 = false, bool DIRECT = false>
 int launch_tile(const F8Params& p, hipStream_t stream, std::string* err) {
   constexpr int BM = WAVES_M * TM * 16, BN = WAVES_N * TN * 16;
   constexpr uint32_t operand_bytes = 2 * (BM + BN) * BK, epilogue_bytes = WAVES_M * WAVES_N * TM * 16 * 256;
   constexpr uint32_t lds_bytes = operand_bytes > epilogue_bytes ? operand_bytes : epilogue_bytes;
   static_assert(TN % 4 == 0, "the epilogue moves 64 columns (4 tiles) per pass");
-  auto kernel = fp8mm_mfma<WAVES_M, WAVES_N, TM, TN, FA, FB, DBG>;
+  auto kernel = fp8mm_mfma<WAVES_M, WAVES_N, TM, TN, FA, FB, MF32, DIRECT>;
   static bool configured = false;  // guarded by the runtime's stream mutex
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -398,18 +491,20 @@ int launch_tile(const F8Params& p, hipStream_t stream, std::string* err) {
 
 template <int FA, int FB>
 int launch_formats(const F8Params& p, uint32_t variant, hipStream_t stream, std::string* err) {
-  // variant 0: planned; 1: 128x128 tiles (4 waves of 64x64); 2: 256x256 (4 waves of 128x128);
-  // 3: 256x128 (4 waves of 128x64); 255: the one-thread-per-output kernel.  An explicit
-  // tile variant runs the MFMA kernel whatever the output dtype (tests, tuning).
-  if (variant == 0) variant = (uint64_t(p.m) * p.n >= (1ull << 22)) ? 2 : 1;
+  // variant 0: planned.  Explicit variants run the MFMA kernel whatever the output dtype
+  // (tests, tuning): 1: 128x128 tiles (4 waves of 64x64, 16x16x128 MFMA); 2: 256x256 (4 waves of
+  // 128x128, 16x16x128); 3: 256x128; 4: 256x256 with the 32x32x64 MFMA (measured ~10 % faster
+  // than 16x16x128 at equal work); 5: as 4 with global-to-LDS direct loads when k is a
+  // multiple of 128 (else 4).  255: the one-thread-per-output kernel.
+  if (variant == 0) variant = (uint64_t(p.m) * p.n >= (1ull << 20)) ? 5 : 1;
   switch (variant) {
     case 1: return launch_tile<2, 2, 4, 4, FA, FB>(p, stream, err);
     case 2: return launch_tile<2, 2, 8, 8, FA, FB>(p, stream, err);
     case 3: return launch_tile<2, 2, 8, 4, FA, FB>(p, stream, err);
-    case 101: return launch_tile<2, 2, 8, 8, FA, FB, 1>(p, stream, err);
-    case 102: return launch_tile<2, 2, 8, 8, FA, FB, 2>(p, stream, err);
-    case 103: return launch_tile<2, 2, 8, 8, FA, FB, 3>(p, stream, err);
-    case 107: return launch_tile<2, 2, 8, 8, FA, FB, 7>(p, stream, err);
+    case 4: return launch_tile<2, 2, 8, 8, FA, FB, true>(p, stream, err);
+    case 5:
+      if (p.k % BK == 0) return launch_tile<2, 2, 8, 8, FA, FB, true, true>(p, stream, err);
+      return launch_tile<2, 2, 8, 8, FA, FB, true>(p, stream, err);
   }
   *err = "fp8mm: unknown variant " + std::to_string(variant);
   return -1;
