@@ -113,6 +113,15 @@ typedef struct Q4Params {
   uint32_t m, n, k, bs, has_bias, pad;
 } Q4Params;
 
+/* "qmm4_packvec", spec {}: aten::_dyn_quant_pack_4bit_weight (quant.cpp:127-144): the
+ * float32 vector cat(weights bytes -> f32, scales -> f32, bias -> f32), in one kernel. */
+typedef struct Q4VecParams {
+  uint64_t weights, scales, bias, out; /* bias may be 0 */
+  uint32_t nw, ns, nb;                 /* element counts */
+  uint32_t scales_dtype, bias_dtype;   /* VKT_F32 | VKT_F16 | VKT_BF16 */
+  uint32_t pad;
+} Q4VecParams;
+
 /* "qmm4c_pack", spec {}: packed float32 vector -> compact side-car (nibbles, scales,
  * bias, per-block nibble sums) laid out for the streaming kernels. */
 typedef struct Q4PackParams {

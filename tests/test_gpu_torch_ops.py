@@ -1,0 +1,192 @@
+"""The five quantised aten ops on device "vk", written as the reference's own tests are
+(tests/python/test_quant.py): each op on "vk" against PyTorch's CPU result, with the
+reference's `on_gpu()` assertion that nothing fell back to the CPU (tests/python/_util.py:28-35).
+The C++ op layer (csrc/torch/quant.cpp) reaches the kernels through the C ABI."""
+import contextlib
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+FLOAT8 = [torch.float8_e4m3fn, torch.float8_e5m2]
+# bfloat16 / float8 results come off the fp8 matrix cores, whose products are added in a
+# window ~14 bits below the largest (a hardware property); float32 / float16 results are exact sums
+HW_WINDOW = 2.0**-13
+
+
+@pytest.fixture(scope="module")
+def tv():
+    import torch_vulkan_amd.backend as tv
+    assert tv.is_available() and (tv.capabilities() & 12) == 12  # 8- and 16-bit storage (test_quant.py:12)
+    return tv
+
+
+@contextlib.contextmanager
+def on_gpu(tv):
+    """Fails if anything inside falls back to the CPU."""
+    before = tv.fallback_counts()
+    yield
+    after = tv.fallback_counts()
+    new = {k: v - before.get(k, 0) for k, v in after.items() if v != before.get(k, 0)}
+    assert not new, f"ran on the CPU: {new}"
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def test_device_round_trip(tv):
+    x = torch.randn(5, 7, generator=gen(0))
+    d = x.to("vk")
+    assert d.device.type == "vk" and torch.equal(d.cpu(), x)
+    assert torch.equal(d[::2].cpu(), x[::2]) and torch.equal(d.t().contiguous().cpu(), x.t().contiguous())
+    assert torch.equal(d.to(torch.bfloat16).cpu(), x.bfloat16())  # (a conversion staged through the host)
+    for dt in (torch.int8, torch.uint8, torch.float16, torch.bfloat16, torch.float8_e4m3fn, torch.float8_e5m2):
+        y = (x * 10).to(dt)
+        assert torch.equal(y.to("vk").cpu().view(torch.uint8), y.view(torch.uint8))
+    assert d[1, 2].item() == x[1, 2].item()
+    stats = tv.memory_stats()
+    assert stats["allocated_bytes"] > 0 and stats["reserved_bytes"] >= stats["allocated_bytes"]
+    torch.vk.synchronize()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,k,n", [(32, 64, 48), (1, 4096, 300), (5, 100, 17), (70, 33, 5), (65, 1, 66)])
+def test_weight_int8pack_mm(tv, dtype, m, k, n):
+    a = torch.randn(m, k, generator=gen(1)).to(dtype)
+    b = torch.randint(-128, 128, (n, k), dtype=torch.int8, generator=gen(2))
+    s = (torch.rand(n, generator=gen(3)) / 50).to(dtype)
+    want = (a.float() @ (b.float() * s.float()[:, None]).t()).to(dtype)
+    with on_gpu(tv):
+        got = torch._weight_int8pack_mm(a.to("vk"), b.to("vk"), s.to("vk"))
+        sliced = torch._weight_int8pack_mm(a.to("vk")[::2], b.to("vk"), s.to("vk"))
+    mag = a.float().abs() @ (b.float() * s.float()[:, None]).abs().t()
+    tol = torch.finfo(dtype).eps * want.float().abs() + 2**-20 * mag
+    assert got.dtype == want.dtype and got.shape == want.shape and got.device.type == "vk"
+    assert ((got.cpu().float() - want.float()).abs() <= tol).all()
+    assert ((sliced.cpu().float() - want[::2].float()).abs() <= tol[::2]).all()
+
+
+def test_weight_int8pack_mm_errors(tv):
+    a, b, s = torch.randn(4, 8).to("vk"), torch.zeros(3, 8, dtype=torch.int8).to("vk"), torch.ones(3).to("vk")
+    with pytest.raises(RuntimeError, match="expect B to be int8 tensor"):
+        torch._weight_int8pack_mm(a, b.float(), s)
+    with pytest.raises(RuntimeError, match="expect scales to be 1d tensor with size 3"):
+        torch._weight_int8pack_mm(a, b, s[:2])
+    with pytest.raises(RuntimeError, match="A must be contiguous on the last dimension"):
+        torch._weight_int8pack_mm(a.t().contiguous().t(), b[:, :4], s)
+
+
+def pack_case(n, k, bs, seed, bias):
+    w = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, generator=gen(seed))
+    nb = 1 if bs == k else k // bs
+    sc = torch.rand(n, nb, generator=gen(seed + 1)) / 10
+    sc = sc if bs == k else sc.to(torch.bfloat16)
+    return w, sc, (torch.randn(n, generator=gen(seed + 2)) if bias else None)
+
+
+@pytest.mark.parametrize("m,k,n,bs,bias", [(1, 64, 4096, 32, False), (32, 128, 11008, 32, True), (5, 96, 70, 96, True),
+                                           (3, 100, 9, 100, False), (4, 256, 16, 64, True), (9, 64, 33, 64, False)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_dyn_quant_matmul_4bit_exact(tv, m, k, n, bs, bias, dtype):
+    if dtype == torch.bfloat16 and bs != k:
+        pytest.skip("bfloat16 inputs are channelwise only (the CPU's check)")
+    w, sc, bvec = pack_case(n, k, bs, 7, bias)
+    x = (torch.randn(m, k, generator=gen(11)) * 3).to(dtype)
+    x[0, : k // 2] = 0.0
+    if m > 1:
+        x[1] = -x[1].abs()
+    packed = torch._dyn_quant_pack_4bit_weight(w, sc, bvec, bs, k, n)
+    want = torch._dyn_quant_matmul_4bit(x, packed, bs, k, n)
+    with on_gpu(tv):
+        packed_vk = torch._dyn_quant_pack_4bit_weight(w.to("vk"), sc.to("vk"), None if bvec is None else bvec.to("vk"),
+                                                      bs, k, n)
+        got = torch._dyn_quant_matmul_4bit(x.to("vk"), packed_vk, bs, k, n)
+        again = torch._dyn_quant_matmul_4bit(x.to("vk"), packed_vk, bs, k, n)  # (the cached side-car)
+        got_cpu_packed = torch._dyn_quant_matmul_4bit(x.to("vk"), packed.to("vk"), bs, k, n)
+    assert torch.equal(packed_vk.cpu(), packed)
+    assert got.dtype == want.dtype
+    assert torch.equal(got.cpu(), want) and torch.equal(again.cpu(), want)
+    assert torch.equal(got_cpu_packed.cpu(), want)
+
+
+def test_dyn_quant_sidecar_follows_writes(tv):
+    """The cached side-car is keyed by the packed tensor's version: an in-place change of the
+    packed weights must show in the next product."""
+    w, sc, _ = pack_case(16, 64, 32, 3, False)
+    x = torch.randn(2, 64, generator=gen(5))
+    packed = torch._dyn_quant_pack_4bit_weight(w, sc, None, 32, 64, 16)
+    pv = packed.to("vk")
+    first = torch._dyn_quant_matmul_4bit(x.to("vk"), pv, 32, 64, 16).cpu()
+    packed2 = packed.clone()
+    packed2[: 16 * 32] = 255.0 - packed2[: 16 * 32]
+    pv.copy_(packed2)
+    second = torch._dyn_quant_matmul_4bit(x.to("vk"), pv, 32, 64, 16).cpu()
+    assert torch.equal(first, torch._dyn_quant_matmul_4bit(x, packed, 32, 64, 16))
+    assert torch.equal(second, torch._dyn_quant_matmul_4bit(x, packed2, 32, 64, 16))
+
+
+def test_dyn_quant_errors(tv):
+    x = torch.randn(2, 64).to("vk")
+    w, sc, _ = pack_case(8, 64, 32, 3, False)
+    with pytest.raises(RuntimeError, match="Group size should be multiple of 32"):
+        torch._dyn_quant_pack_4bit_weight(w.to("vk"), sc.to("vk"), None, 48, 64, 8)
+    with pytest.raises(RuntimeError, match="expect weight to be kByte"):
+        torch._dyn_quant_pack_4bit_weight(w.to(torch.int8).to("vk"), sc.to("vk"), None, 32, 64, 8)
+    packed = torch._dyn_quant_pack_4bit_weight(w.to("vk"), sc.to("vk"), None, 32, 64, 8)
+    with pytest.raises(RuntimeError, match="expect input to be float32 or bfloat16 tensor"):
+        torch._dyn_quant_matmul_4bit(x.cpu().bfloat16().to("vk"), packed, 32, 64, 8)
+    with pytest.raises(RuntimeError, match="Invalid packed weight tensor size"):
+        torch._dyn_quant_matmul_4bit(x, packed[:100], 32, 64, 8)
+
+
+@pytest.mark.parametrize("fa,fb", [(FLOAT8[0], FLOAT8[0]), (FLOAT8[1], FLOAT8[0]), (FLOAT8[0], FLOAT8[1])])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32, torch.float16, torch.float8_e4m3fn, None])
+@pytest.mark.parametrize("rowwise", [False, True])
+def test_scaled_mm(tv, fa, fb, out_dtype, rowwise):
+    a = torch.randn(16, 32, generator=gen(1)).to(fa)
+    b = torch.randn(48, 32, generator=gen(2)).to(fb).t()
+    sa = torch.rand(16, 1, generator=gen(3)) + 0.5 if rowwise else torch.tensor(1.25)
+    sb = torch.rand(1, 48, generator=gen(4)) + 0.5 if rowwise else torch.tensor(0.75)
+    bias = torch.randn(48, generator=gen(5)).to(torch.bfloat16) if out_dtype == torch.bfloat16 else None
+    scale_result = torch.tensor(2.0) if out_dtype == torch.float8_e4m3fn else None
+    kw = dict(bias=bias, out_dtype=out_dtype, scale_result=scale_result)
+    res_dtype = out_dtype or fa
+    if rowwise:  # torch 2.10's CPU kernel takes per-tensor scales only: the closed form it emulates
+        want = (a.float() * sa) @ (b.float() * sb)
+        want = want + bias.float() if bias is not None else want
+        want = (want * 0.5 if scale_result is not None else want).to(res_dtype)
+    else:
+        want = torch._scaled_mm(a, b, sa, sb, **kw)
+    vkw = {k: (v.to("vk") if isinstance(v, torch.Tensor) else v) for k, v in kw.items()}
+    with on_gpu(tv):
+        got = torch._scaled_mm(a.to("vk"), b.to("vk"), sa.to("vk"), sb.to("vk"), **vkw)
+        out = torch.empty(0, dtype=want.dtype).to("vk")
+        torch._scaled_mm(a.to("vk"), b.to("vk"), sa.to("vk"), sb.to("vk"), **vkw, out=out)
+    assert got.dtype == want.dtype and got.shape == want.shape
+    mag = (a.float() * sa).abs() @ (b.float() * sb).abs() / (2.0 if scale_result is not None else 1.0)
+    eps = torch.finfo(want.dtype).eps
+    tol = eps * want.float().abs() + 2**-20 * mag
+    if want.dtype not in (torch.float32, torch.float16):
+        tol = tol + HW_WINDOW * mag
+    for res in (got, out):
+        assert ((res.cpu().float() - want.float()).abs() <= tol).all()
+
+
+def test_scaled_mm_errors(tv):
+    a = torch.randn(4, 8).to(FLOAT8[0]).to("vk")
+    b = torch.randn(6, 8).to(FLOAT8[0]).to("vk").t()
+    one = torch.tensor(1.0).to("vk")
+    with pytest.raises(ValueError, match="Invalid scaling configuration"):
+        torch._scaled_mm(a, b, torch.ones(3).to("vk"), one)
+    with pytest.raises(ValueError, match="out_dtype must match output matrix type"):
+        torch._scaled_mm(a, b, one, one, out_dtype=torch.float32, out=torch.empty(0, dtype=torch.half).to("vk"))
+    with pytest.raises(RuntimeError, match="Bias must be size 6"):
+        torch._scaled_mm(a, b, one, one, bias=torch.ones(5).to("vk"), out_dtype=torch.float32)
+
+
+def test_fallback_is_counted(tv):
+    """An op without a vk kernel runs on the CPU and shows in fallback_counts (what on_gpu() watches)."""
+    before = sum(tv.fallback_counts().values())
+    y = torch.ones(3).to("vk") + 1
+    assert torch.equal(y.cpu(), torch.full((3,), 2.0)) and sum(tv.fallback_counts().values()) > before

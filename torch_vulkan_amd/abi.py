@@ -41,6 +41,11 @@ class Q4Params(ctypes.Structure):  # reference quant.cpp:39-43
                 ("k", u32), ("bs", u32), ("has_bias", u32), ("pad", u32)]
 
 
+class Q4VecParams(ctypes.Structure):
+    _fields_ = [("weights", u64), ("scales", u64), ("bias", u64), ("out", u64), ("nw", u32), ("ns", u32), ("nb", u32),
+                ("scales_dtype", u32), ("bias_dtype", u32), ("pad", u32)]
+
+
 class Q4PackParams(ctypes.Structure):
     _fields_ = [("packed", u64), ("compact", u64), ("n", u32), ("k", u32), ("bs", u32), ("has_bias", u32)]
 

@@ -166,6 +166,11 @@ int dispatch_named(Runtime& rt, const char* name, const uint32_t* spec, size_t n
     }
     return launch_qmm8(p, dt, spec_at(1), rt.machine, rt.stream, err);
   }
+  if (!std::strcmp(name, "qmm4_packvec")) {
+    Q4VecParams p;
+    if (!read_push(push, npush, &p, name, err)) return -1;
+    return launch_qmm4_packvec(p, rt.stream, err);
+  }
   if (!std::strncmp(name, "qmm4_", 5)) {
     int dt = dtype_of_suffix(name + 5);
     Q4Params p;

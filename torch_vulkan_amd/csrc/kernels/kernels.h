@@ -21,6 +21,7 @@ int launch_qmm8(const Q8Params& p, int dtype, uint32_t variant, const Machine& m
                 std::string* err);
 int launch_qmm4(const Q4Params& p, int dtype, uint32_t phase, uint32_t groupwise, const Machine& mc,
                 hipStream_t stream, std::string* err);
+int launch_qmm4_packvec(const Q4VecParams& p, hipStream_t stream, std::string* err);
 int launch_qmm4c_pack(const Q4PackParams& p, const Machine& mc, hipStream_t stream, std::string* err);
 int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwise, uint32_t variant,
                  const Machine& mc, hipStream_t stream, std::string* err);

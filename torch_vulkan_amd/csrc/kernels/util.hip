@@ -35,6 +35,24 @@ __global__ __launch_bounds__(256) void copy_kernel(uint64_t dst, uint64_t src, u
   }
 }
 
+__device__ __forceinline__ float any_f32(uint64_t base, uint64_t i, uint32_t dtype) {
+  if (dtype == VKT_F32) return ldg<float>(base + 4 * i);
+  if (dtype == VKT_F16) return f16_to_f32(ldg<uint16_t>(base + 2 * i));
+  return bf16_to_f32(ldg<uint16_t>(base + 2 * i));
+}
+
+// The packed float32 vector of the int4 op: bytes, scales and bias widened (all exact).
+__global__ __launch_bounds__(256) void packvec_kernel(Q4VecParams p) {
+  const uint64_t total = uint64_t(p.nw) + p.ns + p.nb, stride = uint64_t(gridDim.x) * 256;
+  for (uint64_t i = uint64_t(blockIdx.x) * 256 + threadIdx.x; i < total; i += stride) {
+    float v;
+    if (i < p.nw) v = float(ldg<uint8_t>(p.weights + i));
+    else if (i < uint64_t(p.nw) + p.ns) v = any_f32(p.scales, i - p.nw, p.scales_dtype);
+    else v = any_f32(p.bias, i - p.nw - p.ns, p.bias_dtype);
+    stg<float>(p.out + 4 * i, v);
+  }
+}
+
 uint32_t groups_for(uint64_t units) {
   const uint64_t want = (units + 255) / 256 + 1;
   return uint32_t(want < 16384 ? want : 16384);
@@ -46,6 +64,22 @@ int launch_fill(uint64_t dst, uint8_t value, uint64_t nbytes, hipStream_t stream
   hipLaunchKernelGGL(fill_kernel, dim3(groups_for(nbytes / 16)), dim3(256), 0, stream, dst, uint32_t(value), nbytes);
   if (hipGetLastError() != hipSuccess) {
     *err = "fill: kernel launch failed";
+    return -1;
+  }
+  return 0;
+}
+
+int launch_qmm4_packvec(const Q4VecParams& p, hipStream_t stream, std::string* err) {
+  const uint64_t total = uint64_t(p.nw) + p.ns + p.nb;
+  if (total == 0) return 0;
+  if (!p.out || (p.nw && !p.weights) || (p.ns && !p.scales) || (p.nb && !p.bias) || p.scales_dtype > VKT_BF16 ||
+      p.bias_dtype > VKT_BF16) {
+    *err = "qmm4_packvec: null address or unsupported dtype";
+    return -1;
+  }
+  hipLaunchKernelGGL(packvec_kernel, dim3(groups_for(total)), dim3(256), 0, stream, p);
+  if (hipGetLastError() != hipSuccess) {
+    *err = "qmm4_packvec: kernel launch failed";
     return -1;
   }
   return 0;

@@ -1,0 +1,61 @@
+// Shared declarations of the torch layer of device "vk" (the counterpart of the reference's
+// crates/pyvk/csrc/vk.h, cut down to what the quantized-matmul path uses).
+#pragma once
+
+#include <ATen/ATen.h>
+#include <ATen/core/dispatch/Dispatcher.h>
+#include <ATen/core/stack.h>
+
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "../../../include/vkt.h"
+
+namespace vk {
+
+constexpr c10::DeviceType kDevice = c10::DeviceType::PrivateUse1;
+
+// rc of a vkt_* call -> exception "torch_vulkan: <message>" (reference vk.h:75-77).
+void check(int rc);
+
+// Waits for queued GPU work.
+void synchronize();
+
+c10::Allocator* allocator();
+
+// Device address of the first element of `t` (0 for an empty tensor).  The DataPtr of a vk
+// tensor is the device pointer, so this is t.data_ptr() (reference vk.h:117-122 looks it up
+// in a host-pointer map).  The _out form materializes copy-on-write storage first.
+uint64_t gpu_address(const at::TensorBase& t);
+uint64_t gpu_address_out(const at::TensorBase& t);
+
+// Records that `op` ran on the CPU instead of the GPU; under TORCH_VK_STRICT raises
+// NotImplementedError instead (reference vk.h: record_fallback).
+void record_fallback(const std::string& op);
+
+// Runs `op` on CPU copies of the stack's vk tensors, recorded as a fallback.
+void run_fallback(const c10::OperatorHandle& op, torch::jit::Stack* stack, bool error_on_views);
+
+inline bool is_vk(const at::Tensor& t) { return t.device().type() == kDevice; }
+
+// Runs aten op `name.overload` without a vk kernel (reference vk.h:372-379).
+template <typename... Args>
+torch::jit::Stack on_cpu(const char* name, const char* overload, const Args&... args) {
+  auto op = c10::Dispatcher::singleton().findSchemaOrThrow(name, overload);
+  torch::jit::Stack stack;
+  (stack.emplace_back(args), ...);
+  run_fallback(op, &stack, /*error_on_views=*/false);
+  return stack;
+}
+
+// Queues `kernel` with its parameter block (at most 128 bytes) (reference vk.h:383-389).
+template <typename P>
+void dispatch(const std::string& kernel, const std::vector<uint32_t>& spec, const P& params, uint32_t gx,
+              uint32_t gy = 1, uint32_t gz = 1) {
+  static_assert(sizeof(P) <= 128, "parameter blocks are limited to 128 bytes");
+  check(vkt_dispatch(kernel.c_str(), spec.data(), spec.size(), reinterpret_cast<const uint8_t*>(&params), sizeof(P), gx,
+                     gy, gz));
+}
+
+}  // namespace vk
