@@ -50,6 +50,20 @@ def test_qmm8_every_variant(variant, dtype):
         check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=variant), a, b, s, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("variant", [0, 1 | 4 << 8, 2 | 8 << 8, 4 | 16 << 8, 1 << 17])
+@pytest.mark.parametrize("m,k,n", [(5, 1024, 40), (16, 4096, 67), (33, 2048, 130), (64, 4160, 96), (70, 512, 36)])
+def test_qmm8_matrix_core_variants(dtype, variant, m, k, n):
+    """4 < M with 16-bit activations runs on the matrix cores: every (columns, k-split)
+    instantiation, and the GEMV kernels forced on the same problem (bit 17)."""
+    import _dev
+    a, b, s = q8_case(dtype, m, k, n)
+    check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=variant), a, b, s, dtype)
+    sliced_variant = variant if (m + 1) // 2 > 4 else 0  # (4 rows or fewer: the GEMV kernels plan themselves)
+    check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=sliced_variant, row_step=2), a, b, s, dtype,
+             rows=slice(None, None, 2))
+
+
 def test_qmm8_config1_vs_torch_cpu():
     """BASELINE config 1: fp32, M=1, K=N=4096, within rtol/atol 1e-4 of PyTorch's CPU op."""
     import _dev

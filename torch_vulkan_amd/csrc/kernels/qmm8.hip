@@ -16,8 +16,14 @@
 //                two differ by one float32 rounding, inside its test's tolerance).
 //   qmm8_generic any shape, stride or alignment (K not a multiple of 16, unaligned rows):
 //                a wave per output column, byte loads.
-// Rows beyond 16 are served by the launcher in chunks (the weight stream is then re-read
-// per chunk) until the MFMA tile kernel takes them.
+//   qmm8_mfma    4 < M (bfloat16 / float16 activations).  The stream is the same, the
+//                arithmetic moves to the matrix cores: int8 weights widen exactly to
+//                bfloat16 / float16 in registers, V_MFMA_F32_16X16X32_{BF16,F16} multiplies a
+//                16-column weight fragment (converted once) against up to four 16-row
+//                activation tiles, float32 accumulate.  The waves of a workgroup split K and
+//                add their partial tiles in wave order through LDS (deterministic).
+// Rows beyond the largest kernel's are served by the launcher in chunks (the weight stream
+// is then re-read per chunk).
 #include "common.h"
 #include "kernels.h"
 
@@ -139,6 +145,173 @@ __global__ __launch_bounds__(256) void qmm8_generic(Q8Params p) {
   }
 }
 
+using V4F = float __attribute__((ext_vector_type(4)));
+using V8BF = __bf16 __attribute__((ext_vector_type(8)));
+using V8H = _Float16 __attribute__((ext_vector_type(8)));
+
+// 16 int8 weights (one 16-byte load) as two MFMA operands of 8 elements in T (exact).
+template <class T>
+__device__ __forceinline__ void widen16_to_operands(const U4& v, U4* lo, U4* hi) {
+  uint32_t out[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float f0 = float(int(int8_t(v[i]))), f1 = float(int(int8_t(v[i] >> 8)));
+    const float f2 = float(int(int8_t(v[i] >> 16))), f3 = float(int(int8_t(v[i] >> 24)));
+    if constexpr (T::dtype == VKT_BF16) {
+      // an integer of magnitude <= 128 is its float32's upper 16 bits
+      out[2 * i] = __builtin_amdgcn_perm(f32_bits(f1), f32_bits(f0), 0x07060302u);
+      out[2 * i + 1] = __builtin_amdgcn_perm(f32_bits(f3), f32_bits(f2), 0x07060302u);
+    } else {
+      out[2 * i] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(f0, f1));
+      out[2 * i + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(f2, f3));
+    }
+  }
+  *lo = U4{out[0], out[1], out[2], out[3]};
+  *hi = U4{out[4], out[5], out[6], out[7]};
+}
+
+template <class T>
+__device__ __forceinline__ V4F mfma16(const U4& w, const U4& a, const V4F& acc) {
+  if constexpr (T::dtype == VKT_BF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(V8BF, w), __builtin_bit_cast(V8BF, a), acc, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(V8H, w), __builtin_bit_cast(V8H, a), acc, 0, 0, 0);
+}
+
+// A workgroup owns 16*NT output columns; its WAVES waves take the 64-wide k-steps in turn.
+// Lane (c = lane % 16, g = lane / 16) streams 16 bytes of weight row n0 + 16 t + c at
+// k0 + 16 g (two MFMA operands) and the matching 16 activations of rows 16 mt + c; the
+// MFMA's first operand is the weights, so the lane ends with C[16 mt + c][n0 + 16 t + 4 g + r].
+template <class T, int MT, int NT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void qmm8_mfma(Q8Params p) {
+  constexpr uint64_t item = 2;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
+  const uint32_t n0 = blockIdx.x * 16 * NT;
+  uint64_t brow[NT], arow[MT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const uint32_t n = n0 + 16 * t + c < p.n ? n0 + 16 * t + c : p.n - 1;
+    brow[t] = p.b + uint64_t(n) * p.k + 16 * g;
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const uint32_t m = uint32_t(16 * mt + c) < p.m ? 16 * mt + c : p.m - 1;
+    arow[mt] = p.a + uint64_t(int64_t(m) * p.a_sm * int64_t(item)) + 32 * g;
+  }
+  V4F acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[mt][t] = V4F{0.0f, 0.0f, 0.0f, 0.0f};
+
+  const U4 zero = {0, 0, 0, 0};
+#pragma unroll 2
+  for (uint32_t k0 = wave * 64; k0 < p.k; k0 += WAVES * 64) {
+    const bool inside = k0 + 16 * g < p.k;  // (k is a multiple of 16)
+    U4 wv[NT], a0[MT], a1[MT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) wv[t] = inside ? ldg_stream<U4>(brow[t] + k0) : zero;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      a0[mt] = inside ? ldg<U4>(arow[mt] + k0 * item) : zero;
+      a1[mt] = inside ? ldg<U4>(arow[mt] + k0 * item + 16) : zero;
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      U4 wlo, whi;
+      widen16_to_operands<T>(wv[t], &wlo, &whi);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        acc[mt][t] = mfma16<T>(wlo, a0[mt], acc[mt][t]);
+        acc[mt][t] = mfma16<T>(whi, a1[mt], acc[mt][t]);
+      }
+    }
+  }
+
+  // partial tiles of waves 1.. are added to wave 0's in wave order
+  __shared__ V4F part[MT * NT][64];
+  for (int w = 1; w < WAVES; ++w) {
+    __syncthreads();
+    if (wave == w) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) part[mt * NT + t][lane] = acc[mt][t];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[mt][t] += part[mt * NT + t][lane];
+    }
+  }
+  if (wave != 0) return;
+  const bool vec_ok = (p.n & 3u) == 0 && (p.c & 7u) == 0;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const uint32_t n = n0 + 16 * t + 4 * g;
+    float scale[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) scale[r] = load_f32<T>(p.scales + (n + r < p.n ? n + r : p.n - 1) * item);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const uint32_t m = 16 * mt + c;
+      if (m >= p.m || n >= p.n) continue;
+      const uint64_t at = p.c + (uint64_t(m) * p.n + n) * item;
+      uint32_t h[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float v = acc[mt][t][r] * scale[r];
+        h[r] = T::dtype == VKT_BF16 ? f32_to_bf16(v) : f32_to_f16(v);
+      }
+      if (vec_ok && n + 3 < p.n) {
+        stg<U2>(at, U2{h[0] | h[1] << 16, h[2] | h[3] << 16});
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (n + r < p.n) stg<uint16_t>(at + r * item, uint16_t(h[r]));
+      }
+    }
+  }
+}
+
+template <class T, int MT, int NT>
+void launch_mfma_waves(const Q8Params& p, int waves, hipStream_t stream) {
+  const dim3 grid((p.n + 16 * NT - 1) / (16 * NT));
+  switch (waves) {
+    case 4: hipLaunchKernelGGL((qmm8_mfma<T, MT, NT, 4>), grid, dim3(256), 0, stream, p); break;
+    case 8: hipLaunchKernelGGL((qmm8_mfma<T, MT, NT, 8>), grid, dim3(512), 0, stream, p); break;
+    default: hipLaunchKernelGGL((qmm8_mfma<T, MT, NT, 16>), grid, dim3(1024), 0, stream, p); break;
+  }
+}
+
+// Rows (<= 64) of 16-bit activations on the matrix cores.  Columns per workgroup and waves
+// per workgroup are chosen so that the grid covers the machine: many small workgroups
+// when N is large, more k-splitting when it is not.
+template <class T>
+void launch_mfma(const Q8Params& p, uint32_t variant, const Machine& mc, hipStream_t stream) {
+  const int mt = p.m <= 16 ? 1 : p.m <= 32 ? 2 : 4;
+  // measured on MI355X (bf16, K = 4096 / 14336): with many columns, 64 per workgroup and 8
+  // k-slices (the activation fragments are then reused over 4 weight fragments); with few
+  // columns the grid matters more than the reuse: 16 per workgroup, 16 k-slices
+  (void)mc;
+  int nt = p.n >= 8192 ? 4 : 1, waves = p.n >= 8192 ? 8 : 16;
+  while (waves > 4 && p.k < uint32_t(waves) * 64) waves /= 2;
+  if (variant & 0xffff) {
+    nt = variant & 0xff;
+    waves = (variant >> 8) & 0xff;
+  }
+#define VKT_MFMA_CASE(MT_, NT_) \
+  if (mt == MT_ && nt == NT_) return launch_mfma_waves<T, MT_, NT_>(p, waves, stream);
+  VKT_MFMA_CASE(1, 1) VKT_MFMA_CASE(1, 2) VKT_MFMA_CASE(1, 4)
+  VKT_MFMA_CASE(2, 1) VKT_MFMA_CASE(2, 2) VKT_MFMA_CASE(2, 4)
+  VKT_MFMA_CASE(4, 1) VKT_MFMA_CASE(4, 2) VKT_MFMA_CASE(4, 4)
+#undef VKT_MFMA_CASE
+  launch_mfma_waves<T, 4, 1>(p, waves, stream);
+}
+
+
 template <class T, int ROWS, int COLS, int KSPLIT>
 void launch_gemv(const Q8Params& p, hipStream_t stream) {
   constexpr int per_wg = COLS * (4 / KSPLIT);
@@ -181,6 +354,19 @@ int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipSt
     const uint32_t gy = p0.m <= 8 ? 1 : (p0.m + 7) / 8 < 64 ? (p0.m + 7) / 8 : 64;
     hipLaunchKernelGGL((qmm8_generic<T>), dim3((p0.n + 3) / 4, gy), dim3(256), 0, stream, p0);
     return 0;
+  }
+  if constexpr (T::dtype != VKT_F32) {
+    // variant bit 17 forces the GEMV kernels (tests, tuning)
+    if (p0.m > 4 && !((variant >> 17) & 1)) {
+      for (uint32_t r0 = 0; r0 < p0.m; r0 += 64) {
+        Q8Params p = p0;
+        p.m = p0.m - r0 < 64 ? p0.m - r0 : 64;
+        p.a = p0.a + uint64_t(int64_t(r0) * p0.a_sm * int64_t(item));
+        p.c = p0.c + uint64_t(r0) * p0.n * item;
+        launch_mfma<T>(p, variant, mc, stream);
+      }
+      return 0;
+    }
   }
   for (uint32_t r0 = 0; r0 < p0.m; r0 += 16) {
     Q8Params p = p0;
