@@ -132,7 +132,7 @@ typedef struct Q4PackParams {
 /* "qmm4c_f32" | "qmm4c_bf16", spec {PHASE, GROUPWISE}: as qmm4 but PHASE 0 writes int8
  * activations (+ per-unit sums) into q (vkt_qmm4c_q_bytes) and PHASE 1 streams the
  * compact side-car.  PHASE 2 does both, in one launch per 4 rows where the rows can be
- * quantised from registers (k a multiple of 8, at most 8192), else as PHASE 0 then 1.
+ * quantised from registers (k a multiple of 8, at most 16384), else as PHASE 0 then 1.
  * Results are bit-identical to qmm4. */
 typedef struct Q4CParams {
   uint64_t inp, q, rows, compact, out;

@@ -42,7 +42,7 @@ constexpr int kUnit = 32;          // values of k per 16-byte load of nibbles
 constexpr int kUnitsPerLane = 8;   // units a lane handles per round
 constexpr int kRoundUnits = 128;   // 16 k-parts * 8 units
 constexpr int kTileCols = 16;      // output columns per workgroup
-constexpr int kFusedGroups = 4;    // groups of 8 activations a thread quantises in the fused kernel
+constexpr int kFusedGroups = 8;    // groups of 8 activations a thread quantises in the fused kernel
 
 __device__ __forceinline__ float round_away(float x) {  // std::round, qmm4.slang:112-118
   float t = truncf(x);
