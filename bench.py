@@ -107,7 +107,8 @@ def wl_q8(abi, m, k, n, dtype, steps, warmup, seed=1020):
 
 
 def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030):
-    """_dyn_quant_matmul_4bit on the compact side-car (row quantisation fused into the launch)."""
+    """_dyn_quant_matmul_4bit on the compact side-car: up to 4 rows the streaming layout with
+    row quantisation fused into the launch, above that the matrix-core layout (two launches)."""
     import torch
     g = torch.Generator().manual_seed(seed)
     w4 = torch.randint(0, 16, (n, k), dtype=torch.uint8, generator=g)
@@ -120,7 +121,8 @@ def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030):
     cbytes = L.vkt_qmm4c_bytes(n, k, bs)
     dp = abi.Buffer.from_numpy(packed.numpy())
     first = abi.Buffer(cbytes)
-    abi.dispatch("qmm4c_pack", [], abi.Q4PackParams(packed=dp.address, compact=first.address, n=n, k=k, bs=bs,
+    layout = 1 if m > 4 else 0
+    abi.dispatch("qmm4c_pack", [layout], abi.Q4PackParams(packed=dp.address, compact=first.address, n=n, k=k, bs=bs,
                                                     has_bias=1))
     abi.synchronize()
     dp.free()
@@ -136,7 +138,7 @@ def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030):
     for c in copies:
         p = abi.Q4CParams(inp=dx.address, q=dq.address, rows=dr.address, compact=c.address, out=out.address, m=m, n=n,
                           k=k, bs=bs, has_bias=1)
-        fns.append(Launch(abi, "qmm4c_f32", [2, 1], p))  # row quantisation + product in one launch
+        fns.append(Launch(abi, "qmm4c_f32", [2, 1, layout], p))  # row quantisation + product
     wall, ev = time_steps(abi, fns, steps, warmup)
     work = n * k // 2 + 4 * n * (k // bs) + 4 * n + 4 * m * k + 4 * m * n
     return dict(kind="hbm", work=work, wall_ms=wall, event_ms=ev, flops=2 * m * n * k, inputs=(x, packed),

@@ -122,18 +122,23 @@ typedef struct Q4VecParams {
   uint32_t pad;
 } Q4VecParams;
 
-/* "qmm4c_pack", spec {}: packed float32 vector -> compact side-car (nibbles, scales,
- * bias, per-block nibble sums) laid out for the streaming kernels. */
+/* "qmm4c_pack", spec {LAYOUT}: packed float32 vector -> compact side-car (two nibbles per
+ * byte, float32 scales, bias; vkt_qmm4c_bytes bytes) in one of two layouts:
+ *   LAYOUT 0  for the streaming kernel (v_dot8_i32_i4; at most 4 rows per launch: the
+ *             decode case)
+ *   LAYOUT 1  for the matrix-core kernel (v_mfma_i32_16x16x32_i8; tiles of 16 rows).
+ * A side-car serves only products of the layout it was packed for. */
 typedef struct Q4PackParams {
   uint64_t packed, compact;
   uint32_t n, k, bs, has_bias;
 } Q4PackParams;
 
-/* "qmm4c_f32" | "qmm4c_bf16", spec {PHASE, GROUPWISE}: as qmm4 but PHASE 0 writes int8
- * activations (+ per-unit sums) into q (vkt_qmm4c_q_bytes) and PHASE 1 streams the
- * compact side-car.  PHASE 2 does both, in one launch per 4 rows where the rows can be
- * quantised from registers (k a multiple of 8, at most 16384), else as PHASE 0 then 1.
- * Results are bit-identical to qmm4. */
+/* "qmm4c_f32" | "qmm4c_bf16", spec {PHASE, GROUPWISE, LAYOUT}: as qmm4, over the compact
+ * side-car of that LAYOUT.  PHASE 0 writes the quantised activations into q
+ * (vkt_qmm4c_q_bytes; the arrangement differs per layout) and rows; PHASE 1 is the
+ * product; PHASE 2 does both: with LAYOUT 0 in one launch per 4 rows where the rows can
+ * be quantised from registers (k a multiple of 8, at most 16384), otherwise as PHASE 0
+ * then 1.  Results are bit-identical to qmm4. */
 typedef struct Q4CParams {
   uint64_t inp, q, rows, compact, out;
   uint32_t m, n, k, bs, has_bias, pad;

@@ -58,8 +58,9 @@ def q4_reference_layout(x, odt, packed, bs, k, n, want_intermediates=False):
 class CompactWeights:
     """The compact side-car of a packed float32 vector ("qmm4c_pack"), built once."""
 
-    def __init__(self, packed, bs, k, n):
+    def __init__(self, packed, bs, k, n, layout=0):
         packed = np.ascontiguousarray(packed, dtype=np.float32)
+        self.layout = layout  # 0: streaming (at most 4 rows at a time), 1: matrix cores
         nbytes = abi.lib().vkt_qmm4c_bytes(n, k, bs)
         assert nbytes, "no compact form"
         self.n, self.k, self.bs = n, k, bs
@@ -67,7 +68,7 @@ class CompactWeights:
         dp = abi.Buffer.from_numpy(packed)
         self.buf = abi.Buffer(nbytes)
         p = abi.Q4PackParams(packed=dp.address, compact=self.buf.address, n=n, k=k, bs=bs, has_bias=self.has_bias)
-        abi.dispatch("qmm4c_pack", [], p)
+        abi.dispatch("qmm4c_pack", [layout], p)
         abi.synchronize()
         dp.free()
 
@@ -86,10 +87,10 @@ def q4_compact(x, odt, cw, fused=True):
     g = int(bs != k)
     name = "qmm4c_" + abi.SUFFIX[odt]
     if m and n and fused:
-        abi.dispatch(name, [2, g], p, ((n + 31) // 32, (m + 7) // 8))
+        abi.dispatch(name, [2, g, cw.layout], p, ((n + 31) // 32, (m + 7) // 8))
     elif m and n:
-        abi.dispatch(name, [0, g], p, (m,))
-        abi.dispatch(name, [1, g], p, ((n + 31) // 32, (m + 7) // 8))
+        abi.dispatch(name, [0, g, cw.layout], p, (m,))
+        abi.dispatch(name, [1, g, cw.layout], p, ((n + 31) // 32, (m + 7) // 8))
     return do.to_numpy(_NP[odt], (m, n))
 
 

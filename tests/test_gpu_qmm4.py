@@ -14,7 +14,10 @@ from test_oracle_pins import Q4_CASES, pack_case, q4_input
 pytestmark = pytest.mark.gpu
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 EXTRA = [(2, 4096, 300, 32, True), (3, 14336, 20, 32, True), (9, 28672, 6, 128, False), (4, 4096 + 2048, 12, 64, False), (7, 8192, 9, 128, True), (3, 512, 5, 256, False),
-         (6, 4160, 10, 4160, True), (1, 32, 1, 32, False), (5, 8, 3, 8, True)]
+         (6, 4160, 10, 4160, True), (1, 32, 1, 32, False), (5, 8, 3, 8, True),
+         # more than 4 rows: the matrix-core layout's row tiles (16 rows each, 64 rows per launch)
+         (70, 512, 40, 64, True), (33, 1056, 17, 32, False), (16, 4096, 64, 128, True), (20, 4160, 10, 4160, False),
+         (130, 96, 33, 32, True), (17, 2048, 16, 256, False)]
 
 
 @pytest.mark.parametrize("m,k,n,bs,bias", Q4_CASES + EXTRA)
@@ -39,6 +42,9 @@ def test_q4_bit_exact(m, k, n, bs, bias, dtype):
         cw = _dev.CompactWeights(packed.numpy(), bs, k, n)
         assert np.array_equal(_dev.q4_compact(bits(x), odt, cw, fused=True), want)
         assert np.array_equal(_dev.q4_compact(bits(x), odt, cw, fused=False), want)
+        cm = _dev.CompactWeights(packed.numpy(), bs, k, n, layout=1)
+        assert np.array_equal(_dev.q4_compact(bits(x), odt, cm, fused=True), want)
+        assert np.array_equal(_dev.q4_compact(bits(x), odt, cm, fused=False), want)
 
 
 @pytest.mark.parametrize("m", [1, 32])
@@ -64,6 +70,8 @@ def test_q4_config3(m):
     got = _dev.q4_compact(x.numpy(), oracle.F32, cw)
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
     assert np.allclose(got, cpu, rtol=1e-4, atol=1e-4)
+    got = _dev.q4_compact(x.numpy(), oracle.F32, _dev.CompactWeights(packed.numpy(), bs, k, n, layout=1))
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
     if m == 1:
         got = _dev.q4_reference_layout(x.numpy(), oracle.F32, packed.numpy(), bs, k, n)
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
@@ -87,6 +95,8 @@ def test_q4_golden_fixtures():
                                   g[key + "_out"]), key
             cw = _dev.CompactWeights(g[f"c{i}_packed"], bs, k, n)
             assert np.array_equal(_dev.q4_compact(g[key + "_x"], odt, cw), g[key + "_out"]), key
+            cm = _dev.CompactWeights(g[f"c{i}_packed"], bs, k, n, layout=1)
+            assert np.array_equal(_dev.q4_compact(g[key + "_x"], odt, cm), g[key + "_out"]), key
 
 
 def test_q4_errors():
@@ -105,6 +115,8 @@ def test_q4_errors():
                       k=64, bs=32, has_bias=0)
     with pytest.raises(abi.VktError, match="PHASE"):
         abi.dispatch("qmm4c_f32", [3, 1], c)
+    with pytest.raises(abi.VktError, match="LAYOUT"):
+        abi.dispatch("qmm4c_f32", [2, 1, 2], c)
     with pytest.raises(abi.VktError, match="unknown kernel"):
         abi.dispatch("qmm4_f16", [0, 1], p)
     assert abi.lib().vkt_qmm4c_bytes(8, 96, 96) > 0 and abi.lib().vkt_qmm4c_bytes(8, 192, 96) == 0

@@ -60,7 +60,10 @@ def test_compact_sizes():
     total = L.vkt_qmm4c_bytes(n, k, 32)
     assert n * k // 2 + 4 * n * k // 32 + 4 * n <= total <= n * k // 2 + 4 * n * k // 32 + 4 * n + 512
     assert L.vkt_qmm4c_bytes(n, k, 96) == 0 and L.vkt_qmm4c_bytes(n, k, k) > 0
-    assert L.vkt_qmm4c_q_bytes(1, 4096) == 4096 and L.vkt_qmm4c_q_bytes(3, 100) == 3 * 4096
+    # the activation scratch serves either layout: rows * K rounded up to 4096 for the streaming
+    # kernel, tiles of 16 rows * K rounded up to 2048 for the matrix-core kernel
+    assert L.vkt_qmm4c_q_bytes(1, 4096) == 16 * 4096 and L.vkt_qmm4c_q_bytes(3, 100) == 16 * 2048
+    assert L.vkt_qmm4c_q_bytes(40, 8192) == 48 * 8192 and L.vkt_qmm4c_q_bytes(0, 64) == 0
 
 
 # ------------------------------------------------------------------ pool policy

@@ -181,7 +181,7 @@ int dispatch_named(Runtime& rt, const char* name, const uint32_t* spec, size_t n
   if (!std::strcmp(name, "qmm4c_pack")) {
     Q4PackParams p;
     if (!read_push(push, npush, &p, name, err)) return -1;
-    return launch_qmm4c_pack(p, rt.machine, rt.stream, err);
+    return launch_qmm4c_pack(p, spec_at(0), rt.machine, rt.stream, err);
   }
   if (!std::strncmp(name, "qmm4c_", 6)) {
     int dt = dtype_of_suffix(name + 6);

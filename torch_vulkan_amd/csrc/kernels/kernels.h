@@ -22,8 +22,8 @@ int launch_qmm8(const Q8Params& p, int dtype, uint32_t variant, const Machine& m
 int launch_qmm4(const Q4Params& p, int dtype, uint32_t phase, uint32_t groupwise, const Machine& mc,
                 hipStream_t stream, std::string* err);
 int launch_qmm4_packvec(const Q4VecParams& p, hipStream_t stream, std::string* err);
-int launch_qmm4c_pack(const Q4PackParams& p, const Machine& mc, hipStream_t stream, std::string* err);
-int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwise, uint32_t variant,
+int launch_qmm4c_pack(const Q4PackParams& p, uint32_t layout, const Machine& mc, hipStream_t stream, std::string* err);
+int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwise, uint32_t layout,
                  const Machine& mc, hipStream_t stream, std::string* err);
 int launch_fp8mm(const F8Params& p, uint32_t variant, const Machine& mc, hipStream_t stream, std::string* err);
 int launch_fill(uint64_t dst, uint8_t value, uint64_t nbytes, hipStream_t stream, std::string* err);

@@ -14,10 +14,12 @@
 // Two families behind the C ABI:
 //   "qmm4_*"   the reference's parameter block and buffers as they are (int32 q, the
 //              float32-expanded packed vector: 4 bytes of traffic per byte of nibbles).
-//   "qmm4c_*"  the streaming path.  "qmm4c_pack" rewrites the packed vector once into a
+//   "qmm4c_*"  the compact path.  "qmm4c_pack" rewrites the packed vector once into a
 //              compact side-car (two nibbles per byte, 16 bytes per lane per load, laid out
-//              so that every load instruction of a wave reads 1 KiB contiguous), and the
-//              product is an HBM stream over it:
+//              so that every load instruction of a wave reads 1 KiB contiguous), in one of
+//              two layouts: for the matrix cores (more than 4 rows; described further down)
+//              or for the streaming kernel (at most 4 rows per launch), where the product
+//              is an HBM stream over it:
 //                - a workgroup of 4 waves owns 16 output columns; lane = (column, k-part):
 //                  the 16 k-parts (4 waves x 4 groups of 16 lanes) split K into runs of
 //                  8 units per round (a unit = 32 values of k = one 16-byte load);
@@ -31,6 +33,8 @@
 //                  waves through LDS.  Starting from -0.0f and padding with -0.0f makes every
 //                  step a plain addition (x + -0 = x, -0 + t = t) with the reference's bits.
 #pragma clang fp contract(off)
+
+#include <type_traits>
 
 #include "common.h"
 #include "kernels.h"
@@ -519,6 +523,349 @@ __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L
   }
 }
 
+// ------------------------------------------------------------------ compact path on the matrix cores
+//
+// For more than 4 rows the integer sums move to v_mfma_i32_16x16x32_i8, over a second
+// side-car layout ("matrix layout"):
+//   - a unit (32 values of k) of a tile of 16 columns against a tile of 16 rows is one MFMA
+//     shape: lane (x = lane % 16, kg = lane / 16) supplies 8 values k = 32 u + 8 kg .. + 7 of
+//     activation row x (first operand) and of weight column x (second operand), and
+//     receives the sums of column x for rows 4 kg .. + 3;
+//   - weights stay unsigned: a word of 8 nibbles becomes the operand's 8 bytes with two ANDs
+//     and a shift, and
+//       sum (q + nzp) (nib - 8) = sum q nib + sum q (-8) + nzp sum nib - 256 nzp
+//     is four chained MFMAs: the activations against the nibbles, the activations against a
+//     constant operand of -8, and two whose first operand holds nzp in every position, split
+//     in two halves that fit a signed byte (nzp reaches 128); the last term enters as the
+//     first MFMA's accumulator input.  No integer work is left for the vector ALU;
+//   - the float32 block terms are produced 4 waves wide and added in block order by the
+//     thread that owns the output (see qmm4m_tile);
+//   - blocks beyond K hold nibble 8 (weight 0) and scale -1: their term is (+0) * -1 = -0.0f,
+//     which leaves the running sum as it is, bit for bit.
+
+struct MatrixLayout {
+  uint32_t nunits, quads, tiles, upb;  // quads: groups of 4 units, padded to a multiple of 16
+  uint64_t nib_bytes, scale_off, scale_bytes, bias_off, total;
+};
+
+__host__ __device__ inline bool matrix_layout(uint32_t n, uint32_t k, uint32_t bs, MatrixLayout* L) {
+  if (n == 0 || k == 0 || bs == 0) return false;
+  const bool channelwise = bs == k;
+  if (!channelwise && !(bs == 32 || bs == 64 || bs == 128 || bs == 256)) return false;
+  if (!channelwise && k % bs != 0) return false;
+  L->nunits = (k + kUnit - 1) / kUnit;
+  L->quads = (L->nunits + 63) / 64 * 16;
+  L->tiles = (n + kTileCols - 1) / kTileCols;
+  L->upb = channelwise ? 0 : bs / kUnit;
+  // [quad][tile][lane 64] x 16 bytes: word j of a lane = 8 nibbles of unit 4 quad + j.  Quad-major:
+  // the waves of a launch advance through K together, and what they read at any one time is then
+  // one contiguous run over all tiles, spread evenly over the memory channels
+  L->nib_bytes = uint64_t(L->tiles) * L->quads * 64 * 16;
+  L->scale_off = L->nib_bytes;
+  // groupwise: [quad][tile][column 16][unit 4] float32 (a block's scale repeated for each of
+  // its units); channelwise: [n]
+  L->scale_bytes = channelwise ? round_up_u64(uint64_t(n) * 4, 256) : uint64_t(L->tiles) * L->quads * 16 * 16;
+  L->bias_off = L->scale_off + L->scale_bytes;
+  L->total = L->bias_off + round_up_u64(uint64_t(n) * 4, 256);
+  return true;
+}
+
+__global__ __launch_bounds__(256) void qmm4m_pack_kernel(Q4PackParams p, MatrixLayout L) {
+  const uint32_t rstride = (p.k + 1) / 2, nblocks = (p.k + p.bs - 1) / p.bs;
+  const uint64_t wcount = uint64_t(p.n) * p.k / 2;
+  const uint64_t slots = L.nib_bytes / 16;
+  const uint64_t id = uint64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (id < slots) {
+    const uint32_t lane = id & 63;
+    const uint64_t tq = id >> 6;
+    const uint32_t tile = tq % L.tiles, quad = tq / L.tiles;
+    const uint32_t n = tile * kTileCols + (lane & 15), kg = lane >> 4;
+    U4 out;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      uint32_t word = 0;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const uint32_t byte_index = (quad * 4 + j) * 16 + kg * 4 + b;
+        uint32_t byte = 0x88;  // weight 0
+        if (n < p.n && byte_index < rstride) {
+          byte = uint32_t(ldg<float>(p.packed + (uint64_t(n) * rstride + byte_index) * 4)) & 0xffu;
+          if ((p.k & 1) && byte_index == rstride - 1) byte = (byte & 0x0f) | 0x80;
+        }
+        word |= byte << (8 * b);
+      }
+      out[j] = word;
+    }
+    stg<U4>(p.compact + id * 16, out);
+    return;
+  }
+  uint64_t sid = id - slots;
+  if (L.upb != 0) {
+    const uint64_t sslots = L.scale_bytes / 4;
+    if (sid < sslots) {
+      const uint32_t j = sid & 3, col = (sid >> 2) & 15;
+      const uint64_t tq = sid >> 6;
+      const uint32_t tile = tq % L.tiles, quad = tq / L.tiles;
+      const uint32_t n = tile * kTileCols + col, blk = (quad * 4 + j) / L.upb;
+      float s = -1.0f;
+      if (n < p.n && blk < nblocks) s = ldg<float>(p.packed + (wcount + uint64_t(n) * nblocks + blk) * 4);
+      stg<float>(p.compact + L.scale_off + sid * 4, s);
+      return;
+    }
+    sid -= sslots;
+  } else {
+    if (sid < p.n) {
+      stg<float>(p.compact + L.scale_off + sid * 4, ldg<float>(p.packed + (wcount + sid) * 4));
+      return;
+    }
+    sid -= p.n;
+  }
+  if (sid < p.n) {
+    const float b = p.has_bias ? ldg<float>(p.packed + (wcount + uint64_t(p.n) * nblocks + sid) * 4) : 0.0f;
+    stg<float>(p.compact + L.bias_off + sid * 4, b);
+  }
+}
+
+// 8 quantised values as the MFMA operand's 8 bytes: even positions, then odd positions
+// (the order in which the weight nibbles come apart).
+__device__ __forceinline__ U2 operand_bytes(const int (&q)[8]) {
+  U2 r;
+  r.x = (uint32_t(q[0]) & 255u) | (uint32_t(q[2]) & 255u) << 8 | (uint32_t(q[4]) & 255u) << 16 | uint32_t(q[6]) << 24;
+  r.y = (uint32_t(q[1]) & 255u) | (uint32_t(q[3]) & 255u) << 8 | (uint32_t(q[5]) & 255u) << 16 | uint32_t(q[7]) << 24;
+  return r;
+}
+
+// The activation scratch of the matrix layout: [row tile][quad][half 2][lane = kg * 16 + m % 16]
+// [unit 2] x 8 bytes (a wave reads a half of a quad as 64 consecutive 16-byte pieces).
+__device__ __forceinline__ uint64_t operand_offset(uint32_t m, uint32_t g, uint32_t quads) {
+  const uint32_t unit = g >> 2, kg = g & 3, j = unit & 3;
+  return (((uint64_t(m >> 4) * quads + (unit >> 2)) * 2 + (j >> 1)) * 64 + kg * 16 + (m & 15)) * 16 + (j & 1) * 8;
+}
+
+// Phase 0 for the matrix layout, one workgroup per row.  FAST: k is a multiple of 8, at most
+// 2048 * kFusedGroups, rows 16-byte aligned: the row is read once, into registers.
+template <class T, bool FAST>
+__global__ __launch_bounds__(256) void qmm4m_rowquant(Q4CParams p, uint32_t groupwise, uint32_t quads) {
+  constexpr uint64_t item = sizeof(typename T::storage);
+  const uint32_t m = blockIdx.x, tid = threadIdx.x;
+  const uint64_t row = p.inp + uint64_t(m) * p.k * item;
+  const uint32_t groups_all = quads * 16;
+  if constexpr (FAST) {
+    const uint32_t groups = p.k / 8;
+    float x[kFusedGroups][8];
+    float mn = 3.40282347e38f, mx = -3.40282347e38f;
+#pragma unroll
+    for (int i = 0; i < kFusedGroups; ++i) {
+      const uint32_t g = tid + 256 * i;
+      if (g < groups) load8_f32<T>(row + g * 8 * item, x[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < kFusedGroups; ++i) {
+      if (uint32_t(tid + 256 * i) < groups) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) mn = fminf(mn, x[i][e]), mx = fmaxf(mx, x[i][e]);
+      }
+    }
+    block_range(&mn, &mx);
+    const RowQuant rq = row_quant(mn, mx, groupwise != 0);
+    if (tid == 0) {
+      stg<uint32_t>(p.rows + 8ull * m, f32_bits(rq.recip));
+      stg<int32_t>(p.rows + 8ull * m + 4, -rq.izp);
+    }
+#pragma unroll
+    for (int i = 0; i < kFusedGroups; ++i) {
+      const uint32_t g = tid + 256 * i;
+      if (g < groups_all) {
+        U2 v = {0u, 0u};
+        if (g < groups) {
+          int q[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) q[e] = quantise(x[i][e], rq);
+          v = operand_bytes(q);
+        }
+        stg<U2>(p.q + operand_offset(m, g, quads), v);
+      }
+    }
+  } else {
+    float mn, mx;
+    row_range<T>(row, p.k, &mn, &mx);
+    const RowQuant rq = row_quant(mn, mx, groupwise != 0);
+    if (tid == 0) {
+      stg<uint32_t>(p.rows + 8ull * m, f32_bits(rq.recip));
+      stg<int32_t>(p.rows + 8ull * m + 4, -rq.izp);
+    }
+    for (uint32_t g = tid; g < groups_all; g += 256) {
+      int q[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t k = g * 8 + e;
+        q[e] = k < p.k ? quantise(load_f32<T>(row + k * item), rq) : 0;
+      }
+      stg<U2>(p.q + operand_offset(m, g, quads), operand_bytes(q));
+    }
+  }
+}
+
+using V4I = int __attribute__((ext_vector_type(4)));
+
+constexpr int kGroupQuads = 16;  // quads per workgroup and load group: 4 per wave
+
+// The matrix-core kernel.  A workgroup is one tile of 16 columns against one tile of 16 rows
+// (blockIdx.y, starting at row m0); its 4 waves share K.  Work proceeds in steps of 4 quads
+// (8 for blocks of 256), one quad (two) per wave: each wave turns its units into float32
+// block terms - four MFMAs per unit, then convert and scale - and leaves them in LDS;
+// after a barrier, thread (row, column) adds the step's terms to its running sum in block
+// order.  That addition is the only part of the operator that has to be sequential, and it
+// is 1/16 of the terms per thread; everything else runs 4 waves wide per tile, with several
+// workgroups per compute unit to hide each other's latencies.  The term buffer is double
+// buffered, so a step costs one barrier.  Weights and scales are loaded a group of 4 quads
+// per wave ahead (two register sets, used alternately), activations - which every
+// workgroup of the row tile re-reads, from L2 - one step ahead.
+template <class T, int UPB>
+__global__ __launch_bounds__(256) void qmm4m_tile(Q4CParams p, MatrixLayout L, uint32_t m0) {
+  constexpr uint64_t item = sizeof(typename T::storage);
+  constexpr int QW = UPB == 8 ? 2 : 1;               // quads per wave per step
+  constexpr int SPG = 4 / QW;                         // steps per group
+  constexpr int BW = UPB ? 4 * QW / UPB : 0;          // blocks per wave per step
+  constexpr int NB = 4 * BW;                          // blocks per step
+  __shared__ __attribute__((aligned(16))) float terms[2][NB ? NB : 1][256];  // [buffer][block][output]
+  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t tile = blockIdx.x;
+  const uint32_t col = lane & 15, kg = lane >> 4;
+  const uint32_t row0 = m0 + blockIdx.y * 16;  // a multiple of 16, below p.m
+
+  V4I unit_const;  // -256 nzp: per unit, for the rows this lane receives
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const uint32_t m = row0 + kg * 4 + r < p.m ? row0 + kg * 4 + r : p.m - 1;
+    unit_const[r] = -256 * ldg<int32_t>(p.rows + 8ull * m + 4);
+  }
+  // -zero_point of the row this lane feeds as first operand, in two halves that fit a byte
+  long nz_a, nz_b;
+  {
+    const uint32_t m = row0 + col < p.m ? row0 + col : p.m - 1;
+    const int nzp = ldg<int32_t>(p.rows + 8ull * m + 4);
+    const int h1 = nzp >> 1, h2 = nzp - h1;
+    const uint32_t w1 = (uint32_t(h1) & 255u) * 0x01010101u, w2 = (uint32_t(h2) & 255u) * 0x01010101u;
+    nz_a = long(uint64_t(w1) | uint64_t(w1) << 32);
+    nz_b = long(uint64_t(w2) | uint64_t(w2) << 32);
+  }
+  const long minus8 = long(0xf8f8f8f8f8f8f8f8ull);
+
+  const uint64_t wbase = p.compact + (uint64_t(tile) * 64 + lane) * 16;             // + quad * wstep
+  const uint64_t sbase = p.compact + L.scale_off + (uint64_t(tile) * 16 + col) * 16;  // + quad * sstep
+  const uint64_t wstep = uint64_t(L.tiles) * 1024, sstep = uint64_t(L.tiles) * 256;
+  const uint64_t qbase = p.q + (uint64_t(row0 >> 4) * L.quads * 128 + lane) * 16;    // + quad * 2048 (+ 1024)
+
+  // the quad of this wave's slot sl (0..3) in group g: consecutive waves take consecutive
+  // quads (pairs of quads), so that a step's blocks lie in LDS in the order of K
+  auto quad_of = [&](uint32_t g, int sl) -> uint32_t {
+    return QW == 1 ? g * kGroupQuads + sl * 4 + wave : g * kGroupQuads + (sl >> 1) * 8 + wave * 2 + (sl & 1);
+  };
+  struct Set {
+    U4 w[4];
+    F4 s[4];
+  };
+  auto load_set = [&](Set& set, uint32_t g) {
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {
+      const uint32_t quad = quad_of(g, sl);
+      set.w[sl] = ldg_stream<U4>(wbase + quad * wstep);
+      if constexpr (UPB != 0) set.s[sl] = ldg<F4>(sbase + quad * sstep);
+    }
+  };
+
+  const uint32_t groups = L.quads / kGroupQuads;
+  Set set_a, set_b;
+  load_set(set_a, 0);
+  U4 qn[QW][2];  // the next step's activations
+  auto load_q = [&](uint32_t g, int st) {
+#pragma unroll
+    for (int x = 0; x < QW; ++x) {
+      const uint64_t at = qbase + uint64_t(quad_of(g, st * QW + x)) * 2048;
+      qn[x][0] = ldg<U4>(at), qn[x][1] = ldg<U4>(at + 1024);
+    }
+  };
+  load_q(0, 0);
+
+  float acc = -0.0f;       // of this thread's output
+  V4I d = {0, 0, 0, 0};    // (channelwise: the wave's integer sums over all its units)
+  uint32_t parity = 0;
+
+  auto process = [&](const Set& set, uint32_t g) {
+#pragma unroll
+    for (int st = 0; st < SPG; ++st) {
+      U4 qc[QW][2];
+#pragma unroll
+      for (int x = 0; x < QW; ++x) qc[x][0] = qn[x][0], qc[x][1] = qn[x][1];
+      // the next step's activations (of the next group at the last step; beyond the end the
+      // last group again, unused)
+      if (st + 1 < SPG) load_q(g, st + 1);
+      else load_q(g + 1 < groups ? g + 1 : g, 0);
+#pragma unroll
+      for (int x = 0; x < QW; ++x) {
+        const int sl = st * QW + x;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t v = set.w[sl][j];
+          const long b = long(uint64_t(v & 0x0f0f0f0fu) | uint64_t((v >> 4) & 0x0f0f0f0fu) << 32);
+          const U4& qq = qc[x][j >> 1];
+          const long a = long(uint64_t(qq[(j & 1) * 2]) | uint64_t(qq[(j & 1) * 2 + 1]) << 32);
+          constexpr int mask = UPB ? UPB - 1 : 0;
+          const int u = x * 4 + j;  // unit within the wave's step
+          const bool first = UPB != 0 && (u & mask) == 0;
+          d = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, first ? unit_const * (UPB ? UPB : 1) : d, 0, 0, 0);
+          d = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, minus8, d, 0, 0, 0);
+          d = __builtin_amdgcn_mfma_i32_16x16x32_i8(nz_a, b, d, 0, 0, 0);
+          d = __builtin_amdgcn_mfma_i32_16x16x32_i8(nz_b, b, d, 0, 0, 0);
+          if constexpr (UPB != 0) {
+            if ((u & mask) == mask) {  // the block's last unit
+              // position r * 64 + lane for row 4 kg + r: a wave's 64 stores of one r fall on 64 banks
+              float* at = &terms[parity][wave * BW + u / UPB][lane];
+#pragma unroll
+              for (int r = 0; r < 4; ++r) at[r * 64] = float(d[r]) * set.s[sl][j];
+            }
+          }
+        }
+      }
+      if constexpr (UPB != 0) {
+        __syncthreads();
+#pragma unroll
+        for (int blk = 0; blk < NB; ++blk) acc = acc + terms[parity][blk][tid];
+        parity ^= 1;
+      }
+    }
+  };
+
+  for (uint32_t g = 0; g < groups; g += 2) {
+    if (g + 1 < groups) load_set(set_b, g + 1);
+    process(set_a, g);
+    if (g + 1 < groups) {
+      if (g + 2 < groups) load_set(set_a, g + 2);
+      process(set_b, g + 1);
+    }
+  }
+
+  // thread tid = r * 64 + kg * 16 + column owns row 4 kg + r
+  const uint32_t row = ((tid >> 4) & 3) * 4 + (tid >> 6), n = tile * kTileCols + (tid & 15), m = row0 + row;
+  if constexpr (UPB == 0) {
+    // one block: the waves' integer sums meet in LDS, then one scaling
+    __shared__ int totals[4][256];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) totals[wave][r * 64 + lane] = d[r];
+    __syncthreads();
+    const uint32_t mc = m < p.m ? m : p.m - 1;
+    const int nzp = ldg<int32_t>(p.rows + 8ull * mc + 4);
+    const int iacc = totals[0][tid] + totals[1][tid] + totals[2][tid] + totals[3][tid] - 256 * nzp * int(L.quads * 4);
+    acc = float(iacc) * ldg<float>(p.compact + L.scale_off + (n < p.n ? n : p.n - 1) * 4ull);
+  }
+  if (n < p.n && m < p.m) {
+    const float recip = bits_f32(ldg<uint32_t>(p.rows + 8ull * m));
+    const float bias = ldg<float>(p.compact + L.bias_off + n * 4ull);
+    finish_store<T>(p.out + (uint64_t(m) * p.n + n) * item, acc, recip, p.has_bias != 0, bias);
+  }
+}
+
 bool check_q4_shape(uint32_t m, uint32_t n, uint32_t k, uint32_t bs, std::string* err) {
   if (bs == 0 || !(bs == k || (bs % 32 == 0 && k % bs == 0))) {
     *err = "qmm4: block size must equal k or be a multiple of 32 dividing k";
@@ -590,13 +937,17 @@ int launch_stream_rows(const Q4CParams& p, const CompactLayout& L, uint32_t grou
 
 uint64_t qmm4c_bytes(uint32_t n, uint32_t k, uint32_t bs) {
   CompactLayout L;
-  return compact_layout(n, k, bs, &L) ? L.total : 0;
+  MatrixLayout M;
+  if (!compact_layout(n, k, bs, &L) || !matrix_layout(n, k, bs, &M)) return 0;
+  return L.total > M.total ? L.total : M.total;  // either layout fits
 }
 
 uint64_t qmm4c_q_bytes(uint32_t m, uint32_t k) {
   if (m == 0 || k == 0) return 0;
   const uint64_t nunits = (k + kUnit - 1) / kUnit, rounds = (nunits + kRoundUnits - 1) / kRoundUnits;
-  return round_up_u64(uint64_t(m) * rounds * kRoundUnits * kUnit, 256);
+  const uint64_t streaming = uint64_t(m) * rounds * kRoundUnits * kUnit;
+  const uint64_t matrix = uint64_t((m + 15) / 16) * ((nunits + 63) / 64 * 16) * 2048;
+  return round_up_u64(streaming > matrix ? streaming : matrix, 256);
 }
 
 int launch_qmm4(const Q4Params& p, int dtype, uint32_t phase, uint32_t groupwise, const Machine&, hipStream_t stream,
@@ -633,24 +984,31 @@ int launch_qmm4(const Q4Params& p, int dtype, uint32_t phase, uint32_t groupwise
   return 0;
 }
 
-int launch_qmm4c_pack(const Q4PackParams& p, const Machine&, hipStream_t stream, std::string* err) {
+int launch_qmm4c_pack(const Q4PackParams& p, uint32_t layout, const Machine&, hipStream_t stream, std::string* err) {
   CompactLayout L;
+  MatrixLayout M;
   if (!check_q4_shape(1, p.n, p.k, p.bs, err)) return -1;
-  if (!compact_layout(p.n, p.k, p.bs, &L)) {
+  if (!compact_layout(p.n, p.k, p.bs, &L) || !matrix_layout(p.n, p.k, p.bs, &M)) {
     *err = "qmm4c_pack: this shape has no compact form (groupwise block sizes: 32, 64, 128, 256)";
+    return -1;
+  }
+  if (layout > 1) {
+    *err = "qmm4c_pack: LAYOUT must be 0 (streaming) or 1 (matrix cores)";
     return -1;
   }
   if (!p.packed || !p.compact || (p.compact & 15)) {
     *err = "qmm4c_pack: null or unaligned address";
     return -1;
   }
-  const uint64_t threads = L.nib_bytes / 16 + (L.upb ? L.scale_bytes / 4 : p.n) + p.n;
+  const uint64_t threads = layout == 0 ? L.nib_bytes / 16 + (L.upb ? L.scale_bytes / 4 : p.n) + p.n
+                                       : M.nib_bytes / 16 + (M.upb ? M.scale_bytes / 4 : p.n) + p.n;
   const uint64_t groups = (threads + 255) / 256;
   if (groups >= (1ull << 31)) {
     *err = "qmm4c_pack: too large";
     return -1;
   }
-  hipLaunchKernelGGL(qmm4c_pack_kernel, dim3(uint32_t(groups)), dim3(256), 0, stream, p, L);
+  if (layout == 0) hipLaunchKernelGGL(qmm4c_pack_kernel, dim3(uint32_t(groups)), dim3(256), 0, stream, p, L);
+  else hipLaunchKernelGGL(qmm4m_pack_kernel, dim3(uint32_t(groups)), dim3(256), 0, stream, p, M);
   if (hipGetLastError() != hipSuccess) {
     *err = "qmm4c_pack: kernel launch failed";
     return -1;
@@ -658,11 +1016,76 @@ int launch_qmm4c_pack(const Q4PackParams& p, const Machine&, hipStream_t stream,
   return 0;
 }
 
-int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwise, uint32_t, const Machine& mc,
+// The matrix-layout form of the product: phase 0, 1 or 2 (= 0 then 1).
+template <class T>
+int launch_matrix(const Q4CParams& p, uint32_t phase, uint32_t groupwise, hipStream_t stream, std::string* err) {
+  constexpr uint32_t item = sizeof(typename T::storage);
+  MatrixLayout M;
+  if (!matrix_layout(p.n, p.k, p.bs, &M)) {
+    *err = "qmm4c: this shape has no compact form (groupwise block sizes: 32, 64, 128, 256)";
+    return -1;
+  }
+  if (!p.q || !p.rows || (p.q & 15)) {
+    *err = "qmm4c: null or unaligned tensor address";
+    return -1;
+  }
+  if (phase == 0 || phase == 2) {
+    if (p.m > 65535) {
+      *err = "qmm4c: at most 65535 rows per dispatch";
+      return -1;
+    }
+    const bool fast = p.k % 8 == 0 && p.k <= 2048u * kFusedGroups && (p.inp & 15) == 0 && (uint64_t(p.k) * item) % 16 == 0;
+    if (fast) hipLaunchKernelGGL((qmm4m_rowquant<T, true>), dim3(p.m), dim3(256), 0, stream, p, groupwise, M.quads);
+    else hipLaunchKernelGGL((qmm4m_rowquant<T, false>), dim3(p.m), dim3(256), 0, stream, p, groupwise, M.quads);
+  }
+  if (phase == 1 || phase == 2) {
+    if (!p.compact || (p.compact & 15)) {
+      *err = "qmm4c: null or unaligned side-car address";
+      return -1;
+    }
+    for (uint32_t m0 = 0; m0 < p.m; m0 += 16 * 1024) {
+      const uint32_t rows = p.m - m0 < 16 * 1024 ? p.m - m0 : 16 * 1024;
+      const dim3 grid(M.tiles, (rows + 15) / 16);
+      switch (M.upb) {
+        case 0: hipLaunchKernelGGL((qmm4m_tile<T, 0>), grid, dim3(256), 0, stream, p, M, m0); break;
+        case 1: hipLaunchKernelGGL((qmm4m_tile<T, 1>), grid, dim3(256), 0, stream, p, M, m0); break;
+        case 2: hipLaunchKernelGGL((qmm4m_tile<T, 2>), grid, dim3(256), 0, stream, p, M, m0); break;
+        case 4: hipLaunchKernelGGL((qmm4m_tile<T, 4>), grid, dim3(256), 0, stream, p, M, m0); break;
+        case 8: hipLaunchKernelGGL((qmm4m_tile<T, 8>), grid, dim3(256), 0, stream, p, M, m0); break;
+        default: *err = "qmm4c: bad layout"; return -1;
+      }
+    }
+  }
+  return 0;
+}
+
+int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwise, uint32_t layout, const Machine& mc,
                  hipStream_t stream, std::string* err) {
   if (p.m == 0 || p.n == 0) return 0;
   CompactLayout L;
   if (!check_q4_shape(p.m, p.n, p.k, p.bs, err)) return -1;
+  if (layout > 1) {
+    *err = "qmm4c: LAYOUT must be 0 (streaming) or 1 (matrix cores)";
+    return -1;
+  }
+  if (layout == 1) {
+    if (groupwise != (p.bs != p.k ? 1u : 0u)) {
+      *err = "qmm4c: GROUPWISE must be 1 exactly when bs != k";
+      return -1;
+    }
+    if (!p.inp || !p.out || phase > 2) {
+      *err = phase > 2 ? "qmm4c: PHASE must be 0, 1 or 2" : "qmm4c: null or unaligned tensor address";
+      return -1;
+    }
+    const int rc = dtype == VKT_F32 ? launch_matrix<f32_t>(p, phase, groupwise, stream, err)
+                                    : launch_matrix<bf16_t>(p, phase, groupwise, stream, err);
+    if (rc != 0) return rc;
+    if (hipGetLastError() != hipSuccess) {
+      *err = "qmm4c: kernel launch failed";
+      return -1;
+    }
+    return 0;
+  }
   if (!compact_layout(p.n, p.k, p.bs, &L)) {
     *err = "qmm4c: this shape has no compact form (groupwise block sizes: 32, 64, 128, 256)";
     return -1;

@@ -124,21 +124,24 @@ at::Tensor dyn_quant_pack_4bit_weight(const at::Tensor& weights, const at::Tenso
   return out;
 }
 
-// Compact side-cars of packed weight vectors, one per live packed tensor: keyed by the
-// storage, its data pointer and the tensor's version counter, dropped when the storage
-// dies or the tensor is written to.  (The reference streams the float32-expanded vector
+// Compact side-cars of packed weight vectors, per live packed tensor and layout (0: streamed
+// by the kernel for at most 4 rows, 1: for the matrix cores; a weight that sees both kinds of
+// call holds both, each the size of the nibbles plus scales): keyed by the storage, its data
+// pointer and the tensor's version counter, dropped when the storage dies or the tensor is
+// written to.  (The reference streams the float32-expanded vector
 // itself: 4 bytes of traffic per byte of nibbles.)
 struct SideCar {
   c10::weak_intrusive_ptr<c10::StorageImpl> storage;
   const void* data;
-  uint32_t version;
+  int64_t version;
   int64_t offset, numel, bs, k, n;
+  uint32_t layout;
   at::Tensor compact;
 };
 std::mutex g_sidecar_mutex;
 std::list<SideCar> g_sidecars;
 
-at::Tensor sidecar_for(const at::Tensor& packed, int64_t bs, int64_t K, int64_t N, bool has_bias) {
+at::Tensor sidecar_for(const at::Tensor& packed, int64_t bs, int64_t K, int64_t N, bool has_bias, uint32_t layout) {
   const uint64_t bytes = vkt_qmm4c_bytes(static_cast<uint32_t>(N), static_cast<uint32_t>(K), static_cast<uint32_t>(bs));
   if (bytes == 0) return at::Tensor();
   std::lock_guard<std::mutex> lock(g_sidecar_mutex);
@@ -149,7 +152,7 @@ at::Tensor sidecar_for(const at::Tensor& packed, int64_t bs, int64_t K, int64_t 
     }
     if (it->storage._unsafe_get_target() == packed.storage().unsafeGetStorageImpl() && it->data == packed.const_data_ptr() &&
         it->version == packed._version() && it->offset == packed.storage_offset() && it->numel == packed.numel() &&
-        it->bs == bs && it->k == K && it->n == N) {
+        it->bs == bs && it->k == K && it->n == N && it->layout == layout) {
       return it->compact;
     }
     ++it;
@@ -162,11 +165,11 @@ at::Tensor sidecar_for(const at::Tensor& packed, int64_t bs, int64_t K, int64_t 
   p.k = static_cast<uint32_t>(K);
   p.bs = static_cast<uint32_t>(bs);
   p.has_bias = has_bias ? 1u : 0u;
-  dispatch("qmm4c_pack", {}, p, 1);
+  dispatch("qmm4c_pack", {layout}, p, 1);
   if (g_sidecars.size() >= 64) g_sidecars.pop_front();
   g_sidecars.push_back(SideCar{c10::weak_intrusive_ptr<c10::StorageImpl>(packed.storage().getWeakStorageImpl()),
                                packed.const_data_ptr(), packed._version(), packed.storage_offset(), packed.numel(), bs,
-                               K, N, compact});
+                               K, N, layout, compact});
   return compact;
 }
 
@@ -203,7 +206,8 @@ at::Tensor dyn_quant_matmul_4bit(const at::Tensor& inp, const at::Tensor& packed
   const uint32_t groupwise = block_size != K ? 1u : 0u;
   const int64_t item = x.element_size();
 
-  at::Tensor compact = sidecar_for(packed, block_size, K, N, bias_elements != 0);
+  const uint32_t layout = M > 4 ? 1u : 0u;
+  at::Tensor compact = sidecar_for(packed, block_size, K, N, bias_elements != 0, layout);
   if (compact.defined()) {
     for (int64_t r0 = 0; r0 < M; r0 += kMaxRows) {
       const int64_t rows_here = std::min<int64_t>(M - r0, kMaxRows);
@@ -222,7 +226,7 @@ at::Tensor dyn_quant_matmul_4bit(const at::Tensor& inp, const at::Tensor& packed
       p.k = static_cast<uint32_t>(K);
       p.bs = static_cast<uint32_t>(block_size);
       p.has_bias = bias_elements != 0 ? 1u : 0u;
-      dispatch(std::string("qmm4c_") + label, {2u, groupwise}, p, 1);
+      dispatch(std::string("qmm4c_") + label, {2u, groupwise, layout}, p, 1);
     }
     return output;
   }
