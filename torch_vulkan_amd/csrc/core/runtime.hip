@@ -64,12 +64,14 @@ struct Runtime {
   std::atomic<uint64_t> dispatches{0};
   bool trace = false;
   uint64_t generation = 0;
+  void* workspace_base = nullptr;
 
   ~Runtime() {
     if (stream) {
       (void)hipStreamSynchronize(stream);
     }
     pool.reset();
+    if (workspace_base) (void)hipFree(workspace_base);
     if (stream) (void)hipStreamDestroy(stream);
   }
 };
@@ -117,6 +119,21 @@ std::shared_ptr<Runtime> runtime(std::string* err) {
     return nullptr;
   }
   rt->machine.compute_units = rt->props.multiProcessorCount;
+  // The kernels' own workspace (partial tiles of products that are split over workgroups).
+  // Held outside the pool until shutdown: it is not the caller's memory and does not show
+  // in vkt_memory_stats.  Every use is queued on the runtime's one stream, so uses do not
+  // overlap.
+  {
+    constexpr uint64_t kWorkspaceBytes = 32ull << 20;
+    void* base = nullptr;
+    if ((e = hipMalloc(&base, kWorkspaceBytes)) != hipSuccess) {
+      *err = hip_message("workspace allocation", e);
+      return nullptr;
+    }
+    rt->workspace_base = base;
+    rt->machine.workspace = reinterpret_cast<uint64_t>(base);
+    rt->machine.workspace_bytes = kWorkspaceBytes;
+  }
   rt->pool = std::make_unique<Pool<HipSource>>(HipSource{});
   rt->pool->set_idle_hook(&idle_hook, rt.get());
   const char* tr = std::getenv("TORCH_VK_TRACE");  // reference ffi.rs:144-148

@@ -13,6 +13,9 @@ namespace vkt {
 
 struct Machine {
   int compute_units = 256;
+  // device memory the runtime owns for kernels that split one product over several
+  // workgroups: partial results between a kernel and the one that adds them up
+  uint64_t workspace = 0, workspace_bytes = 0;
 };
 
 // spec[1] of the qmm8 kernels: 0 = planned by the library; otherwise an explicit

@@ -182,10 +182,48 @@ __device__ __forceinline__ V4F mfma16(const U4& w, const U4& a, const V4F& acc) 
 // Lane (c = lane % 16, g = lane / 16) streams 16 bytes of weight row n0 + 16 t + c at
 // k0 + 16 g (two MFMA operands) and the matching 16 activations of rows 16 mt + c; the
 // MFMA's first operand is the weights, so the lane ends with C[16 mt + c][n0 + 16 t + 4 g + r].
+// The epilogue of the matrix-core kernels: lane (c = lane % 16, g = lane / 16) holds, per
+// tile (mt, t), the sums of row 16 mt + c for columns n0 + 16 t + 4 g .. + 3.
+template <class T, int MT, int NT>
+__device__ __forceinline__ void store_tiles(const Q8Params& p, uint32_t n0, const V4F (&acc)[MT][NT], int lane) {
+  constexpr uint64_t item = 2;
+  const int c = lane & 15, g = lane >> 4;
+  const bool vec_ok = (p.n & 3u) == 0 && (p.c & 7u) == 0;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const uint32_t n = n0 + 16 * t + 4 * g;
+    float scale[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) scale[r] = load_f32<T>(p.scales + (n + r < p.n ? n + r : p.n - 1) * item);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const uint32_t m = 16 * mt + c;
+      if (m >= p.m || n >= p.n) continue;
+      const uint64_t at = p.c + (uint64_t(m) * p.n + n) * item;
+      uint32_t h[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float v = acc[mt][t][r] * scale[r];
+        h[r] = T::dtype == VKT_BF16 ? f32_to_bf16(v) : f32_to_f16(v);
+      }
+      if (vec_ok && n + 3 < p.n) {
+        stg<U2>(at, U2{h[0] | h[1] << 16, h[2] | h[3] << 16});
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (n + r < p.n) stg<uint16_t>(at + r * item, uint16_t(h[r]));
+      }
+    }
+  }
+}
+
 template <class T, int MT, int NT, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void qmm8_mfma(Q8Params p) {
+__global__ __launch_bounds__(WAVES * 64) void qmm8_mfma(Q8Params p, uint32_t chunks_per_slice, uint64_t workspace) {
   constexpr uint64_t item = 2;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
+  // gridDim.y slices of K (in chunks of 64 values), one per workgroup of the column group
+  const uint32_t k_begin = blockIdx.y * chunks_per_slice * 64;
+  const uint32_t k_end = k_begin + chunks_per_slice * 64 < p.k ? k_begin + chunks_per_slice * 64 : p.k;
   const uint32_t n0 = blockIdx.x * 16 * NT;
   uint64_t brow[NT], arow[MT];
 #pragma unroll
@@ -206,7 +244,7 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma(Q8Params p) {
 
   const U4 zero = {0, 0, 0, 0};
 #pragma unroll 2
-  for (uint32_t k0 = wave * 64; k0 < p.k; k0 += WAVES * 64) {
+  for (uint32_t k0 = k_begin + wave * 64; k0 < k_end; k0 += WAVES * 64) {
     const bool inside = k0 + 16 * g < p.k;  // (k is a multiple of 16)
     U4 wv[NT], a0[MT], a1[MT];
 #pragma unroll
@@ -247,68 +285,81 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma(Q8Params p) {
     }
   }
   if (wave != 0) return;
-  const bool vec_ok = (p.n & 3u) == 0 && (p.c & 7u) == 0;
+  if (gridDim.y > 1) {
+    // one of several slices of K: the tile goes to the workspace, and qmm8_mfma_finish adds
+    // the slices up in slice order
+    V4F* const mine = reinterpret_cast<V4F*>(workspace) + (uint64_t(blockIdx.x) * gridDim.y + blockIdx.y) * (MT * NT * 64);
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const uint32_t n = n0 + 16 * t + 4 * g;
-    float scale[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) scale[r] = load_f32<T>(p.scales + (n + r < p.n ? n + r : p.n - 1) * item);
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const uint32_t m = 16 * mt + c;
-      if (m >= p.m || n >= p.n) continue;
-      const uint64_t at = p.c + (uint64_t(m) * p.n + n) * item;
-      uint32_t h[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float v = acc[mt][t][r] * scale[r];
-        h[r] = T::dtype == VKT_BF16 ? f32_to_bf16(v) : f32_to_f16(v);
-      }
-      if (vec_ok && n + 3 < p.n) {
-        stg<U2>(at, U2{h[0] | h[1] << 16, h[2] | h[3] << 16});
-      } else {
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (n + r < p.n) stg<uint16_t>(at + r * item, uint16_t(h[r]));
-      }
-    }
+    for (int i = 0; i < MT * NT; ++i) mine[i * 64 + lane] = acc[i / NT][i % NT];
+    return;
   }
+  store_tiles<T, MT, NT>(p, n0, acc, lane);
+}
+
+// Adds up the slices of one column group (one wave per group), in slice order.
+template <class T, int MT, int NT>
+__global__ __launch_bounds__(64) void qmm8_mfma_finish(Q8Params p, uint32_t slices, uint64_t workspace) {
+  const int lane = threadIdx.x;
+  const V4F* const tiles = reinterpret_cast<const V4F*>(workspace) + uint64_t(blockIdx.x) * slices * (MT * NT * 64);
+  V4F acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT * NT; ++i) acc[i / NT][i % NT] = tiles[i * 64 + lane];
+  for (uint32_t sl = 1; sl < slices; ++sl) {
+#pragma unroll
+    for (int i = 0; i < MT * NT; ++i) acc[i / NT][i % NT] += tiles[uint64_t(sl) * (MT * NT * 64) + i * 64 + lane];
+  }
+  store_tiles<T, MT, NT>(p, blockIdx.x * 16 * NT, acc, lane);
 }
 
 template <class T, int MT, int NT>
-void launch_mfma_waves(const Q8Params& p, int waves, hipStream_t stream) {
-  const dim3 grid((p.n + 16 * NT - 1) / (16 * NT));
+void launch_mfma_waves(const Q8Params& p, int waves, uint32_t slices, const Machine& mc, hipStream_t stream) {
+  const dim3 grid((p.n + 16 * NT - 1) / (16 * NT), slices);
+  const uint32_t chunks = (p.k + 63) / 64, per_slice = (chunks + slices - 1) / slices;
   switch (waves) {
-    case 4: hipLaunchKernelGGL((qmm8_mfma<T, MT, NT, 4>), grid, dim3(256), 0, stream, p); break;
-    case 8: hipLaunchKernelGGL((qmm8_mfma<T, MT, NT, 8>), grid, dim3(512), 0, stream, p); break;
-    default: hipLaunchKernelGGL((qmm8_mfma<T, MT, NT, 16>), grid, dim3(1024), 0, stream, p); break;
+    case 4: hipLaunchKernelGGL((qmm8_mfma<T, MT, NT, 4>), grid, dim3(256), 0, stream, p, per_slice, mc.workspace); break;
+    case 8: hipLaunchKernelGGL((qmm8_mfma<T, MT, NT, 8>), grid, dim3(512), 0, stream, p, per_slice, mc.workspace); break;
+    default: hipLaunchKernelGGL((qmm8_mfma<T, MT, NT, 16>), grid, dim3(1024), 0, stream, p, per_slice, mc.workspace); break;
   }
+  if (slices > 1) hipLaunchKernelGGL((qmm8_mfma_finish<T, MT, NT>), dim3(grid.x), dim3(64), 0, stream, p, slices, mc.workspace);
 }
 
-// Rows (<= 64) of 16-bit activations on the matrix cores.  Columns per workgroup and waves
-// per workgroup are chosen so that the grid covers the machine: many small workgroups
-// when N is large, more k-splitting when it is not.
+// Rows (<= 64) of 16-bit activations on the matrix cores.  A workgroup takes 64 columns
+// where there are that many, so that an activation fragment is reused over 4 weight
+// fragments (every workgroup reads all the activations of its slice of K from L2: with 16
+// columns per workgroup that traffic is several times the weight stream once M reaches 64),
+// and K is cut into slices across workgroups until the grid covers the machine about
+// twice.  variant = NT | WAVES << 8 | SLICES << 24 overrides the plan (tuning, tests).
 template <class T>
 void launch_mfma(const Q8Params& p, uint32_t variant, const Machine& mc, hipStream_t stream) {
   const int mt = p.m <= 16 ? 1 : p.m <= 32 ? 2 : 4;
-  // measured on MI355X (bf16, K = 4096 / 14336): with many columns, 64 per workgroup and 8
-  // k-slices (the activation fragments are then reused over 4 weight fragments); with few
-  // columns the grid matters more than the reuse: 16 per workgroup, 16 k-slices
-  (void)mc;
-  int nt = p.n >= 8192 ? 4 : 1, waves = p.n >= 8192 ? 8 : 16;
-  while (waves > 4 && p.k < uint32_t(waves) * 64) waves /= 2;
+  int nt = p.n >= 64 ? 4 : 1, waves = p.m > 32 ? 4 : 8;  // (measured: K = 4096 and 14336, N = 14336 and 4096)
+  uint32_t slices = 1;
   if (variant & 0xffff) {
     nt = variant & 0xff;
     waves = (variant >> 8) & 0xff;
+    slices = (variant >> 24) ? (variant >> 24) : 1;
+  } else {
+    const uint32_t groups = (p.n + 16 * nt - 1) / (16 * nt), chunks = (p.k + 63) / 64;
+    while (waves > 4 && chunks < uint32_t(waves)) waves /= 2;
+    const uint32_t want = (uint32_t(mc.compute_units) + groups / 2) / groups;  // about one workgroup per compute unit
+    const uint32_t most = chunks / (2u * waves) ? chunks / (2u * waves) : 1;   // >= 2 chunks per wave
+    slices = want < most ? want : most;
+    if (slices < 1) slices = 1;
+    if (slices > 16) slices = 16;
   }
+  // the workspace holds groups * slices tiles of MT * NT KiB
+  const uint64_t groups = (p.n + 16 * nt - 1) / (16 * nt);
+  while (slices > 1 && groups * slices * mt * nt * 1024 > mc.workspace_bytes) --slices;
+  const uint32_t chunks = (p.k + 63) / 64;
+  while (slices > 1 && (chunks + slices - 1) / slices * (slices - 1) >= chunks) --slices;  // no empty slice
 #define VKT_MFMA_CASE(MT_, NT_) \
-  if (mt == MT_ && nt == NT_) return launch_mfma_waves<T, MT_, NT_>(p, waves, stream);
+  if (mt == MT_ && nt == NT_) return launch_mfma_waves<T, MT_, NT_>(p, waves, slices, mc, stream);
   VKT_MFMA_CASE(1, 1) VKT_MFMA_CASE(1, 2) VKT_MFMA_CASE(1, 4)
   VKT_MFMA_CASE(2, 1) VKT_MFMA_CASE(2, 2) VKT_MFMA_CASE(2, 4)
   VKT_MFMA_CASE(4, 1) VKT_MFMA_CASE(4, 2) VKT_MFMA_CASE(4, 4)
+  VKT_MFMA_CASE(1, 8) VKT_MFMA_CASE(2, 8) VKT_MFMA_CASE(4, 8)
 #undef VKT_MFMA_CASE
-  launch_mfma_waves<T, 4, 1>(p, waves, stream);
+  launch_mfma_waves<T, 4, 1>(p, waves, slices, mc, stream);
 }
 
 
