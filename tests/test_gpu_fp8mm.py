@@ -19,12 +19,14 @@ FLOAT8 = [torch.float8_e4m3fn, torch.float8_e5m2]
 
 # The fp8 matrix core adds the 128 products of one instruction in a fixed-point window
 # ~14 bits below the largest product (a hardware property, measured: ~2^-15.3 of sum|a||b| on
-# random data); bfloat16 / float8 outputs take that path, float32 / float16 outputs do not.
+# random data); bfloat16 / float8 outputs take that path, float32 / float16 outputs (and
+# variants 6, 7) run the bfloat16 matrix core on exactly widened operands, inside the
+# reference's own bound.
 HW_WINDOW = 2.0**-13
 
 
 def on_matrix_cores(odt, variant, k):
-    if variant == 255 or k % 16:
+    if variant in (6, 7, 255) or k % 16:
         return False
     return variant in (1, 2, 3, 4, 5) or odt in (oracle.BF16, oracle.E4M3, oracle.E5M2)
 
@@ -77,7 +79,7 @@ def test_scaled_mm_reference_cases(fa, fb, out_dtype, rowwise):
 
 @pytest.mark.parametrize("m,k,n", [(1, 16, 1), (130, 256, 70), (257, 384, 129), (64, 1040, 300), (300, 128, 520),
                                    (5, 100, 7), (33, 48, 17)])
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 255])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 255])
 @pytest.mark.parametrize("rowwise", [False, True])
 def test_scaled_mm_tile_edges(m, k, n, variant, rowwise):
     """Shapes that are not multiples of any tile, K tails (K % 128 != 0, K % 16 != 0 -> the
@@ -138,6 +140,28 @@ def test_scaled_mm_config4_8192_cubed():
     assert np.array_equal(oracle.bf16_to_f32(got2), oracle.bf16_to_f32(got) * 2)
 
 
+@pytest.mark.parametrize("fa,fb", [(FLOAT8[0], FLOAT8[0]), (FLOAT8[1], FLOAT8[0]), (FLOAT8[1], FLOAT8[1])])
+def test_scaled_mm_float32_output_large(fa, fb):
+    """float32 output at a size where the path matters (the exact kernel on 256x256 tiles,
+    direct-to-LDS loads): sampled rows / columns inside the reference's bound
+    eps*|want| + 2^-20*sum|a||b|, and within the stated 1e-4 of the float64 closed form."""
+    import _dev
+    m, k, n = 1024, 8192, 1280
+    a = torch.randn(m, k, generator=gen(1060)).to(fa)
+    bt = torch.randn(n, k, generator=gen(1061)).to(fb)
+    sa = torch.empty(m, 1).uniform_(0.5, 2, generator=gen(1062)).numpy()
+    sb = torch.empty(1, n).uniform_(0.5, 2, generator=gen(1063)).numpy()
+    got = _dev.scaled_mm(bits(a), ODT[fa], bits(bt), ODT[fb], sa, sb, True, out_dtype=oracle.F32)
+    rows, cols = np.array([0, 31, 32, 255, 256, 700, 1023]), np.array([0, 1, 127, 128, 255, 256, 1279])
+    af = oracle.fp8_table(ODT[fa])[bits(a)[rows]].astype(np.float64)
+    bf = oracle.fp8_table(ODT[fb])[bits(bt)[cols]].astype(np.float64)
+    scale = sa.reshape(-1)[rows][:, None].astype(np.float64) * sb.reshape(-1)[cols][None, :]
+    truth, mag = (af @ bf.T) * scale, (np.abs(af) @ np.abs(bf).T) * scale
+    sub = got[np.ix_(rows, cols)].astype(np.float64)
+    assert (np.abs(sub - truth) <= ref_tol(truth, mag, oracle.F32)).all()
+    assert np.allclose(sub, truth, rtol=1e-4, atol=1e-4)
+
+
 def test_scaled_mm_config5_rowwise_70b():
     """BASELINE config 5: rowwise scales, M=4096, K=8192, N=28672, bf16 out."""
     import _dev
@@ -165,4 +189,4 @@ def test_scaled_mm_errors():
         abi.dispatch("fp8mm", [0], p)
     p.lda = 16
     with pytest.raises(abi.VktError, match="unknown variant"):
-        abi.dispatch("fp8mm", [9], p)
+        abi.dispatch("fp8mm", [99], p)

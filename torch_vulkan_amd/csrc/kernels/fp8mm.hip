@@ -13,9 +13,11 @@
 // sum|a||b| per output, invisible at bfloat16 / float8 output precision (eps >= 2^-8) but
 // not at float32.  So the path is chosen by the precision the caller asked for:
 //   bfloat16 / float8 outputs  -> fp8mm_mfma (this is the 5 PFLOP/s path)
-//   float32 / float16 outputs  -> exact float32 products and sums (fp8mm_generic), inside the
-//                                 reference test's bound eps*|want| + 2^-20 * sum|a||b|
-//                                 (tests/python/test_quant.py:124-126)
+//   float32 / float16 outputs  -> the same kernel with each float8 fragment widened (exactly)
+//                                 to bfloat16 in registers and fed to the bfloat16 matrix
+//                                 core, which keeps float32 precision (half the rate: 2.5
+//                                 PFLOP/s peak); inside the reference test's bound
+//                                 eps*|want| + 2^-20 * sum|a||b| (tests/python/test_quant.py:124-126)
 // The scales multiply once per output instead of once per operand element (one rounding
 // less than the reference, inside the same bound).
 //
@@ -120,6 +122,24 @@ __device__ __forceinline__ V16F mfma_f8_32(const V8I& first, const V8I& second, 
   return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(first, second, acc, FB, FA, 0, 0, 0, 0);
 }
 
+// The exact path: float8 values widen exactly to bfloat16 (two per instruction), and the
+// bfloat16 matrix core adds its products at float32 precision (measured: within 2^-27 of
+// sum|a||b|).  Slice q of a 32-byte fragment = its bytes 8 q .. 8 q + 7: both operands are
+// sliced alike, so every product pairs the same k.
+using V8BF = __bf16 __attribute__((ext_vector_type(8)));
+using V2BF = __bf16 __attribute__((ext_vector_type(2)));
+template <int F, bool HI>
+__device__ __forceinline__ V2BF widen_pair(int word) {
+  if constexpr (F == 0) return __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(word, 1.0f, HI);
+  else return __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(word, 1.0f, HI);
+}
+template <int F>
+__device__ __forceinline__ V8BF widen_slice(const V8I& frag, int q) {
+  const V2BF p0 = widen_pair<F, false>(frag[2 * q]), p1 = widen_pair<F, true>(frag[2 * q]);
+  const V2BF p2 = widen_pair<F, false>(frag[2 * q + 1]), p3 = widen_pair<F, true>(frag[2 * q + 1]);
+  return V8BF{p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
+}
+
 // LDS tile: rows of 128 bytes; 16-byte chunk c of row r sits at chunk c ^ ((r >> 1) & 7).
 // The LDS serves 16 lanes of a 128-bit read per clock from 64 banks (256 bytes), and the 16
 // lanes of a fragment read hold 16 consecutive rows at one logical chunk: two rows share a
@@ -130,7 +150,7 @@ __device__ __forceinline__ uint32_t tile_offset(uint32_t row, uint32_t chunk) {
   return row * BK + ((chunk ^ ((row >> 1) & 7u)) << 4);
 }
 
-template <int WAVES_M, int WAVES_N, int TM, int TN, int FA, int FB, bool MF32 = false, bool DIRECT = false>
+template <int WAVES_M, int WAVES_N, int TM, int TN, int FA, int FB, bool MF32 = false, bool DIRECT = false, bool WIDE = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, uint32_t tiles_m, uint32_t tiles_n) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * TM * 16, BN = WAVES_N * TN * 16;
@@ -293,6 +313,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, 
         const int kk = gi / TM2, i = gi % TM2;
         V8I next = af;
         if (gi + 1 < 2 * TM2) next = frag32(ta, (wm * TM2 + (gi + 1) % TM2) * 32 + l32, (gi + 1) / TM2);
+        V8BF af_wide[WIDE ? 4 : 1];
+        if constexpr (WIDE) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) af_wide[q] = widen_slice<FA>(af, q);
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < TN2; ++j) {
@@ -303,7 +328,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, 
             side(op, s, steady);
             __builtin_amdgcn_sched_barrier(0);
           }
-          acc32[i][j] = mfma_f8_32<FA, FB>(bf[kk][j], af, acc32[i][j]);
+          if constexpr (WIDE) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              acc32[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(widen_slice<FB>(bf[kk][j], q), af_wide[q], acc32[i][j], 0, 0, 0);
+          } else {
+            acc32[i][j] = mfma_f8_32<FA, FB>(bf[kk][j], af, acc32[i][j]);
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
         af = next;
@@ -461,13 +492,14 @@ __global__ __launch_bounds__(256) void fp8mm_generic(F8Params p) {
   store_out(p, uint64_t(m) * p.ldo + n, finish(p, acc, sa, sb, n, output_inv(p)));
 }
 
-template <int WAVES_M, int WAVES_N, int TM, int TN, int FA, int FB, bool MF32 = false, bool DIRECT = false>
+template <int WAVES_M, int WAVES_N, int TM, int TN, int FA, int FB, bool MF32 = false, bool DIRECT = false, bool WIDE = false>
 int launch_tile(const F8Params& p, hipStream_t stream, std::string* err) {
   constexpr int BM = WAVES_M * TM * 16, BN = WAVES_N * TN * 16;
   constexpr uint32_t operand_bytes = 2 * (BM + BN) * BK, epilogue_bytes = WAVES_M * WAVES_N * TM * 16 * 256;
   constexpr uint32_t lds_bytes = operand_bytes > epilogue_bytes ? operand_bytes : epilogue_bytes;
   static_assert(TN % 4 == 0, "the epilogue moves 64 columns (4 tiles) per pass");
-  auto kernel = fp8mm_mfma<WAVES_M, WAVES_N, TM, TN, FA, FB, MF32, DIRECT>;
+  static_assert(!WIDE || MF32, "the exact path is built on the 32x32 tiles");
+  auto kernel = fp8mm_mfma<WAVES_M, WAVES_N, TM, TN, FA, FB, MF32, DIRECT, WIDE>;
   static bool configured = false;  // guarded by the runtime's stream mutex
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -496,8 +528,15 @@ int launch_formats(const F8Params& p, uint32_t variant, hipStream_t stream, std:
   // 128x128, 16x16x128); 3: 256x128; 4: 256x256 with the 32x32x64 MFMA (measured ~10 % faster
   // than 16x16x128 at equal work); 5: as 4 with global-to-LDS direct loads when k is a
   // multiple of 128 (else 4).  255: the one-thread-per-output kernel.
-  if (variant == 0) variant = (uint64_t(p.m) * p.n >= (1ull << 20)) ? 5 : 1;
+  // 6 / 7: the exact path (float8 widened to bfloat16 in registers, 32x32x16 bfloat16 MFMA) on
+  // 256x256 / 128x128 tiles: what float32 and float16 outputs get.
+  const bool big = uint64_t(p.m) * p.n >= (1ull << 20);
+  if (variant == 0) variant = (p.out_dtype == VKT_F32 || p.out_dtype == VKT_F16) ? (big ? 6 : 7) : (big ? 5 : 1);
   switch (variant) {
+    case 6:
+      if (p.k % BK == 0) return launch_tile<2, 2, 8, 8, FA, FB, true, true, true>(p, stream, err);
+      return launch_tile<2, 2, 8, 4, FA, FB, true, false, true>(p, stream, err);  // (256x256 without the direct loads runs out of registers)
+    case 7: return launch_tile<2, 2, 4, 4, FA, FB, true, false, true>(p, stream, err);
     case 1: return launch_tile<2, 2, 4, 4, FA, FB>(p, stream, err);
     case 2: return launch_tile<2, 2, 8, 8, FA, FB>(p, stream, err);
     case 3: return launch_tile<2, 2, 8, 4, FA, FB>(p, stream, err);
@@ -536,8 +575,7 @@ int launch_fp8mm(const F8Params& p, uint32_t variant, const Machine&, hipStream_
     return -1;
   }
   int rc;
-  const bool wants_exact = (p.out_dtype == VKT_F32 || p.out_dtype == VKT_F16) && variant == 0;
-  if (p.k == 0 || p.k % 16 || p.lda % 16 || p.ldb % 16 || (p.a & 15) || (p.b & 15) || variant == 255 || wants_exact) {
+  if (p.k == 0 || p.k % 16 || p.lda % 16 || p.ldb % 16 || (p.a & 15) || (p.b & 15) || variant == 255) {
     if ((p.m + 3) / 4 > 65535) {
       *err = "fp8mm: too many rows for the unaligned path";
       return -1;
