@@ -104,6 +104,16 @@ __device__ __forceinline__ void store_out(const F8Params& p, uint64_t index, flo
   }
 }
 
+// Two float32 -> two bfloat16 in one word: v_cvt_pk_bf16_f32 (round to nearest even); NaN
+// becomes 0x7fc0 as c10 writes it.
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  using V2 = __bf16 __attribute__((ext_vector_type(2)));
+  const float qnan = bits_f32(0x7fc00000u);
+  a = a != a ? qnan : a;
+  b = b != b ? qnan : b;
+  return __builtin_bit_cast(uint32_t, V2{static_cast<__bf16>(a), static_cast<__bf16>(b)});
+}
+
 __device__ __forceinline__ float output_inv(const F8Params& p) {
   if (!(p.out_dtype == VKT_E4M3 || p.out_dtype == VKT_E5M2)) return 1.0f;
   return 1.0f / (p.scale_result ? ldg<float>(p.scale_result) : 1.0f);
@@ -163,13 +173,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, 
   // workgroup w runs on XCD w % 8.  Each XCD is given a contiguous band of tiles in
   // column-major order within a panel of `PANEL` tile rows, which keeps the operand rows
   // it touches resident in that XCD's L2.
-  const uint32_t total = tiles_m * tiles_n;
-  uint32_t w = blockIdx.x;
-  {
-    const uint32_t xcd = w & 7u, slot = w >> 3, per = (total + 7) / 8;
-    w = xcd * per + slot;
-    if (w >= total) return;  // whole workgroups only: before any barrier
-  }
+  // The grid is persistent: about as many workgroups as fit the machine at once, each
+  // walking through the slots of its XCD's band.  A tile's output stores then drain while
+  // the next tile's main loop runs, instead of all compute units writing (and then all
+  // starting cold) at the same moments.
+  const uint32_t total = tiles_m * tiles_n, per = (total + 7) / 8;
+  for (uint32_t slot = blockIdx.x >> 3; slot < per; slot += gridDim.x >> 3) {
+  const uint32_t w = (blockIdx.x & 7u) * per + slot;
+  if (w >= total) break;  // whole workgroups only, and between barriers
   constexpr uint32_t PANEL = 8;
   const uint32_t panel = w / (PANEL * tiles_n), in_panel = w % (PANEL * tiles_n);
   const uint32_t rows_here = tiles_m - panel * PANEL < PANEL ? tiles_m - panel * PANEL : PANEL;
@@ -302,17 +313,26 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, 
         const V4I hi = *reinterpret_cast<const V4I*>(tile + tile_offset(row, 4 * kk + 2 * h + 1));
         return V8I{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
       };
+      // LDS answers in the order asked: the first MFMA needs the first row fragment and the
+      // first column fragment, so those are asked for first; the column fragments of the
+      // second half of k are asked for once the first MFMAs are under way
+      // (row fragments are asked for two groups of MFMAs ahead: one group, 256 cycles, is
+      // less than an LDS read takes while the direct loads are writing into the same LDS)
+      auto row_frag = [&](int gi) { return frag32(ta, (wm * TM2 + gi % TM2) * 32 + l32, gi / TM2); };
+      V8I af = row_frag(0);
       V8I bf[2][TN2];
 #pragma unroll
-      for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-        for (int j = 0; j < TN2; ++j) bf[kk][j] = frag32(tb, (wn * TN2 + j) * 32 + l32, kk);
-      V8I af = frag32(ta, (wm * TM2) * 32 + l32, 0);
+      for (int j = 0; j < TN2; ++j) bf[0][j] = frag32(tb, (wn * TN2 + j) * 32 + l32, 0);
+      V8I next = row_frag(1 < 2 * TM2 ? 1 : 0);
 #pragma unroll
       for (int gi = 0; gi < 2 * TM2; ++gi) {
         const int kk = gi / TM2, i = gi % TM2;
-        V8I next = af;
-        if (gi + 1 < 2 * TM2) next = frag32(ta, (wm * TM2 + (gi + 1) % TM2) * 32 + l32, (gi + 1) / TM2);
+        V8I next2 = next;
+        if (gi + 2 < 2 * TM2) next2 = row_frag(gi + 2);
+        if (gi == 0) {
+#pragma unroll
+          for (int j = 0; j < TN2; ++j) bf[1][j] = frag32(tb, (wn * TN2 + j) * 32 + l32, 1);
+        }
         V8BF af_wide[WIDE ? 4 : 1];
         if constexpr (WIDE) {
 #pragma unroll
@@ -322,7 +342,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, 
 #pragma unroll
         for (int j = 0; j < TN2; ++j) {
           const int n = gi * TN2 + j;
-          const int lo_op = n * NSIDE / NMFMA, hi_op = (n + 1) * NSIDE / NMFMA;
+          // DIRECT: the step ends by waiting for its loads, so they are all issued at its
+          // start (FRONT per MFMA), not spread over it: the last one then has most of the
+          // step to land instead of none of it
+          constexpr int FRONT = 2;
+          const int lo_op = DIRECT ? (n * FRONT < NSIDE ? n * FRONT : NSIDE) : n * NSIDE / NMFMA;
+          const int hi_op = DIRECT ? ((n + 1) * FRONT < NSIDE ? (n + 1) * FRONT : NSIDE) : (n + 1) * NSIDE / NMFMA;
 #pragma unroll
           for (int op = lo_op; op < hi_op; ++op) {
             side(op, s, steady);
@@ -338,6 +363,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, 
         }
         __builtin_amdgcn_sched_barrier(0);
         af = next;
+        next = next2;
       }
     } else {
       V8I bf[TN];
@@ -441,43 +467,59 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, 
       sb[r] = p.rowwise ? ldg<float>(p.scale_b + 4ull * nn) : sb_all;
       bias[r] = p.bias ? load_any_f32(p.bias, nn, p.bias_dtype) : 0.0f;
     }
-    const bool fp8_out = p.out_dtype == VKT_E4M3 || p.out_dtype == VKT_E5M2;
-#pragma unroll 1
-    for (uint32_t it = 0; it < TM * 4; ++it) {
-      const uint32_t row = it * 4 + (lane >> 4), m = wm0 + row;
-      const V4F t = *reinterpret_cast<const V4F*>(reinterpret_cast<const uint8_t*>(ep) + row * EP_ROW +
-                                                   ((chunk ^ (row & 15u)) << 4));
-      if (m >= p.m || n >= p.n) continue;
-      const float sa = p.rowwise ? ldg<float>(p.scale_a + 4ull * m) : sa_all;
-      float v[4];
+    // The row loop, once per output type (chosen outside the loop, so that its body is
+    // straight-line and four rows' LDS reads and scale loads are in flight together).
+    // DT < 0: any type, element by element (unaligned outputs and the columns past n).
+    auto rows = [&](auto dt) {
+      constexpr int DT = decltype(dt)::value;
+      // (the register-staged 256x256 kernels have no registers to spare for the unrolling)
+      constexpr int UNROLL = (DIRECT || TM * TN < 64) ? 4 : 1;
+#pragma unroll UNROLL
+      for (uint32_t it = 0; it < TM * 4; ++it) {
+        const uint32_t row = it * 4 + (lane >> 4), m = wm0 + row;
+        const V4F t = *reinterpret_cast<const V4F*>(reinterpret_cast<const uint8_t*>(ep) + row * EP_ROW +
+                                                     ((chunk ^ (row & 15u)) << 4));
+        if (m >= p.m || n >= p.n) continue;
+        const float sa = p.rowwise ? ldg<float>(p.scale_a + 4ull * m) : sa_all;
+        float v[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        v[r] = t[r] * (sa * sb[r]);
-        if (p.bias) v[r] += bias[r];
-        if (fp8_out) v[r] *= inv;
-      }
-      const uint64_t index = uint64_t(m) * p.ldo + n;
-      if (vec_ok && n + 3 < p.n) {
-        if (p.out_dtype == VKT_F32) {
+        for (int r = 0; r < 4; ++r) {
+          v[r] = t[r] * (sa * sb[r]);
+          if (p.bias) v[r] += bias[r];
+          if (DT < 0 || DT == VKT_E4M3 || DT == VKT_E5M2) v[r] *= inv;  // (inv is 1 for the other types)
+        }
+        const uint64_t index = uint64_t(m) * p.ldo + n;
+        if constexpr (DT == VKT_F32) {
           stg<F4>(p.out + index * 4, F4{v[0], v[1], v[2], v[3]});
-        } else if (p.out_dtype == VKT_BF16) {
-          stg<U2>(p.out + index * 2, U2{uint32_t(f32_to_bf16(v[0])) | uint32_t(f32_to_bf16(v[1])) << 16,
-                                        uint32_t(f32_to_bf16(v[2])) | uint32_t(f32_to_bf16(v[3])) << 16});
-        } else if (p.out_dtype == VKT_F16) {
+        } else if constexpr (DT == VKT_BF16) {
+          stg<U2>(p.out + index * 2, U2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])});
+        } else if constexpr (DT == VKT_F16) {
           stg<U2>(p.out + index * 2, U2{uint32_t(f32_to_f16(v[0])) | uint32_t(f32_to_f16(v[1])) << 16,
                                         uint32_t(f32_to_f16(v[2])) | uint32_t(f32_to_f16(v[3])) << 16});
+        } else if constexpr (DT == VKT_E4M3 || DT == VKT_E5M2) {
+          stg<uint32_t>(p.out + index, f32_to_fp8(v[0], DT) | f32_to_fp8(v[1], DT) << 8 | f32_to_fp8(v[2], DT) << 16 |
+                                           f32_to_fp8(v[3], DT) << 24);
         } else {
-          const int f = int(p.out_dtype);
-          stg<uint32_t>(p.out + index, f32_to_fp8(v[0], f) | f32_to_fp8(v[1], f) << 8 | f32_to_fp8(v[2], f) << 16 |
-                                           f32_to_fp8(v[3], f) << 24);
-        }
-      } else {
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (n + r < p.n) store_out(p, index + r, v[r]);
+          for (int r = 0; r < 4; ++r)
+            if (n + r < p.n) store_out(p, index + r, v[r]);
+        }
       }
+    };
+    if (vec_ok && n + 3 < p.n) {
+      switch (p.out_dtype) {
+        case VKT_F32: rows(std::integral_constant<int, VKT_F32>{}); break;
+        case VKT_BF16: rows(std::integral_constant<int, VKT_BF16>{}); break;
+        case VKT_F16: rows(std::integral_constant<int, VKT_F16>{}); break;
+        case VKT_E4M3: rows(std::integral_constant<int, VKT_E4M3>{}); break;
+        default: rows(std::integral_constant<int, VKT_E5M2>{}); break;
+      }
+    } else {
+      rows(std::integral_constant<int, -1>{});
     }
   }
+  __syncthreads();  // the next tile's operands overwrite the LDS the epilogue has just read
+  }  // (tile loop)
 }
 
 // Any shape, stride or alignment: one thread per output.
@@ -493,7 +535,7 @@ __global__ __launch_bounds__(256) void fp8mm_generic(F8Params p) {
 }
 
 template <int WAVES_M, int WAVES_N, int TM, int TN, int FA, int FB, bool MF32 = false, bool DIRECT = false, bool WIDE = false>
-int launch_tile(const F8Params& p, hipStream_t stream, std::string* err) {
+int launch_tile(const F8Params& p, int compute_units, hipStream_t stream, std::string* err) {
   constexpr int BM = WAVES_M * TM * 16, BN = WAVES_N * TN * 16;
   constexpr uint32_t operand_bytes = 2 * (BM + BN) * BK, epilogue_bytes = WAVES_M * WAVES_N * TM * 16 * 256;
   constexpr uint32_t lds_bytes = operand_bytes > epilogue_bytes ? operand_bytes : epilogue_bytes;
@@ -512,17 +554,20 @@ int launch_tile(const F8Params& p, hipStream_t stream, std::string* err) {
   }
   const uint32_t tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
   const uint64_t total = uint64_t(tiles_m) * tiles_n;
-  const uint64_t grid = (total + 7) / 8 * 8;
-  if (grid >= (1ull << 31)) {
+  if (total >= (1ull << 31)) {
     *err = "fp8mm: too many tiles";
     return -1;
   }
+  // as many workgroups as are resident at once (LDS decides), in multiples of 8 (one per XCD)
+  const uint32_t per_cu = lds_bytes > 80 * 1024 ? 1 : (lds_bytes > 53 * 1024 ? 2 : 3);
+  const uint64_t resident = (uint64_t(compute_units) * per_cu + 7) / 8 * 8;
+  const uint64_t grid = (total + 7) / 8 * 8 < resident ? (total + 7) / 8 * 8 : resident;
   hipLaunchKernelGGL(kernel, dim3(uint32_t(grid)), dim3(WAVES_M * WAVES_N * 64), lds_bytes, stream, p, tiles_m, tiles_n);
   return 0;
 }
 
 template <int FA, int FB>
-int launch_formats(const F8Params& p, uint32_t variant, hipStream_t stream, std::string* err) {
+int launch_formats(const F8Params& p, uint32_t variant, int compute_units, hipStream_t stream, std::string* err) {
   // variant 0: planned.  Explicit variants run the MFMA kernel whatever the output dtype
   // (tests, tuning): 1: 128x128 tiles (4 waves of 64x64, 16x16x128 MFMA); 2: 256x256 (4 waves of
   // 128x128, 16x16x128); 3: 256x128; 4: 256x256 with the 32x32x64 MFMA (measured ~10 % faster
@@ -534,16 +579,16 @@ int launch_formats(const F8Params& p, uint32_t variant, hipStream_t stream, std:
   if (variant == 0) variant = (p.out_dtype == VKT_F32 || p.out_dtype == VKT_F16) ? (big ? 6 : 7) : (big ? 5 : 1);
   switch (variant) {
     case 6:
-      if (p.k % BK == 0) return launch_tile<2, 2, 8, 8, FA, FB, true, true, true>(p, stream, err);
-      return launch_tile<2, 2, 8, 4, FA, FB, true, false, true>(p, stream, err);  // (256x256 without the direct loads runs out of registers)
-    case 7: return launch_tile<2, 2, 4, 4, FA, FB, true, false, true>(p, stream, err);
-    case 1: return launch_tile<2, 2, 4, 4, FA, FB>(p, stream, err);
-    case 2: return launch_tile<2, 2, 8, 8, FA, FB>(p, stream, err);
-    case 3: return launch_tile<2, 2, 8, 4, FA, FB>(p, stream, err);
-    case 4: return launch_tile<2, 2, 8, 8, FA, FB, true>(p, stream, err);
+      if (p.k % BK == 0) return launch_tile<2, 2, 8, 8, FA, FB, true, true, true>(p, compute_units, stream, err);
+      return launch_tile<2, 2, 8, 4, FA, FB, true, false, true>(p, compute_units, stream, err);  // (256x256 without the direct loads runs out of registers)
+    case 7: return launch_tile<2, 2, 4, 4, FA, FB, true, false, true>(p, compute_units, stream, err);
+    case 1: return launch_tile<2, 2, 4, 4, FA, FB>(p, compute_units, stream, err);
+    case 2: return launch_tile<2, 2, 8, 8, FA, FB>(p, compute_units, stream, err);
+    case 3: return launch_tile<2, 2, 8, 4, FA, FB>(p, compute_units, stream, err);
+    case 4: return launch_tile<2, 2, 8, 8, FA, FB, true>(p, compute_units, stream, err);
     case 5:
-      if (p.k % BK == 0) return launch_tile<2, 2, 8, 8, FA, FB, true, true>(p, stream, err);
-      return launch_tile<2, 2, 8, 8, FA, FB, true>(p, stream, err);
+      if (p.k % BK == 0) return launch_tile<2, 2, 8, 8, FA, FB, true, true>(p, compute_units, stream, err);
+      return launch_tile<2, 2, 8, 8, FA, FB, true>(p, compute_units, stream, err);
   }
   *err = "fp8mm: unknown variant " + std::to_string(variant);
   return -1;
@@ -551,7 +596,7 @@ int launch_formats(const F8Params& p, uint32_t variant, hipStream_t stream, std:
 
 }  // namespace
 
-int launch_fp8mm(const F8Params& p, uint32_t variant, const Machine&, hipStream_t stream, std::string* err) {
+int launch_fp8mm(const F8Params& p, uint32_t variant, const Machine& mc, hipStream_t stream, std::string* err) {
   if (p.m == 0 || p.n == 0) return 0;
   auto fp8 = [](uint32_t f) { return f == VKT_E4M3 || f == VKT_E5M2; };
   if (!fp8(p.fmt_a) || !fp8(p.fmt_b)) {
@@ -583,13 +628,13 @@ int launch_fp8mm(const F8Params& p, uint32_t variant, const Machine&, hipStream_
     hipLaunchKernelGGL(fp8mm_generic, dim3((p.n + 63) / 64, (p.m + 3) / 4), dim3(256), 0, stream, p);
     rc = 0;
   } else if (p.fmt_a == VKT_E4M3 && p.fmt_b == VKT_E4M3) {
-    rc = launch_formats<0, 0>(p, variant, stream, err);
+    rc = launch_formats<0, 0>(p, variant, mc.compute_units, stream, err);
   } else if (p.fmt_a == VKT_E5M2 && p.fmt_b == VKT_E4M3) {
-    rc = launch_formats<1, 0>(p, variant, stream, err);
+    rc = launch_formats<1, 0>(p, variant, mc.compute_units, stream, err);
   } else if (p.fmt_a == VKT_E4M3 && p.fmt_b == VKT_E5M2) {
-    rc = launch_formats<0, 1>(p, variant, stream, err);
+    rc = launch_formats<0, 1>(p, variant, mc.compute_units, stream, err);
   } else {
-    rc = launch_formats<1, 1>(p, variant, stream, err);
+    rc = launch_formats<1, 1>(p, variant, mc.compute_units, stream, err);
   }
   if (rc == 0 && hipGetLastError() != hipSuccess) {
     *err = "fp8mm: kernel launch failed";
