@@ -146,12 +146,16 @@ def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030):
                 reference_layout_bytes=int(packed.numel()) * 4 + 4 * m * k + 4 * m * n)
 
 
-def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040):
-    """_scaled_mm e4m3fn x e4m3fn -> bf16; A row-major, B column-major."""
+def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False):
+    """_scaled_mm e4m3fn x e4m3fn -> bf16; A row-major, B column-major.  zero_operands: the same
+    launch on all-zero matrices: the matrix cores' sustained rate depends on how many operand
+    bits toggle (the part is power limited), and this is the data-independent end of that range."""
     import torch
     g = torch.Generator().manual_seed(seed)
     a = torch.randn(m, k, generator=g).clamp(-448, 448).to(torch.float8_e4m3fn)
     bt = torch.randn(n, k, generator=g).clamp(-448, 448).to(torch.float8_e4m3fn)
+    if zero_operands:
+        a, bt = torch.zeros_like(a), torch.zeros_like(bt)
     if rowwise:
         sa = torch.empty(m).uniform_(0.5, 2, generator=g)
         sb = torch.empty(n).uniform_(0.5, 2, generator=g)
@@ -166,7 +170,8 @@ def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040):
     wall, ev = time_steps(abi, fns, steps, warmup)
     return dict(kind="mfma", work=2 * m * n * k, wall_ms=wall, event_ms=ev, bytes=m * k + n * k + 2 * m * n,
                 inputs=(a, bt, sa, sb), copies=1,
-                name=f"_scaled_mm e4m3fn {'rowwise' if rowwise else 'per-tensor'} M={m} K={k} N={n} -> bf16")
+                name=f"_scaled_mm e4m3fn {'rowwise' if rowwise else 'per-tensor'} M={m} K={k} N={n} -> bf16"
+                     + (" (all-zero operands)" if zero_operands else ""))
 
 
 def wl_copy(abi, nbytes, steps, warmup):
@@ -196,6 +201,10 @@ WORKLOADS = {
     "c4_fp8_8192": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 10, 5), max(w // 4, 3)),
     "c5_fp8_rowwise_70b": lambda abi, s, w: wl_fp8(abi, 4096, 8192, 28672, True, max(s // 10, 5), max(w // 4, 3),
                                                    seed=1050),
+    # config 4's launch on all-zero operands (not a BASELINE configuration: it shows how much of the
+    # distance to the published peak is the data's, not the kernel's)
+    "c4_fp8_8192_zero_operands": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 10, 5),
+                                                          max(w // 4, 3), zero_operands=True),
 }
 # not a BASELINE configuration: selected by name only (counter calibration)
 CALIBRATION = {"copy_256mib": lambda abi, s, w: wl_copy(abi, 256 << 20, max(s // 4, 5), w)}
