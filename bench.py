@@ -174,6 +174,33 @@ def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False)
                      + (" (all-zero operands)" if zero_operands else ""))
 
 
+def wl_cast(abi, n, steps, warmup, seed=1070):
+    """bfloat16 -> e4m3fn elementwise cast of n values (the float8 step in front of _scaled_mm)."""
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(1 << 20, generator=g).bfloat16().repeat(n >> 20)
+    dx = abi.Buffer.from_numpy(x.view(torch.int16).numpy())
+    out = abi.Buffer(n)
+    p = abi.CastParams(src=dx.address, dst=out.address, n=n, src_dtype=abi.BF16, dst_dtype=abi.E4M3)
+    wall, ev = time_steps(abi, [Launch(abi, "cast_fp8", [], p)], steps, warmup)
+    return dict(kind="hbm", work=3 * n, wall_ms=wall, event_ms=ev, flops=0, inputs=None, copies=1,
+                name=f"cast bf16 -> e4m3fn, {n >> 20} Mi values")
+
+
+def wl_quant(abi, m, k, steps, warmup, seed=1080):
+    """The rowwise float8 producer: bfloat16 [m,k] -> e4m3fn [m,k] + float32 scales [m]."""
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    dx = abi.Buffer.from_numpy(x.view(torch.int16).numpy())
+    out, scales = abi.Buffer(m * k), abi.Buffer(m * 4)
+    p = abi.F8QuantParams(src=dx.address, dst=out.address, scale=scales.address, m=m, k=k, lds=k, ldd=k,
+                          src_dtype=abi.BF16, dst_fmt=abi.E4M3)
+    wall, ev = time_steps(abi, [Launch(abi, "fp8_quant", [1], p)], steps, warmup)
+    return dict(kind="hbm", work=3 * m * k + 4 * m, wall_ms=wall, event_ms=ev, flops=0, inputs=None, copies=1,
+                name=f"fp8_quant rowwise bf16 -> e4m3fn M={m} K={k}")
+
+
 def wl_copy(abi, nbytes, steps, warmup):
     """A plain device-to-device copy of known size (calibrates the HBM traffic counters)."""
     src, dst = abi.Buffer(nbytes), abi.Buffer(nbytes)
@@ -201,6 +228,10 @@ WORKLOADS = {
     "c4_fp8_8192": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 10, 5), max(w // 4, 3)),
     "c5_fp8_rowwise_70b": lambda abi, s, w: wl_fp8(abi, 4096, 8192, 28672, True, max(s // 10, 5), max(w // 4, 3),
                                                    seed=1050),
+    # the float8 steps in front of _scaled_mm (not BASELINE configurations: the next rows of the path),
+    # at the size of config 4's A operand and beyond the L2 / MALL capacity
+    "f8_cast_bf16_e4m3_256mi": lambda abi, s, w: wl_cast(abi, 1 << 28, max(s // 10, 5), max(w // 4, 3)),
+    "f8_quant_rowwise_bf16_16384x16384": lambda abi, s, w: wl_quant(abi, 16384, 16384, max(s // 10, 5), max(w // 4, 3)),
     # config 4's launch on all-zero operands (not a BASELINE configuration: it shows how much of the
     # distance to the published peak is the data's, not the kernel's)
     "c4_fp8_8192_zero_operands": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 10, 5),

@@ -144,6 +144,28 @@ typedef struct Q4CParams {
   uint32_t m, n, k, bs, has_bias, pad;
 } Q4CParams;
 
+/* "cast_fp8", spec {}: dst[i] = convert(src[i]), i < n, where one side is VKT_E4M3 / VKT_E5M2
+ * and the other VKT_F32 / VKT_F16 / VKT_BF16 (or the other float8 format): through float32,
+ * bit for bit as the CPU converts (what the reference's copy between a float8 tensor and
+ * a float tensor does with lookup tables, backend.cpp:534-586).  32 bytes. */
+typedef struct CastParams {
+  uint64_t src, dst, n;
+  uint32_t src_dtype, dst_dtype;
+} CastParams;
+
+/* "fp8_quant", spec {ROWWISE}: the float8 producer in front of _scaled_mm.  src [m,k]
+ * (float32 / float16 / bfloat16, rows lds elements apart) -> dst [m,k] float8 (rows ldd bytes
+ * apart).  ROWWISE 1: scale[r] = max(max_k |src[r,k]|, 1e-12) / fmax is written (float32 [m],
+ * what _scaled_mm takes as a rowwise scale); ROWWISE 0: scale[0] is read (one scale for the
+ * tensor).  dst = convert(clamp(src * (fmax / (scale * fmax)), -fmax, fmax)), every step one
+ * float32 operation; fmax = 448 (e4m3fn) or 57344 (e5m2).  No counterpart in the reference
+ * (its float8 tensors come from casts alone).  48 bytes. */
+typedef struct F8QuantParams {
+  uint64_t src, dst, scale;
+  uint32_t m, k, lds, ldd;
+  uint32_t src_dtype, dst_fmt;
+} F8QuantParams;
+
 /* "fp8mm", spec {}: out = cast((f32(A)*sa) @ (f32(B)*sb) + bias) [* 1/scale_result]
  * (quant.cpp:279-300 fused into one kernel).  A: fp8 [m,k] row-major (lda bytes);
  * B: fp8, column-major, i.e. [n,k] rows ldb bytes apart.  104 bytes. */

@@ -180,3 +180,23 @@ def scaled_mm(a, fmt_a, bt, fmt_b, sa, sb, rowwise, bias=None, bias_dtype=F32, s
     lib().orc_scaled_mm(_p(a), fmt_a, _p(bt), fmt_b, _p(sa), _p(sb), int(bool(rowwise)), _p(bias), bias_dtype, _p(sr),
                         _p(out), out_dtype, _p(mag), I64(M), I64(N), I64(K))
     return (out, mag) if want_mag else out
+
+
+def cast(a, src_dtype, dst_dtype):
+    """Elementwise conversion where one side is float8 (through float32, as c10)."""
+    a = _c(a, _NP[src_dtype])
+    out = np.empty(a.shape, _NP[dst_dtype])
+    lib().orc_cast(_p(a), src_dtype, _p(out), dst_dtype, I64(a.size))
+    return out
+
+
+def fp8_quant(x, dtype, fmt, scale=None):
+    """The float8 producer: rowwise scales computed (scale is None) or one given scale.
+    Returns (codes uint8 [M,K], scales float32 [M] or [1])."""
+    x = _c(x, _NP[dtype])
+    m, k = x.shape
+    q = np.empty((m, k), np.uint8)
+    rowwise = scale is None
+    scales = np.empty(m, np.float32) if rowwise else np.asarray([scale], np.float32)
+    lib().orc_fp8_quant_rows(_p(x), dtype, I64(m), I64(k), I64(k), fmt, int(rowwise), _p(q), I64(k), _p(scales))
+    return q, scales

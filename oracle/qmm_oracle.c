@@ -24,6 +24,13 @@
  *   orc_q4_matmul       pinned: torch CPU _dyn_quant_matmul_4bit (bit-exact), golden
  *   orc_scaled_mm       pinned: torch CPU _scaled_mm (per-tensor), f64 closed form,
  *                               identity / power-of-two cases that are exact
+ *   orc_cast            pinned: torch CPU Tensor.to() between float32 / float16 / bfloat16 and
+ *                               both float8 formats (the reference's own vectors,
+ *                               tests/python/test_fallback_ops.py:469-485, plus all 256 codes)
+ *   orc_fp8_quant_rows  pinned: the same steps composed from torch CPU operators (amax, clamp,
+ *                               true_divide, mul, clamp, to(float8)), rows whose maximum is
+ *                               fmax exactly (the scale is 1: a plain cast), power-of-two
+ *                               rescaling, zero rows
  */
 #include <math.h>
 #include <stdint.h>
@@ -341,4 +348,44 @@ void orc_scaled_mm(const uint8_t* a, int fmt_a, const uint8_t* bt, int fmt_b, co
     }
   }
   free(arow);
+}
+
+/* ------------------------------------------------------------------ float8 casts and producer */
+
+/* Elementwise conversion where one side is float8: through float32, as the reference's copy
+ * between a float8 tensor and a float tensor (crates/pyvk/csrc/backend.cpp:534-586, tables
+ * built from c10's conversions) and as c10 itself converts. */
+void orc_cast(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t n) {
+  for (int64_t i = 0; i < n; i++) store_from_f32(dst, i, dst_dtype, load_as_f32(src, i, src_dtype));
+}
+
+/* The float8 producer in front of _scaled_mm (no counterpart in the reference; SURVEY lists it
+ * as the step a float8 pipeline needs on the device).  Per row, or with one given scale:
+ *   a = max(max_k |x|, 1e-12) (NaN elements do not count); scale = a / fmax;
+ *   q = cast(clamp(x * (fmax / a), -fmax, fmax)); every step one float32 operation.
+ * rowwise 0: scales[0] is an input and a = scales[0] * fmax. */
+void orc_fp8_quant_rows(const void* x, int dtype, int64_t M, int64_t K, int64_t ldx, int fmt, int rowwise, uint8_t* q,
+                        int64_t ldq, float* scales) {
+  const float fmax = fmt == ORC_E4M3 ? 448.0f : 57344.0f;
+  for (int64_t m = 0; m < M; m++) {
+    float a;
+    if (rowwise) {
+      float amax = 0.0f;
+      for (int64_t k = 0; k < K; k++) {
+        const float v = fabsf(load_as_f32(x, m * ldx + k, dtype));
+        if (v > amax) amax = v; /* (a NaN compares false) */
+      }
+      a = amax > 1e-12f ? amax : 1e-12f;
+      scales[m] = a / fmax;
+    } else {
+      a = scales[0] * fmax;
+    }
+    const volatile float inv = fmax / a;
+    for (int64_t k = 0; k < K; k++) {
+      volatile float y = load_as_f32(x, m * ldx + k, dtype) * inv;
+      if (y < -fmax) y = -fmax;
+      if (fmax < y) y = fmax;
+      q[m * ldq + k] = orc_f32_to_fp8(y, fmt);
+    }
+  }
 }

@@ -115,3 +115,41 @@ def scaled_mm(a, fmt_a, bt, fmt_b, sa, sb, rowwise, bias=None, bias_dtype=oracle
     if m and n:
         abi.dispatch("fp8mm", [variant], p)
     return do.to_numpy(_NP[out_dtype], (m, n))
+
+
+def cast(a, src_dtype, dst_dtype, skew=0):
+    """Elementwise float8 cast ("cast_fp8").  skew: elements by which both device addresses are
+    moved off their 16-element alignment (the element-by-element form of the kernel)."""
+    a = np.ascontiguousarray(a, dtype=_NP[src_dtype]).reshape(-1)
+    n = a.size
+    si, di = a.itemsize, np.dtype(_NP[dst_dtype]).itemsize
+    dsrc = abi.Buffer(max((n + skew) * si, 1))
+    ddst = abi.Buffer(max((n + skew) * di, 1))
+    if n:
+        abi.check(abi.lib().vkt_copy_to_device(dsrc.address + skew * si, a.ctypes.data, n * si))
+        p = abi.CastParams(src=dsrc.address + skew * si, dst=ddst.address + skew * di, n=n, src_dtype=src_dtype,
+                           dst_dtype=dst_dtype)
+        abi.dispatch("cast_fp8", [], p)
+    return ddst.to_numpy(_NP[dst_dtype], (n + skew,))[skew:]
+
+
+def fp8_quant(x, dtype, fmt, scale=None, pad=0):
+    """The float8 producer ("fp8_quant"): rowwise scales computed, or one given scale.
+    pad: extra elements between rows on both sides (row strides larger than k)."""
+    x = np.ascontiguousarray(x, dtype=_NP[dtype])
+    m, k = x.shape
+    lds = ldd = k + pad
+    xs = np.zeros((m, lds), _NP[dtype])
+    xs[:, :k] = x
+    dx = abi.Buffer.from_numpy(xs)
+    dq = abi.Buffer(max(m * ldd, 1))
+    abi.check(abi.lib().vkt_fill(dq.address, 0xAB, max(m * ldd, 1)))
+    rowwise = scale is None
+    ds = abi.Buffer(max(m * 4, 4)) if rowwise else abi.Buffer.from_numpy(np.asarray([scale], np.float32))
+    p = abi.F8QuantParams(src=dx.address, dst=dq.address, scale=ds.address, m=m, k=k, lds=lds, ldd=ldd, src_dtype=dtype,
+                          dst_fmt=fmt)
+    if m and k:
+        abi.dispatch("fp8_quant", [int(rowwise)], p)
+    q = dq.to_numpy(np.uint8, (m, ldd))
+    assert (q[:, k:] == 0xAB).all(), "the producer wrote between rows"
+    return q[:, :k], ds.to_numpy(np.float32, (m if rowwise else 1,))

@@ -190,3 +190,55 @@ def test_fallback_is_counted(tv):
     before = sum(tv.fallback_counts().values())
     y = torch.ones(3).to("vk") + 1
     assert torch.equal(y.cpu(), torch.full((3,), 2.0)) and sum(tv.fallback_counts().values()) > before
+
+
+@pytest.mark.parametrize("f8", FLOAT8, ids=str)
+@pytest.mark.parametrize("src", [torch.float32, torch.float16, torch.bfloat16], ids=str)
+def test_float8_casts(tv, f8, src):
+    """The reference's float8 cast test for the types _scaled_mm takes
+    (tests/python/test_fallback_ops.py:469-485): every float8 code to the wider type, and values
+    that round, saturate, overflow and are NaN, inf or -0 to float8, bit for bit as the CPU's,
+    converted on the device (cast_fp8 counts its dispatches)."""
+    codes = torch.arange(256, dtype=torch.int32).to(torch.uint8).view(f8)
+    x = torch.cat([torch.randn(300, generator=gen(0)) * 3, torch.randn(300, generator=gen(1)) * 300,
+                   torch.tensor([0.0, -0.0, float("inf"), -float("inf"), float("nan"), 448.0, 464.0, 57344.0, 61440.0,
+                                 1e-9, -1e-9, 2.0 ** -9, 2.0 ** -10, 2.0 ** -17, 1e30])]).to(src)
+    dx = x.to("vk")
+    dcodes = codes.to("vk")
+    before = tv.dispatch_count()
+    with on_gpu(tv):
+        got = dx.to(f8)
+        back = dcodes.to(src)
+    assert tv.dispatch_count() - before == 2  # both conversions ran as kernels
+    assert torch.equal(got.cpu().view(torch.uint8), x.to(f8).view(torch.uint8))
+    torch.testing.assert_close(back.cpu(), codes.to(src), equal_nan=True, atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("f8", FLOAT8, ids=str)
+@pytest.mark.parametrize("src", [torch.float32, torch.bfloat16], ids=str)
+def test_fp8_quant_rowwise_into_scaled_mm(tv, f8, src):
+    """torch.ops.vk.fp8_quant_rowwise (the producer in front of _scaled_mm): bit for bit the same
+    steps composed from PyTorch's CPU operators, and its outputs go straight into _scaled_mm."""
+    fmax = 448.0 if f8 == torch.float8_e4m3fn else 57344.0
+    a = (torch.randn(48, 256, generator=gen(5)) * 0.7).to(src)
+    w = (torch.randn(80, 256, generator=gen(6)) * 0.04).to(src)
+    with on_gpu(tv):
+        qa, sa = torch.ops.vk.fp8_quant_rowwise(a.to("vk"), f8)
+        qw, sw = torch.ops.vk.fp8_quant_rowwise(w.to("vk"), torch.float8_e4m3fn)
+        out = torch._scaled_mm(qa, qw.t(), sa, sw.t(), out_dtype=torch.float32)
+
+    def on_cpu(x, dt, top):
+        amax = torch.clamp(x.float().abs().amax(dim=1, keepdim=True), min=1e-12)
+        scale = torch.true_divide(amax, torch.tensor(top))
+        y = torch.clamp(x.float() * torch.true_divide(torch.tensor(top), amax), -top, top)
+        return y.to(dt), scale
+
+    ca, csa = on_cpu(a, f8, fmax)
+    cw, csw = on_cpu(w, torch.float8_e4m3fn, 448.0)
+    assert torch.equal(qa.cpu().view(torch.uint8), ca.view(torch.uint8)) and torch.equal(sa.cpu(), csa)
+    assert torch.equal(qw.cpu().view(torch.uint8), cw.view(torch.uint8)) and torch.equal(sw.cpu(), csw)
+    want = (ca.float() * csa).double() @ (cw.float() * csw).double().t()
+    mag = (ca.float() * csa).abs().double() @ (cw.float() * csw).abs().double().t()
+    assert ((out.cpu().double() - want).abs() <= 2.0**-23 * want.abs() + 2.0**-20 * mag).all()
+    with pytest.raises(RuntimeError, match="float8_e4m3fn or float8_e5m2"):
+        torch.ops.vk.fp8_quant_rowwise(a.to("vk"), torch.bfloat16)

@@ -28,6 +28,7 @@ def test_parameter_block_sizes():
     # quant.cpp:37,43 static_asserts; at most 128 bytes of push constants (vk.h:386)
     assert ctypes.sizeof(abi.Q8Params) == 56
     assert ctypes.sizeof(abi.Q4Params) == 64
+    assert ctypes.sizeof(abi.CastParams) == 32 and ctypes.sizeof(abi.F8QuantParams) == 48
     for t in (abi.Q4PackParams, abi.Q4CParams, abi.F8Params):
         assert ctypes.sizeof(t) <= 128
     assert ctypes.sizeof(abi.VktAlloc) == 32

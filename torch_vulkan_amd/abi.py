@@ -61,7 +61,17 @@ class F8Params(ctypes.Structure):
                 ("fmt_a", u32), ("fmt_b", u32), ("out_dtype", u32), ("bias_dtype", u32), ("rowwise", u32), ("pad", u32)]
 
 
+class CastParams(ctypes.Structure):
+    _fields_ = [("src", u64), ("dst", u64), ("n", u64), ("src_dtype", u32), ("dst_dtype", u32)]
+
+
+class F8QuantParams(ctypes.Structure):
+    _fields_ = [("src", u64), ("dst", u64), ("scale", u64), ("m", u32), ("k", u32), ("lds", u32), ("ldd", u32),
+                ("src_dtype", u32), ("dst_fmt", u32)]
+
+
 assert ctypes.sizeof(Q8Params) == 56 and ctypes.sizeof(Q4Params) == 64 and ctypes.sizeof(F8Params) == 104
+assert ctypes.sizeof(CastParams) == 32 and ctypes.sizeof(F8QuantParams) == 48
 
 # every symbol include/vkt.h declares
 SYMBOLS = ["vkt_last_error", "vkt_alloc", "vkt_free", "vkt_synchronize", "vkt_empty_cache", "vkt_memory_stats",

@@ -207,6 +207,16 @@ int dispatch_named(Runtime& rt, const char* name, const uint32_t* spec, size_t n
     if (!read_push(push, npush, &p, name, err)) return -1;
     return launch_qmm4c(p, dt, spec_at(0), spec_at(1), spec_at(2), rt.machine, rt.stream, err);
   }
+  if (!std::strcmp(name, "cast_fp8")) {
+    CastParams p;
+    if (!read_push(push, npush, &p, name, err)) return -1;
+    return launch_cast_fp8(p, rt.machine, rt.stream, err);
+  }
+  if (!std::strcmp(name, "fp8_quant")) {
+    F8QuantParams p;
+    if (!read_push(push, npush, &p, name, err)) return -1;
+    return launch_fp8_quant(p, spec_at(0), rt.machine, rt.stream, err);
+  }
   if (!std::strcmp(name, "fp8mm")) {
     F8Params p;
     if (!read_push(push, npush, &p, name, err)) return -1;
@@ -346,7 +356,10 @@ uint32_t vkt_kernel_subgroup_size(const char* name) {
   if (!name) return 0;
   std::string err;
   if (!runtime(&err)) return 0;
-  return (!std::strncmp(name, "qmm", 3) || !std::strcmp(name, "fp8mm")) ? 64u : 0u;
+  return (!std::strncmp(name, "qmm", 3) || !std::strcmp(name, "fp8mm") || !std::strcmp(name, "cast_fp8") ||
+          !std::strcmp(name, "fp8_quant"))
+             ? 64u
+             : 0u;
 }
 
 int vkt_copy_to_device(uint64_t dst, const void* src, uint64_t nbytes) {

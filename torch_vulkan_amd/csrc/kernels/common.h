@@ -132,6 +132,58 @@ __device__ __forceinline__ void widen16_i8(const U4& v, float (&w)[16]) {
   }
 }
 
+// ---- float8 element conversions (exact decode; encode as c10 converts: round to nearest even,
+// e4m3fn overflow -> NaN, e5m2 overflow -> inf) ----
+__device__ __forceinline__ float fp8_to_f32(uint32_t c, int fmt) {
+  const uint32_t sign = (c & 0x80u) << 24;
+  if (fmt == VKT_E4M3) {
+    const uint32_t e = (c >> 3) & 15u, m = c & 7u;
+    if (e == 15 && m == 7) return bits_f32(sign | 0x7ff00000u);
+    if (e == 0) return bits_f32(sign | f32_bits(float(m) * 0.001953125f));  // m * 2^-9
+    return bits_f32(sign | ((e + 120u) << 23) | (m << 20));
+  }
+  const uint32_t e = (c >> 2) & 31u, m = c & 3u;
+  if (e == 31) return bits_f32(sign | 0x7f800000u | (m << 21));
+  if (e == 0) return bits_f32(sign | f32_bits(float(m) * 1.52587890625e-05f));  // m * 2^-16
+  return bits_f32(sign | ((e + 112u) << 23) | (m << 21));
+}
+
+__device__ __forceinline__ uint32_t f32_to_fp8(float f, int fmt) {
+  const uint32_t u = f32_bits(f), sign = (u >> 24) & 0x80u, mag = u & 0x7fffffffu;
+  const int mbits = fmt == VKT_E4M3 ? 3 : 2, bias = fmt == VKT_E4M3 ? 7 : 15;
+  if (mag > 0x7f800000u) return sign | 0x7fu;
+  if (fmt == VKT_E4M3) {
+    if (mag >= 0x43f00000u) return sign | 0x7fu;  // >= 480: NaN (no saturation)
+  } else {
+    if (mag >= 0x47800000u) return sign | 0x7cu;  // >= 65536: inf
+  }
+  if ((mag >> 23) == 0) return sign;  // zero and float32 denormals
+  const int e = int(mag >> 23) - 127, emin = 1 - bias;
+  const uint32_t m = (mag & 0x7fffffu) | 0x800000u;
+  const int shift = 23 - mbits + (e < emin ? emin - e : 0);
+  if (shift > 25) return sign;
+  uint32_t keep = m >> shift;
+  const uint32_t rem = m & ((1u << shift) - 1u), half = 1u << (shift - 1);
+  if (rem > half || (rem == half && (keep & 1u))) ++keep;
+  const uint32_t out = e < emin ? keep : ((uint32_t(e + bias) << mbits) + (keep - (1u << mbits)));
+  return sign | out;
+}
+
+// Two float32 -> two float8 codes (low 16 bits) with the hardware conversion.  On gfx950
+// v_cvt_pk_fp8_f32 / v_cvt_pk_bf8_f32 agree with f32_to_fp8 above on every one of the 2^32
+// float32 bit patterns that is not a NaN (checked exhaustively on the device: overflow to
+// NaN / inf, subnormals and ties included); a NaN comes out with another payload, so NaNs are
+// given the code c10 writes, sign | 0x7f.
+template <int FMT>
+__device__ __forceinline__ uint32_t pack2_fp8(float a, float b) {
+  const uint32_t na = ((f32_bits(a) >> 24) & 0x80u) | 0x7fu, nb = ((f32_bits(b) >> 24) & 0x80u) | 0x7fu;
+  uint32_t r;
+  if constexpr (FMT == VKT_E4M3) r = uint32_t(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false));
+  else r = uint32_t(__builtin_amdgcn_cvt_pk_bf8_f32(a, b, 0, false));
+  const uint32_t ca = a != a ? na : (r & 0xffu), cb = b != b ? nb : ((r >> 8) & 0xffu);
+  return ca | cb << 8;
+}
+
 // ---- wave64 reductions through DPP (no LDS traffic) ----
 template <int CTRL, int ROW_MASK = 0xf>
 __device__ __forceinline__ float dpp_f32(float v) {

@@ -44,43 +44,6 @@ using V4F = float __attribute__((ext_vector_type(4)));
 
 constexpr int BK = 128;  // bytes (= fp8 values) of K per step, one MFMA deep
 
-// ---- element conversions (exact decode; encode as c10 converts: round to nearest even,
-// e4m3fn overflow -> NaN, e5m2 overflow -> inf) ----
-__device__ __forceinline__ float fp8_to_f32(uint32_t c, int fmt) {
-  const uint32_t sign = (c & 0x80u) << 24;
-  if (fmt == VKT_E4M3) {
-    const uint32_t e = (c >> 3) & 15u, m = c & 7u;
-    if (e == 15 && m == 7) return bits_f32(sign | 0x7ff00000u);
-    if (e == 0) return bits_f32(sign | f32_bits(float(m) * 0.001953125f));  // m * 2^-9
-    return bits_f32(sign | ((e + 120u) << 23) | (m << 20));
-  }
-  const uint32_t e = (c >> 2) & 31u, m = c & 3u;
-  if (e == 31) return bits_f32(sign | 0x7f800000u | (m << 21));
-  if (e == 0) return bits_f32(sign | f32_bits(float(m) * 1.52587890625e-05f));  // m * 2^-16
-  return bits_f32(sign | ((e + 112u) << 23) | (m << 21));
-}
-
-__device__ __forceinline__ uint32_t f32_to_fp8(float f, int fmt) {
-  const uint32_t u = f32_bits(f), sign = (u >> 24) & 0x80u, mag = u & 0x7fffffffu;
-  const int mbits = fmt == VKT_E4M3 ? 3 : 2, bias = fmt == VKT_E4M3 ? 7 : 15;
-  if (mag > 0x7f800000u) return sign | 0x7fu;
-  if (fmt == VKT_E4M3) {
-    if (mag >= 0x43f00000u) return sign | 0x7fu;  // >= 480: NaN (no saturation)
-  } else {
-    if (mag >= 0x47800000u) return sign | 0x7cu;  // >= 65536: inf
-  }
-  if ((mag >> 23) == 0) return sign;  // zero and float32 denormals
-  const int e = int(mag >> 23) - 127, emin = 1 - bias;
-  const uint32_t m = (mag & 0x7fffffu) | 0x800000u;
-  const int shift = 23 - mbits + (e < emin ? emin - e : 0);
-  if (shift > 25) return sign;
-  uint32_t keep = m >> shift;
-  const uint32_t rem = m & ((1u << shift) - 1u), half = 1u << (shift - 1);
-  if (rem > half || (rem == half && (keep & 1u))) ++keep;
-  const uint32_t out = e < emin ? keep : ((uint32_t(e + bias) << mbits) + (keep - (1u << mbits)));
-  return sign | out;
-}
-
 __device__ __forceinline__ float load_any_f32(uint64_t base, uint64_t i, uint32_t dtype) {
   if (dtype == VKT_F32) return ldg<float>(base + 4 * i);
   if (dtype == VKT_F16) return f16_to_f32(ldg<uint16_t>(base + 2 * i));
@@ -497,8 +460,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void fp8mm_mfma(F8Params p, 
           stg<U2>(p.out + index * 2, U2{uint32_t(f32_to_f16(v[0])) | uint32_t(f32_to_f16(v[1])) << 16,
                                         uint32_t(f32_to_f16(v[2])) | uint32_t(f32_to_f16(v[3])) << 16});
         } else if constexpr (DT == VKT_E4M3 || DT == VKT_E5M2) {
-          stg<uint32_t>(p.out + index, f32_to_fp8(v[0], DT) | f32_to_fp8(v[1], DT) << 8 | f32_to_fp8(v[2], DT) << 16 |
-                                           f32_to_fp8(v[3], DT) << 24);
+          stg<uint32_t>(p.out + index, pack2_fp8<DT>(v[0], v[1]) | pack2_fp8<DT>(v[2], v[3]) << 16);
         } else {
 #pragma unroll
           for (int r = 0; r < 4; ++r)

@@ -217,6 +217,26 @@ at::Tensor copy_from(const at::Tensor& src, const at::Tensor& dst, bool non_bloc
     }
     return dst;
   }
+  // float8 <-> float32 / float16 / bfloat16 between two vk tensors of the same dense layout:
+  // converted on the device, bit for bit as the CPU converts (reference backend.cpp:534-586)
+  if (is_vk(src) && is_vk(dst) && src.sizes() == dst.sizes() && src.strides() == dst.strides() && plain(src) &&
+      plain(dst) && !src.is_conj() && !src.is_neg()) {
+    const int sdt = vkt_dtype(src.scalar_type()), ddt = vkt_dtype(dst.scalar_type());
+    const bool s8 = sdt == VKT_E4M3 || sdt == VKT_E5M2, d8 = ddt == VKT_E4M3 || ddt == VKT_E5M2;
+    if (sdt >= 0 && ddt >= 0 && (s8 || d8)) {
+      const auto [slo, shi] = element_span(src);
+      const auto [dlo, dhi] = element_span(dst);
+      (void)shi, (void)dhi;
+      CastParams p{};
+      p.src = reinterpret_cast<uint64_t>(src.const_data_ptr()) + uint64_t(slo * src.element_size());
+      p.dst = reinterpret_cast<uint64_t>(dst.mutable_data_ptr()) + uint64_t(dlo * dst.element_size());
+      p.n = uint64_t(dst.numel());
+      p.src_dtype = uint32_t(sdt);
+      p.dst_dtype = uint32_t(ddt);
+      dispatch("cast_fp8", {}, p, 1);
+      return dst;
+    }
+  }
   // anything else (dtype conversion, strides, broadcast): through host mirrors
   at::Tensor s = is_vk(src) ? host_mirror(src, true) : src;
   if (!is_vk(dst)) {

@@ -23,17 +23,6 @@ namespace {
 
 constexpr int64_t kMaxRows = 65535;  // rows per dispatch of the int4 kernels (quant.cpp:29)
 
-int vkt_dtype(at::ScalarType t) {
-  switch (t) {
-    case at::kFloat: return VKT_F32;
-    case at::kHalf: return VKT_F16;
-    case at::kBFloat16: return VKT_BF16;
-    case at::kFloat8_e4m3fn: return VKT_E4M3;
-    case at::kFloat8_e5m2: return VKT_E5M2;
-    default: return -1;
-  }
-}
-
 const char* float_label(at::ScalarType t) {  // (reference quant.cpp:47-51)
   if (t == at::kFloat) return "f32";
   if (t == at::kHalf) return "f16";
@@ -388,6 +377,50 @@ at::Tensor scaled_mm(const at::Tensor& mat_a, const at::Tensor& mat_b, const at:
 
 }  // namespace
 }  // namespace vk
+
+namespace vk {
+namespace {
+
+// vk::fp8_quant_rowwise(x [M,K] float32 / float16 / bfloat16, dtype) -> (q [M,K] float8, scale [M,1]
+// float32): the producer in front of _scaled_mm (kernel "fp8_quant"), scale as _scaled_mm
+// takes a rowwise scale_a (for mat2 quantise the [N,K] weight and pass q.t(), scale.t()).
+// No counterpart in the reference: its float8 tensors come from casts alone.
+std::tuple<at::Tensor, at::Tensor> fp8_quant_rowwise(const at::Tensor& x, at::ScalarType dtype) {
+  TORCH_CHECK(x.dim() == 2, "fp8_quant_rowwise: expected a 2-D input, got ", x.sizes());
+  TORCH_CHECK(dtype == at::kFloat8_e4m3fn || dtype == at::kFloat8_e5m2,
+              "fp8_quant_rowwise: dtype must be float8_e4m3fn or float8_e5m2, got ", dtype);
+  const int sdt = vkt_dtype(x.scalar_type());
+  TORCH_CHECK(sdt >= 0 && sdt <= VKT_BF16, "fp8_quant_rowwise: input must be float32, float16 or bfloat16, got ",
+              x.scalar_type());
+  TORCH_CHECK(is_vk(x), "fp8_quant_rowwise: input must be on the vk device");
+  const int64_t M = x.size(0), K = x.size(1);
+  TORCH_CHECK(M < (int64_t(1) << 31) && K < (int64_t(1) << 31), "fp8_quant_rowwise: too large");
+  at::Tensor xc = x.contiguous();
+  at::Tensor q = at::empty({M, K}, x.options().dtype(dtype));
+  at::Tensor scale = at::empty({M, 1}, x.options().dtype(at::kFloat));
+  if (M == 0 || K == 0) {
+    // (rows without elements: the scale of an all-zero row)
+    if (M != 0) scale.fill_(1e-12f / (dtype == at::kFloat8_e4m3fn ? 448.0f : 57344.0f));
+    return {q, scale};
+  }
+  F8QuantParams p{};
+  p.src = gpu_address(xc);
+  p.dst = gpu_address_out(q);
+  p.scale = gpu_address_out(scale);
+  p.m = static_cast<uint32_t>(M);
+  p.k = static_cast<uint32_t>(K);
+  p.lds = p.ldd = static_cast<uint32_t>(K);
+  p.src_dtype = static_cast<uint32_t>(sdt);
+  p.dst_fmt = static_cast<uint32_t>(vkt_dtype(dtype));
+  dispatch("fp8_quant", {1u}, p, static_cast<uint32_t>(M));
+  return {q, scale};
+}
+
+}  // namespace
+}  // namespace vk
+
+TORCH_LIBRARY(vk, m) { m.def("fp8_quant_rowwise(Tensor x, ScalarType dtype) -> (Tensor, Tensor)"); }
+TORCH_LIBRARY_IMPL(vk, PrivateUse1, m) { m.impl("fp8_quant_rowwise", &vk::fp8_quant_rowwise); }
 
 TORCH_LIBRARY_IMPL(aten, PrivateUse1, m) {
   using namespace vk;

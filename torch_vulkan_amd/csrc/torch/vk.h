@@ -39,6 +39,18 @@ void run_fallback(const c10::OperatorHandle& op, torch::jit::Stack* stack, bool 
 
 inline bool is_vk(const at::Tensor& t) { return t.device().type() == kDevice; }
 
+// The library's code of an element type (-1: not one of its types).
+inline int vkt_dtype(at::ScalarType t) {
+  switch (t) {
+    case at::kFloat: return VKT_F32;
+    case at::kHalf: return VKT_F16;
+    case at::kBFloat16: return VKT_BF16;
+    case at::kFloat8_e4m3fn: return VKT_E4M3;
+    case at::kFloat8_e5m2: return VKT_E5M2;
+    default: return -1;
+  }
+}
+
 // Runs aten op `name.overload` without a vk kernel (reference vk.h:372-379).
 template <typename... Args>
 torch::jit::Stack on_cpu(const char* name, const char* overload, const Args&... args) {
