@@ -144,6 +144,21 @@ typedef struct Q4CParams {
   uint32_t m, n, k, bs, has_bias, pad;
 } Q4CParams;
 
+/* "gemmcm_bf16" | "gemmcm_f16", spec {USE_CIN, (ignored), (ignored), VARIANT}; grid z = batches:
+ * C[b] = alpha * A[b] @ B[b] (+ beta * Cin[b] when USE_CIN), 16-bit operands, float32
+ * accumulation, one rounding (the reference's block, linalg.cpp:25-34, and kernel,
+ * shaders/gemmcm.slang).  Strides in elements; alpha and beta hold float32 bits in their low
+ * words.  112 bytes. */
+typedef struct GemmParams {
+  uint64_t a, b, c, cin;
+  uint64_t alpha, beta;
+  uint32_t m, n, k, pad;
+  int32_t a_sm, a_sk, a_sb;
+  int32_t b_sk, b_sn, b_sb;
+  int32_t c_sm, c_sn, c_sb;
+  int32_t cin_sm, cin_sn, cin_sb;
+} GemmParams;
+
 /* "cast_fp8", spec {}: dst[i] = convert(src[i]), i < n, where one side is VKT_E4M3 / VKT_E5M2
  * and the other VKT_F32 / VKT_F16 / VKT_BF16 (or the other float8 format): through float32,
  * bit for bit as the CPU converts (what the reference's copy between a float8 tensor and

@@ -200,3 +200,36 @@ def fp8_quant(x, dtype, fmt, scale=None):
     scales = np.empty(m, np.float32) if rowwise else np.asarray([scale], np.float32)
     lib().orc_fp8_quant_rows(_p(x), dtype, I64(m), I64(k), I64(k), fmt, int(rowwise), _p(q), I64(k), _p(scales))
     return q, scales
+
+
+def _strided(a):
+    """(base pointer, element strides) of a numpy array viewed as [B, R, C]."""
+    a3 = a if a.ndim == 3 else a[None]
+    st = np.array([x // a.itemsize for x in a3.strides], np.int64)
+    return a3, st
+
+
+def gemm16(a, b, dtype, cin=None, alpha=1.0, beta=0.0, want_mag=False):
+    """alpha * a @ b (+ beta * cin) for uint16 views of bfloat16 / float16 arrays [B,]M,K and [B,]K,N
+    (any strides); cin broadcastable to the result.  Returns the 16-bit result [B,]M,N (and the magnitude bound)."""
+    a3, sa = _strided(np.asarray(a))
+    b3, sb = _strided(np.asarray(b))
+    B, M, K = a3.shape
+    N = b3.shape[2]
+    out = np.empty((B, M, N), np.uint16)
+    sc = np.array([M * N, N, 1], np.int64)
+    mag = np.empty((B, M, N), np.float64) if want_mag else None
+    if cin is not None:
+        c3 = np.broadcast_to(np.asarray(cin), (B, M, N))
+        scin = np.array([x // 2 for x in c3.strides], np.int64)
+        cp = ctypes.c_void_p(c3.__array_interface__["data"][0])
+    else:
+        scin, cp = np.zeros(3, np.int64), None
+    # base pointers at element (0,0,0): negative strides are handled by the element offsets
+    lib().orc_gemm16(ctypes.c_void_p(a3.__array_interface__["data"][0]), ctypes.c_void_p(b3.__array_interface__["data"][0]),
+                     cp, _p(out), dtype, I64(B), I64(M), I64(N), I64(K), _p(sa), _p(sb), _p(sc), _p(scin),
+                     ctypes.c_float(alpha), ctypes.c_float(beta), _p(mag) if want_mag else None)
+    res = out if np.asarray(a).ndim == 3 else out[0]
+    if want_mag:
+        return res, (mag if np.asarray(a).ndim == 3 else mag[0])
+    return res

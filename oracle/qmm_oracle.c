@@ -24,6 +24,9 @@
  *   orc_q4_matmul       pinned: torch CPU _dyn_quant_matmul_4bit (bit-exact), golden
  *   orc_scaled_mm       pinned: torch CPU _scaled_mm (per-tensor), f64 closed form,
  *                               identity / power-of-two cases that are exact
+ *   orc_gemm16          pinned: float64 closed form by numpy, torch CPU float32 matmul of the same
+ *                               16-bit values (inside the reference test's bound), exactly
+ *                               representable cases (small integers, identity, powers of two)
  *   orc_cast            pinned: torch CPU Tensor.to() between float32 / float16 / bfloat16 and
  *                               both float8 formats (the reference's own vectors,
  *                               tests/python/test_fallback_ops.py:469-485, plus all 256 codes)
@@ -388,4 +391,38 @@ void orc_fp8_quant_rows(const void* x, int dtype, int64_t M, int64_t K, int64_t 
       q[m * ldq + k] = orc_f32_to_fp8(y, fmt);
     }
   }
+}
+
+/* ------------------------------------------------------------------ 16-bit matrix product */
+
+/* C[b] = alpha * A[b] @ B[b] (+ beta * Cin[b]) for bfloat16 / float16 operands as the reference's
+ * cooperative-matrix kernel specifies it (crates/vkcore/shaders/gemmcm.slang:293-310,
+ * crates/pyvk/csrc/linalg.cpp:227-255): products accumulated in float32, alpha and beta
+ * applied in float32, one rounding to the 16-bit type.  The summation order is an
+ * implementation detail (the reference's test allows eps*|want| + 2^-20 * sum|a||b|,
+ * tests/python/test_matmul.py:250-264); this restatement sums in float64, the centre of that
+ * band.  Strides in elements (any sign, 0 for a broadcast Cin); mag (optional) receives
+ * |alpha| sum|a||b| + |beta||cin|. */
+void orc_gemm16(const void* a, const void* b, const void* cin, void* c, int dtype, int64_t B, int64_t M, int64_t N, int64_t K,
+                const int64_t* sa, const int64_t* sb, const int64_t* sc, const int64_t* scin, float alpha, float beta,
+                double* mag) {
+  for (int64_t bb = 0; bb < B; bb++)
+    for (int64_t m = 0; m < M; m++)
+      for (int64_t n = 0; n < N; n++) {
+        double acc = 0.0, am = 0.0;
+        for (int64_t k = 0; k < K; k++) {
+          const double x = load_as_f32(a, bb * sa[0] + m * sa[1] + k * sa[2], dtype);
+          const double y = load_as_f32(b, bb * sb[0] + k * sb[1] + n * sb[2], dtype);
+          acc += x * y;
+          am += fabs(x * y);
+        }
+        double v = (double)alpha * acc, vm = fabs((double)alpha) * am;
+        if (cin) {
+          const double ci = load_as_f32(cin, bb * scin[0] + m * scin[1] + n * scin[2], dtype);
+          v += (double)beta * ci;
+          vm += fabs((double)beta * ci);
+        }
+        store_from_f32(c, bb * sc[0] + m * sc[1] + n * sc[2], dtype, (float)v);
+        if (mag) mag[(bb * M + m) * N + n] = vm;
+      }
 }

@@ -1,6 +1,8 @@
 """Runs the quantized-matmul kernels through the C ABI (vkt_alloc / vkt_copy_* /
 vkt_dispatch) on numpy storage arrays, the way the reference's C++ op layer drives its
 runtime (crates/pyvk/csrc/quant.cpp).  GPU tests only."""
+import ctypes
+
 import numpy as np
 
 import oracle
@@ -153,3 +155,40 @@ def fp8_quant(x, dtype, fmt, scale=None, pad=0):
     q = dq.to_numpy(np.uint8, (m, ldd))
     assert (q[:, k:] == 0xAB).all(), "the producer wrote between rows"
     return q[:, :k], ds.to_numpy(np.float32, (m if rowwise else 1,))
+
+
+def _device_view(arr):
+    """Uploads the bytes a (possibly strided) numpy array spans; returns (buffer, address of
+    element [0,...,0], element strides)."""
+    arr = np.asarray(arr)
+    lo = sum(min(0, (n - 1) * st) for n, st in zip(arr.shape, arr.strides))
+    hi = sum(max(0, (n - 1) * st) for n, st in zip(arr.shape, arr.strides)) + arr.itemsize
+    base = arr.__array_interface__["data"][0] + lo
+    raw = (ctypes.c_uint8 * (hi - lo)).from_address(base)
+    buf = abi.Buffer(max(hi - lo, 1))
+    abi.check(abi.lib().vkt_copy_to_device(buf.address, ctypes.addressof(raw), hi - lo))
+    return buf, buf.address - lo, [st // arr.itemsize for st in arr.strides]
+
+
+def gemm16(a, b, dtype, cin=None, alpha=1.0, beta=0.0, variant=0):
+    """alpha * a @ b (+ beta * cin) through "gemmcm_<T>": a [B,]M,K and b [B,]K,N as uint16 views with
+    any strides; cin broadcastable to the result (zero strides)."""
+    a3 = np.asarray(a) if np.asarray(a).ndim == 3 else np.asarray(a)[None]
+    b3 = np.asarray(b) if np.asarray(b).ndim == 3 else np.asarray(b)[None]
+    B, M, K = a3.shape
+    N = b3.shape[2]
+    ba, pa, sa = _device_view(a3)
+    bb, pb, sb = _device_view(b3)
+    out = abi.Buffer(max(B * M * N * 2, 1))
+    p = abi.GemmParams(a=pa, b=pb, c=out.address, m=M, n=N, k=K, a_sb=sa[0], a_sm=sa[1], a_sk=sa[2], b_sb=sb[0],
+                       b_sk=sb[1], b_sn=sb[2], c_sb=M * N, c_sm=N, c_sn=1,
+                       alpha=int(np.float32(alpha).view(np.uint32)), beta=int(np.float32(beta).view(np.uint32)))
+    use_cin = cin is not None and beta != 0.0
+    if use_cin:
+        c3 = np.broadcast_to(np.asarray(cin), (B, M, N))
+        bc, pc, sc = _device_view(c3)
+        p.cin, p.cin_sb, p.cin_sm, p.cin_sn = pc, sc[0], sc[1], sc[2]
+    if B and M and N:
+        abi.dispatch("gemmcm_" + abi.SUFFIX[dtype], [int(use_cin), 0, 0, variant], p, (1, 1, B))
+    res = out.to_numpy(np.uint16, (B, M, N))
+    return res if np.asarray(a).ndim == 3 else res[0]

@@ -1,0 +1,97 @@
+"""GPU parity of the 16-bit matrix product ("gemmcm_bf16" / "gemmcm_f16") through the C ABI, as
+the reference tests its cooperative-matrix kernel (tests/python/test_matmul.py:250-284): every
+layout of the operands, edges of every size, strided views, batches, alpha / beta and a
+broadcast bias, inside eps*|want| + 2^-20 * sum|a||b| of the oracle and of PyTorch's CPU product."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from _util import ODT, bits, gen
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.bfloat16, torch.float16]
+
+
+def close(got, want, mag, dtype):
+    gf, wf = oracle.to_f32(got, ODT[dtype]).astype(np.float64), oracle.to_f32(want, ODT[dtype]).astype(np.float64)
+    tol = torch.finfo(dtype).eps * np.maximum(np.abs(wf), 2.0**-14) + 2.0**-20 * mag
+    assert (np.abs(gf - wf) <= tol).all(), float(np.max(np.abs(gf - wf) - tol))
+
+
+def col_major(x):
+    """The same values with the last two dims stored column by column."""
+    return np.ascontiguousarray(np.swapaxes(x, -1, -2)).swapaxes(-1, -2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("m,k,n", [(64, 32, 64), (65, 33, 63), (17, 200, 129), (128, 1, 96), (3, 1000, 5), (256, 64, 256),
+                                   (300, 136, 260), (1, 64, 1)])
+def test_gemm16_layouts(dtype, m, k, n):
+    import _dev
+    a = bits(torch.randn(m, k, generator=gen(1)).to(dtype))
+    b = bits(torch.randn(k, n, generator=gen(2)).to(dtype))
+    want, mag = oracle.gemm16(a, b, ODT[dtype], want_mag=True)
+    for x, y in [(a, b), (col_major(a), col_major(b)), (a, col_major(b)), (col_major(a), b)]:
+        close(_dev.gemm16(x, y, ODT[dtype]), want, mag, dtype)
+    close(_dev.gemm16(a[::2], b, ODT[dtype]), want[::2], mag[::2], dtype)  # a strided view
+    cpu = bits((torch.from_numpy(oracle.to_f32(a, ODT[dtype])) @ torch.from_numpy(oracle.to_f32(b, ODT[dtype]))).to(dtype))
+    close(_dev.gemm16(a, col_major(b), ODT[dtype]), cpu, mag, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 255])
+@pytest.mark.parametrize("m,k,n", [(130, 256, 70), (257, 384, 129), (64, 1088, 300), (300, 128, 520)])
+def test_gemm16_tile_variants(dtype, variant, m, k, n):
+    """The Linear layout (both operands contiguous along k) through every tile variant and the strided kernel."""
+    import _dev
+    a = bits((torch.randn(m, k, generator=gen(3)) * 0.5).to(dtype))
+    w = bits((torch.randn(n, k, generator=gen(4)) * 0.5).to(dtype))  # B = w.T: rows of k
+    want, mag = oracle.gemm16(a, w.T, ODT[dtype], want_mag=True)
+    close(_dev.gemm16(a, w.T, ODT[dtype], variant=variant), want, mag, dtype)
+    bias = bits(torch.randn(n, generator=gen(5)).to(dtype))
+    want2, mag2 = oracle.gemm16(a, w.T, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, want_mag=True)
+    close(_dev.gemm16(a, w.T, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, variant=variant), want2, mag2, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_gemm16_batches_and_bias(dtype):
+    import _dev
+    a = bits(torch.randn(3, 40, 72, generator=gen(6)).to(dtype))
+    w = bits(torch.randn(3, 50, 72, generator=gen(7)).to(dtype))
+    bias = bits(torch.randn(50, generator=gen(8)).to(dtype))
+    want, mag = oracle.gemm16(a, w.transpose(0, 2, 1), ODT[dtype], want_mag=True)
+    close(_dev.gemm16(a, w.transpose(0, 2, 1), ODT[dtype]), want, mag, dtype)
+    want, mag = oracle.gemm16(a[0], w[0].T, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, want_mag=True)
+    close(_dev.gemm16(a[0], w[0].T, ODT[dtype], cin=bias, alpha=2.0, beta=0.5), want, mag, dtype)
+    # beta == 0 ignores Cin entirely, NaN included (gemmcm.slang:309)
+    nan_bias = np.full(50, 0x7FC0 if dtype == torch.bfloat16 else 0x7E00, np.uint16)
+    want0, mag0 = oracle.gemm16(a[0], w[0].T, ODT[dtype], want_mag=True)
+    close(_dev.gemm16(a[0], w[0].T, ODT[dtype], cin=nan_bias, beta=0.0), want0, mag0, dtype)
+
+
+def test_gemm16_config_8192_cubed():
+    """The reference's adjacent benchmark shape (bf16 8192^3): sampled rows / columns against the float64 closed form."""
+    import _dev
+    m = n = k = 8192
+    a = torch.randn(m, k, generator=gen(9)).bfloat16()
+    w = torch.randn(n, k, generator=gen(10)).bfloat16()
+    got = _dev.gemm16(bits(a), bits(w).T, oracle.BF16)
+    rows, cols = np.array([0, 1, 255, 256, 4095, 8191]), np.array([0, 3, 127, 128, 5000, 8191])
+    exact = a[rows].double().numpy() @ w[cols].double().numpy().T
+    mag = np.abs(a[rows].double().numpy()) @ np.abs(w[cols].double().numpy()).T
+    sub = oracle.bf16_to_f32(got[np.ix_(rows, cols)]).astype(np.float64)
+    assert (np.abs(sub - exact) <= 2.0**-7 * np.maximum(np.abs(exact), 2.0**-14) + 2.0**-20 * mag).all()
+
+
+def test_gemm16_errors():
+    from torch_vulkan_amd import abi
+    buf = abi.Buffer(4096)
+    p = abi.GemmParams(a=buf.address, b=buf.address, c=buf.address, m=4, n=4, k=8, a_sm=8, a_sk=1, b_sk=1, b_sn=8, c_sm=4,
+                       c_sn=1)
+    with pytest.raises(abi.VktError, match="null tensor address"):
+        abi.dispatch("gemmcm_bf16", [1], p)
+    with pytest.raises(abi.VktError, match="unknown kernel"):
+        abi.dispatch("gemmcm_f32", [0], p)
+    with pytest.raises(abi.VktError, match="unknown variant"):
+        abi.dispatch("gemmcm_bf16", [0, 0, 0, 9], p)

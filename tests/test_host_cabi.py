@@ -29,6 +29,7 @@ def test_parameter_block_sizes():
     assert ctypes.sizeof(abi.Q8Params) == 56
     assert ctypes.sizeof(abi.Q4Params) == 64
     assert ctypes.sizeof(abi.CastParams) == 32 and ctypes.sizeof(abi.F8QuantParams) == 48
+    assert ctypes.sizeof(abi.GemmParams) == 112  # the reference's block (linalg.cpp:25-34)
     for t in (abi.Q4PackParams, abi.Q4CParams, abi.F8Params):
         assert ctypes.sizeof(t) <= 128
     assert ctypes.sizeof(abi.VktAlloc) == 32

@@ -61,6 +61,13 @@ class F8Params(ctypes.Structure):
                 ("fmt_a", u32), ("fmt_b", u32), ("out_dtype", u32), ("bias_dtype", u32), ("rowwise", u32), ("pad", u32)]
 
 
+class GemmParams(ctypes.Structure):
+    _fields_ = [("a", u64), ("b", u64), ("c", u64), ("cin", u64), ("alpha", u64), ("beta", u64),
+                ("m", u32), ("n", u32), ("k", u32), ("pad", u32)] + [
+                    (name, ctypes.c_int32) for name in ("a_sm", "a_sk", "a_sb", "b_sk", "b_sn", "b_sb", "c_sm", "c_sn", "c_sb",
+                                                        "cin_sm", "cin_sn", "cin_sb")]
+
+
 class CastParams(ctypes.Structure):
     _fields_ = [("src", u64), ("dst", u64), ("n", u64), ("src_dtype", u32), ("dst_dtype", u32)]
 
@@ -71,7 +78,7 @@ class F8QuantParams(ctypes.Structure):
 
 
 assert ctypes.sizeof(Q8Params) == 56 and ctypes.sizeof(Q4Params) == 64 and ctypes.sizeof(F8Params) == 104
-assert ctypes.sizeof(CastParams) == 32 and ctypes.sizeof(F8QuantParams) == 48
+assert ctypes.sizeof(CastParams) == 32 and ctypes.sizeof(F8QuantParams) == 48 and ctypes.sizeof(GemmParams) == 112
 
 # every symbol include/vkt.h declares
 SYMBOLS = ["vkt_last_error", "vkt_alloc", "vkt_free", "vkt_synchronize", "vkt_empty_cache", "vkt_memory_stats",

@@ -27,6 +27,7 @@ SOURCES = {
     # (and its MFMA results go to ordinary registers, where the float32 chain consumes them)
     "kernels/qmm4.hip": ["-ffp-contract=off", "-mllvm", "-amdgpu-mfma-vgpr-form"],
     "kernels/fp8mm.hip": [],
+    "kernels/gemm16.hip": [],
     # (single float32 operations in the float8 producer, as specified)
     "kernels/cast.hip": ["-ffp-contract=off"],
     "kernels/util.hip": [],

@@ -168,7 +168,7 @@ bool read_push(const uint8_t* push, size_t npush, P* out, const char* name, std:
 
 // name + specialisation constants -> launcher (the role of kernels.rs:72-140 KernelCache::get).
 int dispatch_named(Runtime& rt, const char* name, const uint32_t* spec, size_t nspec, const uint8_t* push, size_t npush,
-                   std::string* err) {
+                   uint32_t gz, std::string* err) {
   auto spec_at = [&](size_t i) { return i < nspec ? spec[i] : 0u; };
   if (!std::strncmp(name, "qmm8_", 5)) {
     int dt = dtype_of_suffix(name + 5);
@@ -206,6 +206,13 @@ int dispatch_named(Runtime& rt, const char* name, const uint32_t* spec, size_t n
     if (dt != VKT_F32 && dt != VKT_BF16) goto unknown;
     if (!read_push(push, npush, &p, name, err)) return -1;
     return launch_qmm4c(p, dt, spec_at(0), spec_at(1), spec_at(2), rt.machine, rt.stream, err);
+  }
+  if (!std::strncmp(name, "gemmcm_", 7)) {
+    int dt = dtype_of_suffix(name + 7);
+    GemmParams p;
+    if (dt != VKT_BF16 && dt != VKT_F16) goto unknown;
+    if (!read_push(push, npush, &p, name, err)) return -1;
+    return launch_gemm16(p, dt, spec_at(0), gz, spec_at(3), rt.machine, rt.stream, err);
   }
   if (!std::strcmp(name, "cast_fp8")) {
     CastParams p;
@@ -307,7 +314,7 @@ int vkt_dispatch(const char* name, const uint32_t* spec, size_t nspec, const uin
   if (npush != 0 && !push) return fail("parameter block is null");
   if (gx == 0 || gy == 0 || gz == 0) return fail("empty grid");
   std::lock_guard<std::mutex> lock(rt->stream_mutex);
-  if (dispatch_named(*rt, name, spec, nspec, push, npush, &err) != 0) return fail(err);
+  if (dispatch_named(*rt, name, spec, nspec, push, npush, gz, &err) != 0) return fail(err);
   rt->dispatches.fetch_add(1, std::memory_order_relaxed);
   if (rt->trace) {
     // each kernel runs to completion before the next is queued, so a kernel that
@@ -356,7 +363,7 @@ uint32_t vkt_kernel_subgroup_size(const char* name) {
   if (!name) return 0;
   std::string err;
   if (!runtime(&err)) return 0;
-  return (!std::strncmp(name, "qmm", 3) || !std::strcmp(name, "fp8mm") || !std::strcmp(name, "cast_fp8") ||
+  return (!std::strncmp(name, "qmm", 3) || !std::strcmp(name, "fp8mm") || !std::strcmp(name, "cast_fp8") || !std::strncmp(name, "gemmcm_", 7) ||
           !std::strcmp(name, "fp8_quant"))
              ? 64u
              : 0u;

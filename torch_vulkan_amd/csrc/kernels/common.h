@@ -37,6 +37,7 @@ __device__ __forceinline__ void stg(uint64_t addr, X v) {
 }
 
 __device__ __forceinline__ float bits_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+inline float bits_f32_host(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t f32_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
 
 // Storage element types.  16-bit floats are carried as raw bits so that every rounding
@@ -182,6 +183,16 @@ __device__ __forceinline__ uint32_t pack2_fp8(float a, float b) {
   else r = uint32_t(__builtin_amdgcn_cvt_pk_bf8_f32(a, b, 0, false));
   const uint32_t ca = a != a ? na : (r & 0xffu), cb = b != b ? nb : ((r >> 8) & 0xffu);
   return ca | cb << 8;
+}
+
+// Two float32 -> two bfloat16 in one word: v_cvt_pk_bf16_f32 (round to nearest even); NaN
+// becomes 0x7fc0 as c10 writes it.
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  using V2 = __bf16 __attribute__((ext_vector_type(2)));
+  const float qnan = bits_f32(0x7fc00000u);
+  a = a != a ? qnan : a;
+  b = b != b ? qnan : b;
+  return __builtin_bit_cast(uint32_t, V2{static_cast<__bf16>(a), static_cast<__bf16>(b)});
 }
 
 // ---- wave64 reductions through DPP (no LDS traffic) ----

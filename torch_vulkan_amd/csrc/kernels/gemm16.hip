@@ -1,0 +1,140 @@
+// The unquantised Linear next to the quantised ops: C[b] = alpha * A[b] @ B[b] (+ beta * Cin[b])
+// for bfloat16 / float16 matrices, products accumulated in float32 and rounded once - the
+// contract of the reference's cooperative-matrix kernel (crates/vkcore/shaders/gemmcm.slang,
+// host side crates/pyvk/csrc/linalg.cpp:227-255), behind its kernel names ("gemmcm_bf16",
+// "gemmcm_f16"), parameter block (GemmParams, strides in elements) and spec {USE_CIN, ..}.
+//   - A rows and B columns both contiguous along k (x @ W.t(), the Linear layout), 16-byte
+//     aligned, k a multiple of 8: the tile kernel of _scaled_mm (mma_tile.h: 256x256x64-value
+//     workgroup tiles, direct global-to-LDS loads, persistent grid) with
+//     V_MFMA_F32_32X32X16_{BF16,F16} and an alpha / beta epilogue;
+//   - every other layout (row-major B, column-major A, strided views): one thread per output
+//     over the strides as given.  Correct for any strides, and slow.
+#include "kernels.h"
+#include "mma_tile.h"
+
+namespace vkt {
+namespace {
+
+__device__ __forceinline__ float slot_float(uint64_t slot) { return bits_f32(uint32_t(slot)); }
+
+template <class T>
+struct GemmProblem {
+  // operands as the tile kernel takes them (bytes)
+  uint64_t a, b;
+  uint32_t m, n, k, lda, ldb, batches;
+  uint64_t a_batch, b_batch;
+  // epilogue
+  uint64_t c, cin;
+  float alpha, beta;
+  int32_t c_sm, c_sb, cin_sm, cin_sn, cin_sb;  // elements (c_sn is 1 here)
+  struct Whole {
+    bool vec_ok;
+  };
+  struct Columns {};
+  __device__ __forceinline__ Whole whole() const { return Whole{(c_sm & 3) == 0 && (c_sb & 3) == 0 && (c & 7u) == 0}; }
+  __device__ __forceinline__ Columns columns(uint32_t, uint32_t, const Whole&) const { return Columns{}; }
+  template <int DT>
+  __device__ __forceinline__ void store(uint32_t batch, uint32_t row, uint32_t col, const V4F& t, const Columns&,
+                                        const Whole&) const {
+    float v[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      v[r] = alpha * t[r];
+      if (cin != 0 && (DT >= 0 || col + r < n)) {  // beta == 0 never reads Cin (it may hold NaN): then cin is 0
+        const int64_t at = int64_t(batch) * cin_sb + int64_t(row) * cin_sm + int64_t(col + r) * cin_sn;
+        v[r] += beta * load_f32<T>(cin + uint64_t(at * 2));
+      }
+    }
+    const uint64_t out = c + uint64_t((int64_t(batch) * c_sb + int64_t(row) * c_sm + int64_t(col)) * 2);
+    if constexpr (DT >= 0) {
+      if constexpr (T::dtype == VKT_BF16) stg<U2>(out, U2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])});
+      else stg<U2>(out, U2{uint32_t(f32_to_f16(v[0])) | uint32_t(f32_to_f16(v[1])) << 16,
+                           uint32_t(f32_to_f16(v[2])) | uint32_t(f32_to_f16(v[3])) << 16});
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (col + r < n) store_f32<T>(out + 2 * r, v[r]);
+    }
+  }
+  template <class F>
+  __device__ __forceinline__ void for_output_type(bool full, const Whole& w, F&& f) const {
+    if (w.vec_ok && full) f(std::integral_constant<int, T::dtype>{});
+    else f(std::integral_constant<int, -1>{});
+  }
+};
+
+// Any strides: one thread per output, float32 accumulation.
+template <class T>
+__global__ __launch_bounds__(256) void gemm16_generic(GemmParams p, uint32_t use_cin) {
+  const uint32_t n = blockIdx.x * 64 + (threadIdx.x & 63), m = blockIdx.y * 4 + (threadIdx.x >> 6), batch = blockIdx.z;
+  if (m >= p.m || n >= p.n) return;
+  const int64_t a0 = int64_t(batch) * p.a_sb + int64_t(m) * p.a_sm, b0 = int64_t(batch) * p.b_sb + int64_t(n) * p.b_sn;
+  float acc = 0.0f;
+  for (uint32_t k = 0; k < p.k; ++k)
+    acc = fmaf(load_f32<T>(p.a + uint64_t((a0 + int64_t(k) * p.a_sk) * 2)), load_f32<T>(p.b + uint64_t((b0 + int64_t(k) * p.b_sk) * 2)), acc);
+  float v = slot_float(p.alpha) * acc;
+  if (use_cin) {
+    const int64_t at = int64_t(batch) * p.cin_sb + int64_t(m) * p.cin_sm + int64_t(n) * p.cin_sn;
+    v += slot_float(p.beta) * load_f32<T>(p.cin + uint64_t(at * 2));
+  }
+  store_f32<T>(p.c + uint64_t((int64_t(batch) * p.c_sb + int64_t(m) * p.c_sm + int64_t(n) * p.c_sn) * 2), v);
+}
+
+template <class T>
+int launch_gemm16_t(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t variant, const Machine& mc,
+                    hipStream_t stream, std::string* err) {
+  constexpr int MATH = T::dtype == VKT_BF16 ? kMathBf16 : kMathF16;
+  const bool tiles_ok = p.k != 0 && p.k % 8 == 0 && p.a_sk == 1 && p.b_sk == 1 && p.c_sn == 1 && p.a_sm > 0 && p.b_sn > 0 &&
+                        p.c_sm > 0 && p.a_sm % 8 == 0 && p.b_sn % 8 == 0 && p.a_sb % 8 == 0 && p.b_sb % 8 == 0 &&
+                        p.a_sb >= 0 && p.b_sb >= 0 && p.c_sb >= 0 && p.a % 16 == 0 && p.b % 16 == 0 &&
+                        uint32_t(p.a_sm) >= p.k && uint32_t(p.b_sn) >= p.k && variant != 255;
+  if (!tiles_ok) {
+    if ((p.m + 3) / 4 > 65535 || batch > 65535) {
+      *err = "gemmcm: too many rows or batches for the strided kernel";
+      return -1;
+    }
+    hipLaunchKernelGGL((gemm16_generic<T>), dim3((p.n + 63) / 64, (p.m + 3) / 4, batch), dim3(256), 0, stream, p, use_cin);
+    return 0;
+  }
+  GemmProblem<T> g;
+  g.a = p.a, g.b = p.b, g.m = p.m, g.n = p.n, g.k = p.k * 2, g.lda = uint32_t(p.a_sm) * 2, g.ldb = uint32_t(p.b_sn) * 2;
+  g.batches = batch, g.a_batch = uint64_t(p.a_sb) * 2, g.b_batch = uint64_t(p.b_sb) * 2;
+  g.c = p.c, g.cin = use_cin ? p.cin : 0;
+  g.alpha = bits_f32_host(uint32_t(p.alpha)), g.beta = bits_f32_host(uint32_t(p.beta));
+  g.c_sm = p.c_sm, g.c_sb = p.c_sb, g.cin_sm = p.cin_sm, g.cin_sn = p.cin_sn, g.cin_sb = p.cin_sb;
+  // variant 0: planned; 1: 128x128 tiles; 2: 256x128; 3: 256x256 with direct loads (k a multiple of 64)
+  if (variant == 0) variant = uint64_t(p.m) * p.n >= (1ull << 20) ? (g.k % BK == 0 ? 3 : 2) : 1;
+  switch (variant) {
+    case 1: return launch_mma_tile<2, 2, 4, 4, 0, 0, true, false, MATH>(g, mc.compute_units, stream, err, "gemmcm");
+    case 2: return launch_mma_tile<2, 2, 8, 4, 0, 0, true, false, MATH>(g, mc.compute_units, stream, err, "gemmcm");
+    case 3:
+      if (g.k % BK != 0) break;
+      return launch_mma_tile<2, 2, 8, 8, 0, 0, true, true, MATH>(g, mc.compute_units, stream, err, "gemmcm");
+  }
+  *err = "gemmcm: unknown variant " + std::to_string(variant) + " for this k";
+  return -1;
+}
+
+}  // namespace
+
+int launch_gemm16(const GemmParams& p, int dtype, uint32_t use_cin, uint32_t batch, uint32_t variant, const Machine& mc,
+                  hipStream_t stream, std::string* err) {
+  if (p.m == 0 || p.n == 0 || batch == 0) return 0;
+  if (!p.a || !p.b || !p.c || (use_cin && !p.cin)) {
+    *err = "gemmcm: null tensor address";
+    return -1;
+  }
+  if (use_cin > 1) {
+    *err = "gemmcm: USE_CIN must be 0 or 1";
+    return -1;
+  }
+  const int rc = dtype == VKT_BF16 ? launch_gemm16_t<bf16_t>(p, use_cin, batch, variant, mc, stream, err)
+                                   : launch_gemm16_t<f16_t>(p, use_cin, batch, variant, mc, stream, err);
+  if (rc == 0 && hipGetLastError() != hipSuccess) {
+    *err = "gemmcm: kernel launch failed";
+    return -1;
+  }
+  return rc;
+}
+
+}  // namespace vkt

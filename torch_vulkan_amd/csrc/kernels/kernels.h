@@ -29,6 +29,8 @@ int launch_qmm4c_pack(const Q4PackParams& p, uint32_t layout, const Machine& mc,
 int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwise, uint32_t layout,
                  const Machine& mc, hipStream_t stream, std::string* err);
 int launch_fp8mm(const F8Params& p, uint32_t variant, const Machine& mc, hipStream_t stream, std::string* err);
+int launch_gemm16(const GemmParams& p, int dtype, uint32_t use_cin, uint32_t batch, uint32_t variant, const Machine& mc,
+                  hipStream_t stream, std::string* err);
 int launch_cast_fp8(const CastParams& p, const Machine& mc, hipStream_t stream, std::string* err);
 int launch_fp8_quant(const F8QuantParams& p, uint32_t rowwise, const Machine& mc, hipStream_t stream, std::string* err);
 int launch_fill(uint64_t dst, uint8_t value, uint64_t nbytes, hipStream_t stream, std::string* err);
