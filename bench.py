@@ -31,6 +31,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 FP8_PEAK_TFLOPS = 5000.0    # MI355X dense fp8 MFMA, published
+BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 / fp16 MFMA, published
 
 
 def _abi():
@@ -174,6 +175,20 @@ def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False)
                      + (" (all-zero operands)" if zero_operands else ""))
 
 
+def wl_gemm16(abi, m, k, n, steps, warmup, seed=1090):
+    """bfloat16 mm in the Linear layout (x [m,k] @ w[n,k]^T -> [m,n]): the unquantised product next to the path."""
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    a, w = torch.randn(m, k, generator=g).bfloat16(), torch.randn(n, k, generator=g).bfloat16()
+    da, dw = abi.Buffer.from_numpy(a.view(torch.int16).numpy()), abi.Buffer.from_numpy(w.view(torch.int16).numpy())
+    out = abi.Buffer(m * n * 2)
+    p = abi.GemmParams(a=da.address, b=dw.address, c=out.address, m=m, n=n, k=k, a_sm=k, a_sk=1, b_sk=1, b_sn=k, c_sm=n,
+                       c_sn=1, alpha=int(np.float32(1).view(np.uint32)))
+    wall, ev = time_steps(abi, [Launch(abi, "gemmcm_bf16", [0], p)], steps, warmup)
+    return dict(kind="mfma", peak=BF16_PEAK_TFLOPS, metric="bf16 mm TFLOP/s (% of MFMA peak)", work=2 * m * n * k, wall_ms=wall, event_ms=ev,
+                bytes=2 * (m * k + n * k + m * n), inputs=None, copies=1, name=f"mm bf16 M={m} K={k} N={n} (Linear layout)")
+
+
 def wl_cast(abi, n, steps, warmup, seed=1070):
     """bfloat16 -> e4m3fn elementwise cast of n values (the float8 step in front of _scaled_mm)."""
     import torch
@@ -232,6 +247,8 @@ WORKLOADS = {
     # at the size of config 4's A operand and beyond the L2 / MALL capacity
     "f8_cast_bf16_e4m3_256mi": lambda abi, s, w: wl_cast(abi, 1 << 28, max(s // 10, 5), max(w // 4, 3)),
     "f8_quant_rowwise_bf16_16384x16384": lambda abi, s, w: wl_quant(abi, 16384, 16384, max(s // 10, 5), max(w // 4, 3)),
+    # the unquantised 16-bit product beside the path (not a BASELINE configuration), at the reference's own shape
+    "mm_bf16_8192": lambda abi, s, w: wl_gemm16(abi, 8192, 8192, 8192, max(s // 10, 5), max(w // 4, 3)),
     # config 4's launch on all-zero operands (not a BASELINE configuration: it shows how much of the
     # distance to the published peak is the data's, not the kernel's)
     "c4_fp8_8192_zero_operands": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 10, 5),
@@ -248,7 +265,7 @@ def summarise(r):
         value, unit, peak = r["work"] / r["wall_ms"] / 1e6, "GB/s", HBM_PEAK_GBPS
         achieved = r["work"] / r["event_ms"] / 1e6
     else:
-        value, unit, peak = r["work"] / r["wall_ms"] / 1e9, "TFLOP/s", FP8_PEAK_TFLOPS
+        value, unit, peak = r["work"] / r["wall_ms"] / 1e9, "TFLOP/s", r.get("peak", FP8_PEAK_TFLOPS)
         achieved = r["work"] / r["event_ms"] / 1e9
     return value, unit, dict(bound=r["kind"], achieved=round(achieved, 1), peak=peak, unit=unit,
                              frac=round(achieved / peak, 4), traffic=None)
@@ -317,7 +334,8 @@ def main():
     value, unit, roof = summarise(r)
     roof["traffic"] = traffic.get(args.workload)
     line = {
-        "metric": "M=1 int8 GEMV GB/s (% of HBM peak)" if r["kind"] == "hbm" else "fp8 _scaled_mm TFLOP/s (% of MFMA peak)",
+        "metric": r.get("metric") or ("M=1 int8 GEMV GB/s (% of HBM peak)" if r["kind"] == "hbm"
+                                      else "fp8 _scaled_mm TFLOP/s (% of MFMA peak)"),
         "value": round(value, 1), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(r["wall_ms"], 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32 accumulate (bf16 activations, int8 weights)" if args.workload.startswith("c2") else "see workload",

@@ -242,3 +242,53 @@ def test_fp8_quant_rowwise_into_scaled_mm(tv, f8, src):
     assert ((out.cpu().double() - want).abs() <= 2.0**-23 * want.abs() + 2.0**-20 * mag).all()
     with pytest.raises(RuntimeError, match="float8_e4m3fn or float8_e5m2"):
         torch.ops.vk.fp8_quant_rowwise(a.to("vk"), torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_16bit_matrix_products(tv, dtype):
+    """mm / bmm / addmm of 16-bit tensors on the matrix cores, as the reference tests its
+    cooperative-matrix kernel (tests/python/test_matmul.py:250-284): float32 sums rounded once, one
+    ulp from the CPU's float32 product plus summation-order error relative to the products'
+    magnitudes; every layout, a strided view, batches, alpha / beta with a broadcast bias."""
+
+    def want(x, y):
+        return (x.float() @ y.float()).to(dtype)
+
+    def close(got, ref, mag):
+        assert got.device.type == "vk" and got.dtype == dtype and got.shape == ref.shape
+        got, ref = got.cpu().float(), ref.float()
+        tol = torch.finfo(dtype).eps * ref.abs().clamp_min(2**-14) + 2**-20 * mag
+        assert ((got - ref).abs() <= tol).all(), (got - ref).abs().max().item()
+
+    for m, k, n in [(64, 32, 64), (65, 33, 63), (17, 200, 129), (128, 1, 96), (3, 1000, 5), (300, 256, 260)]:
+        a, b = torch.randn(m, k, generator=gen(1)).to(dtype), torch.randn(k, n, generator=gen(2)).to(dtype)
+        at, bt = a.t().contiguous().t(), b.t().contiguous().t()  # (column-major)
+        for x, y in [(a, b), (at, bt), (a, bt), (at, b)]:
+            with on_gpu(tv):
+                got = x.to("vk") @ y.to("vk")
+            close(got, want(a, b), a.float().abs() @ b.float().abs())
+        with on_gpu(tv):
+            got = a.to("vk")[::2] @ b.to("vk")
+        close(got, want(a[::2], b), a[::2].float().abs() @ b.float().abs())
+    a, b = torch.randn(3, 40, 72, generator=gen(3)).to(dtype), torch.randn(3, 50, 72, generator=gen(4)).to(dtype)
+    bias = torch.randn(50, generator=gen(5)).to(dtype)
+    with on_gpu(tv):
+        got_t = torch.bmm(a.to("vk"), b.to("vk").transpose(1, 2))
+        got_add = torch.addmm(bias.to("vk"), a[0].to("vk"), b[0].to("vk").t(), beta=0.5, alpha=2.0)
+        got_lin = torch.nn.functional.linear(a.to("vk"), b[0].to("vk"), bias.to("vk"))  # [3,40,72] x [50,72]^T + bias
+        got_badd = torch.baddbmm(bias.to("vk"), a.to("vk"), b.to("vk").transpose(1, 2), beta=0.5, alpha=2.0)
+        out = torch.empty(0, dtype=dtype, device="vk")
+        torch.mm(a[1].to("vk"), b[1].to("vk").t(), out=out)
+        empty_k = torch.mm(a[0, :, :0].to("vk"), b[0, :, :0].to("vk").t())
+    mag_t = a.float().abs() @ b.float().abs().transpose(1, 2)
+    close(got_t, want(a, b.transpose(1, 2)), mag_t)
+    close(out, want(a[1], b[1].t()), mag_t[1])
+    close(got_add, (0.5 * bias.float() + 2.0 * (a[0].float() @ b[0].float().t())).to(dtype), 0.5 * bias.float().abs() + 2.0 * mag_t[0])
+    close(got_badd, (0.5 * bias.float() + 2.0 * (a.float() @ b.float().transpose(1, 2))).to(dtype), 0.5 * bias.float().abs() + 2.0 * mag_t)
+    close(got_lin, (a.float() @ b[0].float().t() + bias.float()).to(dtype), a.float().abs() @ b[0].float().abs().t() + bias.float().abs())
+    assert empty_k.shape == (40, 50) and (empty_k.cpu() == 0).all()  # (k = 0: sums of nothing)
+    assert tv.kernel_subgroup_size("gemmcm_bf16") == 64 and tv.kernel_subgroup_size("gemmcm_f16") == 64
+    with pytest.raises(RuntimeError, match="cannot be multiplied"):
+        torch.mm(a[0].to("vk"), b[0].to("vk"))
+    with pytest.raises(RuntimeError, match="same dtype"):
+        torch.mm(a[0].to("vk"), b[0].t().float().to("vk"))

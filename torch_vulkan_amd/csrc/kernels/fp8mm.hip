@@ -12,7 +12,7 @@
 // input itself is added in full float32).  On random data that is an error of ~2^-16 of
 // sum|a||b| per output, invisible at bfloat16 / float8 output precision (eps >= 2^-8) but
 // not at float32.  So the path is chosen by the precision the caller asked for:
-//   bfloat16 / float8 outputs  -> fp8mm_mfma (this is the 5 PFLOP/s path)
+//   bfloat16 / float8 outputs  -> mma_tile on the fp8 matrix cores (this is the 5 PFLOP/s path)
 //   float32 / float16 outputs  -> the same kernel with each float8 fragment widened (exactly)
 //                                 to bfloat16 in registers and fed to the bfloat16 matrix
 //                                 core, which keeps float32 precision (half the rate: 2.5
@@ -21,7 +21,7 @@
 // The scales multiply once per output instead of once per operand element (one rounding
 // less than the reference, inside the same bound).
 //
-//   fp8mm_mfma     V_MFMA_F32_32X32X64_F8F6F4 / 16X16X128 (8192 flop/clk/CU: the only fp8 rate
+//   mma_tile       (mma_tile.h) V_MFMA_F32_32X32X64_F8F6F4 / 16X16X128 (8192 flop/clk/CU: the only fp8 rate
 //                  that reaches the 5 PFLOP/s peak; the 16x16x32 fp8 instruction runs at half).
 //                  A workgroup computes a BM x BN tile, K in steps of 128 bytes; both
 //                  operand tiles are staged in LDS (double buffered, 16-byte chunks XOR-

@@ -120,7 +120,7 @@ int launch_gemm16_t(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint3
 int launch_gemm16(const GemmParams& p, int dtype, uint32_t use_cin, uint32_t batch, uint32_t variant, const Machine& mc,
                   hipStream_t stream, std::string* err) {
   if (p.m == 0 || p.n == 0 || batch == 0) return 0;
-  if (!p.a || !p.b || !p.c || (use_cin && !p.cin)) {
+  if ((p.k != 0 && (!p.a || !p.b)) || !p.c || (use_cin && !p.cin)) {
     *err = "gemmcm: null tensor address";
     return -1;
   }
