@@ -216,6 +216,27 @@ def wl_quant(abi, m, k, steps, warmup, seed=1080):
                 name=f"fp8_quant rowwise bf16 -> e4m3fn M={m} K={k}")
 
 
+def wl_move(abi, kind, steps, warmup, rows=16384, cols=16384):
+    """Strided same-size copies of bfloat16 [rows, cols]: "transpose" (x.t().contiguous()) or "rows"
+    (x[::2].contiguous()): bytes read + bytes written per launch."""
+    src, item = abi.Buffer(rows * cols * 2), 2
+    abi.check(abi.lib().vkt_fill(src.address, 1, rows * cols * 2))
+    p = abi.StridedParams(a=src.address, ndim=2)
+    if kind == "transpose":
+        out = abi.Buffer(rows * cols * 2)
+        p.n, sizes, so, sa, name, work = rows * cols, (rows, cols), (1, rows), (cols, 1), "move_b2", 2 * rows * cols * item
+    else:
+        out = abi.Buffer(rows * cols)
+        p.n, sizes, so, sa, name, work = rows // 2 * cols, (cols, rows // 2), (1, cols), (1, 2 * cols), "move_b2", rows * cols * item
+    p.out = out.address
+    for d in range(4):
+        p.size[d], p.so[d], p.sa[d] = (sizes[d], so[d], sa[d]) if d < 2 else (1, 0, 0)
+    wall, ev = time_steps(abi, [Launch(abi, name, [abi.MOVE_COPY], p)], steps, warmup)
+    label = {"transpose": "x.t().contiguous()", "rows": "x[::2].contiguous()"}[kind]
+    return dict(kind="hbm", metric="strided copy GB/s (% of HBM peak)", work=work, wall_ms=wall, event_ms=ev, flops=0, inputs=None,
+                copies=1, name=f"{name} {label}, bfloat16 [{rows}, {cols}]")
+
+
 def wl_copy(abi, nbytes, steps, warmup):
     """A plain device-to-device copy of known size (calibrates the HBM traffic counters)."""
     src, dst = abi.Buffer(nbytes), abi.Buffer(nbytes)
@@ -249,6 +270,9 @@ WORKLOADS = {
     "f8_quant_rowwise_bf16_16384x16384": lambda abi, s, w: wl_quant(abi, 16384, 16384, max(s // 10, 5), max(w // 4, 3)),
     # the unquantised 16-bit product beside the path (not a BASELINE configuration), at the reference's own shape
     "mm_bf16_8192": lambda abi, s, w: wl_gemm16(abi, 8192, 8192, 8192, max(s // 10, 5), max(w // 4, 3)),
+    # strided device copies either side of the path (not BASELINE configurations)
+    "move_transpose_bf16_16384": lambda abi, s, w: wl_move(abi, "transpose", max(s // 10, 5), max(w // 4, 3)),
+    "move_rows_bf16_16384": lambda abi, s, w: wl_move(abi, "rows", max(s // 10, 5), max(w // 4, 3)),
     # config 4's launch on all-zero operands (not a BASELINE configuration: it shows how much of the
     # distance to the published peak is the data's, not the kernel's)
     "c4_fp8_8192_zero_operands": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 10, 5),

@@ -159,8 +159,37 @@ typedef struct GemmParams {
   int32_t cin_sm, cin_sn, cin_sb;
 } GemmParams;
 
+/* "move_b1" | "move_b2" | "move_b4" | "move_b8" | "move_b16", spec {OP}: data movement by
+ * element size, strided (the reference's block, launch.cpp:18-27, and kernel, shaders/move.slang).
+ *   OP VKT_MOVE_COPY  out[sum c_d so[d]] = a[sum c_d sa[d]] over 0 <= c_d < size[d]
+ *   OP VKT_MOVE_FILL  out[...] = the value whose bits are in alpha (and beta for 16 bytes)
+ * Dims innermost first, ndim <= 4, n = product of the sizes, strides in elements (0 =
+ * broadcast); b, sb, gamma and stride are not used (the library sizes its own grid).  The
+ * gather / scatter opcodes of the reference are not built.
+ * Also "cast_<src>_<dst>" with src, dst in f32 | f16 | bf16, spec {}: out = dst(a) over the same
+ * block (shaders/cast.slang: through float32, round to nearest even).  128 bytes. */
+typedef struct StridedParams {
+  uint64_t out, a, b;
+  uint64_t alpha, beta, gamma;
+  uint32_t n, ndim, stride, pad;
+  uint32_t size[4];
+  int32_t so[4], sa[4], sb[4];
+} StridedParams;
+
+/* "copy8_b1" ... "copy8_b16", spec {}: out = a, strided over up to 8 dims (the reference's
+ * block, launch.cpp:84-90, and kernel, shaders/copy8.slang).  128 bytes. */
+typedef struct Copy8Params {
+  uint64_t out, a;
+  uint32_t n, ndim, stride, pad;
+  uint32_t size[8];
+  int32_t so[8], sa[8];
+} Copy8Params;
+
+enum { VKT_MOVE_COPY = 0, VKT_MOVE_FILL = 1 }; /* shaders/opcodes.txt:206-207 */
+
 /* "cast_fp8", spec {}: dst[i] = convert(src[i]), i < n, where one side is VKT_E4M3 / VKT_E5M2
- * and the other VKT_F32 / VKT_F16 / VKT_BF16 (or the other float8 format): through float32,
+ * and the other VKT_F32 / VKT_F16 / VKT_BF16 (or the other float8 format; two non-float8 types are
+ * accepted too: the dense form of "cast_<src>_<dst>"): through float32,
  * bit for bit as the CPU converts (what the reference's copy between a float8 tensor and
  * a float tensor does with lookup tables, backend.cpp:534-586).  32 bytes. */
 typedef struct CastParams {

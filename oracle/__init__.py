@@ -202,6 +202,46 @@ def fp8_quant(x, dtype, fmt, scale=None):
     return q, scales
 
 
+def _layout(dst, src):
+    """(sizes, dst strides, src strides) in elements, innermost dim first, src broadcast to dst."""
+    size = np.array(dst.shape[::-1], np.int64)
+    so = np.array([x // dst.itemsize for x in dst.strides[::-1]], np.int64)
+    if src is None:
+        return size, so, np.zeros_like(so)
+    src = np.broadcast_to(src, dst.shape)
+    return size, so, np.array([x // src.itemsize for x in src.strides[::-1]], np.int64)
+
+
+def _base(a):
+    return ctypes.c_void_p(a.__array_interface__["data"][0])
+
+
+def move(dst, src=None, value=None):
+    """dst[...] = src (any strides either side, src broadcast to dst), or the fill value's bytes: the strided
+    move kernel's index arithmetic.  dst is a numpy array (written in place); non-negative strides."""
+    size, so, sa = _layout(dst, src)
+    if dst.size == 0:
+        return dst
+    if src is not None:
+        src = np.broadcast_to(src, dst.shape)
+        assert src.itemsize == dst.itemsize
+        lib().orc_move(_base(dst), _base(src), I64(dst.itemsize), I64(dst.size), len(size), _p(size), _p(so), _p(sa), 0, None)
+    else:
+        v = np.frombuffer(np.asarray(value).tobytes(), np.uint8).copy()
+        assert v.size == dst.itemsize
+        lib().orc_move(_base(dst), None, I64(dst.itemsize), I64(dst.size), len(size), _p(size), _p(so), _p(sa), 1, _p(v))
+    return dst
+
+
+def cast_strided(dst, dst_dtype, src, src_dtype):
+    """dst[...] = dst_dtype(src) over strided views (uint16 views for the 16-bit types, float32 else)."""
+    size, so, sa = _layout(dst, src)
+    if dst.size:
+        src = np.broadcast_to(src, dst.shape)
+        lib().orc_cast_strided(_base(dst), dst_dtype, _base(src), src_dtype, I64(dst.size), len(size), _p(size), _p(so), _p(sa))
+    return dst
+
+
 def _strided(a):
     """(base pointer, element strides) of a numpy array viewed as [B, R, C]."""
     a3 = a if a.ndim == 3 else a[None]

@@ -30,6 +30,9 @@
  *   orc_cast            pinned: torch CPU Tensor.to() between float32 / float16 / bfloat16 and
  *                               both float8 formats (the reference's own vectors,
  *                               tests/python/test_fallback_ops.py:469-485, plus all 256 codes)
+ *   orc_move            pinned: numpy strided views (as_strided) and torch CPU copy_ / contiguous() /
+ *                               fill_ on the same layouts: transposes, slices, broadcasts, up to 8 dims
+ *   orc_cast_strided    pinned: torch CPU Tensor.to() over the same strided views
  *   orc_fp8_quant_rows  pinned: the same steps composed from torch CPU operators (amax, clamp,
  *                               true_divide, mul, clamp, to(float8)), rows whose maximum is
  *                               fmax exactly (the scale is 1: a plain cast), power-of-two
@@ -360,6 +363,40 @@ void orc_scaled_mm(const uint8_t* a, int fmt_a, const uint8_t* bt, int fmt_b, co
  * built from c10's conversions) and as c10 itself converts. */
 void orc_cast(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t n) {
   for (int64_t i = 0; i < n; i++) store_from_f32(dst, i, dst_dtype, load_as_f32(src, i, src_dtype));
+}
+
+/* Strided data movement by element size (crates/vkcore/shaders/move.slang:37-52 with the index
+ * arithmetic of _strided.slang:68-86, copy8.slang:36-66): linear index i is split into per-dim
+ * coordinates, innermost dim first; out[sum c so] = a[sum c sa] (fill = 0) or the fill value.
+ * Strides in elements of `item` bytes. */
+void orc_move(uint8_t* out, const uint8_t* a, int64_t item, int64_t n, int ndim, const int64_t* size, const int64_t* so,
+              const int64_t* sa, int fill, const uint8_t* value) {
+  for (int64_t i = 0; i < n; i++) {
+    int64_t rem = i, o = 0, s = 0;
+    for (int d = 0; d < ndim; d++) {
+      const int64_t c = rem % size[d];
+      rem /= size[d];
+      o += c * so[d];
+      if (!fill) s += c * sa[d];
+    }
+    memcpy(out + o * item, fill ? value : a + s * item, (size_t)item);
+  }
+}
+
+/* out = dst_dtype(a) over the same index space (crates/vkcore/shaders/cast.slang: through
+ * float32, round to nearest even); strides in elements of each side. */
+void orc_cast_strided(void* out, int dst_dtype, const void* a, int src_dtype, int64_t n, int ndim, const int64_t* size,
+                      const int64_t* so, const int64_t* sa) {
+  for (int64_t i = 0; i < n; i++) {
+    int64_t rem = i, o = 0, s = 0;
+    for (int d = 0; d < ndim; d++) {
+      const int64_t c = rem % size[d];
+      rem /= size[d];
+      o += c * so[d];
+      s += c * sa[d];
+    }
+    store_from_f32(out, o, dst_dtype, load_as_f32(a, s, src_dtype));
+  }
 }
 
 /* The float8 producer in front of _scaled_mm (no counterpart in the reference; SURVEY lists it

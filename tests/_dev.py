@@ -192,3 +192,61 @@ def gemm16(a, b, dtype, cin=None, alpha=1.0, beta=0.0, variant=0):
         abi.dispatch("gemmcm_" + abi.SUFFIX[dtype], [int(use_cin), 0, 0, variant], p, (1, 1, B))
     res = out.to_numpy(np.uint16, (B, M, N))
     return res if np.asarray(a).ndim == 3 else res[0]
+
+
+def _span(arr):
+    """(lowest byte offset, byte length) of the memory a strided numpy view touches, relative to element [0,..,0]."""
+    lo = sum(min(0, (n - 1) * st) for n, st in zip(arr.shape, arr.strides))
+    hi = sum(max(0, (n - 1) * st) for n, st in zip(arr.shape, arr.strides)) + arr.itemsize
+    return lo, hi - lo
+
+
+def _upload_span(arr):
+    lo, length = _span(arr)
+    raw = (ctypes.c_uint8 * length).from_address(arr.__array_interface__["data"][0] + lo)
+    buf = abi.Buffer(length)
+    abi.check(abi.lib().vkt_copy_to_device(buf.address, ctypes.addressof(raw), length))
+    return buf, buf.address - lo, raw
+
+
+def _dims(dst, src):
+    size = list(dst.shape[::-1])
+    so = [st // dst.itemsize for st in dst.strides[::-1]]
+    sa = [st // src.itemsize for st in np.broadcast_to(src, dst.shape).strides[::-1]] if src is not None else [0] * len(size)
+    return size, so, sa
+
+
+def move(dst, src=None, value=None, variant=0, cast=None):
+    """dst[...] = src (broadcast) or the fill value, on the device, through "move_b<S>" (up to 4 dims) or
+    "copy8_b<S>" (5 to 8); cast=(src_label, dst_label) runs "cast_<src>_<dst>" instead.  dst's memory is
+    uploaded first and read back, so untouched elements show as unchanged."""
+    if dst.size == 0:
+        return dst
+    size, so, sa = _dims(dst, src)
+    dbuf, daddr, draw = _upload_span(dst)
+    if src is not None:
+        src = np.broadcast_to(src, dst.shape)
+        sbuf, saddr, _ = _upload_span(src)
+    label = "b%d" % dst.itemsize
+    if len(size) <= 4:
+        p = abi.StridedParams(out=daddr, a=saddr if src is not None else 0, n=dst.size, ndim=len(size))
+        for d in range(len(size)):
+            p.size[d], p.so[d], p.sa[d] = size[d], so[d], sa[d]
+        for d in range(len(size), 4):
+            p.size[d] = 1
+        if cast is not None:
+            abi.dispatch("cast_%s_%s" % cast, [], p)
+        elif src is not None:
+            abi.dispatch("move_" + label, [abi.MOVE_COPY, 0, variant], p)
+        else:
+            bits = np.frombuffer(np.asarray(value).tobytes().ljust(16, b"\0"), np.uint64)
+            p.alpha, p.beta = int(bits[0]), int(bits[1])
+            abi.dispatch("move_" + label, [abi.MOVE_FILL, 0, variant], p)
+    else:
+        assert src is not None and cast is None and len(size) <= 8
+        p = abi.Copy8Params(out=daddr, a=saddr, n=dst.size, ndim=len(size))
+        for d in range(8):
+            p.size[d], p.so[d], p.sa[d] = (size[d], so[d], sa[d]) if d < len(size) else (1, 0, 0)
+        abi.dispatch("copy8_" + label, [variant], p)
+    abi.check(abi.lib().vkt_copy_to_host(ctypes.addressof(draw), dbuf.address, len(draw)))
+    return dst

@@ -40,7 +40,7 @@ def test_device_round_trip(tv):
     d = x.to("vk")
     assert d.device.type == "vk" and torch.equal(d.cpu(), x)
     assert torch.equal(d[::2].cpu(), x[::2]) and torch.equal(d.t().contiguous().cpu(), x.t().contiguous())
-    assert torch.equal(d.to(torch.bfloat16).cpu(), x.bfloat16())  # (a conversion staged through the host)
+    assert torch.equal(d.to(torch.bfloat16).cpu(), x.bfloat16())  # (converted on the device: cast_f32_bf16)
     for dt in (torch.int8, torch.uint8, torch.float16, torch.bfloat16, torch.float8_e4m3fn, torch.float8_e5m2):
         y = (x * 10).to(dt)
         assert torch.equal(y.to("vk").cpu().view(torch.uint8), y.view(torch.uint8))
@@ -292,3 +292,41 @@ def test_16bit_matrix_products(tv, dtype):
         torch.mm(a[0].to("vk"), b[0].to("vk"))
     with pytest.raises(RuntimeError, match="same dtype"):
         torch.mm(a[0].to("vk"), b[0].t().float().to("vk"))
+
+
+def test_strided_copies_and_fills_on_the_device(tv):
+    """contiguous(), copy_ between strided / broadcast views, float conversions and fill_ / zero_ run as
+    device kernels (the dispatch count moves, nothing falls back), bit for bit as the CPU."""
+    x = torch.randn(6, 40, 66, generator=gen(21))
+    d = x.to("vk")
+    with on_gpu(tv):
+        n0 = tv.dispatch_count()
+        t = d.transpose(1, 2).contiguous()
+        p = d.permute(2, 0, 1)[:, ::2].contiguous()
+        h = d.to(torch.float16)
+        b = d.transpose(0, 2).to(torch.bfloat16)
+        back = b.to(torch.float32)
+        z = torch.empty(5, 7, device="vk").fill_(2.5)
+        z[:, ::2].zero_()
+        w = torch.empty(4, 66, device="vk")
+        w.copy_(d[0, 3])  # a broadcast row
+        e = torch.empty(3, 4, dtype=torch.int64, device="vk").fill_(-7)
+        assert tv.dispatch_count() - n0 == 9  # one kernel each
+    assert torch.equal(t.cpu(), x.transpose(1, 2).contiguous()) and t.is_contiguous()
+    assert torch.equal(p.cpu(), x.permute(2, 0, 1)[:, ::2].contiguous())
+    assert torch.equal(h.cpu(), x.half()) and torch.equal(b.cpu(), x.transpose(0, 2).bfloat16())
+    assert torch.equal(back.cpu(), x.transpose(0, 2).bfloat16().float())
+    want = torch.full((5, 7), 2.5)
+    want[:, ::2] = 0
+    assert torch.equal(z.cpu(), want) and torch.equal(w.cpu(), x[0, 3].expand(4, 66)) and (e.cpu() == -7).all()
+    # host <-> device with strides on the device side: staged densely, scattered / gathered by the kernels
+    y = torch.zeros(8, 10).to("vk")
+    y[::2, 1:9].copy_(x[0, :4, :8])
+    ref = torch.zeros(8, 10)
+    ref[::2, 1:9] = x[0, :4, :8]
+    assert torch.equal(y.cpu(), ref) and torch.equal(y[::2, 1:9].cpu(), x[0, :4, :8])
+    # what the quantised ops take: a non-contiguous activation and int8 weight made contiguous on the device
+    wq = torch.randint(-128, 128, (48, 64), dtype=torch.int8, generator=gen(22))
+    with on_gpu(tv):
+        wt = wq.to("vk").t().contiguous().t().contiguous()
+    assert torch.equal(wt.cpu(), wq)

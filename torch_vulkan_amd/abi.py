@@ -68,6 +68,20 @@ class GemmParams(ctypes.Structure):
                                                         "cin_sm", "cin_sn", "cin_sb")]
 
 
+class StridedParams(ctypes.Structure):
+    _fields_ = [("out", u64), ("a", u64), ("b", u64), ("alpha", u64), ("beta", u64), ("gamma", u64),
+                ("n", u32), ("ndim", u32), ("stride", u32), ("pad", u32), ("size", u32 * 4),
+                ("so", i32 * 4), ("sa", i32 * 4), ("sb", i32 * 4)]
+
+
+class Copy8Params(ctypes.Structure):
+    _fields_ = [("out", u64), ("a", u64), ("n", u32), ("ndim", u32), ("stride", u32), ("pad", u32),
+                ("size", u32 * 8), ("so", i32 * 8), ("sa", i32 * 8)]
+
+
+MOVE_COPY, MOVE_FILL = 0, 1
+
+
 class CastParams(ctypes.Structure):
     _fields_ = [("src", u64), ("dst", u64), ("n", u64), ("src_dtype", u32), ("dst_dtype", u32)]
 
@@ -79,6 +93,7 @@ class F8QuantParams(ctypes.Structure):
 
 assert ctypes.sizeof(Q8Params) == 56 and ctypes.sizeof(Q4Params) == 64 and ctypes.sizeof(F8Params) == 104
 assert ctypes.sizeof(CastParams) == 32 and ctypes.sizeof(F8QuantParams) == 48 and ctypes.sizeof(GemmParams) == 112
+assert ctypes.sizeof(StridedParams) == 128 and ctypes.sizeof(Copy8Params) == 128
 
 # every symbol include/vkt.h declares
 SYMBOLS = ["vkt_last_error", "vkt_alloc", "vkt_free", "vkt_synchronize", "vkt_empty_cache", "vkt_memory_stats",

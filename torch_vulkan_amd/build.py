@@ -30,6 +30,7 @@ SOURCES = {
     "kernels/gemm16.hip": [],
     # (single float32 operations in the float8 producer, as specified)
     "kernels/cast.hip": ["-ffp-contract=off"],
+    "kernels/move.hip": [],
     "kernels/util.hip": [],
 }
 

@@ -214,6 +214,27 @@ int dispatch_named(Runtime& rt, const char* name, const uint32_t* spec, size_t n
     if (!read_push(push, npush, &p, name, err)) return -1;
     return launch_gemm16(p, dt, spec_at(0), gz, spec_at(3), rt.machine, rt.stream, err);
   }
+  if (!std::strncmp(name, "move_", 5)) {
+    StridedParams p;
+    if (!read_push(push, npush, &p, name, err)) return -1;
+    return launch_move(p, name + 5, spec_at(0), spec_at(2), rt.machine, rt.stream, err);
+  }
+  if (!std::strncmp(name, "copy8_", 6)) {
+    Copy8Params p;
+    if (!read_push(push, npush, &p, name, err)) return -1;
+    return launch_copy8(p, name + 6, spec_at(0), rt.machine, rt.stream, err);
+  }
+  if (!std::strncmp(name, "cast_", 5) && std::strcmp(name, "cast_fp8")) {
+    // "cast_<src>_<dst>"
+    const char* second = std::strchr(name + 5, '_');
+    if (!second) goto unknown;
+    const std::string from(name + 5, second);
+    const int sdt = dtype_of_suffix(from.c_str()), ddt = dtype_of_suffix(second + 1);
+    StridedParams p;
+    if (sdt < 0 || ddt < 0 || sdt == ddt) goto unknown;
+    if (!read_push(push, npush, &p, name, err)) return -1;
+    return launch_cast_strided(p, sdt, ddt, rt.machine, rt.stream, err);
+  }
   if (!std::strcmp(name, "cast_fp8")) {
     CastParams p;
     if (!read_push(push, npush, &p, name, err)) return -1;

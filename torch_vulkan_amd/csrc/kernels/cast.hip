@@ -12,8 +12,8 @@
 //               every step a single float32 operation, fmax = 448 (e4m3fn) or 57344 (e5m2).
 //               The reference has no such kernel (its float8 tensors come from casts alone).
 // Both read and write each byte once: 16 elements per thread, 16-byte accesses.
-#include "common.h"
 #include "kernels.h"
+#include "strided.h"
 
 namespace vkt {
 namespace {
@@ -87,6 +87,18 @@ __global__ __launch_bounds__(256) void cast_kernel(CastParams p, uint32_t vector
     if (i0 < (p.n & 15)) store1_any<DST>(p.dst, body * 16 + i0, load1_any<SRC>(p.src, body * 16 + i0));
   } else {
     for (uint64_t j = i0; j < p.n; j += stride) store1_any<DST>(p.dst, j, load1_any<SRC>(p.src, j));
+  }
+}
+
+// out = DST(a) over a strided index space, one element per thread (the reference's
+// shaders/cast.slang); dense layouts take cast_kernel instead.
+template <uint32_t SRC, uint32_t DST>
+__global__ __launch_bounds__(256) void cast_strided(MovePlan p) {
+  const uint64_t stride = uint64_t(gridDim.x) * 256;
+  for (uint64_t i = uint64_t(blockIdx.x) * 256 + threadIdx.x; i < p.n; i += stride) {
+    int64_t o, a;
+    plan_offsets(p, uint32_t(i), &o, &a);
+    store1_any<DST>(p.out, uint64_t(o), load1_any<SRC>(p.a, uint64_t(a)));
   }
 }
 
@@ -185,8 +197,8 @@ void launch_quant(const F8QuantParams& p, uint32_t rowwise, hipStream_t stream) 
 
 int launch_cast_fp8(const CastParams& p, const Machine& mc, hipStream_t stream, std::string* err) {
   if (p.n == 0) return 0;
-  if (p.src_dtype > VKT_E5M2 || p.dst_dtype > VKT_E5M2 || (!is_fp8_host(p.src_dtype) && !is_fp8_host(p.dst_dtype))) {
-    *err = "cast_fp8: one side must be e4m3fn or e5m2, the other float32, float16, bfloat16 or float8";
+  if (p.src_dtype > VKT_E5M2 || p.dst_dtype > VKT_E5M2) {
+    *err = "cast_fp8: the types are float32, float16, bfloat16, e4m3fn and e5m2";
     return -1;
   }
   if (!p.src || !p.dst) {
@@ -210,6 +222,35 @@ int launch_cast_fp8(const CastParams& p, const Machine& mc, hipStream_t stream, 
     return -1;
   }
   return rc;
+}
+
+int launch_cast_strided(const StridedParams& s, int src_dtype, int dst_dtype, const Machine& mc, hipStream_t stream,
+                        std::string* err) {
+  if (s.n == 0) return 0;
+  const uint32_t si = item_size(uint32_t(src_dtype)), di = item_size(uint32_t(dst_dtype));
+  if (!s.out || !s.a || s.out % di != 0 || s.a % si != 0) {
+    *err = "cast: null or misaligned tensor address";
+    return -1;
+  }
+  MovePlan p;
+  if (!plan_from(s.out, s.a, s.n, s.ndim, 4, s.size, s.so, s.sa, di, "cast", &p, err)) return -1;
+  if (p.ndim == 0 || (p.ndim == 1 && p.so[0] == 1 && p.sa[0] == 1)) {  // dense: 16 elements per thread
+    CastParams c{};
+    c.src = s.a, c.dst = s.out, c.n = s.n, c.src_dtype = uint32_t(src_dtype), c.dst_dtype = uint32_t(dst_dtype);
+    return launch_cast_fp8(c, mc, stream, err);
+  }
+  const uint64_t want = (p.n + 255) / 256, cap = uint64_t(mc.compute_units) * 64;
+  const dim3 grid(uint32_t(want < cap ? want : cap));
+#define VKT_CAST_CASE(S, D) \
+  if (src_dtype == S && dst_dtype == D) hipLaunchKernelGGL((cast_strided<S, D>), grid, dim3(256), 0, stream, p);
+  VKT_CAST_CASE(VKT_F32, VKT_F16) VKT_CAST_CASE(VKT_F32, VKT_BF16) VKT_CAST_CASE(VKT_F16, VKT_F32)
+  VKT_CAST_CASE(VKT_F16, VKT_BF16) VKT_CAST_CASE(VKT_BF16, VKT_F32) VKT_CAST_CASE(VKT_BF16, VKT_F16)
+#undef VKT_CAST_CASE
+  if (hipGetLastError() != hipSuccess) {
+    *err = "cast: kernel launch failed";
+    return -1;
+  }
+  return 0;
 }
 
 int launch_fp8_quant(const F8QuantParams& p, uint32_t rowwise, const Machine&, hipStream_t stream, std::string* err) {

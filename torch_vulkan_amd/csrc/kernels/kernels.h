@@ -32,6 +32,14 @@ int launch_fp8mm(const F8Params& p, uint32_t variant, const Machine& mc, hipStre
 int launch_gemm16(const GemmParams& p, int dtype, uint32_t use_cin, uint32_t batch, uint32_t variant, const Machine& mc,
                   hipStream_t stream, std::string* err);
 int launch_cast_fp8(const CastParams& p, const Machine& mc, hipStream_t stream, std::string* err);
+int launch_cast_strided(const StridedParams& s, int src_dtype, int dst_dtype, const Machine& mc, hipStream_t stream,
+                        std::string* err);
+// "move_<size_label>" (op: VKT_MOVE_COPY | VKT_MOVE_FILL) and "copy8_<size_label>"; variant 0 plans the
+// form from the strides, 1 moves element by element as given, 2 widens units but never tiles.
+int launch_move(const StridedParams& s, const char* size_label, uint32_t op, uint32_t variant, const Machine& mc,
+                hipStream_t stream, std::string* err);
+int launch_copy8(const Copy8Params& c, const char* size_label, uint32_t variant, const Machine& mc, hipStream_t stream,
+                 std::string* err);
 int launch_fp8_quant(const F8QuantParams& p, uint32_t rowwise, const Machine& mc, hipStream_t stream, std::string* err);
 int launch_fill(uint64_t dst, uint8_t value, uint64_t nbytes, hipStream_t stream, std::string* err);
 int launch_copy(uint64_t dst, uint64_t src, uint64_t nbytes, hipStream_t stream, std::string* err);

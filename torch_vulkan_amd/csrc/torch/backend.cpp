@@ -8,8 +8,10 @@
 //                        t.data_ptr() and the reference's address map (:170-192) is gone
 //   device guard, hooks  :286-369 (one device, one stream)
 //   empty / resize / views / set_   :391-465
-//   _copy_from, _local_scalar_dense :765-805; host <-> device through vkt_copy_*; anything
-//                        that is not a same-dtype contiguous move is staged through the CPU
+//   _copy_from, _local_scalar_dense :765-805; host <-> device through vkt_copy_*; strided,
+//                        broadcasting and float32 / float16 / bfloat16-converting copies and
+//                        fills run on the device ("move_b<S>", "copy8_b<S>", "cast_<s>_<d>":
+//                        :633-717, :806-826); other conversions are staged through the CPU
 //   boxed CPU fallback   :1696-1740, counted per op (fallback_counts), an error under
 //                        TORCH_VK_STRICT
 // The aten kernels of the path live in quant.cpp.
@@ -26,6 +28,7 @@
 #include <torch/library.h>
 
 #include <cstdlib>
+#include <cstring>
 #include <map>
 #include <mutex>
 
@@ -191,6 +194,129 @@ at::Tensor host_mirror(const at::Tensor& t, bool download) {
 
 bool plain(const at::Tensor& t) { return t.is_non_overlapping_and_dense(); }
 
+// ---- strided moves on the device (reference launch.cpp:55-83 launch<K>, :108-150 copy_many_dims;
+// strided.h:35-121 merge_dims / for_each_dispatch)
+
+struct MergedDims {
+  std::vector<int64_t> size, so, sa;  // innermost first
+};
+
+// dst's index space with src broadcast to it: dims of size 1 dropped, dims that are contiguous on
+// both sides merged.
+MergedDims merged_dims(const at::Tensor& dst, const at::Tensor* src) {
+  MergedDims m;
+  const int64_t pad = src ? dst.dim() - src->dim() : 0;
+  for (int64_t i = dst.dim() - 1; i >= 0; --i) {
+    const int64_t n = dst.size(i);
+    if (n == 1) continue;
+    const int64_t o = dst.stride(i);
+    const int64_t a = (src && i >= pad && src->size(i - pad) != 1) ? src->stride(i - pad) : 0;
+    if (!m.size.empty() && o == m.so.back() * m.size.back() && a == m.sa.back() * m.size.back()) {
+      m.size.back() *= n;
+      continue;
+    }
+    m.size.push_back(n), m.so.push_back(o), m.sa.push_back(a);
+  }
+  return m;
+}
+
+// Runs `emit(count, ndim, out offset, a offset)` over the innermost `inner` dims for every index of the rest.
+template <class F>
+bool for_each_launch(const MergedDims& m, size_t inner_max, F&& emit) {
+  const size_t inner = std::min(m.size.size(), inner_max);
+  int64_t count = 1, span_o = 0, span_a = 0;
+  for (size_t d = 0; d < inner; ++d) {
+    count *= m.size[d];
+    span_o += (m.size[d] - 1) * m.so[d], span_a += (m.size[d] - 1) * m.sa[d];
+  }
+  if (count >= (int64_t(1) << 32) || span_o >= (int64_t(1) << 31) || span_a >= (int64_t(1) << 31)) return false;
+  for (size_t d = 0; d < inner; ++d)
+    if (m.so[d] < 0 || m.sa[d] < 0) return false;
+  std::vector<int64_t> index(m.size.size() - inner, 0);
+  while (true) {
+    int64_t oo = 0, ao = 0;
+    for (size_t j = 0; j < index.size(); ++j) oo += index[j] * m.so[inner + j], ao += index[j] * m.sa[inner + j];
+    emit(count, inner, oo, ao);
+    size_t j = 0;
+    for (; j < index.size(); ++j) {
+      if (++index[j] < m.size[inner + j]) break;
+      index[j] = 0;
+    }
+    if (j == index.size()) return true;
+  }
+}
+
+const char* size_label(int64_t item) {
+  switch (item) {
+    case 1: return "b1";
+    case 2: return "b2";
+    case 4: return "b4";
+    case 8: return "b8";
+    case 16: return "b16";
+    default: return nullptr;
+  }
+}
+
+const char* float_label(at::ScalarType t) {
+  return t == at::kFloat ? "f32" : t == at::kHalf ? "f16" : t == at::kBFloat16 ? "bf16" : nullptr;
+}
+
+// dst (vk) <- src (vk) with strides, broadcasting and float32 / float16 / bfloat16 conversion, on
+// the device (reference backend.cpp:633-690 copy_vk_to_vk).  False where no kernel covers it.
+bool copy_on_device(const at::Tensor& dst, const at::Tensor& src) {
+  if (src.is_conj() || src.is_neg() || dst.is_conj() || dst.is_neg()) return false;
+  const bool same = src.scalar_type() == dst.scalar_type();
+  const char* label = size_label(dst.element_size());
+  std::string kernel;
+  if (same && label) kernel = std::string("move_") + label;
+  else if (!same && float_label(src.scalar_type()) && float_label(dst.scalar_type()))
+    kernel = std::string("cast_") + float_label(src.scalar_type()) + "_" + float_label(dst.scalar_type());
+  else return false;
+  const MergedDims m = merged_dims(dst, &src);
+  const uint64_t out = reinterpret_cast<uint64_t>(dst.mutable_data_ptr()), a = reinterpret_cast<uint64_t>(src.const_data_ptr());
+  const int64_t oi = dst.element_size(), ai = src.element_size();
+  if (same && m.size.size() > 4) {  // up to 8 dims in one launch (reference copy_many_dims)
+    const std::string k8 = std::string("copy8_") + label;
+    return for_each_launch(m, 8, [&](int64_t count, size_t ndim, int64_t oo, int64_t ao) {
+      Copy8Params p{};
+      p.out = out + uint64_t(oo * oi), p.a = a + uint64_t(ao * ai), p.n = uint32_t(count), p.ndim = uint32_t(ndim);
+      for (size_t d = 0; d < 8; ++d) {
+        p.size[d] = d < ndim ? uint32_t(m.size[d]) : 1u;
+        p.so[d] = d < ndim ? int32_t(m.so[d]) : 0, p.sa[d] = d < ndim ? int32_t(m.sa[d]) : 0;
+      }
+      dispatch(k8, {}, p, 1);
+    });
+  }
+  return for_each_launch(m, 4, [&](int64_t count, size_t ndim, int64_t oo, int64_t ao) {
+    StridedParams p{};
+    p.out = out + uint64_t(oo * oi), p.a = a + uint64_t(ao * ai), p.n = uint32_t(count), p.ndim = uint32_t(ndim);
+    for (size_t d = 0; d < 4; ++d) {
+      p.size[d] = d < ndim ? uint32_t(m.size[d]) : 1u;
+      p.so[d] = d < ndim ? int32_t(m.so[d]) : 0, p.sa[d] = d < ndim ? int32_t(m.sa[d]) : 0;
+    }
+    dispatch(kernel, {VKT_MOVE_COPY}, p, 1);
+  });
+}
+
+// self[...] = value on the device (reference backend.cpp:806-816 fill_scalar).
+bool fill_on_device(const at::Tensor& self, const at::Scalar& value) {
+  const char* label = size_label(self.element_size());
+  if (!label || self.is_conj() || self.is_neg()) return false;
+  if (self.numel() == 0) return true;
+  at::Tensor v = at::scalar_tensor(value, at::TensorOptions().dtype(self.scalar_type()));
+  uint64_t bits[2] = {0, 0};
+  std::memcpy(bits, v.const_data_ptr(), size_t(v.element_size()));
+  const MergedDims m = merged_dims(self, nullptr);
+  const uint64_t out = reinterpret_cast<uint64_t>(self.mutable_data_ptr());
+  const int64_t item = self.element_size();
+  return for_each_launch(m, 4, [&](int64_t count, size_t ndim, int64_t oo, int64_t) {
+    StridedParams p{};
+    p.out = out + uint64_t(oo * item), p.alpha = bits[0], p.beta = bits[1], p.n = uint32_t(count), p.ndim = uint32_t(ndim);
+    for (size_t d = 0; d < 4; ++d) p.size[d] = d < ndim ? uint32_t(m.size[d]) : 1u, p.so[d] = d < ndim ? int32_t(m.so[d]) : 0;
+    dispatch(std::string("move_") + label, {VKT_MOVE_FILL}, p, 1);
+  });
+}
+
 // dst <- src where at least one is on vk (reference backend.cpp:765-790).
 at::Tensor copy_from(const at::Tensor& src, const at::Tensor& dst, bool non_blocking) {
   TORCH_CHECK(src.sizes() == dst.sizes() || src.numel() == 1 || at::is_expandable_to(src.sizes(), dst.sizes()),
@@ -237,7 +363,27 @@ at::Tensor copy_from(const at::Tensor& src, const at::Tensor& dst, bool non_bloc
       return dst;
     }
   }
-  // anything else (dtype conversion, strides, broadcast): through host mirrors
+  // strides, broadcasting, float conversions: on the device (host <-> device through a dense staging tensor,
+  // reference backend.cpp:697-717 copy_cpu_to_vk)
+  if (is_vk(src) && is_vk(dst) && copy_on_device(dst, src)) return dst;
+  if (is_vk(dst) && !is_vk(src) && size_label(dst.element_size()) && !dst.is_conj() && !dst.is_neg()) {
+    at::Tensor host = src.to(dst.scalar_type()).expand(dst.sizes()).contiguous();
+    at::Tensor staging = at::empty(dst.sizes(), dst.options());
+    check(vkt_copy_to_device(reinterpret_cast<uint64_t>(staging.mutable_data_ptr()), host.const_data_ptr(), nbytes));
+    if (copy_on_device(dst, staging)) return dst;
+  }
+  if (is_vk(src) && !is_vk(dst) && size_label(src.element_size()) && !src.is_conj() && !src.is_neg() &&
+      !plain(src) && src.numel() > 0) {
+    at::Tensor staging = at::empty(src.sizes(), src.options());
+    if (copy_on_device(staging, src)) {
+      at::Tensor host = at::empty(src.sizes(), src.options().device(at::kCPU));
+      check(vkt_copy_to_host(host.mutable_data_ptr(), reinterpret_cast<uint64_t>(staging.const_data_ptr()),
+                             uint64_t(src.numel()) * src.element_size()));
+      dst.copy_(host);
+      return dst;
+    }
+  }
+  // anything else: through host mirrors
   at::Tensor s = is_vk(src) ? host_mirror(src, true) : src;
   if (!is_vk(dst)) {
     dst.copy_(s);
@@ -261,6 +407,23 @@ at::Scalar local_scalar_dense(const at::Tensor& self) {
   TORCH_CHECK(self.numel() == 1, "a Tensor with ", self.numel(), " elements cannot be converted to Scalar");
   return host_mirror(self, true).item();
 }
+
+at::Tensor& fill_scalar(at::Tensor& self, const at::Scalar& value) {
+  if (!fill_on_device(self, value)) {
+    record_fallback("aten::fill_.Scalar");
+    at::Tensor host = at::full(self.sizes(), value, self.options().device(at::kCPU));
+    copy_from(host, self, false);
+  }
+  return self;
+}
+
+at::Tensor& fill_tensor(at::Tensor& self, const at::Tensor& value) {
+  TORCH_CHECK(value.dim() == 0, "fill_ only supports 0-dimension value tensor but got tensor with ", value.dim(),
+              " dimensions.");
+  return fill_scalar(self, value.item());
+}
+
+at::Tensor& zero_(at::Tensor& self) { return fill_scalar(self, 0); }
 
 // ------------------------------------------------------------------ CPU fallback
 
@@ -291,6 +454,9 @@ TORCH_LIBRARY_IMPL(aten, PrivateUse1, m) {
   m.impl("_copy_from", &copy_from);
   m.impl("_copy_from_and_resize", &copy_from_and_resize);
   m.impl("_local_scalar_dense", &local_scalar_dense);
+  m.impl("fill_.Scalar", &fill_scalar);
+  m.impl("fill_.Tensor", &fill_tensor);
+  m.impl("zero_", &zero_);
 }
 
 TORCH_LIBRARY_IMPL(_, PrivateUse1, m) { m.fallback(torch::CppFunction::makeFromBoxedFunction<&vk::boxed_fallback>()); }
