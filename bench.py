@@ -175,8 +175,9 @@ def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False)
                      + (" (all-zero operands)" if zero_operands else ""))
 
 
-def wl_gemm16(abi, m, k, n, steps, warmup, seed=1090):
-    """bfloat16 mm in the Linear layout (x [m,k] @ w[n,k]^T -> [m,n]): the unquantised product next to the path."""
+def wl_gemm16(abi, m, k, n, steps, warmup, seed=1090, layout="nt"):
+    """bfloat16 mm, x [m,k] @ w -> [m,n]: the unquantised product next to the path.  layout "nt": w stored
+    [n,k] (x @ w.T, the Linear layout); "nn": w stored [k,n] (x @ w); "tn": x stored [k,m] as well (x.t() @ w)."""
     import torch
     g = torch.Generator().manual_seed(seed)
     a, w = torch.randn(m, k, generator=g).bfloat16(), torch.randn(n, k, generator=g).bfloat16()
@@ -184,9 +185,13 @@ def wl_gemm16(abi, m, k, n, steps, warmup, seed=1090):
     out = abi.Buffer(m * n * 2)
     p = abi.GemmParams(a=da.address, b=dw.address, c=out.address, m=m, n=n, k=k, a_sm=k, a_sk=1, b_sk=1, b_sn=k, c_sm=n,
                        c_sn=1, alpha=int(np.float32(1).view(np.uint32)))
+    if layout in ("nn", "tn"):  # (the same bytes read as the other layout: the values do not matter to the timing)
+        p.b_sk, p.b_sn = n, 1
+    if layout == "tn":
+        p.a_sm, p.a_sk = 1, m
     wall, ev = time_steps(abi, [Launch(abi, "gemmcm_bf16", [0], p)], steps, warmup)
     return dict(kind="mfma", peak=BF16_PEAK_TFLOPS, metric="bf16 mm TFLOP/s (% of MFMA peak)", work=2 * m * n * k, wall_ms=wall, event_ms=ev,
-                bytes=2 * (m * k + n * k + m * n), inputs=None, copies=1, name=f"mm bf16 M={m} K={k} N={n} (Linear layout)")
+                bytes=2 * (m * k + n * k + m * n), inputs=None, copies=1, name=f"mm bf16 M={m} K={k} N={n} ({layout}: " + {"nt": "x @ w.T, the Linear layout", "nn": "x @ w", "tn": "x.T @ w"}[layout] + ")")
 
 
 def wl_cast(abi, n, steps, warmup, seed=1070):
@@ -270,6 +275,8 @@ WORKLOADS = {
     "f8_quant_rowwise_bf16_16384x16384": lambda abi, s, w: wl_quant(abi, 16384, 16384, max(s // 10, 5), max(w // 4, 3)),
     # the unquantised 16-bit product beside the path (not a BASELINE configuration), at the reference's own shape
     "mm_bf16_8192": lambda abi, s, w: wl_gemm16(abi, 8192, 8192, 8192, max(s // 10, 5), max(w // 4, 3)),
+    "mm_bf16_8192_nn": lambda abi, s, w: wl_gemm16(abi, 8192, 8192, 8192, max(s // 10, 5), max(w // 4, 3), layout="nn"),
+    "mm_bf16_8192_tn": lambda abi, s, w: wl_gemm16(abi, 8192, 8192, 8192, max(s // 10, 5), max(w // 4, 3), layout="tn"),
     # strided device copies either side of the path (not BASELINE configurations)
     "move_transpose_bf16_16384": lambda abi, s, w: wl_move(abi, "transpose", max(s // 10, 5), max(w // 4, 3)),
     "move_rows_bf16_16384": lambda abi, s, w: wl_move(abi, "rows", max(s // 10, 5), max(w // 4, 3)),

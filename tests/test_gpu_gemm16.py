@@ -55,6 +55,27 @@ def test_gemm16_tile_variants(dtype, variant, m, k, n):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("variant", [0, 3, 4])
+@pytest.mark.parametrize("m,k,n", [(128, 64, 136), (264, 192, 520), (1032, 128, 1024), (8, 64, 8)])
+def test_gemm16_k_major_operands(dtype, variant, m, k, n):
+    """Operands contiguous along m / n (x @ W with W row-major, x.t() @ y): the matrix-core tiles read them
+    through the transposing LDS load; every combination with the k-contiguous form, batched, with a bias."""
+    import _dev
+    a = bits((torch.randn(2, m, k, generator=gen(11)) * 0.5).to(dtype))
+    b = bits((torch.randn(2, k, n, generator=gen(12)) * 0.5).to(dtype))
+    bias = bits(torch.randn(n, generator=gen(13)).to(dtype))
+    want, mag = oracle.gemm16(a, b, ODT[dtype], want_mag=True)
+    want2, mag2 = oracle.gemm16(a, b, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, want_mag=True)
+    for x, y in [(a, b), (col_major(a), b), (a, col_major(b)), (col_major(a), col_major(b))]:
+        close(_dev.gemm16(x, y, ODT[dtype], variant=variant), want, mag, dtype)
+    close(_dev.gemm16(col_major(a), b, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, variant=variant), want2, mag2, dtype)
+    # one matrix of a larger one: rows further apart than they are long
+    big_a, big_b = np.zeros((2, m, k + 64), np.uint16), np.zeros((2, k, n + 8), np.uint16)
+    big_a[:, :, :k], big_b[:, :, :n] = a, b
+    close(_dev.gemm16(big_a[:, :, :k], big_b[:, :, :n], ODT[dtype], variant=variant), want, mag, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
 def test_gemm16_batches_and_bias(dtype):
     import _dev
     a = bits(torch.randn(3, 40, 72, generator=gen(6)).to(dtype))

@@ -260,7 +260,7 @@ def test_16bit_matrix_products(tv, dtype):
         tol = torch.finfo(dtype).eps * ref.abs().clamp_min(2**-14) + 2**-20 * mag
         assert ((got - ref).abs() <= tol).all(), (got - ref).abs().max().item()
 
-    for m, k, n in [(64, 32, 64), (65, 33, 63), (17, 200, 129), (128, 1, 96), (3, 1000, 5), (300, 256, 260)]:
+    for m, k, n in [(64, 32, 64), (65, 33, 63), (17, 200, 129), (128, 1, 96), (3, 1000, 5), (300, 256, 260), (304, 256, 264)]:
         a, b = torch.randn(m, k, generator=gen(1)).to(dtype), torch.randn(k, n, generator=gen(2)).to(dtype)
         at, bt = a.t().contiguous().t(), b.t().contiguous().t()  # (column-major)
         for x, y in [(a, b), (at, bt), (a, bt), (at, b)]:

@@ -67,6 +67,7 @@ __device__ __forceinline__ float output_inv(const F8Params& p) {
 // _scaled_mm as a problem of the tile kernel: float8 operands, and in the epilogue the scales,
 // the bias, the output scale and the cast.
 struct F8Problem : F8Params {
+  static constexpr bool kTransA = false, kTransB = false;  // float8 operands are rows of k
   uint32_t batches = 1;
   uint64_t a_batch = 0, b_batch = 0;
   struct Whole {

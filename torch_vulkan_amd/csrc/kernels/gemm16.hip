@@ -3,12 +3,15 @@
 // contract of the reference's cooperative-matrix kernel (crates/vkcore/shaders/gemmcm.slang,
 // host side crates/pyvk/csrc/linalg.cpp:227-255), behind its kernel names ("gemmcm_bf16",
 // "gemmcm_f16"), parameter block (GemmParams, strides in elements) and spec {USE_CIN, ..}.
-//   - A rows and B columns both contiguous along k (x @ W.t(), the Linear layout), 16-byte
-//     aligned, k a multiple of 8: the tile kernel of _scaled_mm (mma_tile.h: 256x256x64-value
-//     workgroup tiles, direct global-to-LDS loads, persistent grid) with
-//     V_MFMA_F32_32X32X16_{BF16,F16} and an alpha / beta epilogue;
-//   - every other layout (row-major B, column-major A, strided views): one thread per output
-//     over the strides as given.  Correct for any strides, and slow.
+//   - operands whose rows are 16-byte aligned and contiguous along one of their two dims, C
+//     contiguous along n: the tile kernel of _scaled_mm (mma_tile.h: 256x256x64-value workgroup
+//     tiles, direct global-to-LDS loads, persistent grid) with V_MFMA_F32_32X32X16_{BF16,F16}
+//     and an alpha / beta epilogue.  A contiguous along k and B along k (x @ W.t(), the Linear
+//     layout) takes k a multiple of 8; an operand contiguous along m or n (x @ W, x.t() @ y:
+//     what backward passes produce) is read through the transposing LDS load and takes k a
+//     multiple of 64 and m (n) of 8;
+//   - everything else (strided views, odd sizes): one thread per output over the strides as
+//     given.  Correct for any strides, and slow.
 #include "kernels.h"
 #include "mma_tile.h"
 
@@ -17,8 +20,9 @@ namespace {
 
 __device__ __forceinline__ float slot_float(uint64_t slot) { return bits_f32(uint32_t(slot)); }
 
-template <class T>
+template <class T, bool TRA = false, bool TRB = false>
 struct GemmProblem {
+  static constexpr bool kTransA = TRA, kTransB = TRB;
   // operands as the tile kernel takes them (bytes)
   uint64_t a, b;
   uint32_t m, n, k, lda, ldb, batches;
@@ -80,14 +84,47 @@ __global__ __launch_bounds__(256) void gemm16_generic(GemmParams p, uint32_t use
   store_f32<T>(p.c + uint64_t((int64_t(batch) * p.c_sb + int64_t(m) * p.c_sm + int64_t(n) * p.c_sn) * 2), v);
 }
 
+template <class T, bool TRA, bool TRB>
+int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t variant, const Machine& mc, hipStream_t stream,
+                 std::string* err) {
+  constexpr int MATH = T::dtype == VKT_BF16 ? kMathBf16 : kMathF16;
+  GemmProblem<T, TRA, TRB> g;
+  g.a = p.a, g.b = p.b, g.m = p.m, g.n = p.n, g.k = p.k * 2;
+  g.lda = uint32_t(TRA ? p.a_sk : p.a_sm) * 2, g.ldb = uint32_t(TRB ? p.b_sk : p.b_sn) * 2;
+  g.batches = batch, g.a_batch = uint64_t(p.a_sb) * 2, g.b_batch = uint64_t(p.b_sb) * 2;
+  g.c = p.c, g.cin = use_cin ? p.cin : 0;
+  g.alpha = bits_f32_host(uint32_t(p.alpha)), g.beta = bits_f32_host(uint32_t(p.beta));
+  g.c_sm = p.c_sm, g.c_sb = p.c_sb, g.cin_sm = p.cin_sm, g.cin_sn = p.cin_sn, g.cin_sb = p.cin_sb;
+  const bool direct_ok = g.k % BK == 0;
+  // variant 0: planned; 1: 128x128 tiles; 2: 256x128; 3: 256x256 with direct loads; 4: 128x128 with direct loads
+  // (direct loads: k a multiple of 64; k-major operands run on the direct forms only)
+  if (variant == 0) {
+    const bool large = uint64_t(p.m) * p.n >= (1ull << 20);
+    variant = large ? (direct_ok ? 3 : 2) : (TRA || TRB ? 4 : 1);
+  }
+  if constexpr (!TRA && !TRB) {
+    if (variant == 1) return launch_mma_tile<2, 2, 4, 4, 0, 0, true, false, MATH>(g, mc.compute_units, stream, err, "gemmcm");
+    if (variant == 2) return launch_mma_tile<2, 2, 8, 4, 0, 0, true, false, MATH>(g, mc.compute_units, stream, err, "gemmcm");
+  }
+  if (variant == 3 && direct_ok) return launch_mma_tile<2, 2, 8, 8, 0, 0, true, true, MATH>(g, mc.compute_units, stream, err, "gemmcm");
+  if (variant == 4 && direct_ok) return launch_mma_tile<2, 2, 4, 4, 0, 0, true, true, MATH>(g, mc.compute_units, stream, err, "gemmcm");
+  *err = "gemmcm: unknown variant " + std::to_string(variant) + " for this k and layout";
+  return -1;
+}
+
 template <class T>
 int launch_gemm16_t(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t variant, const Machine& mc,
                     hipStream_t stream, std::string* err) {
-  constexpr int MATH = T::dtype == VKT_BF16 ? kMathBf16 : kMathF16;
-  const bool tiles_ok = p.k != 0 && p.k % 8 == 0 && p.a_sk == 1 && p.b_sk == 1 && p.c_sn == 1 && p.a_sm > 0 && p.b_sn > 0 &&
-                        p.c_sm > 0 && p.a_sm % 8 == 0 && p.b_sn % 8 == 0 && p.a_sb % 8 == 0 && p.b_sb % 8 == 0 &&
-                        p.a_sb >= 0 && p.b_sb >= 0 && p.c_sb >= 0 && p.a % 16 == 0 && p.b % 16 == 0 &&
-                        uint32_t(p.a_sm) >= p.k && uint32_t(p.b_sn) >= p.k && variant != 255;
+  // an operand is k-contiguous (rows of k), or k-major (contiguous along m / n, rows of k apart)
+  auto rows_ok = [](int32_t contiguous, int32_t pitch, int32_t batch_stride, uint64_t base, uint32_t row_len) {
+    return contiguous == 1 && pitch > 0 && pitch % 8 == 0 && uint32_t(pitch) >= row_len && batch_stride >= 0 &&
+           batch_stride % 8 == 0 && base % 16 == 0;
+  };
+  const bool a_k = rows_ok(p.a_sk, p.a_sm, p.a_sb, p.a, p.k), b_k = rows_ok(p.b_sk, p.b_sn, p.b_sb, p.b, p.k);
+  const bool a_m = !a_k && p.m % 8 == 0 && rows_ok(p.a_sm, p.a_sk, p.a_sb, p.a, p.m);
+  const bool b_n = !b_k && p.n % 8 == 0 && rows_ok(p.b_sn, p.b_sk, p.b_sb, p.b, p.n);
+  const bool k_ok = p.k != 0 && (a_m || b_n ? p.k % 64 == 0 : p.k % 8 == 0);
+  const bool tiles_ok = (a_k || a_m) && (b_k || b_n) && k_ok && p.c_sn == 1 && p.c_sm > 0 && p.c_sb >= 0 && variant != 255;
   if (!tiles_ok) {
     if ((p.m + 3) / 4 > 65535 || batch > 65535) {
       *err = "gemmcm: too many rows or batches for the strided kernel";
@@ -96,23 +133,10 @@ int launch_gemm16_t(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint3
     hipLaunchKernelGGL((gemm16_generic<T>), dim3((p.n + 63) / 64, (p.m + 3) / 4, batch), dim3(256), 0, stream, p, use_cin);
     return 0;
   }
-  GemmProblem<T> g;
-  g.a = p.a, g.b = p.b, g.m = p.m, g.n = p.n, g.k = p.k * 2, g.lda = uint32_t(p.a_sm) * 2, g.ldb = uint32_t(p.b_sn) * 2;
-  g.batches = batch, g.a_batch = uint64_t(p.a_sb) * 2, g.b_batch = uint64_t(p.b_sb) * 2;
-  g.c = p.c, g.cin = use_cin ? p.cin : 0;
-  g.alpha = bits_f32_host(uint32_t(p.alpha)), g.beta = bits_f32_host(uint32_t(p.beta));
-  g.c_sm = p.c_sm, g.c_sb = p.c_sb, g.cin_sm = p.cin_sm, g.cin_sn = p.cin_sn, g.cin_sb = p.cin_sb;
-  // variant 0: planned; 1: 128x128 tiles; 2: 256x128; 3: 256x256 with direct loads (k a multiple of 64)
-  if (variant == 0) variant = uint64_t(p.m) * p.n >= (1ull << 20) ? (g.k % BK == 0 ? 3 : 2) : 1;
-  switch (variant) {
-    case 1: return launch_mma_tile<2, 2, 4, 4, 0, 0, true, false, MATH>(g, mc.compute_units, stream, err, "gemmcm");
-    case 2: return launch_mma_tile<2, 2, 8, 4, 0, 0, true, false, MATH>(g, mc.compute_units, stream, err, "gemmcm");
-    case 3:
-      if (g.k % BK != 0) break;
-      return launch_mma_tile<2, 2, 8, 8, 0, 0, true, true, MATH>(g, mc.compute_units, stream, err, "gemmcm");
-  }
-  *err = "gemmcm: unknown variant " + std::to_string(variant) + " for this k";
-  return -1;
+  if (a_m && b_n) return launch_tiles<T, true, true>(p, use_cin, batch, variant, mc, stream, err);
+  if (a_m) return launch_tiles<T, true, false>(p, use_cin, batch, variant, mc, stream, err);
+  if (b_n) return launch_tiles<T, false, true>(p, use_cin, batch, variant, mc, stream, err);
+  return launch_tiles<T, false, false>(p, use_cin, batch, variant, mc, stream, err);
 }
 
 }  // namespace

@@ -9,6 +9,13 @@
 //   columns(batch, n, whole)             per-lane constants of columns n .. n + 3
 //   store<DT>(batch, m, n, t, cols, whole)   finish and store 4 outputs of row m
 //   for_output_type(full, whole, f)      call f(integral_constant<int, DT>) for the output type
+//   kTransA, kTransB                     16-bit operands only: the operand is stored k-major, i.e.
+//                                        as [k, m] (or [k, n]) rows lda (ldb) bytes apart, contiguous
+//                                        along m (n); m (n) a multiple of 8, k of 64 values
+// A k-major operand keeps its global layout in LDS ([64 k][BM or BN values], 16-byte chunks
+// swizzled by the row's low bits) and the matrix-core fragments come out of it through the
+// transposing LDS read (ds_read_b64_tr_b16: 16 lanes read a 4 (k) x 16 block of 2-byte
+// values and each receives the 4 values of one column), so no layout costs a pass over memory.
 #pragma once
 
 #include <type_traits>
@@ -85,6 +92,9 @@ template <int WAVES_M, int WAVES_N, int TM, int TN, int FA, int FB, bool MF32, b
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void mma_tile(P p, uint32_t tiles_m, uint32_t tiles_n) {
   constexpr bool WIDE = MATH == kMathFp8Wide;
   static_assert(MATH == kMathFp8 || MF32, "the widened and 16-bit forms are built on the 32x32 tiles");
+  constexpr bool TRA = P::kTransA, TRB = P::kTransB;
+  static_assert(!(TRA || TRB) || (DIRECT && MF32 && (MATH == kMathBf16 || MATH == kMathF16)),
+                "k-major operands: 16-bit values, direct loads, 32x32 tiles");
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * TM * 16, BN = WAVES_N * TN * 16;
   constexpr int A_CHUNKS = BM * 8 / NT, B_CHUNKS = BN * 8 / NT;  // 16-byte chunks per thread per step
@@ -123,6 +133,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void mma_tile(P p, uint32_t 
   for (int i = 0; i < A_CHUNKS; ++i) {
     // DIRECT: the load lands at LDS slot id (lane order), so the lane fetches the logical
     // chunk that the swizzle keeps in that slot
+    if constexpr (TRA) {
+      // slot id of the [64 k][BM values] tile -> (k row, chunk of 8 values along m); chunks past m repeat the last one
+      const uint32_t id = tid + NT * i, row = id / (BM / 8), c = (id % (BM / 8)) ^ ((row & 3u) << 2);
+      const uint32_t mc = m0 / 8 + c < p.m / 8 ? m0 / 8 + c : p.m / 8 - 1;
+      a_src[i] = a_base + uint64_t(row) * p.lda + mc * 16;
+      a_dst[i] = 0, a_k[i] = 0;
+      continue;
+    }
     const uint32_t id = tid + NT * i, row = id >> 3, c = DIRECT ? (id & 7u) ^ ((row >> 1) & 7u) : id & 7u;
     const uint32_t m = m0 + row < p.m ? m0 + row : p.m - 1;
     a_src[i] = a_base + uint64_t(m) * p.lda + c * 16;
@@ -131,6 +149,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void mma_tile(P p, uint32_t 
   }
 #pragma unroll
   for (int i = 0; i < B_CHUNKS; ++i) {
+    if constexpr (TRB) {
+      const uint32_t id = tid + NT * i, row = id / (BN / 8), c = (id % (BN / 8)) ^ ((row & 3u) << 2);
+      const uint32_t nc = n0 / 8 + c < p.n / 8 ? n0 / 8 + c : p.n / 8 - 1;
+      b_src[i] = b_base + uint64_t(row) * p.ldb + nc * 16;
+      b_dst[i] = 0, b_k[i] = 0;
+      continue;
+    }
     const uint32_t id = tid + NT * i, row = id >> 3, c = DIRECT ? (id & 7u) ^ ((row >> 1) & 7u) : id & 7u;
     const uint32_t n = n0 + row < p.n ? n0 + row : p.n - 1;
     b_src[i] = b_base + uint64_t(n) * p.ldb + c * 16;
@@ -210,7 +235,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void mma_tile(P p, uint32_t 
     const uint64_t src = c < A_CHUNKS ? a_src[c < A_CHUNKS ? c : 0] : b_src[c < A_CHUNKS ? 0 : c - A_CHUNKS];
     const uint32_t tile_base = c < A_CHUNKS ? uint32_t(c) * NT * 16 : BM * BK + uint32_t(c - A_CHUNKS) * NT * 16;
     uint8_t* dst = lds + (step & 1u) * STAGE + tile_base + uint32_t(wave) * 1024;
-    __builtin_amdgcn_global_load_lds(reinterpret_cast<const VKT_GLOBAL void*>(src + uint64_t(step) * BK),
+    // a step is 128 bytes along a k-contiguous row, or 64 rows of a k-major operand
+    const uint64_t advance = c < A_CHUNKS ? (TRA ? uint64_t(BK / 2) * p.lda : uint64_t(BK)) : (TRB ? uint64_t(BK / 2) * p.ldb : uint64_t(BK));
+    __builtin_amdgcn_global_load_lds(reinterpret_cast<const VKT_GLOBAL void*>(src + uint64_t(step) * advance),
                                      (__attribute__((address_space(3))) void*)(dst), 16, 0, 0);
   };
   auto side = [&](int op, uint32_t s, auto steady) {
@@ -243,11 +270,36 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void mma_tile(P p, uint32_t 
       // second half of k are asked for once the first MFMAs are under way
       // (row fragments are asked for two groups of MFMAs ahead: one group, 256 cycles, is
       // less than an LDS read takes while the direct loads are writing into the same LDS)
-      auto row_frag = [&](int gi) { return frag32(ta, (wm * TM2 + gi % TM2) * 32 + l32, gi / TM2); };
+      // The same fragment out of a k-major tile [64 k][W values]: for each half q of the fragment the 8
+      // values k = 32 kk + 16 h + 8 q .. + 7 of column `col`, by two transposing reads of 4 k each.  Lane i
+      // of a group of 16 points at row k + i / 4, values 4 (i % 4) .. + 3 of the group's 16 columns.
+      auto frag32_t = [&](const uint8_t* tile, uint32_t width, uint32_t col0, int kk) {
+        using V4S = short __attribute__((ext_vector_type(4)));
+        V8I f;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const uint32_t k = 32 * kk + 16 * h + 4 * t + (l16 >> 2);
+          const uint32_t value = col0 + 16 * ((lane >> 4) & 1) + 4 * (l16 & 3);  // first of the 4 values this lane points at
+          const uint32_t chunk = (value >> 3) ^ ((k & 3u) << 2);
+          const V4S v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (__attribute__((address_space(3))) V4S*)(tile + k * width * 2 + chunk * 16 + (value & 7u) * 2));
+          const U2 w = __builtin_bit_cast(U2, v);
+          f[2 * t] = int(w.x), f[2 * t + 1] = int(w.y);
+        }
+        return f;
+      };
+      auto row_frag = [&](int gi) {
+        if constexpr (TRA) return frag32_t(ta, BM, (wm * TM2 + gi % TM2) * 32, gi / TM2);
+        else return frag32(ta, (wm * TM2 + gi % TM2) * 32 + l32, gi / TM2);
+      };
+      auto col_frag = [&](int j, int kk) {
+        if constexpr (TRB) return frag32_t(tb, BN, (wn * TN2 + j) * 32, kk);
+        else return frag32(tb, (wn * TN2 + j) * 32 + l32, kk);
+      };
       V8I af = row_frag(0);
       V8I bf[2][TN2];
 #pragma unroll
-      for (int j = 0; j < TN2; ++j) bf[0][j] = frag32(tb, (wn * TN2 + j) * 32 + l32, 0);
+      for (int j = 0; j < TN2; ++j) bf[0][j] = col_frag(j, 0);
       V8I next = row_frag(1 < 2 * TM2 ? 1 : 0);
 #pragma unroll
       for (int gi = 0; gi < 2 * TM2; ++gi) {
@@ -256,7 +308,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void mma_tile(P p, uint32_t 
         if (gi + 2 < 2 * TM2) next2 = row_frag(gi + 2);
         if (gi == 0) {
 #pragma unroll
-          for (int j = 0; j < TN2; ++j) bf[1][j] = frag32(tb, (wn * TN2 + j) * 32 + l32, 1);
+          for (int j = 0; j < TN2; ++j) bf[1][j] = col_frag(j, 1);
         }
         V8BF af_wide[WIDE ? 4 : 1];
         if constexpr (WIDE) {
