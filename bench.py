@@ -242,6 +242,29 @@ def wl_move(abi, kind, steps, warmup, rows=16384, cols=16384):
                 copies=1, name=f"{name} {label}, bfloat16 [{rows}, {cols}]")
 
 
+def wl_affine(abi, kind, n, steps, warmup, seed=1100):
+    """Per-tensor affine quantisation of n float32 values: "quantize" (-> quint8), "dequantize" (quint8 -> float32),
+    "fake_quant" (-> float32 + mask bytes): bytes read + written per launch."""
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(1 << 20, generator=g) * 20).repeat(n >> 20)
+    scale_bits = int(np.float32(0.1).view(np.uint32))
+    if kind == "quantize":
+        src, dst = abi.Buffer.from_numpy(x.numpy()), abi.Buffer(n)
+        p, name, spec, work = abi.QuantParams(src=src.address, dst=dst.address, n=n, scale_bits=scale_bits, zero_point=5), "quantize_affine", [0], 5 * n
+    elif kind == "dequantize":
+        src, dst = abi.Buffer.from_numpy(torch.quantize_per_tensor(x, 0.1, 5, torch.quint8).int_repr().numpy()), abi.Buffer(4 * n)
+        p, name, spec, work = abi.QuantParams(src=src.address, dst=dst.address, n=n, scale_bits=scale_bits, zero_point=5), "dequantize_affine", [0], 5 * n
+    else:
+        src, dst, mask = abi.Buffer.from_numpy(x.numpy()), abi.Buffer(4 * n), abi.Buffer(n)
+        p = abi.QuantParams(src=src.address, dst=dst.address, mask=mask.address, n=n, scale_bits=scale_bits, zero_point=5, qmin=0,
+                            qmax=255, dtype=abi.F32)
+        name, spec, work = "fake_quant", [0, 0], 9 * n
+    wall, ev = time_steps(abi, [Launch(abi, name, spec, p)], steps, warmup)
+    return dict(kind="hbm", metric="affine quantisation GB/s (% of HBM peak)", work=work, wall_ms=wall, event_ms=ev, flops=0,
+                inputs=None, copies=1, name=f"{name} float32 / quint8 per tensor, {n >> 20} Mi values")
+
+
 def wl_copy(abi, nbytes, steps, warmup):
     """A plain device-to-device copy of known size (calibrates the HBM traffic counters)."""
     src, dst = abi.Buffer(nbytes), abi.Buffer(nbytes)
@@ -280,6 +303,10 @@ WORKLOADS = {
     # strided device copies either side of the path (not BASELINE configurations)
     "move_transpose_bf16_16384": lambda abi, s, w: wl_move(abi, "transpose", max(s // 10, 5), max(w // 4, 3)),
     "move_rows_bf16_16384": lambda abi, s, w: wl_move(abi, "rows", max(s // 10, 5), max(w // 4, 3)),
+    # per-tensor affine quantised tensors and fake quantisation (not BASELINE configurations)
+    "affine_quantize_256mi": lambda abi, s, w: wl_affine(abi, "quantize", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
+    "affine_dequantize_256mi": lambda abi, s, w: wl_affine(abi, "dequantize", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
+    "affine_fake_quant_256mi": lambda abi, s, w: wl_affine(abi, "fake_quant", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
     # config 4's launch on all-zero operands (not a BASELINE configuration: it shows how much of the
     # distance to the published peak is the data's, not the kernel's)
     "c4_fp8_8192_zero_operands": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 10, 5),

@@ -210,6 +210,25 @@ typedef struct F8QuantParams {
   uint32_t src_dtype, dst_fmt;
 } F8QuantParams;
 
+/* Per-tensor affine quantised tensors and fake quantisation, each one fused kernel (the reference
+ * composes them from elementwise operators: quantized.cpp:72-130, _kernels.py:1613-1676), bit
+ * for bit what PyTorch's x86 CPU kernels compute:
+ *   "quantize_affine", spec {QTYPE}    src float32 [n] -> dst quint8 (QTYPE 0) | qint8 (1) | qint32 (2)
+ *   "dequantize_affine", spec {QTYPE}  src integers [n] -> dst float32 = scale * float(q - zero_point)
+ *   "fake_quant", spec {PER_CHANNEL, ZP_FLOAT}   src [n] (dtype) -> dst [n] (dtype), mask [n] bytes;
+ *        per tensor: scale_bits, zero_point; per channel: scales float32 [channels], zero_points
+ *        int32 or float32 [channels], element i in channel (i / inner) % channels.
+ * Dense tensors.  88 bytes. */
+typedef struct QuantParams {
+  uint64_t src, dst, mask, scales, zero_points, n;
+  uint32_t scale_bits; /* float32 bits of the scale */
+  int32_t zero_point;
+  int64_t qmin, qmax;
+  uint32_t channels, inner;
+  uint32_t dtype; /* fake_quant: VKT_F32 | VKT_F16 | VKT_BF16 */
+  uint32_t pad;
+} QuantParams;
+
 /* "fp8mm", spec {}: out = cast((f32(A)*sa) @ (f32(B)*sb) + bias) [* 1/scale_result]
  * (quant.cpp:279-300 fused into one kernel).  A: fp8 [m,k] row-major (lda bytes);
  * B: fp8, column-major, i.e. [n,k] rows ldb bytes apart.  104 bytes. */

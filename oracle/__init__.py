@@ -242,6 +242,41 @@ def cast_strided(dst, dst_dtype, src, src_dtype):
     return dst
 
 
+QUINT8, QINT8, QINT32 = 0, 1, 2
+_QNP = {QUINT8: np.uint8, QINT8: np.int8, QINT32: np.int32}
+
+
+def quantize_affine(x, scale, zero_point, qtype):
+    """quantize_per_tensor's integers (x86 / FBGEMM semantics) of a float32 array."""
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, _QNP[qtype])
+    lib().orc_quantize_affine(_p(x), I64(x.size), ctypes.c_float(scale), ctypes.c_int32(zero_point), qtype, _p(out))
+    return out
+
+
+def dequantize_affine(q, scale, zero_point, qtype):
+    q = _c(q, _QNP[qtype])
+    out = np.empty(q.shape, np.float32)
+    lib().orc_dequantize_affine(_p(q), qtype, I64(q.size), ctypes.c_float(scale), ctypes.c_int32(zero_point), _p(out))
+    return out
+
+
+def fake_quant(x, dtype, scales, zero_points, qmin, qmax, axis=None):
+    """(output in x's type, mask uint8) of fake quantisation: per tensor (axis None; scales / zero_points of one
+    element) or per channel along `axis` (zero_points int32 or float32)."""
+    x = _c(x, _NP[dtype])
+    scales = _c(np.atleast_1d(scales), np.float32)
+    zps = np.atleast_1d(zero_points)
+    zp_float = int(zps.dtype.kind == "f")
+    zps = _c(zps, np.float32 if zp_float else np.int32)
+    channels = x.shape[axis] if axis is not None else 1
+    inner = int(np.prod(x.shape[axis + 1:])) if axis is not None else 1
+    out, mask = np.empty(x.shape, _NP[dtype]), np.empty(x.shape, np.uint8)
+    lib().orc_fake_quant(_p(x), dtype, I64(x.size), _p(scales), _p(zps), zp_float, I64(channels), I64(inner),
+                         int(axis is not None), I64(qmin), I64(qmax), _p(out), _p(mask))
+    return out, mask
+
+
 def _strided(a):
     """(base pointer, element strides) of a numpy array viewed as [B, R, C]."""
     a3 = a if a.ndim == 3 else a[None]

@@ -33,6 +33,12 @@
  *   orc_move            pinned: numpy strided views (as_strided) and torch CPU copy_ / contiguous() /
  *                               fill_ on the same layouts: transposes, slices, broadcasts, up to 8 dims
  *   orc_cast_strided    pinned: torch CPU Tensor.to() over the same strided views
+ *   orc_quantize_affine, orc_dequantize_affine   pinned: torch CPU quantize_per_tensor / int_repr /
+ *                               dequantize (the x86 FBGEMM build) for quint8, qint8, qint32 on random
+ *                               values, every rounding tie, NaN, infinities and values beyond int32
+ *   orc_fake_quant      pinned: torch CPU _fake_quantize_per_tensor_affine_cachemask_tensor_qparams and
+ *                               fake_quantize_per_channel_affine_cachemask (int32 and float zero points)
+ *                               on the same kinds of values, outputs and masks bit for bit
  *   orc_fp8_quant_rows  pinned: the same steps composed from torch CPU operators (amax, clamp,
  *                               true_divide, mul, clamp, to(float8)), rows whose maximum is
  *                               fmax exactly (the scale is 1: a plain cast), power-of-two
@@ -396,6 +402,92 @@ void orc_cast_strided(void* out, int dst_dtype, const void* a, int src_dtype, in
       s += c * sa[d];
     }
     store_from_f32(out, o, dst_dtype, load_as_f32(a, s, src_dtype));
+  }
+}
+
+/* ------------------------------------------------------------------ per-tensor affine quantised tensors */
+
+enum { ORC_QUINT8 = 0, ORC_QINT8 = 1, ORC_QINT32 = 2 };
+
+/* quantize_per_tensor as PyTorch's x86 CPU build computes it (FBGEMM's Quantize), restated from the
+ * reference's composition (crates/pyvk/csrc/quantized.cpp:72-116):
+ *   8-bit: t = x * (1.0f / scale) clipped at the largest float below 2^31 (a NaN too), rounded to
+ *          nearest even as int32 (below -2^31: INT32_MIN), plus the zero point (wrapping), clamped;
+ *   qint32: float(nearbyint(t) + zero_point), a NaN -> qmin, clamped. */
+void orc_quantize_affine(const float* x, int64_t n, float scale, int32_t zero_point, int qtype, void* out) {
+  const float inv = 1.0f / scale;
+  for (int64_t i = 0; i < n; i++) {
+    const float t = x[i] * inv;
+    if (qtype == ORC_QINT32) {
+      const float r = nearbyintf(t) + (float)zero_point;
+      int64_t q;
+      if (isnan(r)) q = INT32_MIN;
+      else if (r >= 2147483648.0f) q = INT32_MAX;
+      else if (r <= -2147483648.0f) q = INT32_MIN;
+      else q = (int64_t)r;
+      ((int32_t*)out)[i] = (int32_t)q;
+      continue;
+    }
+    const float top = 2147483520.0f;
+    const float tc = isnan(t) ? top : (t < top ? t : top);
+    const float r = nearbyintf(tc);
+    const int64_t base = r < -2147483648.0f ? (int64_t)INT32_MIN : (int64_t)r;
+    int32_t q = (int32_t)(uint32_t)(uint64_t)(base + zero_point); /* (wraps as the int32 add does) */
+    const int32_t lo = qtype == ORC_QUINT8 ? 0 : -128, hi = qtype == ORC_QUINT8 ? 255 : 127;
+    q = q < lo ? lo : (q > hi ? hi : q);
+    if (qtype == ORC_QUINT8) ((uint8_t*)out)[i] = (uint8_t)q;
+    else ((int8_t*)out)[i] = (int8_t)q;
+  }
+}
+
+/* dequantize: scale * float(q - zero_point), the difference in wrapping int32
+ * (crates/pyvk/csrc/quantized.cpp:123-130). */
+void orc_dequantize_affine(const void* q, int qtype, int64_t n, float scale, int32_t zero_point, float* out) {
+  for (int64_t i = 0; i < n; i++) {
+    const int32_t v = qtype == ORC_QUINT8 ? ((const uint8_t*)q)[i] : qtype == ORC_QINT8 ? ((const int8_t*)q)[i] : ((const int32_t*)q)[i];
+    const int32_t d = (int32_t)((uint32_t)v - (uint32_t)zero_point);
+    out[i] = (float)d * scale;
+  }
+}
+
+/* Fake quantisation with its mask (python/torch_vulkan/_kernels.py:1613-1630, which restates ATen's CPU
+ * kernels).  x: float32 values of element type dtype's tensor; element i belongs to channel
+ * (i / inner) % channels.  scales float32 [channels]; zero points int32 (zp_float 0) or float32 (1).
+ *   per tensor (per_channel 0): q = nearbyint(x * inv) + zp in float32; mask = qmin <= q <= qmax;
+ *       a NaN q counts as qmin; out = (clamp(q) - zp) * scale.
+ *   per channel: q is converted to int64 before the mask and the clamp (as ATen does): a q that
+ *       int64 cannot hold (NaN, infinities, |q| >= 2^63) becomes INT64_MIN, so qmin; with a float zero
+ *       point q = lrintf(zp + x * inv), which PyTorch's x86 build evaluates as one fused multiply-add
+ *       (measured: 7 of 8 million random values differ otherwise; the reference's composition rounds the
+ *       product first); the output is computed in double and rounded once.
+ * The output is rounded to dtype. */
+void orc_fake_quant(const void* x, int dtype, int64_t n, const float* scales, const void* zps, int zp_float,
+                    int64_t channels, int64_t inner, int per_channel, int64_t qmin, int64_t qmax, void* out,
+                    uint8_t* mask) {
+  for (int64_t i = 0; i < n; i++) {
+    const int64_t c = per_channel ? (i / inner) % channels : 0;
+    const float sc = scales[c], inv = 1.0f / sc; /* (a zero scale divides to infinity, as the CPU's) */
+    const float zp = zp_float ? ((const float*)zps)[c] : (float)((const int32_t*)zps)[c];
+    const float v = load_as_f32(x, i, dtype);
+    float q;
+    if (per_channel && zp_float) q = nearbyintf(fmaf(v, inv, zp)); /* (one rounding: see above) */
+    else q = nearbyintf(v * inv) + zp;
+    int inside;
+    float result;
+    if (per_channel) {
+      const int fits = q > -9223372036854775808.0f && q < 9223372036854775808.0f; /* (false for a NaN) */
+      const int64_t qi = fits ? (int64_t)q : INT64_MIN;
+      inside = qi >= qmin && qi <= qmax;
+      const int64_t qc = qi < qmin ? qmin : (qi > qmax ? qmax : qi);
+      /* (ATen clamps with fmin / fmax, i.e. in double, and stays there: one rounding at the end) */
+      result = (float)(((double)qc - (double)zp) * (double)sc);
+    } else {
+      inside = q >= (float)qmin && q <= (float)qmax;
+      const float qc = isnan(q) ? (float)qmin : (q < (float)qmin ? (float)qmin : (q > (float)qmax ? (float)qmax : q));
+      result = (qc - zp) * sc;
+    }
+    store_from_f32(out, i, dtype, result);
+    mask[i] = (uint8_t)inside;
   }
 }
 

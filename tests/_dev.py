@@ -250,3 +250,58 @@ def move(dst, src=None, value=None, variant=0, cast=None):
         abi.dispatch("copy8_" + label, [variant], p)
     abi.check(abi.lib().vkt_copy_to_host(ctypes.addressof(draw), dbuf.address, len(draw)))
     return dst
+
+
+_QNP = {0: np.uint8, 1: np.int8, 2: np.int32}
+
+
+def quantize_affine(x, scale, zero_point, qtype, skew=0):
+    """float32 array -> integers of quint8 (0) / qint8 (1) / qint32 (2); skew: elements by which both
+    buffers are offset from their allocations (exercises the unaligned form)."""
+    x = np.ascontiguousarray(x, np.float32)
+    qdt = np.dtype(_QNP[qtype])
+    src, dst = abi.Buffer(x.nbytes + 4 * skew + 4), abi.Buffer(x.size * qdt.itemsize + skew * qdt.itemsize + 4)
+    abi.check(abi.lib().vkt_copy_to_device(src.address + 4 * skew, x.ctypes.data, x.nbytes))
+    p = abi.QuantParams(src=src.address + 4 * skew, dst=dst.address + qdt.itemsize * skew, n=x.size,
+                        scale_bits=int(np.float32(scale).view(np.uint32)), zero_point=zero_point)
+    abi.dispatch("quantize_affine", [qtype], p)
+    out = np.empty(x.shape, qdt)
+    abi.check(abi.lib().vkt_copy_to_host(out.ctypes.data, dst.address + qdt.itemsize * skew, out.nbytes))
+    return out
+
+
+def dequantize_affine(q, scale, zero_point, qtype, skew=0):
+    q = np.ascontiguousarray(q, _QNP[qtype])
+    src, dst = abi.Buffer(q.nbytes + q.itemsize * skew + 4), abi.Buffer(q.size * 4 + 4 * skew + 4)
+    abi.check(abi.lib().vkt_copy_to_device(src.address + q.itemsize * skew, q.ctypes.data, q.nbytes))
+    p = abi.QuantParams(src=src.address + q.itemsize * skew, dst=dst.address + 4 * skew, n=q.size,
+                        scale_bits=int(np.float32(scale).view(np.uint32)), zero_point=zero_point)
+    abi.dispatch("dequantize_affine", [qtype], p)
+    out = np.empty(q.shape, np.float32)
+    abi.check(abi.lib().vkt_copy_to_host(out.ctypes.data, dst.address + 4 * skew, out.nbytes))
+    return out
+
+
+def fake_quant(x, dtype, scales, zero_points, qmin, qmax, axis=None, skew=0):
+    """(output in x's type, mask uint8): x a float32 array (dtype F32) or a uint16 view (F16 / BF16)."""
+    x = np.ascontiguousarray(x)
+    item = x.itemsize
+    src, dst, mask = abi.Buffer(x.nbytes + item * skew + 4), abi.Buffer(x.nbytes + item * skew + 4), abi.Buffer(x.size + skew + 4)
+    abi.check(abi.lib().vkt_copy_to_device(src.address + item * skew, x.ctypes.data, x.nbytes))
+    scales = np.ascontiguousarray(np.atleast_1d(scales), np.float32)
+    zps = np.atleast_1d(zero_points)
+    zp_float = int(zps.dtype.kind == "f")
+    zps = np.ascontiguousarray(zps, np.float32 if zp_float else np.int32)
+    p = abi.QuantParams(src=src.address + item * skew, dst=dst.address + item * skew, mask=mask.address + skew, n=x.size,
+                        qmin=qmin, qmax=qmax, dtype=dtype)
+    if axis is None:
+        p.scale_bits, p.zero_point = int(scales[0].view(np.uint32)), int(zps[0])
+        abi.dispatch("fake_quant", [0, 0], p)
+    else:
+        ds, dz = abi.Buffer.from_numpy(scales), abi.Buffer.from_numpy(zps)
+        p.scales, p.zero_points, p.channels, p.inner = ds.address, dz.address, x.shape[axis], int(np.prod(x.shape[axis + 1:]))
+        abi.dispatch("fake_quant", [1, zp_float], p)
+    out, m = np.empty(x.shape, x.dtype), np.empty(x.shape, np.uint8)
+    abi.check(abi.lib().vkt_copy_to_host(out.ctypes.data, dst.address + item * skew, out.nbytes))
+    abi.check(abi.lib().vkt_copy_to_host(m.ctypes.data, mask.address + skew, m.nbytes))
+    return out, m

@@ -330,3 +330,59 @@ def test_strided_copies_and_fills_on_the_device(tv):
     with on_gpu(tv):
         wt = wq.to("vk").t().contiguous().t().contiguous()
     assert torch.equal(wt.cpu(), wq)
+
+
+@pytest.mark.parametrize("qdtype", [torch.quint8, torch.qint8, torch.qint32])
+def test_quantized_per_tensor(tv, qdtype):
+    """Legacy quantised tensors on vk as the reference tests them (tests/python/test_fallback_ops.py:986-1006):
+    quantize_per_tensor, the getters, int_repr, dequantize, flip, clone and copies, bit for bit as the CPU's."""
+    x = torch.cat([torch.randn(40, generator=gen(0)) * 20,
+                   torch.tensor([float("nan"), float("inf"), -float("inf"), 0.05, 0.15, -0.05, 1e30, 3e9])]).view(6, 8)
+    c = torch.quantize_per_tensor(x, 0.1, 5, qdtype)
+    with on_gpu(tv):
+        v = torch.quantize_per_tensor(x.to("vk"), 0.1, 5, qdtype)
+        assert v.is_quantized and v.device.type == "vk" and v.dtype == qdtype
+        assert (v.q_scale(), v.q_zero_point(), v.qscheme()) == (c.q_scale(), c.q_zero_point(), c.qscheme())
+        ints, deq, flipped, cloned = v.int_repr(), v.dequantize(), v.flip((0, 1)), v.clone()
+        t = torch.quantize_per_tensor(x.to("vk").t(), 0.1, 5, qdtype)  # a strided input
+        by_tensor = torch.quantize_per_tensor(x.to("vk"), torch.tensor(0.1).to("vk"), torch.tensor(5).to("vk"), qdtype)
+        e = torch._empty_affine_quantized([5, 5, 5, 5], scale=2, zero_point=3, dtype=qdtype, device="vk")
+    assert torch.equal(ints.cpu(), c.int_repr()) and torch.equal(deq.cpu(), c.dequantize())
+    assert torch.equal(flipped.int_repr().cpu(), c.flip((0, 1)).int_repr()) and torch.equal(cloned.int_repr().cpu(), c.int_repr())
+    assert torch.equal(t.int_repr().cpu(), c.int_repr().t()) and torch.equal(by_tensor.int_repr().cpu(), c.int_repr())
+    assert torch.equal(v.cpu().int_repr(), c.int_repr())
+    back = c.to("vk")
+    assert back.is_quantized and torch.equal(back.int_repr().cpu(), c.int_repr())
+    assert e.flatten(0, -1).shape == (625,) and e.ravel().shape == (625,)
+    with pytest.raises(RuntimeError, match="only works on Float"):
+        torch.quantize_per_tensor(x.half().to("vk"), 0.1, 5, qdtype)
+
+
+def test_fake_quantize_cachemask_ops(tv):
+    """As the reference's test (tests/python/test_fallback_ops.py:972-984), plus float zero points and 16-bit inputs."""
+    x = torch.tensor([[-1.3, 0.0, 0.26, 4.0], [float("nan"), float("inf"), -0.5, 1e-3]])
+    v = lambda t: t.to("vk")
+    sc, zp = torch.tensor([0.05]), torch.tensor([3], dtype=torch.int32)
+    on = torch.ones(1, dtype=torch.long)
+    f = torch.ops.aten._fake_quantize_per_tensor_affine_cachemask_tensor_qparams
+    with on_gpu(tv):
+        got = f(v(x), v(sc), v(zp), v(on), 0, 255)
+        off = f(v(x), v(sc), v(zp), v(torch.zeros(1, dtype=torch.long)), 0, 255)
+    for a, b in zip(got, f(x, sc, zp, on, 0, 255)):
+        assert torch.equal(a.cpu().nan_to_num(), b.nan_to_num())
+    assert torch.equal(off[0].cpu().nan_to_num(), x.nan_to_num()) and off[1].cpu().all()
+    scs, zps = torch.tensor([0.05, 0.2]), torch.tensor([3, 250], dtype=torch.int32)
+    g = torch.ops.aten.fake_quantize_per_channel_affine_cachemask
+    big = torch.randn(2, 3, 500, generator=gen(4)) * 4
+    for inp, axis, s, z in [(x, 0, scs, zps), (x, 0, scs, torch.tensor([3.25, 250.5])), (big, 1, torch.tensor([0.05, 0.2, 0.01]), torch.tensor([3, 250, 128], dtype=torch.int32)),
+                            (big.bfloat16(), 2, torch.rand(500, generator=gen(5)) * 0.1 + 0.01, torch.randint(0, 255, (500,), dtype=torch.int32, generator=gen(6))),
+                            (big.transpose(0, 2), 0, torch.rand(500, generator=gen(5)) * 0.1 + 0.01, torch.rand(500, generator=gen(7)) * 200)]:
+        with on_gpu(tv):
+            got = g(v(inp), v(s), v(z), axis, 0, 255)
+        for a, b in zip(got, g(inp, s, z, axis, 0, 255)):
+            assert a.shape == b.shape and torch.equal(a.cpu().float().nan_to_num(), b.float().nan_to_num())
+    with on_gpu(tv):
+        got = torch.fake_quantize_per_tensor_affine(v(big), 0.05, 3, 0, 255)
+    assert torch.equal(got.cpu(), torch.fake_quantize_per_tensor_affine(big, 0.05, 3, 0, 255))
+    with pytest.raises(RuntimeError, match="must be between"):
+        g(v(x), v(scs), v(torch.tensor([3, 300], dtype=torch.int32)), 0, 0, 255)

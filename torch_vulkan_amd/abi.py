@@ -79,6 +79,12 @@ class Copy8Params(ctypes.Structure):
                 ("size", u32 * 8), ("so", i32 * 8), ("sa", i32 * 8)]
 
 
+class QuantParams(ctypes.Structure):
+    _fields_ = [("src", u64), ("dst", u64), ("mask", u64), ("scales", u64), ("zero_points", u64), ("n", u64),
+                ("scale_bits", u32), ("zero_point", i32), ("qmin", ctypes.c_int64), ("qmax", ctypes.c_int64),
+                ("channels", u32), ("inner", u32), ("dtype", u32), ("pad", u32)]
+
+
 MOVE_COPY, MOVE_FILL = 0, 1
 
 
@@ -93,7 +99,7 @@ class F8QuantParams(ctypes.Structure):
 
 assert ctypes.sizeof(Q8Params) == 56 and ctypes.sizeof(Q4Params) == 64 and ctypes.sizeof(F8Params) == 104
 assert ctypes.sizeof(CastParams) == 32 and ctypes.sizeof(F8QuantParams) == 48 and ctypes.sizeof(GemmParams) == 112
-assert ctypes.sizeof(StridedParams) == 128 and ctypes.sizeof(Copy8Params) == 128
+assert ctypes.sizeof(StridedParams) == 128 and ctypes.sizeof(Copy8Params) == 128 and ctypes.sizeof(QuantParams) == 88
 
 # every symbol include/vkt.h declares
 SYMBOLS = ["vkt_last_error", "vkt_alloc", "vkt_free", "vkt_synchronize", "vkt_empty_cache", "vkt_memory_stats",

@@ -27,7 +27,7 @@ _lib = None
 def build(force=False):
     """Compiles the C++ backend against the installed torch (g++; no GPU or HIP needed)."""
     from torch.utils import cpp_extension
-    srcs = [os.path.join(_SRC, f) for f in ("backend.cpp", "quant.cpp", "linalg.cpp")]
+    srcs = [os.path.join(_SRC, f) for f in ("backend.cpp", "quant.cpp", "linalg.cpp", "quantized.cpp")]
     deps = srcs + [os.path.join(_SRC, "vk.h"), os.path.join(os.path.dirname(_HERE), "include", "vkt.h")]
     if not force and os.path.exists(LIB_PATH) and all(os.path.getmtime(d) <= os.path.getmtime(LIB_PATH) for d in deps):
         return LIB_PATH

@@ -31,6 +31,8 @@ SOURCES = {
     # (single float32 operations in the float8 producer, as specified)
     "kernels/cast.hip": ["-ffp-contract=off"],
     "kernels/move.hip": [],
+    # (the CPU's quantisation arithmetic, operation by operation)
+    "kernels/quantize.hip": ["-ffp-contract=off"],
     "kernels/util.hip": [],
 }
 

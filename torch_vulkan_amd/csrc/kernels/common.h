@@ -36,6 +36,12 @@ __device__ __forceinline__ void stg(uint64_t addr, X v) {
   *reinterpret_cast<VKT_GLOBAL X*>(addr) = v;
 }
 
+// A store of data that this kernel does not read again (a streamed output): non-temporal.
+template <class X>
+__device__ __forceinline__ void stg_stream(uint64_t addr, X v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<VKT_GLOBAL X*>(addr));
+}
+
 __device__ __forceinline__ float bits_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
 inline float bits_f32_host(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t f32_bits(float f) { return __builtin_bit_cast(uint32_t, f); }

@@ -40,6 +40,10 @@ int launch_move(const StridedParams& s, const char* size_label, uint32_t op, uin
                 hipStream_t stream, std::string* err);
 int launch_copy8(const Copy8Params& c, const char* size_label, uint32_t variant, const Machine& mc, hipStream_t stream,
                  std::string* err);
+int launch_quantize_affine(const QuantParams& p, uint32_t qtype, bool dequantize, const Machine& mc, hipStream_t stream,
+                           std::string* err);
+int launch_fake_quant(const QuantParams& p, uint32_t per_channel, uint32_t zp_float, const Machine& mc, hipStream_t stream,
+                      std::string* err);
 int launch_fp8_quant(const F8QuantParams& p, uint32_t rowwise, const Machine& mc, hipStream_t stream, std::string* err);
 int launch_fill(uint64_t dst, uint8_t value, uint64_t nbytes, hipStream_t stream, std::string* err);
 int launch_copy(uint64_t dst, uint64_t src, uint64_t nbytes, hipStream_t stream, std::string* err);

@@ -203,14 +203,13 @@ struct MergedDims {
 
 // dst's index space with src broadcast to it: dims of size 1 dropped, dims that are contiguous on
 // both sides merged.
-MergedDims merged_dims(const at::Tensor& dst, const at::Tensor* src) {
+MergedDims merged_dims(const at::Tensor& dst, const std::vector<int64_t>* src_strides) {
   MergedDims m;
-  const int64_t pad = src ? dst.dim() - src->dim() : 0;
   for (int64_t i = dst.dim() - 1; i >= 0; --i) {
     const int64_t n = dst.size(i);
     if (n == 1) continue;
     const int64_t o = dst.stride(i);
-    const int64_t a = (src && i >= pad && src->size(i - pad) != 1) ? src->stride(i - pad) : 0;
+    const int64_t a = src_strides ? (*src_strides)[size_t(i)] : 0;
     if (!m.size.empty() && o == m.so.back() * m.size.back() && a == m.sa.back() * m.size.back()) {
       m.size.back() *= n;
       continue;
@@ -227,11 +226,9 @@ bool for_each_launch(const MergedDims& m, size_t inner_max, F&& emit) {
   int64_t count = 1, span_o = 0, span_a = 0;
   for (size_t d = 0; d < inner; ++d) {
     count *= m.size[d];
-    span_o += (m.size[d] - 1) * m.so[d], span_a += (m.size[d] - 1) * m.sa[d];
+    span_o += (m.size[d] - 1) * std::abs(m.so[d]), span_a += (m.size[d] - 1) * std::abs(m.sa[d]);
   }
   if (count >= (int64_t(1) << 32) || span_o >= (int64_t(1) << 31) || span_a >= (int64_t(1) << 31)) return false;
-  for (size_t d = 0; d < inner; ++d)
-    if (m.so[d] < 0 || m.sa[d] < 0) return false;
   std::vector<int64_t> index(m.size.size() - inner, 0);
   while (true) {
     int64_t oo = 0, ao = 0;
@@ -261,20 +258,25 @@ const char* float_label(at::ScalarType t) {
   return t == at::kFloat ? "f32" : t == at::kHalf ? "f16" : t == at::kBFloat16 ? "bf16" : nullptr;
 }
 
-// dst (vk) <- src (vk) with strides, broadcasting and float32 / float16 / bfloat16 conversion, on
-// the device (reference backend.cpp:633-690 copy_vk_to_vk).  False where no kernel covers it.
-bool copy_on_device(const at::Tensor& dst, const at::Tensor& src) {
-  if (src.is_conj() || src.is_neg() || dst.is_conj() || dst.is_neg()) return false;
-  const bool same = src.scalar_type() == dst.scalar_type();
+}  // namespace
+
+// The device side of copies between vk tensors (reference backend.cpp:633-690 copy_vk_to_vk):
+// dst[...] = the elements of type src_type at src_base + sum_d index_d * src_strides[d] (element strides, one
+// per dim of dst, 0 where the source broadcasts, negative ones allowed).
+bool copy_strided_on_device(const at::Tensor& dst, uint64_t src_base, const std::vector<int64_t>& src_strides,
+                            at::ScalarType src_type) {
+  if (dst.is_conj() || dst.is_neg()) return false;
+  const bool same = src_type == dst.scalar_type();
   const char* label = size_label(dst.element_size());
   std::string kernel;
   if (same && label) kernel = std::string("move_") + label;
-  else if (!same && float_label(src.scalar_type()) && float_label(dst.scalar_type()))
-    kernel = std::string("cast_") + float_label(src.scalar_type()) + "_" + float_label(dst.scalar_type());
+  else if (!same && float_label(src_type) && float_label(dst.scalar_type()))
+    kernel = std::string("cast_") + float_label(src_type) + "_" + float_label(dst.scalar_type());
   else return false;
-  const MergedDims m = merged_dims(dst, &src);
-  const uint64_t out = reinterpret_cast<uint64_t>(dst.mutable_data_ptr()), a = reinterpret_cast<uint64_t>(src.const_data_ptr());
-  const int64_t oi = dst.element_size(), ai = src.element_size();
+  if (dst.numel() == 0) return true;
+  const MergedDims m = merged_dims(dst, &src_strides);
+  const uint64_t out = reinterpret_cast<uint64_t>(dst.mutable_data_ptr()), a = src_base;
+  const int64_t oi = dst.element_size(), ai = int64_t(c10::elementSize(src_type));
   if (same && m.size.size() > 4) {  // up to 8 dims in one launch (reference copy_many_dims)
     const std::string k8 = std::string("copy8_") + label;
     return for_each_launch(m, 8, [&](int64_t count, size_t ndim, int64_t oo, int64_t ao) {
@@ -296,6 +298,18 @@ bool copy_on_device(const at::Tensor& dst, const at::Tensor& src) {
     }
     dispatch(kernel, {VKT_MOVE_COPY}, p, 1);
   });
+}
+
+namespace {
+
+// dst (vk) <- src (vk) with strides, broadcasting and float32 / float16 / bfloat16 conversion.
+bool copy_on_device(const at::Tensor& dst, const at::Tensor& src) {
+  if (src.is_conj() || src.is_neg()) return false;
+  std::vector<int64_t> strides(size_t(dst.dim()), 0);
+  const int64_t pad = dst.dim() - src.dim();
+  for (int64_t i = pad; i < dst.dim(); ++i)
+    if (src.size(i - pad) != 1) strides[size_t(i)] = src.stride(i - pad);
+  return copy_strided_on_device(dst, reinterpret_cast<uint64_t>(src.const_data_ptr()), strides, src.scalar_type());
 }
 
 // self[...] = value on the device (reference backend.cpp:806-816 fill_scalar).

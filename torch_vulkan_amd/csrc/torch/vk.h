@@ -37,6 +37,15 @@ void record_fallback(const std::string& op);
 // Runs `op` on CPU copies of the stack's vk tensors, recorded as a fallback.
 void run_fallback(const c10::OperatorHandle& op, torch::jit::Stack* stack, bool error_on_views);
 
+// dst[...] = the elements at src_base + sum_d index_d * src_strides[d] (element strides per dim of dst, 0 =
+// broadcast, negative allowed), converting between float32 / float16 / bfloat16 if src_type differs.  False
+// where no device kernel covers the case.
+bool copy_strided_on_device(const at::Tensor& dst, uint64_t src_base, const std::vector<int64_t>& src_strides,
+                            at::ScalarType src_type);
+
+// A dense copy of quantised vk tensor q in memory format mf, with q's quantizer.
+at::Tensor vk_clone_quantized(const at::Tensor& q, at::MemoryFormat mf);
+
 inline bool is_vk(const at::Tensor& t) { return t.device().type() == kDevice; }
 
 // The library's code of an element type (-1: not one of its types).
