@@ -28,10 +28,10 @@
 //                  kept as two signed-nibble planes qh and ql-8, so
 //                  sum (q+nzp) w = 16 dot8(qh,w) + dot8(ql-8,w) + (8+nzp) dot8(1,w):
 //                  four instructions per 8 weights, no unpacking;
-//                - the float32 block terms must be added in block order: each lane adds its
-//                  8 in order, lane groups hand the running sum on with ds_bpermute and
-//                  waves through LDS.  Starting from -0.0f and padding with -0.0f makes every
-//                  step a plain addition (x + -0 = x, -0 + t = t) with the reference's bits.
+//                - the float32 block terms must be added in block order: every lane leaves
+//                  its terms in LDS at their blocks' places and one thread per output adds
+//                  a round's terms in order.  Starting from -0.0f and padding with -0.0f makes
+//                  every step a plain addition (x + -0 = x, -0 + t = t) with the reference's bits.
 #pragma clang fp contract(off)
 
 #include <type_traits>
@@ -288,8 +288,10 @@ __device__ __forceinline__ void nibble_planes(const int (&q)[8], uint32_t* hi, u
 // 256 (one lane's run of 8 units), so that the four k-parts a wave reads at once, 256 bytes
 // apart, fall on different banks.
 __host__ __device__ inline uint32_t q_row_bytes(uint32_t kpad) { return kpad + kpad / 256 * 16; }
+constexpr uint32_t kTermPitch = 132;  // floats per (row, column) of a round's block terms: 128 + 4, so that the 16
+                                      // columns' 16-byte reads fall on different banks
 __host__ __device__ inline uint32_t q_lds_bytes(uint32_t rows, uint32_t kpad) {
-  return rows * q_row_bytes(kpad) + rows * kTileCols * 4 + 64;
+  return rows * q_row_bytes(kpad) + rows * kTileCols * 4 + 64 + rows * kTileCols * kTermPitch * 4;
 }
 __device__ __forceinline__ uint32_t q_group_offset(uint32_t g) {  // byte offset of 8 values' hi word
   const uint32_t unit = g >> 2, d = g & 3;
@@ -342,16 +344,36 @@ __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L
   const uint32_t tile = blockIdx.x, n = tile * kTileCols + col;
   const uint32_t nblocks = UPB ? p.k / p.bs : 1;
   const uint32_t qs = q_row_bytes(L.kpad);
-  float* const carry = reinterpret_cast<float*>(q_lds + MR * qs);      // [MR][16]: running sums between waves
+  float* const carry = reinterpret_cast<float*>(q_lds + MR * qs);      // [MR][16]
   int* const itotal = reinterpret_cast<int*>(carry);                    // (channelwise: integer totals)
+  float* const terms = carry + MR * kTileCols + 16;                     // [MR][16][kTermPitch]: a round's block terms
 
-  // the first round's weights are requested before anything else: they are the long pole
+  // Loads return in the order they were issued.  The first row's activations are asked for first (they come
+  // from L2 and the row quantisation waits for them alone), then the first round's weights and scales: the
+  // HBM stream runs while the row is quantised.  (Weights first made the quantisation wait for the stream:
+  // 2.5 us of 9.7 at K = 4096.)
   U4 w[kUnitsPerLane];
-  {
-    const uint64_t base = (uint64_t(tile) * L.rounds * 4 + wave) * kUnitsPerLane;
+  float s[BPL];
+  auto request_round = [&](uint32_t round) {
+    const uint64_t base = (uint64_t(tile) * L.rounds + round) * 4 + wave;
+    // (scales first: a block's term needs its scale as soon as its weights are in)
+    if constexpr (UPB != 0) {
+      const uint64_t sp = p.compact + L.scale_off + (base * 64 + lane) * BPL * 4;
+      if constexpr (BPL == 8) {
+        const F4 s0 = ldg_stream<F4>(sp), s1 = ldg_stream<F4>(sp + 16);
+        s[0] = s0.x, s[1] = s0.y, s[2] = s0.z, s[3] = s0.w, s[4] = s1.x, s[5] = s1.y, s[6] = s1.z, s[7] = s1.w;
+      } else if constexpr (BPL == 4) {
+        const F4 s0 = ldg<F4>(sp);
+        s[0] = s0.x, s[1] = s0.y, s[2] = s0.z, s[3] = s0.w;
+      } else {
 #pragma unroll
-    for (int j = 0; j < kUnitsPerLane; ++j) w[j] = ldg_stream<U4>(p.compact + ((base + j) * 64 + lane) * 16);
-  }
+        for (int jb = 0; jb < BPL; ++jb) s[jb] = ldg<float>(sp + 4 * jb);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kUnitsPerLane; ++j) w[j] = ldg_stream<U4>(p.compact + ((base * kUnitsPerLane + j) * 64 + lane) * 16);
+  };
+  if constexpr (!FUSED) request_round(0);
 
   int nzp8[MR];  // 8 - zero_point
   float recip[MR];
@@ -372,6 +394,7 @@ __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L
         const uint32_t g = tid + 256 * i;
         if (g < groups) load8_f32<T>(row + g * 8 * item, x[i]);
       }
+      if (r == 0) request_round(0);
 #pragma unroll
       for (int i = 0; i < kFusedGroups; ++i) {
         if (uint32_t(tid + 256 * i) < groups) {
@@ -417,25 +440,6 @@ __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L
   for (int r = 0; r < MR; ++r) acc[r] = 0.0f, tot_a[r] = 0, tot_b[r] = 0;
 
   for (uint32_t round = 0; round < L.rounds; ++round) {
-    const uint64_t base = (uint64_t(tile) * L.rounds + round) * 4 + wave;
-    if (round != 0) {
-#pragma unroll
-      for (int j = 0; j < kUnitsPerLane; ++j) w[j] = ldg_stream<U4>(p.compact + ((base * kUnitsPerLane + j) * 64 + lane) * 16);
-    }
-    float s[BPL];
-    if constexpr (UPB != 0) {
-      const uint64_t sp = p.compact + L.scale_off + (base * 64 + lane) * BPL * 4;
-      if constexpr (BPL == 8) {
-        const F4 s0 = ldg_stream<F4>(sp), s1 = ldg_stream<F4>(sp + 16);
-        s[0] = s0.x, s[1] = s0.y, s[2] = s0.z, s[3] = s0.w, s[4] = s1.x, s[5] = s1.y, s[6] = s1.z, s[7] = s1.w;
-      } else if constexpr (BPL == 4) {
-        const F4 s0 = ldg<F4>(sp);
-        s[0] = s0.x, s[1] = s0.y, s[2] = s0.z, s[3] = s0.w;
-      } else {
-#pragma unroll
-        for (int jb = 0; jb < BPL; ++jb) s[jb] = ldg<float>(sp + 4 * jb);
-      }
-    }
     const uint32_t unit0 = round * kRoundUnits + part * kUnitsPerLane;
     const uint8_t* qbase = q_lds + unit0 * kUnit + unit0 / 8 * 16;
 
@@ -479,29 +483,39 @@ __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L
       }
     }
 
+    // the next round's weights and scales are requested as soon as this round's are used up
+    if (round + 1 < L.rounds) request_round(round + 1);
     if constexpr (UPB != 0) {
-      // the running float32 sums travel through the 16 k-parts in order: wave by wave through
-      // LDS, and inside a wave from one group of 16 lanes to the next
-#pragma unroll 1
-      for (int stage = 0; stage < 4; ++stage) {
-        if (wave == stage) {
+      // The float32 block terms must be added in block order.  Every lane leaves its terms in LDS at the
+      // place of their blocks; then one thread per (row, column) adds the round's 16 * BPL terms in
+      // order (16-byte reads, the only sequential part: ~130 dependent additions per round).
 #pragma unroll
-          for (int r = 0; r < MR; ++r) {
-            float a = carry[r * kTileCols + col];
+      for (int r = 0; r < MR; ++r) {
+        float* at = terms + (r * kTileCols + col) * kTermPitch + part * BPL;
+        if constexpr (BPL % 4 == 0) {
 #pragma unroll
-            for (int gg = 0; gg < 4; ++gg) {
-              if (gg != 0) a = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane - 16) * 4, __builtin_bit_cast(int, acc[r])));
-              if (grp == gg) {
+          for (int jb = 0; jb < BPL; jb += 4) *reinterpret_cast<F4*>(at + jb) = F4{t[r][jb], t[r][jb + 1], t[r][jb + 2], t[r][jb + 3]};
+        } else {
 #pragma unroll
-                for (int jb = 0; jb < BPL; ++jb) a = a + t[r][jb];
-                acc[r] = a;
-              }
-            }
-            if (grp == 3) carry[r * kTileCols + col] = acc[r];
-          }
+          for (int jb = 0; jb < BPL; ++jb) at[jb] = t[r][jb];
         }
-        __syncthreads();
       }
+      __syncthreads();
+      if (wave == 0 && grp < MR) {
+        // (thread (grp, col) of the first wave owns row grp, column col; its sum lives in acc[0])
+        const float* from = terms + (grp * kTileCols + col) * kTermPitch;
+        float a = round == 0 ? -0.0f : acc[0];
+#pragma unroll
+        for (int b = 0; b < 16 * BPL; b += 4) {
+          const F4 v = *reinterpret_cast<const F4*>(from + b);
+          a = a + v.x;
+          a = a + v.y;
+          a = a + v.z;
+          a = a + v.w;
+        }
+        acc[0] = a;
+      }
+      __syncthreads();  // (the next round overwrites the terms)
     }
   }
   if constexpr (UPB == 0) {
@@ -515,7 +529,15 @@ __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L
       for (int r = 0; r < MR; ++r) acc[r] = float(itotal[r * kTileCols + col]) * s;
     }
   }
-  if (part == 15 && n < p.n) {
+  if constexpr (UPB != 0) {
+    if (wave == 0 && grp < MR && n < p.n && m0 + grp < p.m) {
+      const float bias = ldg<float>(p.compact + L.bias_off + n * 4ull);
+      float rc = recip[0];
+#pragma unroll
+      for (int r = 1; r < MR; ++r) rc = grp == r ? recip[r] : rc;
+      finish_store<T>(p.out + (uint64_t(m0 + grp) * p.n + n) * item, acc[0], rc, p.has_bias != 0, bias);
+    }
+  } else if (part == 15 && n < p.n) {
     const float bias = ldg<float>(p.compact + L.bias_off + n * 4ull);
 #pragma unroll
     for (int r = 0; r < MR; ++r)
