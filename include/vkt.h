@@ -229,6 +229,15 @@ typedef struct QuantParams {
   uint32_t pad;
 } QuantParams;
 
+/* "aminmax", spec {}: out_min[r], out_max[r] (float32) = the minimum and maximum of row r of src
+ * [rows, cols] (dtype, rows ld elements apart); a NaN in a row makes both NaN, as torch.aminmax.
+ * The range step of the fake-quantisation observer (_kernels.py:1744-1746).  40 bytes. */
+typedef struct MinMaxParams {
+  uint64_t src, out_min, out_max;
+  uint32_t rows, cols, ld;
+  uint32_t dtype; /* VKT_F32 | VKT_F16 | VKT_BF16 */
+} MinMaxParams;
+
 /* "fp8mm", spec {}: out = cast((f32(A)*sa) @ (f32(B)*sb) + bias) [* 1/scale_result]
  * (quant.cpp:279-300 fused into one kernel).  A: fp8 [m,k] row-major (lda bytes);
  * B: fp8, column-major, i.e. [n,k] rows ldb bytes apart.  104 bytes. */

@@ -277,6 +277,31 @@ def fake_quant(x, dtype, scales, zero_points, qmin, qmax, axis=None):
     return out, mask
 
 
+def choose_qparams(mn, mx, qmin, qmax, symmetric):
+    """(scale float32, zero point) from a range, as the CPU's observer chooses them."""
+    sc, zp = ctypes.c_float(), ctypes.c_int32()
+    rc = lib().orc_choose_qparams(ctypes.c_float(mn), ctypes.c_float(mx), ctypes.c_int32(qmin), ctypes.c_int32(qmax), int(symmetric),
+                                  ctypes.byref(sc), ctypes.byref(zp))
+    if rc != 0:
+        raise ValueError("In ChooseQuantizationParams, min should be less than or equal to max")
+    return np.float32(sc.value), zp.value
+
+
+def observe_fake_quant(x, dtype, run_min, run_max, averaging_const, qmin, qmax, per_row, symmetric):
+    """One step of the fused moving-average observer with fake quantisation on (observer on): updates run_min /
+    run_max (float32 arrays, in place), returns (output, mask, scales float32, zero points int32)."""
+    xf = to_f32(x, dtype) if dtype != F32 else np.asarray(x, np.float32)
+    rows = xf.reshape(xf.shape[0], -1) if per_row else xf.reshape(1, -1)
+    nan = np.isnan(rows).any(axis=1)
+    cur_min = np.where(nan, np.float32("nan"), rows.min(axis=1)).astype(np.float32)
+    cur_max = np.where(nan, np.float32("nan"), rows.max(axis=1)).astype(np.float32)
+    lib().orc_observe(_p(run_min), _p(run_max), _p(cur_min), _p(cur_max), I64(run_min.size), ctypes.c_float(averaging_const))
+    qp = [choose_qparams(a, b, qmin, qmax, symmetric) for a, b in zip(run_min, run_max)]
+    scales, zps = np.array([q[0] for q in qp], np.float32), np.array([q[1] for q in qp], np.int32)
+    out, mask = fake_quant(x, dtype, scales, zps, qmin, qmax, axis=0 if per_row else None)
+    return out, mask, scales, zps
+
+
 def _strided(a):
     """(base pointer, element strides) of a numpy array viewed as [B, R, C]."""
     a3 = a if a.ndim == 3 else a[None]

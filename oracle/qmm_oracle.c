@@ -39,6 +39,9 @@
  *   orc_fake_quant      pinned: torch CPU _fake_quantize_per_tensor_affine_cachemask_tensor_qparams and
  *                               fake_quantize_per_channel_affine_cachemask (int32 and float zero points)
  *                               on the same kinds of values, outputs and masks bit for bit
+ *   orc_choose_qparams, orc_observe   pinned: torch CPU _fused_moving_avg_obs_fq_helper over several steps
+ *                               (running min / max, scale, zero point and the fake-quantised output bit
+ *                               for bit; per tensor and per row, symmetric or not, three averaging constants)
  *   orc_fp8_quant_rows  pinned: the same steps composed from torch CPU operators (amax, clamp,
  *                               true_divide, mul, clamp, to(float8)), rows whose maximum is
  *                               fmax exactly (the scale is 1: a plain cast), power-of-two
@@ -488,6 +491,54 @@ void orc_fake_quant(const void* x, int dtype, int64_t n, const float* scales, co
     }
     store_from_f32(out, i, dtype, result);
     mask[i] = (uint8_t)inside;
+  }
+}
+
+/* Quantisation parameters from a range, as the CPU chooses them (ATen's
+ * quant_utils::ChooseQuantizationParams, restated by the reference in
+ * python/torch_vulkan/_kernels.py:1678-1716): the float32 and double steps as written there.
+ * Returns 0, or -1 where ATen raises (min above max). */
+int orc_choose_qparams(float mn, float mx, int32_t qmin, int32_t qmax, int preserve_sparsity, float* scale_out,
+                       int32_t* zp_out) {
+  if (!(mn <= mx)) return -1;
+  if (mn < 0 && mx > 0 && preserve_sparsity) {
+    const int32_t sqmin = -((qmax - qmin) / 2 + 1), sqmax = (qmax - qmin) / 2;
+    const double a = fabs((double)(mn / (float)sqmin)), b = fabs((double)(mx / (float)sqmax));
+    const double max_scale = a > b ? a : b;
+    mn = (float)(max_scale * sqmin), mx = (float)(max_scale * sqmax);
+  }
+  mn = mn < 0.0f ? mn : 0.0f, mx = mx > 0.0f ? mx : 0.0f;
+  /* (the difference in double, the scale itself a float32: what the zero point below is derived from.
+   * torch 2.10's CPU build behaves so: ranges [-a, a] put the zero point on a tie that tells the two apart;
+   * the reference's restatement keeps the scale in double) */
+  float scale = (float)(((double)mx - (double)mn) / (double)(qmax - qmin));
+  if (scale == 0.0f || isinf(1.0f / scale)) scale = 0.1f;
+  const float small = 6.1e-5f;
+  if (scale < small) {
+    const float org = scale;
+    scale = small;
+    if (mn == 0.0f) mx = small * (float)(qmax - qmin);
+    else if (mx == 0.0f) mn = -small * (float)(qmax - qmin);
+    else {
+      const float amp = small / org;
+      mn = mn * amp, mx = mx * amp;
+    }
+  }
+  const double z_min = qmin - (double)mn / (double)scale, z_max = qmax - (double)mx / (double)scale;
+  const double e_min = fabs((double)qmin) - fabs((double)mn / (double)scale), e_max = fabs((double)qmax) - fabs((double)mx / (double)scale);
+  double z = e_min < e_max ? z_min : z_max;
+  if (mn < 0 && mx > 0 && preserve_sparsity) z = (qmin + qmax) / 2.0;
+  *zp_out = z < qmin ? qmin : (z > qmax ? qmax : (int32_t)nearbyint(z));
+  *scale_out = scale;
+  return 0;
+}
+
+/* One observer step on the running range (python/torch_vulkan/_kernels.py:1740-1750): a running value that
+ * is still infinite takes this batch's, otherwise run + c * (cur - run) in single float32 operations. */
+void orc_observe(float* run_min, float* run_max, const float* cur_min, const float* cur_max, int64_t n, float c) {
+  for (int64_t i = 0; i < n; i++) {
+    run_min[i] = isinf(run_min[i]) ? cur_min[i] : run_min[i] + c * (cur_min[i] - run_min[i]);
+    run_max[i] = isinf(run_max[i]) ? cur_max[i] : run_max[i] + c * (cur_max[i] - run_max[i]);
   }
 }
 

@@ -305,3 +305,17 @@ def fake_quant(x, dtype, scales, zero_points, qmin, qmax, axis=None, skew=0):
     abi.check(abi.lib().vkt_copy_to_host(out.ctypes.data, dst.address + item * skew, out.nbytes))
     abi.check(abi.lib().vkt_copy_to_host(m.ctypes.data, mask.address + skew, m.nbytes))
     return out, m
+
+
+def aminmax(x, dtype, ld=None):
+    """(min, max) float32 per row of a 2-d array (float32, or a uint16 view of float16 / bfloat16 values); ld: row
+    pitch in elements of the device copy (rows further apart than they are long)."""
+    x = np.ascontiguousarray(x)
+    rows, cols = x.shape
+    ld = ld or cols
+    padded = np.zeros((rows, ld), x.dtype)
+    padded[:, :cols] = x
+    src = abi.Buffer.from_numpy(padded)
+    lo, hi = abi.Buffer(4 * rows), abi.Buffer(4 * rows)
+    abi.dispatch("aminmax", [], abi.MinMaxParams(src=src.address, out_min=lo.address, out_max=hi.address, rows=rows, cols=cols, ld=ld, dtype=dtype))
+    return lo.to_numpy(np.float32, (rows,)), hi.to_numpy(np.float32, (rows,))

@@ -87,6 +87,21 @@ def test_fake_quant_large_against_cpu():
     assert np.array_equal(got[0], cpu[0].numpy()) and np.array_equal(got[1].astype(bool), cpu[1].numpy())
 
 
+@pytest.mark.parametrize("dtype", [oracle.F32, oracle.F16, oracle.BF16])
+@pytest.mark.parametrize("rows,cols,ld", [(1, 1, 1), (1, 60, 60), (4, 15, 15), (3, 5000, 5000), (1, 300000, 300000), (7, 70001, 70004), (600, 33, 40),
+                                           (2, 1 << 21, 1 << 21)])
+def test_aminmax(dtype, rows, cols, ld):
+    """Row-wise minimum and maximum as torch.aminmax(x, dim=1) (exact: a selection), NaN rows included."""
+    import _dev
+    x = (torch.randn(rows, cols, generator=torch.Generator().manual_seed(rows + cols)) * 10).to(TD[dtype])
+    if rows > 1 and cols > 3:
+        x[1, cols // 2] = float("nan")
+        x[0, cols - 1] = 1e4
+    lo, hi = _dev.aminmax(as_np(x), dtype, ld=ld)
+    want = torch.aminmax(x.float(), dim=1)
+    assert np.array_equal(lo, want.min.numpy(), equal_nan=True) and np.array_equal(hi, want.max.numpy(), equal_nan=True)
+
+
 def test_errors():
     from torch_vulkan_amd import abi
     buf = abi.Buffer(4096)

@@ -386,3 +386,28 @@ def test_fake_quantize_cachemask_ops(tv):
     assert torch.equal(got.cpu(), torch.fake_quantize_per_tensor_affine(big, 0.05, 3, 0, 255))
     with pytest.raises(RuntimeError, match="must be between"):
         g(v(x), v(scs), v(torch.tensor([3, 300], dtype=torch.int32)), 0, 0, 255)
+
+
+@pytest.mark.parametrize("per_row", [False, True])
+@pytest.mark.parametrize("symmetric", [False, True])
+@pytest.mark.parametrize("qrange", [(0, 255), (-128, 127)])
+def test_fused_moving_avg_obs_fake_quant(tv, per_row, symmetric, qrange):
+    """The QAT observer and fake quantisation as the reference tests them (tests/python/test_fallback_ops.py:947-969):
+    bit for bit as the CPU's over several steps (the running min / max start infinite, then move)."""
+    g = gen(0)
+    size = 4 if per_row else 1
+    state = {d: [torch.full((size,), float("inf")), torch.full((size,), float("-inf")), torch.ones(size),
+                 torch.zeros(size, dtype=torch.int32)] for d in ("cpu", "vk")}
+    state["vk"] = [t.to("vk") for t in state["vk"]]
+    for step in range(4):
+        x = torch.randn(4, 3, 5, generator=g) * (0.1 + step) - 0.5 * step
+        got = {}
+        for d in ("cpu", "vk"):
+            rmin, rmax, s, z = state[d]
+            with (on_gpu(tv) if d == "vk" else contextlib.nullcontext()):
+                out, mask = torch.ops.aten._fused_moving_avg_obs_fq_helper(
+                    x.to(d), torch.tensor([1]).to(d), torch.tensor([1]).to(d), rmin, rmax, s, z, 0.01 if step == 3 else 0.25,
+                    qrange[0], qrange[1], 0, per_row, symmetric)
+            got[d] = [t.cpu() for t in (out, mask, rmin, rmax, s, z)]
+        for a, b in zip(got["cpu"], got["vk"]):
+            assert torch.equal(a, b)

@@ -31,7 +31,7 @@ def test_parameter_block_sizes():
     assert ctypes.sizeof(abi.CastParams) == 32 and ctypes.sizeof(abi.F8QuantParams) == 48
     assert ctypes.sizeof(abi.GemmParams) == 112  # the reference's block (linalg.cpp:25-34)
     assert ctypes.sizeof(abi.StridedParams) == 128 and abi.StridedParams.size.offset == 64  # launch.cpp:28-31
-    assert ctypes.sizeof(abi.QuantParams) == 88
+    assert ctypes.sizeof(abi.QuantParams) == 88 and ctypes.sizeof(abi.MinMaxParams) == 40
     assert ctypes.sizeof(abi.Copy8Params) == 128 and abi.Copy8Params.size.offset == 32 and abi.Copy8Params.sa.offset == 96  # :90-91
     for t in (abi.Q4PackParams, abi.Q4CParams, abi.F8Params):
         assert ctypes.sizeof(t) <= 128

@@ -92,3 +92,38 @@ def test_fake_quant_per_channel(dtype, float_zp, axis):
     want = torch.ops.aten.fake_quantize_per_channel_affine_cachemask(x * 1e6, scales, zps, axis, -(2**26), 2**26)
     out, mask = oracle.fake_quant(as_np(x * 1e6), dtype, scales.numpy(), zps.numpy(), -(2**26), 2**26, axis=axis)
     same((out, mask, dtype), want)
+
+
+@pytest.mark.parametrize("per_row", [False, True])
+@pytest.mark.parametrize("symmetric", [False, True])
+@pytest.mark.parametrize("qrange", [(0, 255), (-128, 127)])
+@pytest.mark.parametrize("c", [0.25, 0.01, 0.9])
+def test_observer_steps(per_row, symmetric, qrange, c):
+    """The QAT observer with fake quantisation as the reference tests it (tests/python/test_fallback_ops.py:947-969),
+    over several steps: the running range starts infinite, then moves; every state and output as the CPU's."""
+    g = torch.Generator().manual_seed(0)
+    size = 4 if per_row else 1
+    cpu = [torch.full((size,), float("inf")), torch.full((size,), float("-inf")), torch.ones(size), torch.zeros(size, dtype=torch.int32)]
+    rmin, rmax = np.full(size, np.inf, np.float32), np.full(size, -np.inf, np.float32)
+    for step in range(5):
+        scale_step = [0.1, 1.1, 1e-7, 30.0, 2.1][step]
+        x = torch.randn(4, 3, 5, generator=g) * scale_step - 0.5 * step
+        out, mask = torch.ops.aten._fused_moving_avg_obs_fq_helper(x, torch.tensor([1]), torch.tensor([1]), cpu[0], cpu[1], cpu[2], cpu[3],
+                                                                   c, qrange[0], qrange[1], 0, per_row, symmetric)
+        got = oracle.observe_fake_quant(x.numpy(), oracle.F32, rmin, rmax, c, qrange[0], qrange[1], per_row, symmetric)
+        assert np.array_equal(rmin, cpu[0].numpy()) and np.array_equal(rmax, cpu[1].numpy())
+        assert np.array_equal(got[2], cpu[2].numpy()) and np.array_equal(got[3], cpu[3].numpy())
+        assert np.array_equal(got[0], out.numpy()) and np.array_equal(got[1].astype(bool), mask.numpy())
+
+
+@pytest.mark.parametrize("mn,mx", [(-1.0, 2.0), (0.0, 0.0), (-1e-9, 1e-9), (0.5, 3.0), (-4.0, -1.0), (-1e-6, 0.0), (0.0, 2e-5), (-3e38, 3e38),
+                                   (-0.7, 0.7), (-1.0, 1.0), (-2e38, 2e38), (-1e-5, 1e-5), (-1e-5, 3e-5)])
+def test_choose_qparams_special_ranges(mn, mx):
+    """Ranges that take the special branches (zero range, tiny scale, one-sided), through the CPU observer itself."""
+    for sym in (False, True):
+        for qr in ((0, 255), (-128, 127)):
+            st = [torch.tensor([mn]), torch.tensor([mx]), torch.ones(1), torch.zeros(1, dtype=torch.int32)]
+            torch.ops.aten._fused_moving_avg_obs_fq_helper(torch.zeros(2, 2), torch.tensor([0]), torch.tensor([1]), st[0], st[1], st[2], st[3],
+                                                           0.25, qr[0], qr[1], 0, False, sym)
+            sc, zp = oracle.choose_qparams(mn, mx, qr[0], qr[1], sym)
+            assert sc == st[2].item() and zp == st[3].item(), (mn, mx, sym, qr, sc, zp, st[2].item(), st[3].item())

@@ -85,6 +85,10 @@ class QuantParams(ctypes.Structure):
                 ("channels", u32), ("inner", u32), ("dtype", u32), ("pad", u32)]
 
 
+class MinMaxParams(ctypes.Structure):
+    _fields_ = [("src", u64), ("out_min", u64), ("out_max", u64), ("rows", u32), ("cols", u32), ("ld", u32), ("dtype", u32)]
+
+
 MOVE_COPY, MOVE_FILL = 0, 1
 
 
@@ -99,7 +103,7 @@ class F8QuantParams(ctypes.Structure):
 
 assert ctypes.sizeof(Q8Params) == 56 and ctypes.sizeof(Q4Params) == 64 and ctypes.sizeof(F8Params) == 104
 assert ctypes.sizeof(CastParams) == 32 and ctypes.sizeof(F8QuantParams) == 48 and ctypes.sizeof(GemmParams) == 112
-assert ctypes.sizeof(StridedParams) == 128 and ctypes.sizeof(Copy8Params) == 128 and ctypes.sizeof(QuantParams) == 88
+assert ctypes.sizeof(StridedParams) == 128 and ctypes.sizeof(Copy8Params) == 128 and ctypes.sizeof(QuantParams) == 88 and ctypes.sizeof(MinMaxParams) == 40
 
 # every symbol include/vkt.h declares
 SYMBOLS = ["vkt_last_error", "vkt_alloc", "vkt_free", "vkt_synchronize", "vkt_empty_cache", "vkt_memory_stats",

@@ -245,14 +245,19 @@ int dispatch_named(Runtime& rt, const char* name, const uint32_t* spec, size_t n
     if (!read_push(push, npush, &p, name, err)) return -1;
     return launch_quantize_affine(p, spec_at(0), name[0] == 'd', rt.machine, rt.stream, err);
   }
-  if (!std::strcmp(name, "fake_quant")) {
+  if (!std::strcmp(name, "aminmax")) {
+    MinMaxParams p;
+    if (!read_push(push, npush, &p, name, err)) return -1;
+    return launch_aminmax(p, rt.machine, rt.stream, err);
+  }
+  if (!std::strcmp(name, "fake_quant") || !std::strcmp(name, "aminmax")) {
     QuantParams p;
     if (!read_push(push, npush, &p, name, err)) return -1;
     return launch_fake_quant(p, spec_at(0), spec_at(1), rt.machine, rt.stream, err);
   }
   if (!std::strcmp(name, "fp8_quant") || !std::strncmp(name, "move_", 5) || !std::strncmp(name, "copy8_", 6) ||
           !std::strncmp(name, "cast_", 5) || !std::strcmp(name, "quantize_affine") || !std::strcmp(name, "dequantize_affine") ||
-          !std::strcmp(name, "fake_quant")) {
+          !std::strcmp(name, "fake_quant") || !std::strcmp(name, "aminmax")) {
     F8QuantParams p;
     if (!read_push(push, npush, &p, name, err)) return -1;
     return launch_fp8_quant(p, spec_at(0), rt.machine, rt.stream, err);
@@ -399,7 +404,7 @@ uint32_t vkt_kernel_subgroup_size(const char* name) {
   return (!std::strncmp(name, "qmm", 3) || !std::strcmp(name, "fp8mm") || !std::strcmp(name, "cast_fp8") || !std::strncmp(name, "gemmcm_", 7) ||
           !std::strcmp(name, "fp8_quant") || !std::strncmp(name, "move_", 5) || !std::strncmp(name, "copy8_", 6) ||
           !std::strncmp(name, "cast_", 5) || !std::strcmp(name, "quantize_affine") || !std::strcmp(name, "dequantize_affine") ||
-          !std::strcmp(name, "fake_quant"))
+          !std::strcmp(name, "fake_quant") || !std::strcmp(name, "aminmax"))
              ? 64u
              : 0u;
 }

@@ -42,6 +42,7 @@ int launch_copy8(const Copy8Params& c, const char* size_label, uint32_t variant,
                  std::string* err);
 int launch_quantize_affine(const QuantParams& p, uint32_t qtype, bool dequantize, const Machine& mc, hipStream_t stream,
                            std::string* err);
+int launch_aminmax(const MinMaxParams& p, const Machine& mc, hipStream_t stream, std::string* err);
 int launch_fake_quant(const QuantParams& p, uint32_t per_channel, uint32_t zp_float, const Machine& mc, hipStream_t stream,
                       std::string* err);
 int launch_fp8_quant(const F8QuantParams& p, uint32_t rowwise, const Machine& mc, hipStream_t stream, std::string* err);

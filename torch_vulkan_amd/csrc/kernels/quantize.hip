@@ -203,6 +203,63 @@ __global__ __launch_bounds__(256) void fake_quant_kernel(QuantParams p, float sc
       });
 }
 
+// Row-wise minimum and maximum (the observer in front of fake quantisation): block (part, row) reduces
+// columns [part * chunk, (part + 1) * chunk) of its row; a NaN anywhere in the range makes both results NaN,
+// as torch.aminmax.  Results as float32 at out[row * parts + part].
+template <class T>
+__global__ __launch_bounds__(256) void aminmax_kernel(MinMaxParams p, uint64_t out_min, uint64_t out_max, uint32_t parts, uint32_t chunk,
+                                                      uint32_t vec) {
+  constexpr uint32_t ITEM = T::dtype == VKT_F32 ? 4 : 2;
+  const uint32_t part = blockIdx.x, row = blockIdx.y, tid = threadIdx.x;
+  const uint64_t base = p.src + uint64_t(row) * p.ld * ITEM;
+  const uint32_t lo = part * chunk, hi = lo + chunk < p.cols ? lo + chunk : p.cols;
+  float mn = __builtin_inff(), mx = -__builtin_inff(), bad = 0.0f;
+  auto take = [&](float v) {
+    mn = fminf(mn, v), mx = fmaxf(mx, v);  // (both drop a NaN: it is counted apart)
+    bad = v != v ? 1.0f : bad;
+  };
+  if (vec) {  // rows and chunks start on 16 bytes
+    for (uint32_t c = lo + tid * kPer; c + kPer <= hi; c += 256 * kPer) {
+      const auto raw = ldg<typename Raw<ITEM>::type>(base + uint64_t(c) * ITEM);
+#pragma unroll
+      for (int e = 0; e < kPer; ++e) take(element_f32<T>(raw, e));
+    }
+    const uint32_t tail = lo + (hi - lo) / kPer * kPer;
+    if (tail + tid < hi) take(load_f32<T>(base + uint64_t(tail + tid) * ITEM));
+  } else {
+    for (uint32_t c = lo + tid; c < hi; c += 256) take(load_f32<T>(base + uint64_t(c) * ITEM));
+  }
+  mn = wave_min(mn), mx = wave_max(mx), bad = wave_max(bad);
+  __shared__ float part_min[4], part_max[4], part_bad[4];
+  if ((tid & 63) == 0) part_min[tid >> 6] = mn, part_max[tid >> 6] = mx, part_bad[tid >> 6] = bad;
+  __syncthreads();
+  if (tid == 0) {
+    mn = fminf(fminf(part_min[0], part_min[1]), fminf(part_min[2], part_min[3]));
+    mx = fmaxf(fmaxf(part_max[0], part_max[1]), fmaxf(part_max[2], part_max[3]));
+    bad = fmaxf(fmaxf(part_bad[0], part_bad[1]), fmaxf(part_bad[2], part_bad[3]));
+    const float nan = __builtin_nanf("");
+    stg<float>(out_min + 4ull * (uint64_t(row) * parts + part), bad != 0.0f ? nan : mn);
+    stg<float>(out_max + 4ull * (uint64_t(row) * parts + part), bad != 0.0f ? nan : mx);
+  }
+}
+
+// Combines the parts of each row (one thread per row; a NaN part makes the row NaN).
+__global__ __launch_bounds__(256) void aminmax_finish(uint64_t part_min, uint64_t part_max, uint64_t out_min, uint64_t out_max, uint32_t rows,
+                                                      uint32_t parts) {
+  const uint32_t row = blockIdx.x * 256 + threadIdx.x;
+  if (row >= rows) return;
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+  bool bad = false;
+  for (uint32_t q = 0; q < parts; ++q) {
+    const float a = ldg<float>(part_min + 4ull * (uint64_t(row) * parts + q)), b = ldg<float>(part_max + 4ull * (uint64_t(row) * parts + q));
+    bad = bad || a != a;
+    mn = fminf(mn, a), mx = fmaxf(mx, b);
+  }
+  const float nan = __builtin_nanf("");
+  stg<float>(out_min + 4ull * row, bad ? nan : mn);
+  stg<float>(out_max + 4ull * row, bad ? nan : mx);
+}
+
 uint32_t groups_for(uint64_t n, const Machine& mc) {
   const uint64_t want = ((n + kPer - 1) / kPer + 255) / 256, cap = uint64_t(mc.compute_units) * 64;
   return uint32_t(want < 1 ? 1 : (want < cap ? want : cap));
@@ -217,6 +274,38 @@ int done(const char* who, std::string* err) {
 }
 
 }  // namespace
+
+int launch_aminmax(const MinMaxParams& p, const Machine& mc, hipStream_t stream, std::string* err) {
+  if (p.rows == 0) return 0;
+  if (p.dtype > VKT_BF16 || p.cols == 0 || p.ld < p.cols || p.rows > 65535) {
+    *err = "aminmax: float32 / float16 / bfloat16 rows of at least one column, at most 65535 rows, ld >= cols";
+    return -1;
+  }
+  const uint64_t item = p.dtype == VKT_F32 ? 4 : 2;
+  if (!p.src || !p.out_min || !p.out_max || p.src % item != 0 || p.out_min % 4 != 0 || p.out_max % 4 != 0) {
+    *err = "aminmax: null or misaligned tensor address";
+    return -1;
+  }
+  // enough blocks to fill the machine: rows split into parts of whole 4 Ki-column chunks
+  const uint32_t unit = 256 * kPer * 4;
+  uint32_t parts = (uint32_t(mc.compute_units) * 4 + p.rows - 1) / p.rows;
+  const uint32_t most = (p.cols + unit - 1) / unit;
+  parts = parts < 1 ? 1 : (parts > most ? most : parts);
+  const uint32_t chunk = ((p.cols + parts - 1) / parts + unit - 1) / unit * unit;
+  parts = (p.cols + chunk - 1) / chunk;
+  if (parts > 1 && uint64_t(p.rows) * parts * 8 > mc.workspace_bytes) {
+    *err = "aminmax: workspace too small";
+    return -1;
+  }
+  const uint64_t pmin = parts > 1 ? mc.workspace : p.out_min, pmax = parts > 1 ? mc.workspace + uint64_t(p.rows) * parts * 4 : p.out_max;
+  const uint32_t vec = p.src % 16 == 0 && (uint64_t(p.ld) * item) % 16 == 0;
+  const dim3 grid(parts, p.rows);
+  if (p.dtype == VKT_F32) hipLaunchKernelGGL(aminmax_kernel<f32_t>, grid, dim3(256), 0, stream, p, pmin, pmax, parts, chunk, vec);
+  else if (p.dtype == VKT_F16) hipLaunchKernelGGL(aminmax_kernel<f16_t>, grid, dim3(256), 0, stream, p, pmin, pmax, parts, chunk, vec);
+  else hipLaunchKernelGGL(aminmax_kernel<bf16_t>, grid, dim3(256), 0, stream, p, pmin, pmax, parts, chunk, vec);
+  if (parts > 1) hipLaunchKernelGGL(aminmax_finish, dim3((p.rows + 255) / 256), dim3(256), 0, stream, pmin, pmax, p.out_min, p.out_max, p.rows, parts);
+  return done("aminmax", err);
+}
 
 int launch_quantize_affine(const QuantParams& p, uint32_t qtype, bool dequantize, const Machine& mc, hipStream_t stream,
                            std::string* err) {

@@ -13,6 +13,7 @@
 #include <ATen/quantized/Quantizer.h>
 #include <torch/library.h>
 
+#include <cmath>
 #include <cstring>
 #include <limits>
 
@@ -216,6 +217,119 @@ std::tuple<at::Tensor, at::Tensor> fake_quant_per_channel(const at::Tensor& self
   return fake_quant_launch(self, &scale, &zero_point, 0.0, 0, axis, quant_min, quant_max);
 }
 
+// ---------------------------------------------------------------- the QAT observer (reference _kernels.py:1678-1762)
+
+// (scale, zero point) from a range as the CPU chooses them (ATen's quant_utils::ChooseQuantizationParams; the
+// scale is a float32 from the start, the zero point is derived from it in double).
+std::pair<float, int32_t> choose_qparams(float mn, float mx, int32_t qmin, int32_t qmax, bool preserve_sparsity) {
+  TORCH_CHECK(mn <= mx, "In ChooseQuantizationParams, min should be less than or equal to max");
+  if (mn < 0 && mx > 0 && preserve_sparsity) {
+    const int32_t sqmin = -((qmax - qmin) / 2 + 1), sqmax = (qmax - qmin) / 2;
+    const double a = std::fabs(static_cast<double>(mn / static_cast<float>(sqmin)));
+    const double b = std::fabs(static_cast<double>(mx / static_cast<float>(sqmax)));
+    const double max_scale = a > b ? a : b;
+    mn = static_cast<float>(max_scale * sqmin), mx = static_cast<float>(max_scale * sqmax);
+  }
+  mn = mn < 0.0f ? mn : 0.0f, mx = mx > 0.0f ? mx : 0.0f;
+  TORCH_CHECK(qmin < qmax, "In ChooseQuantizationParams, qmin should be less than qmax");
+  float scale = static_cast<float>((static_cast<double>(mx) - static_cast<double>(mn)) / static_cast<double>(qmax - qmin));
+  if (scale == 0.0f || std::isinf(1.0f / scale)) scale = 0.1f;
+  TORCH_CHECK(scale > 0, "quantization scale should be > 0");
+  const float small = 6.1e-5f;
+  if (scale < small) {
+    const float org = scale;
+    scale = small;
+    if (mn == 0.0f) mx = small * static_cast<float>(qmax - qmin);
+    else if (mx == 0.0f) mn = -small * static_cast<float>(qmax - qmin);
+    else {
+      const float amp = small / org;
+      mn = mn * amp, mx = mx * amp;
+    }
+  }
+  const double ds = static_cast<double>(scale);
+  const double z_min = qmin - static_cast<double>(mn) / ds, z_max = qmax - static_cast<double>(mx) / ds;
+  const double e_min = std::fabs(static_cast<double>(qmin)) - std::fabs(static_cast<double>(mn) / ds);
+  const double e_max = std::fabs(static_cast<double>(qmax)) - std::fabs(static_cast<double>(mx) / ds);
+  double z = e_min < e_max ? z_min : z_max;
+  if (mn < 0 && mx > 0 && preserve_sparsity) z = (qmin + qmax) / 2.0;
+  const int32_t zp = z < qmin ? qmin : (z > qmax ? qmax : static_cast<int32_t>(std::nearbyint(z)));
+  return {scale, zp};
+}
+
+std::tuple<at::Tensor, at::Tensor> fused_moving_avg_obs_fq_helper(const at::Tensor& self, const at::Tensor& observer_on,
+                                                                   const at::Tensor& fake_quant_on, at::Tensor& running_min,
+                                                                   at::Tensor& running_max, at::Tensor& scale, at::Tensor& zero_point,
+                                                                   double averaging_const, int64_t quant_min, int64_t quant_max,
+                                                                   int64_t ch_axis, bool per_row_fake_quant, bool symmetric_quant) {
+  TORCH_CHECK(ch_axis < self.dim(), "Error in fused_moving_avg_obs_fake_quant_cpu: ch_axis must be < self.dim()");
+  const int dt = vkt_dtype(self.scalar_type());
+  TORCH_CHECK_NOT_IMPLEMENTED(dt == VKT_F32 || dt == VKT_F16 || dt == VKT_BF16, "torch_vulkan: the fake-quantisation observer takes float32, float16 and bfloat16 tensors");
+  const bool observe = observer_on.reshape({-1})[0].item<int64_t>() != 0;
+  at::Tensor x = self;
+  if (per_row_fake_quant) {
+    if (self.dim() != 2) {
+      std::vector<int64_t> perm(static_cast<size_t>(self.dim()));
+      for (size_t i = 0; i < perm.size(); ++i) perm[i] = static_cast<int64_t>(i);
+      perm[static_cast<size_t>(ch_axis)] = 0, perm[0] = ch_axis;
+      x = self.permute(perm).flatten(1);
+    }
+    const int64_t size = self.size(ch_axis);
+    if (running_min.numel() == 0) {
+      running_min.resize_({size}).fill_(std::numeric_limits<float>::infinity());
+      running_max.resize_({size}).fill_(-std::numeric_limits<float>::infinity());
+      scale.resize_({size});
+      zero_point.resize_({size});
+    }
+  }
+  // the running range lives on the device; its few values are updated on the host, as the reference does
+  at::Tensor rmin = running_min.to(at::kCPU, at::kFloat).contiguous().clone(), rmax = running_max.to(at::kCPU, at::kFloat).contiguous().clone();
+  if (observe) {
+    if (per_row_fake_quant) {
+      TORCH_CHECK(ch_axis == 0, "Per-channel FakeQuant in fused_moving_avg_obs_fake_quant is only supported on axis == 0");
+    }
+    at::Tensor rows = (per_row_fake_quant ? x : x.reshape({1, -1})).contiguous();
+    TORCH_CHECK(rows.size(0) == rmin.numel() && rows.size(0) < 65536 && rows.size(1) > 0 && rows.size(1) < (int64_t(1) << 32),
+                "torch_vulkan: the observer's running range has ", rmin.numel(), " values for ", rows.size(0), " rows");
+    at::Tensor cur_min = at::empty({rows.size(0)}, rows.options().dtype(at::kFloat)), cur_max = at::empty_like(cur_min);
+    MinMaxParams p{};
+    p.src = gpu_address(rows), p.out_min = gpu_address_out(cur_min), p.out_max = gpu_address_out(cur_max);
+    p.rows = static_cast<uint32_t>(rows.size(0)), p.cols = static_cast<uint32_t>(rows.size(1)), p.ld = p.cols;
+    p.dtype = static_cast<uint32_t>(dt);
+    dispatch("aminmax", {}, p, 1);
+    at::Tensor cmin = cur_min.cpu(), cmax = cur_max.cpu();
+    const float c = static_cast<float>(averaging_const);
+    float* lo = rmin.data_ptr<float>();
+    float* hi = rmax.data_ptr<float>();
+    const float* a = cmin.const_data_ptr<float>();
+    const float* b = cmax.const_data_ptr<float>();
+    for (int64_t i = 0; i < rmin.numel(); ++i) {
+      // (a value that is still infinite takes this batch's; single float32 operations, as the CPU's)
+      volatile float dl = a[i] - lo[i], dh = b[i] - hi[i];
+      volatile float pl = c * dl, ph = c * dh;
+      lo[i] = std::isinf(lo[i]) ? a[i] : lo[i] + pl;
+      hi[i] = std::isinf(hi[i]) ? b[i] : hi[i] + ph;
+    }
+    running_min.copy_(rmin.reshape(running_min.sizes()));
+    running_max.copy_(rmax.reshape(running_max.sizes()));
+  }
+  if (fake_quant_on.reshape({-1})[0].item<int64_t>() == 0) {
+    return {self.clone(at::MemoryFormat::Preserve), at::ones_like(self, self.options().dtype(at::kBool))};
+  }
+  const int64_t count = per_row_fake_quant ? rmin.numel() : 1;
+  at::Tensor scales = at::empty({count}, at::kFloat), zps = at::empty({count}, at::kInt);
+  for (int64_t i = 0; i < count; ++i) {
+    auto qp = choose_qparams(rmin.const_data_ptr<float>()[i], rmax.const_data_ptr<float>()[i], static_cast<int32_t>(quant_min),
+                             static_cast<int32_t>(quant_max), symmetric_quant);
+    scales.data_ptr<float>()[i] = qp.first, zps.data_ptr<int32_t>()[i] = qp.second;
+  }
+  scale.reshape({-1}).narrow(0, 0, count).copy_(scales);
+  zero_point.reshape({-1}).narrow(0, 0, count).copy_(zps.to(zero_point.scalar_type()));
+  if (per_row_fake_quant) return fake_quant_per_channel(self, scale, zero_point, ch_axis, quant_min, quant_max);
+  TORCH_CHECK(quant_min <= quant_max, "`quant_min` should be less than or \
+        equal to `quant_max`.");
+  return fake_quant_launch(self, nullptr, nullptr, scales.data_ptr<float>()[0], zps.data_ptr<int32_t>()[0], 0, quant_min, quant_max);
+}
+
 }  // namespace
 
 // A dense copy of quantised tensor q in memory format mf, its quantizer kept.
@@ -234,6 +348,7 @@ TORCH_LIBRARY_IMPL(aten, PrivateUse1, m) {
   m.impl("fake_quantize_per_tensor_affine_cachemask", TORCH_FN(vk::fake_quant_per_tensor));
   m.impl("fake_quantize_per_channel_affine_cachemask", TORCH_FN(vk::fake_quant_per_channel));
   m.impl("flip", TORCH_FN(vk::flip_raw));
+  m.impl("_fused_moving_avg_obs_fq_helper", TORCH_FN(vk::fused_moving_avg_obs_fq_helper));
 }
 
 TORCH_LIBRARY_IMPL(aten, QuantizedPrivateUse1, m) {
