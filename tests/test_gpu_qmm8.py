@@ -52,12 +52,14 @@ def test_qmm8_every_variant(variant, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("variant", [0, 1 | 4 << 8, 2 | 8 << 8, 4 | 16 << 8, 4 | 8 << 8 | 3 << 24, 1 | 4 << 8 | 16 << 24,
-                                     1 << 17])
+                                     1 << 17, 1 << 18, 1 | 4 << 8 | 1 << 18, 2 | 8 << 8 | 1 << 18, 4 | 4 << 8 | 1 << 18,
+                                     4 | 8 << 8 | 3 << 24 | 1 << 18, 2 | 4 << 8 | 16 << 24 | 1 << 18])
 @pytest.mark.parametrize("m,k,n", [(5, 1024, 40), (16, 4096, 67), (33, 2048, 130), (64, 4160, 96), (70, 512, 36)])
 def test_qmm8_matrix_core_variants(dtype, variant, m, k, n):
     """4 < M with 16-bit activations runs on the matrix cores: every (columns, k-split)
     instantiation, K sliced over several workgroups (bits 24+; the slices meet in the
-    library's workspace), and the GEMV kernels forced on the same problem (bit 17)."""
+    library's workspace), the GEMV kernels forced on the same problem (bit 17), and the kernel that stages the
+    weights through LDS (bit 18; up to 32 rows, otherwise the plain one runs)."""
     import _dev
     a, b, s = q8_case(dtype, m, k, n)
     check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=variant), a, b, s, dtype)

@@ -217,6 +217,44 @@ __device__ __forceinline__ void store_tiles(const Q8Params& p, uint32_t n0, cons
   }
 }
 
+// The partial tiles of a workgroup's waves added up in wave 0.  Where LDS holds half the waves' tiles, a
+// tree: in each round the upper half of the remaining waves hands its tiles to the lower half (two
+// barriers per round, log2(WAVES) rounds, a fixed order); otherwise wave by wave.
+template <int MT, int NT, int WAVES>
+constexpr int kPartSlots = (WAVES / 2) * MT * NT <= 32 ? WAVES / 2 : 1;
+
+template <int MT, int NT, int WAVES>
+__device__ __forceinline__ void add_wave_tiles(V4F (&acc)[MT][NT], V4F* part, int wave, int lane) {
+  if constexpr (kPartSlots<MT, NT, WAVES> > 1) {
+#pragma unroll
+    for (int half = WAVES / 2; half >= 1; half /= 2) {
+      if (wave >= half && wave < 2 * half) {
+#pragma unroll
+        for (int i = 0; i < MT * NT; ++i) part[((wave - half) * MT * NT + i) * 64 + lane] = acc[i / NT][i % NT];
+      }
+      __syncthreads();
+      if (wave < half) {
+#pragma unroll
+        for (int i = 0; i < MT * NT; ++i) acc[i / NT][i % NT] += part[(wave * MT * NT + i) * 64 + lane];
+      }
+      if (half > 1) __syncthreads();
+    }
+  } else {
+    for (int w = 1; w < WAVES; ++w) {
+      __syncthreads();
+      if (wave == w) {
+#pragma unroll
+        for (int i = 0; i < MT * NT; ++i) part[i * 64 + lane] = acc[i / NT][i % NT];
+      }
+      __syncthreads();
+      if (wave == 0) {
+#pragma unroll
+        for (int i = 0; i < MT * NT; ++i) acc[i / NT][i % NT] += part[i * 64 + lane];
+      }
+    }
+  }
+}
+
 template <class T, int MT, int NT, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma(Q8Params p, uint32_t chunks_per_slice, uint64_t workspace) {
   constexpr uint64_t item = 2;
@@ -251,8 +289,9 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma(Q8Params p, uint32_t chu
     for (int t = 0; t < NT; ++t) wv[t] = inside ? ldg_stream<U4>(brow[t] + k0) : zero;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      a0[mt] = inside ? ldg<U4>(arow[mt] + k0 * item) : zero;
-      a1[mt] = inside ? ldg<U4>(arow[mt] + k0 * item + 16) : zero;
+      const bool real = inside && uint32_t(16 * mt + c) < p.m;  // (rows past m are zeros, not loads)
+      a0[mt] = real ? ldg<U4>(arow[mt] + k0 * item) : zero;
+      a1[mt] = real ? ldg<U4>(arow[mt] + k0 * item + 16) : zero;
     }
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
@@ -266,24 +305,9 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma(Q8Params p, uint32_t chu
     }
   }
 
-  // partial tiles of waves 1.. are added to wave 0's in wave order
-  __shared__ V4F part[MT * NT][64];
-  for (int w = 1; w < WAVES; ++w) {
-    __syncthreads();
-    if (wave == w) {
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int t = 0; t < NT; ++t) part[mt * NT + t][lane] = acc[mt][t];
-    }
-    __syncthreads();
-    if (wave == 0) {
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[mt][t] += part[mt * NT + t][lane];
-    }
-  }
+  // the waves' partial tiles meet in wave 0
+  __shared__ V4F part[kPartSlots<MT, NT, WAVES>][MT * NT][64];
+  add_wave_tiles<MT, NT, WAVES>(acc, &part[0][0][0], wave, lane);
   if (wave != 0) return;
   if (gridDim.y > 1) {
     // one of several slices of K: the tile goes to the workspace, and qmm8_mfma_finish adds
@@ -291,6 +315,108 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma(Q8Params p, uint32_t chu
     V4F* const mine = reinterpret_cast<V4F*>(workspace) + (uint64_t(blockIdx.x) * gridDim.y + blockIdx.y) * (MT * NT * 64);
 #pragma unroll
     for (int i = 0; i < MT * NT; ++i) mine[i * 64 + lane] = acc[i / NT][i % NT];
+    return;
+  }
+  store_tiles<T, MT, NT>(p, n0, acc, lane);
+}
+
+// The same product with the weights staged through LDS, so that HBM sees long runs: a wave's
+// load instruction fetches 4 weight rows x 256 contiguous bytes (in qmm8_mfma it is 16 rows x 64
+// bytes, a pattern this memory system serves ~30 % slower) straight into the wave's own LDS
+// region (global_load_lds_dwordx4: lane l's 16 bytes land at region + 16 l).  The matrix-core
+// operand layout (lane (c, g): row c, bytes 16 g ..) is then a 16-byte LDS read.  The 16-byte
+// chunk q of row r sits at slot q ^ r, so that the 16 lanes of a read (rows 0..15, one logical
+// chunk) fall on 16 different slots of the 256-byte bank line; the swizzle costs nothing, the
+// lane simply fetches the chunk that belongs in its slot.  A wave works on chunks of 256
+// values of k: all loads of a chunk are issued, awaited (vmcnt(0)) and consumed; the waves of a
+// workgroup drift apart and keep the memory pipeline full between them.
+template <class T, int MT, int NT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void qmm8_mfma_staged(Q8Params p, uint32_t chunks_per_slice, uint64_t workspace) {
+  constexpr uint64_t item = 2;
+  constexpr uint32_t TILE = 16 * 256, REGION = NT * TILE;  // bytes of LDS per tile of 16 rows, per wave
+  extern __shared__ __attribute__((aligned(16))) uint8_t staged[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
+  uint8_t* const mine = staged + uint32_t(wave) * REGION;
+  const uint32_t total = (p.k + 255) / 256;
+  const uint32_t q_begin = blockIdx.y * chunks_per_slice;
+  const uint32_t q_end = q_begin + chunks_per_slice < total ? q_begin + chunks_per_slice : total;
+  const uint32_t n0 = blockIdx.x * 16 * NT;
+  // loads: instruction i of tile t fetches rows 4 i .. 4 i + 3; this lane row 4 i + (lane / 16), slot lane % 16
+  uint64_t wsrc[NT][4];
+  uint32_t wk[4];  // byte offset within the chunk of the 16 bytes this lane fetches
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t row = 4 * i + g;
+    wk[i] = ((uint32_t(c) ^ row) & 15u) * 16;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const uint32_t n = n0 + 16 * t + row < p.n ? n0 + 16 * t + row : p.n - 1;
+      wsrc[t][i] = p.b + uint64_t(n) * p.k;
+    }
+  }
+  uint64_t arow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const uint32_t m = uint32_t(16 * mt + c) < p.m ? 16 * mt + c : p.m - 1;
+    arow[mt] = p.a + uint64_t(int64_t(m) * p.a_sm * int64_t(item)) + 32 * g;
+  }
+  V4F acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[mt][t] = V4F{0.0f, 0.0f, 0.0f, 0.0f};
+
+  const U4 zero = {0, 0, 0, 0};
+  for (uint32_t q = q_begin + wave; q < q_end; q += WAVES) {
+    const uint32_t k0 = q * 256;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        // (bytes past k are fetched from the row's start instead: their activations are zeros below)
+        const uint64_t src = wsrc[t][i] + (k0 + wk[i] < p.k ? k0 + wk[i] : 0u);
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const VKT_GLOBAL void*>(src),
+                                         (__attribute__((address_space(3))) void*)(mine + (t * 16 + 4 * i) * 256), 16, 0, 0);
+      }
+    U4 a0[MT][4], a1[MT][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const bool inside = k0 + 64 * j + 16 * g < p.k;  // (k is a multiple of 16)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        // (rows past m are zeros, not loads: with 8 rows that is half of the activation traffic)
+        const bool real = inside && uint32_t(16 * mt + c) < p.m;
+        a0[mt][j] = real ? ldg<U4>(arow[mt] + (k0 + 64 * j) * item) : zero;
+        a1[mt][j] = real ? ldg<U4>(arow[mt] + (k0 + 64 * j) * item + 16) : zero;
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the chunk's weights are in LDS
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const U4 wv = *reinterpret_cast<const U4*>(mine + (t * 16 + c) * 256 + (((4 * j + g) ^ c) & 15) * 16);
+        U4 wlo, whi;
+        widen16_to_operands<T>(wv, &wlo, &whi);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          acc[mt][t] = mfma16<T>(wlo, a0[mt][j], acc[mt][t]);
+          acc[mt][t] = mfma16<T>(whi, a1[mt][j], acc[mt][t]);
+        }
+      }
+    }
+    // (the next chunk's loads overwrite the region: every read above has returned by then, as its value is used)
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+  }
+
+  // the waves' partial tiles meet in wave 0 (through the staging memory, once every wave is done with it)
+  __syncthreads();
+  add_wave_tiles<MT, NT, WAVES>(acc, reinterpret_cast<V4F*>(staged), wave, lane);
+  if (wave != 0) return;
+  if (gridDim.y > 1) {
+    V4F* const out = reinterpret_cast<V4F*>(workspace) + (uint64_t(blockIdx.x) * gridDim.y + blockIdx.y) * (MT * NT * 64);
+#pragma unroll
+    for (int i = 0; i < MT * NT; ++i) out[i * 64 + lane] = acc[i / NT][i % NT];
     return;
   }
   store_tiles<T, MT, NT>(p, n0, acc, lane);
@@ -323,6 +449,38 @@ void launch_mfma_waves(const Q8Params& p, int waves, uint32_t slices, const Mach
   if (slices > 1) hipLaunchKernelGGL((qmm8_mfma_finish<T, MT, NT>), dim3(grid.x), dim3(64), 0, stream, p, slices, mc.workspace);
 }
 
+template <class T, int MT, int NT, int WAVES>
+bool launch_staged_one(const Q8Params& p, uint32_t slices, const Machine& mc, hipStream_t stream) {
+  auto kernel = qmm8_mfma_staged<T, MT, NT, WAVES>;
+  constexpr uint32_t stage_bytes = WAVES * NT * 16 * 256, part_bytes = kPartSlots<MT, NT, WAVES> * MT * NT * 1024;
+  constexpr uint32_t lds = stage_bytes > part_bytes ? stage_bytes : part_bytes;
+  static bool configured = false;  // guarded by the runtime's stream mutex
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
+      (void)hipGetLastError();
+      return false;
+    }
+    configured = true;
+  }
+  const dim3 grid((p.n + 16 * NT - 1) / (16 * NT), slices);
+  const uint32_t chunks = (p.k + 255) / 256, per_slice = (chunks + slices - 1) / slices;
+  hipLaunchKernelGGL(kernel, grid, dim3(WAVES * 64), lds, stream, p, per_slice, mc.workspace);
+  if (slices > 1) hipLaunchKernelGGL((qmm8_mfma_finish<T, MT, NT>), dim3(grid.x), dim3(64), 0, stream, p, slices, mc.workspace);
+  return true;
+}
+
+// The staged kernel for up to 32 rows (MT <= 2: the activations of a chunk fit in registers next to the
+// accumulators).  variant = NT | WAVES << 8 | SLICES << 24 | 1 << 18.  False if this shape is not built.
+template <class T>
+bool launch_staged(const Q8Params& p, int mt, int nt, int waves, uint32_t slices, const Machine& mc, hipStream_t stream) {
+#define VKT_STAGED_CASE(MT_, NT_, W_) \
+  if (mt == MT_ && nt == NT_ && waves == W_) return launch_staged_one<T, MT_, NT_, W_>(p, slices, mc, stream);
+  VKT_STAGED_CASE(1, 1, 4) VKT_STAGED_CASE(1, 2, 4) VKT_STAGED_CASE(1, 4, 4) VKT_STAGED_CASE(1, 1, 8) VKT_STAGED_CASE(1, 2, 8) VKT_STAGED_CASE(1, 4, 8)
+  VKT_STAGED_CASE(2, 1, 4) VKT_STAGED_CASE(2, 2, 4) VKT_STAGED_CASE(2, 4, 4) VKT_STAGED_CASE(2, 1, 8) VKT_STAGED_CASE(2, 2, 8) VKT_STAGED_CASE(2, 4, 8)
+#undef VKT_STAGED_CASE
+  return false;
+}
+
 // Rows (<= 64) of 16-bit activations on the matrix cores.  A workgroup takes 64 columns
 // where there are that many, so that an activation fragment is reused over 4 weight
 // fragments (every workgroup reads all the activations of its slice of K from L2: with 16
@@ -346,6 +504,20 @@ void launch_mfma(const Q8Params& p, uint32_t variant, const Machine& mc, hipStre
     slices = want < most ? want : most;
     if (slices < 1) slices = 1;
     if (slices > 16) slices = 16;
+  }
+  // Up to 8 rows the kernel that stages the weights through LDS wins (measured at K = 4096 / N = 14336 and the
+  // reverse: 15.8 against 17.1 us, 15.1-16.4 against 17.3-18.4); from 16 rows on the activations' own traffic
+  // levels the two.  variant bit 18 asks for it explicitly, bit 19 for the plain kernel.
+  bool staged = (variant >> 18) & 1;
+  if (!(variant & 0xffff) && !((variant >> 19) & 1) && p.m <= 8 && p.k >= 2048 && p.n >= 64) {
+    staged = true;
+    nt = (p.k >= 16384 || (p.n >= 12288 && p.k <= 4096)) ? 2 : 1, waves = 8, slices = 1;  // (measured on the Llama shapes)
+  }
+  if (staged) {  // chunks of 256 values of k
+    const uint64_t sgroups = (p.n + 16 * nt - 1) / (16 * nt);
+    const uint32_t schunks = (p.k + 255) / 256;
+    while (slices > 1 && (sgroups * slices * mt * nt * 1024 > mc.workspace_bytes || (schunks + slices - 1) / slices * (slices - 1) >= schunks)) --slices;
+    if (mt <= 2 && launch_staged<T>(p, mt, nt, waves, slices, mc, stream)) return;
   }
   // the workspace holds groups * slices tiles of MT * NT KiB
   const uint64_t groups = (p.n + 16 * nt - 1) / (16 * nt);
@@ -407,8 +579,10 @@ int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipSt
     return 0;
   }
   if constexpr (T::dtype != VKT_F32) {
-    // variant bit 17 forces the GEMV kernels (tests, tuning)
-    if (p0.m > 4 && !((variant >> 17) & 1)) {
+    // From 3 rows on the matrix cores win: the GEMV kernels convert every weight and multiply it once per row on
+    // the vector units (measured at K = 4096, N = 14336: 10.5, 16.4, 23.0, 23.4 us for 1 to 4 rows; the matrix
+    // cores take 16 us for up to 8).  variant bit 17 forces the GEMV kernels (tests, tuning).
+    if (p0.m > 2 && !((variant >> 17) & 1)) {
       for (uint32_t r0 = 0; r0 < p0.m; r0 += 64) {
         Q8Params p = p0;
         p.m = p0.m - r0 < 64 ? p0.m - r0 : 64;
