@@ -122,7 +122,7 @@ def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030):
     cbytes = L.vkt_qmm4c_bytes(n, k, bs)
     dp = abi.Buffer.from_numpy(packed.numpy())
     first = abi.Buffer(cbytes)
-    layout = 1 if m > 4 else 0
+    layout = 1 if m > 3 else 0
     abi.dispatch("qmm4c_pack", [layout], abi.Q4PackParams(packed=dp.address, compact=first.address, n=n, k=k, bs=bs,
                                                     has_bias=1))
     abi.synchronize()

@@ -114,7 +114,7 @@ at::Tensor dyn_quant_pack_4bit_weight(const at::Tensor& weights, const at::Tenso
 }
 
 // Compact side-cars of packed weight vectors, per live packed tensor and layout (0: streamed
-// by the kernel for at most 4 rows, 1: for the matrix cores; a weight that sees both kinds of
+// by the kernel for at most 3 rows, 1: for the matrix cores; a weight that sees both kinds of
 // call holds both, each the size of the nibbles plus scales): keyed by the storage, its data
 // pointer and the tensor's version counter, dropped when the storage dies or the tensor is
 // written to.  (The reference streams the float32-expanded vector
@@ -195,7 +195,7 @@ at::Tensor dyn_quant_matmul_4bit(const at::Tensor& inp, const at::Tensor& packed
   const uint32_t groupwise = block_size != K ? 1u : 0u;
   const int64_t item = x.element_size();
 
-  const uint32_t layout = M > 4 ? 1u : 0u;
+  const uint32_t layout = M > 3 ? 1u : 0u;  // (measured at K = 4096, N = 11008: 4 rows take 19.0 us streaming, 15.3 on the matrix cores)
   at::Tensor compact = sidecar_for(packed, block_size, K, N, bias_elements != 0, layout);
   if (compact.defined()) {
     for (int64_t r0 = 0; r0 < M; r0 += kMaxRows) {
