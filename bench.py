@@ -80,8 +80,9 @@ def rotation(nbytes, floor_mib=512):
 
 
 # ------------------------------------------------------------------ workloads
-def wl_q8(abi, m, k, n, dtype, steps, warmup, seed=1020):
-    """_weight_int8pack_mm: x ~N(0,1) [m,k]; w int8 uniform [n,k]; scales ~U(0.005,0.02) [n]."""
+def wl_q8(abi, m, k, n, dtype, steps, warmup, seed=1020, prefill=False):
+    """_weight_int8pack_mm: x ~N(0,1) [m,k]; w int8 uniform [n,k]; scales ~U(0.005,0.02) [n].  prefill: many rows,
+    priced against the matrix cores' bf16 rate (the weights are widened once, then one tile-kernel product)."""
     import torch
     g = torch.Generator().manual_seed(seed)
     tdt = {abi.F32: torch.float32, abi.BF16: torch.bfloat16, abi.F16: torch.float16}[dtype]
@@ -103,6 +104,10 @@ def wl_q8(abi, m, k, n, dtype, steps, warmup, seed=1020):
     wall, ev = time_steps(abi, fns, steps, warmup)
     work = n * k + item * (m * k + n + m * n)  # weights once + activations + scales + output
     keep = (x, w, s)
+    if prefill:
+        return dict(kind="mfma", peak=BF16_PEAK_TFLOPS, metric="int8-weight prefill TFLOP/s (% of bf16 MFMA peak)", work=2 * m * n * k,
+                    wall_ms=wall, event_ms=ev, bytes=work, inputs=None, copies=len(copies),
+                    name=f"_weight_int8pack_mm {abi.SUFFIX[dtype]} M={m} K={k} N={n} (prefill)")
     return dict(kind="hbm", work=work, wall_ms=wall, event_ms=ev, flops=2 * m * n * k, inputs=keep,
                 name=f"_weight_int8pack_mm {abi.SUFFIX[dtype]} M={m} K={k} N={n}", copies=len(copies))
 
@@ -286,6 +291,8 @@ WORKLOADS = {
     "c2_m8_k14336_n4096": lambda abi, s, w: wl_q8(abi, 8, 14336, 4096, abi.BF16, s, w),
     "c2_m64_k4096_n14336": lambda abi, s, w: wl_q8(abi, 64, 4096, 14336, abi.BF16, s, w),
     "c2_m64_k14336_n4096": lambda abi, s, w: wl_q8(abi, 64, 14336, 4096, abi.BF16, s, w),
+    # many rows of the same operator (prefill; not a BASELINE configuration)
+    "c2_prefill_m4096_k4096_n14336": lambda abi, s, w: wl_q8(abi, 4096, 4096, 14336, abi.BF16, max(s // 20, 5), max(w // 4, 3), prefill=True),
     "c1_f32_m1_k4096_n4096": lambda abi, s, w: wl_q8(abi, 1, 4096, 4096, abi.F32, s, w, seed=1010),
     "c3_int4_m1": lambda abi, s, w: wl_q4(abi, 1, 4096, 11008, 32, s, w),
     "c3_int4_m32": lambda abi, s, w: wl_q4(abi, 32, 4096, 11008, 32, max(s // 4, 5), w),

@@ -68,6 +68,19 @@ def test_qmm8_matrix_core_variants(dtype, variant, m, k, n):
              rows=slice(None, None, 2))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,k,n", [(192, 512, 200), (2100, 64, 2060), (300, 1088, 7000), (1024, 256, 4100), (4096, 72, 2056)])
+def test_qmm8_many_rows(dtype, m, k, n):
+    """From 192 rows on (prefill) the weights are widened once into the library's scratch region and the product runs
+    on the tile kernel; the row-block kernels (variant bit 20) give the same results to the test's bound."""
+    import _dev
+    a, b, s = q8_case(dtype, m, k, n)
+    got = _dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s))
+    check_q8(got, a, b, s, dtype)
+    check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=1 << 20), a, b, s, dtype)
+    check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), row_step=2), a, b, s, dtype, rows=slice(None, None, 2))
+
+
 def test_qmm8_config1_vs_torch_cpu():
     """BASELINE config 1: fp32, M=1, K=N=4096, within rtol/atol 1e-4 of PyTorch's CPU op."""
     import _dev

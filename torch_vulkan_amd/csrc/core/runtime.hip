@@ -65,6 +65,29 @@ struct Runtime {
   bool trace = false;
   uint64_t generation = 0;
   void* workspace_base = nullptr;
+  void* scratch_base = nullptr;
+
+  // Grows the scratch region to at least `bytes` (never shrinks before vkt_empty_cache / shutdown).  hipFree waits
+  // for the device, so a region still in use by queued kernels is not pulled away.  Caller holds stream_mutex.
+  bool ensure_scratch(uint64_t bytes, std::string* err) {
+    if (bytes <= machine.scratch_bytes) return true;
+    if (scratch_base) (void)hipFree(scratch_base);
+    scratch_base = nullptr, machine.scratch = 0, machine.scratch_bytes = 0;
+    const uint64_t want = (bytes + (uint64_t(64) << 20) - 1) >> 26 << 26;  // whole 64 MiB
+    void* base = nullptr;
+    const hipError_t e = hipMalloc(&base, want);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      *err = hip_message("scratch allocation", e);
+      return false;
+    }
+    scratch_base = base, machine.scratch = reinterpret_cast<uint64_t>(base), machine.scratch_bytes = want;
+    return true;
+  }
+  void drop_scratch() {
+    if (scratch_base) (void)hipFree(scratch_base);
+    scratch_base = nullptr, machine.scratch = 0, machine.scratch_bytes = 0;
+  }
 
   ~Runtime() {
     if (stream) {
@@ -72,6 +95,7 @@ struct Runtime {
     }
     pool.reset();
     if (workspace_base) (void)hipFree(workspace_base);
+    if (scratch_base) (void)hipFree(scratch_base);
     if (stream) (void)hipStreamDestroy(stream);
   }
 };
@@ -180,6 +204,11 @@ int dispatch_named(Runtime& rt, const char* name, const uint32_t* spec, size_t n
     if (spec_at(0) != 0 && spec_at(0) != p.m) {
       *err = "qmm8: specialisation ROWS=" + std::to_string(spec_at(0)) + " does not match m=" + std::to_string(p.m);
       return -1;
+    }
+    // (many rows: the weights are widened into the scratch region first; without memory for it the row-block kernels run)
+    if (const uint64_t need = q8_gemm_scratch_bytes(p, dt, rt.machine); need != 0 && !((spec_at(1) >> 20) & 1)) {
+      std::string ignored;
+      (void)rt.ensure_scratch(need, &ignored);
     }
     return launch_qmm8(p, dt, spec_at(1), rt.machine, rt.stream, err);
   }
@@ -327,6 +356,10 @@ int vkt_empty_cache(void) {
   int rc = vkt_synchronize();
   std::lock_guard<std::mutex> lock(rt->pool_mutex);
   rt->pool->trim();
+  {
+    std::lock_guard<std::mutex> stream_lock(rt->stream_mutex);
+    rt->drop_scratch();
+  }
   return rc;
 }
 

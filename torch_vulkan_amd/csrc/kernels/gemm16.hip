@@ -99,7 +99,8 @@ int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t
   // variant 0: planned; 1: 128x128 tiles; 2: 256x128; 3: 256x256 with direct loads; 4: 128x128 with direct loads
   // (direct loads: k a multiple of 64; k-major operands run on the direct forms only)
   if (variant == 0) {
-    const bool large = uint64_t(p.m) * p.n >= (1ull << 20);
+    // 256 x 256 tiles where they give every compute unit one, else 128 x 128
+    const bool large = uint64_t((p.m + 255) / 256) * ((p.n + 255) / 256) * batch >= uint64_t(mc.compute_units);
     variant = large ? (direct_ok ? 3 : 2) : (TRA || TRB ? 4 : 1);
   }
   if constexpr (!TRA && !TRB) {
@@ -139,7 +140,114 @@ int launch_gemm16_t(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint3
   return launch_tiles<T, false, false>(p, use_cin, batch, variant, mc, stream, err);
 }
 
+// ---- _weight_int8pack_mm for many rows (prefill): the int8 weights are widened once into a scratch matrix of the
+// activations' type (exact) and the product runs on the tile kernel above, the per-column scales applied to the
+// float32 sums in the epilogue, as the decode kernels do.  The row-block kernels of qmm8.hip re-read every weight
+// once per 64 rows; from a few hundred rows on that costs more than the one extra pass over the weights.
+
+template <class T>
+struct Q8GemmProblem {
+  static constexpr bool kTransA = false, kTransB = false;
+  uint64_t a, b;
+  uint32_t m, n, k, lda, ldb, batches;
+  uint64_t a_batch, b_batch;
+  uint64_t c, scales;
+  struct Whole {
+    bool vec_ok;
+  };
+  struct Columns {
+    float s[4];
+  };
+  __device__ __forceinline__ Whole whole() const { return Whole{(n & 3u) == 0 && (c & 7u) == 0}; }
+  __device__ __forceinline__ Columns columns(uint32_t, uint32_t col, const Whole&) const {
+    Columns cs;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) cs.s[r] = load_f32<T>(scales + uint64_t(col + r < n ? col + r : n - 1) * 2);
+    return cs;
+  }
+  template <int DT>
+  __device__ __forceinline__ void store(uint32_t, uint32_t row, uint32_t col, const V4F& t, const Columns& cs, const Whole&) const {
+    float v[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) v[r] = t[r] * cs.s[r];
+    const uint64_t out = c + (uint64_t(row) * n + col) * 2;
+    if constexpr (DT >= 0) {
+      if constexpr (T::dtype == VKT_BF16) stg<U2>(out, U2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])});
+      else stg<U2>(out, U2{uint32_t(f32_to_f16(v[0])) | uint32_t(f32_to_f16(v[1])) << 16,
+                           uint32_t(f32_to_f16(v[2])) | uint32_t(f32_to_f16(v[3])) << 16});
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (col + r < n) store_f32<T>(out + 2 * r, v[r]);
+    }
+  }
+  template <class F>
+  __device__ __forceinline__ void for_output_type(bool full, const Whole& w, F&& f) const {
+    if (w.vec_ok && full) f(std::integral_constant<int, T::dtype>{});
+    else f(std::integral_constant<int, -1>{});
+  }
+};
+
+// 16 int8 values per thread -> 16 values of T (integers of magnitude <= 128 are exact in both 16-bit types).
+template <class T>
+__global__ __launch_bounds__(256) void widen_i8_kernel(uint64_t src, uint64_t dst, uint64_t groups) {
+  const uint64_t stride = uint64_t(gridDim.x) * 256;
+  for (uint64_t g = uint64_t(blockIdx.x) * 256 + threadIdx.x; g < groups; g += stride) {
+    const U4 v = ldg_stream<U4>(src + g * 16);
+    uint32_t out[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float f0 = float(int(int8_t(v[i]))), f1 = float(int(int8_t(v[i] >> 8)));
+      const float f2 = float(int(int8_t(v[i] >> 16))), f3 = float(int(int8_t(v[i] >> 24)));
+      if constexpr (T::dtype == VKT_BF16) {
+        out[2 * i] = __builtin_amdgcn_perm(f32_bits(f1), f32_bits(f0), 0x07060302u);
+        out[2 * i + 1] = __builtin_amdgcn_perm(f32_bits(f3), f32_bits(f2), 0x07060302u);
+      } else {
+        out[2 * i] = uint32_t(f32_to_f16(f0)) | uint32_t(f32_to_f16(f1)) << 16;
+        out[2 * i + 1] = uint32_t(f32_to_f16(f2)) | uint32_t(f32_to_f16(f3)) << 16;
+      }
+    }
+    stg<U4>(dst + g * 32, U4{out[0], out[1], out[2], out[3]});
+    stg<U4>(dst + g * 32 + 16, U4{out[4], out[5], out[6], out[7]});
+  }
+}
+
+template <class T>
+int launch_q8_gemm_t(const Q8Params& p, const Machine& mc, hipStream_t stream, std::string* err) {
+  constexpr int MATH = T::dtype == VKT_BF16 ? kMathBf16 : kMathF16;
+  const uint64_t groups = uint64_t(p.n) * p.k / 16, want = (groups + 255) / 256, cap = uint64_t(mc.compute_units) * 32;
+  hipLaunchKernelGGL(widen_i8_kernel<T>, dim3(uint32_t(want < cap ? want : cap)), dim3(256), 0, stream, p.b, mc.scratch, groups);
+  Q8GemmProblem<T> g;
+  g.a = p.a, g.b = mc.scratch, g.m = p.m, g.n = p.n, g.k = p.k * 2, g.lda = uint32_t(p.a_sm) * 2, g.ldb = p.k * 2;
+  g.batches = 1, g.a_batch = 0, g.b_batch = 0, g.c = p.c, g.scales = p.scales;
+  const bool large = uint64_t((p.m + 255) / 256) * ((p.n + 255) / 256) >= uint64_t(mc.compute_units);
+  if (g.k % BK == 0) {
+    if (large) return launch_mma_tile<2, 2, 8, 8, 0, 0, true, true, MATH>(g, mc.compute_units, stream, err, "qmm8");
+    return launch_mma_tile<2, 2, 4, 4, 0, 0, true, true, MATH>(g, mc.compute_units, stream, err, "qmm8");
+  }
+  if (large) return launch_mma_tile<2, 2, 8, 4, 0, 0, true, false, MATH>(g, mc.compute_units, stream, err, "qmm8");
+  return launch_mma_tile<2, 2, 4, 4, 0, 0, true, false, MATH>(g, mc.compute_units, stream, err, "qmm8");
+}
+
 }  // namespace
+
+uint64_t q8_gemm_scratch_bytes(const Q8Params& p, int dtype, const Machine& mc) {
+  // (worth it where 128 x 128 tiles give every compute unit one: fewer tiles leave most of the machine idle, and the
+  // row-block kernels, which split K, do better)
+  if (uint64_t((p.m + 127) / 128) * ((p.n + 127) / 128) < uint64_t(mc.compute_units)) return 0;
+  const bool fits = (dtype == VKT_BF16 || dtype == VKT_F16) && p.m >= kQ8GemmRows && p.k % 16 == 0 && p.a % 16 == 0 && p.b % 16 == 0 &&
+                    p.a_sm > 0 && p.a_sm % 8 == 0 && uint32_t(p.a_sm) >= p.k && p.a_sk == 1 && p.n > 0;
+  return fits ? uint64_t(p.n) * p.k * 2 : 0;
+}
+
+int launch_q8_gemm(const Q8Params& p, int dtype, const Machine& mc, hipStream_t stream, std::string* err) {
+  const int rc = dtype == VKT_BF16 ? launch_q8_gemm_t<bf16_t>(p, mc, stream, err) : launch_q8_gemm_t<f16_t>(p, mc, stream, err);
+  if (rc == 0 && hipGetLastError() != hipSuccess) {
+    *err = "qmm8: kernel launch failed";
+    return -1;
+  }
+  return rc;
+}
 
 int launch_gemm16(const GemmParams& p, int dtype, uint32_t use_cin, uint32_t batch, uint32_t variant, const Machine& mc,
                   hipStream_t stream, std::string* err) {

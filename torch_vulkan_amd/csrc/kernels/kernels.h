@@ -16,7 +16,16 @@ struct Machine {
   // device memory the runtime owns for kernels that split one product over several
   // workgroups: partial results between a kernel and the one that adds them up
   uint64_t workspace = 0, workspace_bytes = 0;
+  // a second region that the runtime grows on demand, for whole operands rewritten before a product
+  // (the int8 weights of a many-row product widened to 16 bits); queued uses are ordered by the one stream
+  uint64_t scratch = 0, scratch_bytes = 0;
 };
+
+// _weight_int8pack_mm with at least kQ8GemmRows rows of 16-bit activations runs as one tile-kernel product over
+// weights widened into the scratch region: the bytes of scratch it needs (0: not this path), and the launch.
+constexpr uint32_t kQ8GemmRows = 192;
+uint64_t q8_gemm_scratch_bytes(const Q8Params& p, int dtype, const Machine& mc);
+int launch_q8_gemm(const Q8Params& p, int dtype, const Machine& mc, hipStream_t stream, std::string* err);
 
 // spec[1] of the qmm8 kernels: 0 = planned by the library; otherwise an explicit
 // variant id (COLS | KSPLIT << 8 | FORCE_GENERIC << 16) used by tuning sweeps.

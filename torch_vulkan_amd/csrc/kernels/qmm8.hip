@@ -579,6 +579,10 @@ int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipSt
     return 0;
   }
   if constexpr (T::dtype != VKT_F32) {
+    // many rows (prefill): one product on the tile kernel over weights widened into the runtime's scratch region
+    // (variant bit 20 keeps the row-block kernels, for tests and tuning)
+    const uint64_t need = q8_gemm_scratch_bytes(p0, T::dtype, mc);
+    if (need != 0 && need <= mc.scratch_bytes && !((variant >> 20) & 1) && !(variant & 0xffff)) return launch_q8_gemm(p0, T::dtype, mc, stream, err);
     // From 3 rows on the matrix cores win: the GEMV kernels convert every weight and multiply it once per row on
     // the vector units (measured at K = 4096, N = 14336: 10.5, 16.4, 23.0, 23.4 us for 1 to 4 rows; the matrix
     // cores take 16 us for up to 8).  variant bit 17 forces the GEMV kernels (tests, tuning).
