@@ -81,6 +81,19 @@ def test_qmm8_many_rows(dtype, m, k, n):
     check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), row_step=2), a, b, s, dtype, rows=slice(None, None, 2))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("variant", [0, 1 << 21, 1 << 21 | 1 << 24, 1 << 21 | 3 << 24, 1 << 22])
+@pytest.mark.parametrize("m,k,n", [(16, 256, 128), (64, 1024, 200), (33, 2048, 130), (70, 512, 257), (130, 768, 96), (5, 512, 64)])
+def test_qmm8_tile_kernel(dtype, variant, m, k, n):
+    """More than 32 rows with k a multiple of 256 run on the tile kernel (64 x 128 tiles, K sliced over workgroups,
+    slices met in the workspace): planned, forced with 1 and 3 slices (bit 21; also with fewer rows), and switched off (bit 22)."""
+    import _dev
+    a, b, s = q8_case(dtype, m, k, n)
+    check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=variant), a, b, s, dtype)
+    if m > 8:
+        check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=variant, row_step=2), a, b, s, dtype, rows=slice(None, None, 2))
+
+
 def test_qmm8_config1_vs_torch_cpu():
     """BASELINE config 1: fp32, M=1, K=N=4096, within rtol/atol 1e-4 of PyTorch's CPU op."""
     import _dev

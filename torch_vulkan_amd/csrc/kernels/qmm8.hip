@@ -481,6 +481,195 @@ bool launch_staged(const Q8Params& p, int mt, int nt, int waves, uint32_t slices
   return false;
 }
 
+// 33 to a few hundred rows (batched decode): a tile kernel.  A workgroup of 8 waves owns 64 rows x 128 columns and a
+// slice of K, walked in steps of 256 values.  Both operand tiles of a step come straight into LDS
+// (global_load_lds_dwordx4, double buffered: the next step's loads are in flight while this one is multiplied): the
+// activations [64 rows][512 bytes] once per workgroup instead of once per wave, the raw int8 weights [128 rows][256
+// bytes] in runs of 256 contiguous bytes per row.  16-byte chunks are swizzled by the row's low 4 bits, so that the
+// operand-shaped reads (16 lanes = 16 rows at one logical chunk) are conflict free.  Wave (wm, wn) multiplies rows
+// 32 wm .. + 31 by columns 32 wn .. + 31 with V_MFMA_F32_16X16X32, the weights widened (exactly) as they leave LDS.
+// K is cut into slices across workgroups until the grid fills the machine; the slices' float32 tiles meet in the
+// runtime's workspace and qmm8_tile_finish adds them in slice order, scales and stores.
+constexpr uint32_t kTileStepK = 256;
+template <class T>
+__global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_slice, uint64_t workspace) {
+  constexpr uint32_t A_BYTES = 64 * 512, B_BYTES = 128 * 256, STAGE = A_BYTES + B_BYTES;
+  extern __shared__ __attribute__((aligned(16))) uint8_t tile_lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
+  const int wm = wave >> 2, wn = wave & 3;
+  const uint32_t n0 = blockIdx.x * 128, m0 = blockIdx.y * 64, slice = blockIdx.z;
+  const uint32_t steps = p.k / kTileStepK;
+  const uint32_t s_begin = slice * steps_per_slice, s_end = s_begin + steps_per_slice < steps ? s_begin + steps_per_slice : steps;
+
+  // loads of one step: activations 32 wave-loads of 2 rows x 512 bytes, weights 32 of 4 rows x 256 bytes; a wave issues 4 + 4
+  uint64_t a_src[4], b_src[4];
+  uint32_t a_dst[4], b_dst[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t row = (wave * 4 + i) * 2 + (lane >> 5), slot = lane & 31u;
+    const uint32_t m = m0 + row < p.m ? m0 + row : p.m - 1;
+    a_src[i] = p.a + uint64_t(int64_t(m) * p.a_sm * 2) + ((slot ^ (row & 15u)) * 16);
+    a_dst[i] = (wave * 4 + i) * 1024;  // (+ 16 * lane, by the hardware)
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t row = (wave * 4 + i) * 4 + (lane >> 4), slot = lane & 15u;
+    const uint32_t n = n0 + row < p.n ? n0 + row : p.n - 1;
+    b_src[i] = p.b + uint64_t(n) * p.k + ((slot ^ (row & 15u)) * 16);
+    b_dst[i] = A_BYTES + (wave * 4 + i) * 1024;
+  }
+  auto request = [&](uint32_t step, uint32_t stage) {
+    uint8_t* base = tile_lds + stage * STAGE;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const VKT_GLOBAL void*>(a_src[i] + uint64_t(step) * kTileStepK * 2),
+                                       (__attribute__((address_space(3))) void*)(base + a_dst[i]), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const VKT_GLOBAL void*>(b_src[i] + uint64_t(step) * kTileStepK),
+                                       (__attribute__((address_space(3))) void*)(base + b_dst[i]), 16, 0, 0);
+  };
+
+  V4F acc[2][2];
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+    for (int t = 0; t < 2; ++t) acc[mt][t] = V4F{0.0f, 0.0f, 0.0f, 0.0f};
+
+  if (s_begin < s_end) request(s_begin, 0);
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+  __syncthreads();
+  for (uint32_t step = s_begin; step < s_end; ++step) {
+    const uint32_t stage = (step - s_begin) & 1u;
+    if (step + 1 < s_end) request(step + 1, stage ^ 1u);
+    const uint8_t* ta = tile_lds + stage * STAGE;
+    const uint8_t* tb = ta + A_BYTES;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {  // 64 values of k each
+      U4 a0[2], a1[2];
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+        const uint32_t row = 32 * wm + 16 * mt + c;
+        a0[mt] = *reinterpret_cast<const U4*>(ta + row * 512 + (((8 * j + 2 * g) ^ (row & 15u)) * 16));
+        a1[mt] = *reinterpret_cast<const U4*>(ta + row * 512 + (((8 * j + 2 * g + 1) ^ (row & 15u)) * 16));
+      }
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const uint32_t row = 32 * wn + 16 * t + c;
+        const U4 wv = *reinterpret_cast<const U4*>(tb + row * 256 + (((4 * j + g) ^ (row & 15u)) * 16));
+        U4 wlo, whi;
+        widen16_to_operands<T>(wv, &wlo, &whi);
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+          acc[mt][t] = mfma16<T>(wlo, a0[mt], acc[mt][t]);
+          acc[mt][t] = mfma16<T>(whi, a1[mt], acc[mt][t]);
+        }
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the next step's tiles have landed
+    __syncthreads();                      // ... for every wave, and every wave is done reading this step's
+  }
+
+  // lane (c, g) holds, per tile (mt, t), row 32 wm + 16 mt + c, columns 32 wn + 16 t + 4 g .. + 3
+  const bool sliced = gridDim.z > 1;
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const uint32_t m = m0 + 32 * wm + 16 * mt + c, n = n0 + 32 * wn + 16 * t + 4 * g;
+      if (m >= p.m || n >= p.n) continue;
+      if (sliced) {
+        float* out = reinterpret_cast<float*>(workspace) + (uint64_t(slice) * p.m + m) * p.n + n;
+        if ((p.n & 3u) == 0) *reinterpret_cast<V4F*>(out) = acc[mt][t];
+        else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (n + r < p.n) out[r] = acc[mt][t][r];
+        }
+      } else {
+        uint32_t h[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float v = acc[mt][t][r] * load_f32<T>(p.scales + uint64_t(n + r < p.n ? n + r : p.n - 1) * 2);
+          h[r] = T::dtype == VKT_BF16 ? f32_to_bf16(v) : f32_to_f16(v);
+        }
+        const uint64_t at = p.c + (uint64_t(m) * p.n + n) * 2;
+        if ((p.n & 3u) == 0 && (p.c & 7u) == 0) stg<U2>(at, U2{h[0] | h[1] << 16, h[2] | h[3] << 16});
+        else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (n + r < p.n) stg<uint16_t>(at + 2 * r, uint16_t(h[r]));
+        }
+      }
+    }
+}
+
+// The slices of qmm8_tile added in slice order, scaled and stored: one thread per 4 consecutive outputs (n a multiple
+// of 4) or per output.
+template <class T>
+__global__ __launch_bounds__(256) void qmm8_tile_finish(Q8Params p, uint32_t slices, uint64_t workspace, uint32_t vec) {
+  const uint64_t total = uint64_t(p.m) * p.n, per = vec ? 4 : 1, i = (uint64_t(blockIdx.x) * 256 + threadIdx.x) * per;
+  if (i >= total) return;
+  const float* part = reinterpret_cast<const float*>(workspace);
+  float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (uint32_t s = 0; s < slices; ++s) {
+    if (vec) {
+      const V4F t = *reinterpret_cast<const V4F*>(part + uint64_t(s) * total + i);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) v[r] = s == 0 ? t[r] : v[r] + t[r];
+    } else {
+      const float t = part[uint64_t(s) * total + i];
+      v[0] = s == 0 ? t : v[0] + t;
+    }
+  }
+  const uint32_t n = uint32_t(i % p.n);
+  uint32_t h[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float y = v[r] * load_f32<T>(p.scales + uint64_t(n + r < p.n ? n + r : p.n - 1) * 2);
+    h[r] = T::dtype == VKT_BF16 ? f32_to_bf16(y) : f32_to_f16(y);
+  }
+  if (vec && (p.c & 7u) == 0) stg<U2>(p.c + i * 2, U2{h[0] | h[1] << 16, h[2] | h[3] << 16});
+  else {
+    for (uint32_t r = 0; r < per; ++r) stg<uint16_t>(p.c + (i + r) * 2, uint16_t(h[r]));
+  }
+}
+
+// Whether the tile kernel takes the product (rows a multiple of ... any; k a multiple of 256; 16-byte aligned rows), and its launch.
+template <class T>
+bool launch_tile_kernel(const Q8Params& p, uint32_t want_slices, const Machine& mc, hipStream_t stream) {
+  if (p.k % kTileStepK != 0 || p.k == 0 || (int64_t(p.a_sm) * 2) % 16 != 0 || p.a_sm <= 0) return false;
+  constexpr uint32_t lds = 2 * (64 * 512 + 128 * 256);
+  auto kernel = qmm8_tile<T>;
+  static bool configured = false;  // guarded by the runtime's stream mutex
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
+      (void)hipGetLastError();
+      return false;
+    }
+    configured = true;
+  }
+  const uint32_t gx = (p.n + 127) / 128, gy = (p.m + 63) / 64, steps = p.k / kTileStepK;
+  uint32_t slices = want_slices;
+  if (slices == 0) {  // about one workgroup per compute unit (measured: more slices cost more than they fill), 2 steps per slice at least
+    slices = (uint32_t(mc.compute_units) + gx * gy / 2) / (gx * gy);
+    const uint32_t most = steps / 2 ? steps / 2 : 1;
+    slices = slices > most ? most : slices;
+    slices = slices < 1 ? 1 : slices;
+  }
+  while (slices > 1 && uint64_t(slices) * p.m * p.n * 4 > mc.workspace_bytes) --slices;
+  uint32_t per_slice = (steps + slices - 1) / slices;
+  slices = (steps + per_slice - 1) / per_slice;
+  if (gy > 65535 || slices > 65535) return false;
+  hipLaunchKernelGGL(kernel, dim3(gx, gy, slices), dim3(512), lds, stream, p, per_slice, mc.workspace);
+  if (slices > 1) {
+    const uint32_t vec = (p.n & 3u) == 0;
+    const uint64_t threads = (uint64_t(p.m) * p.n + (vec ? 3 : 0)) / (vec ? 4 : 1);
+    hipLaunchKernelGGL(qmm8_tile_finish<T>, dim3(uint32_t((threads + 255) / 256)), dim3(256), 0, stream, p, slices, mc.workspace, vec);
+  }
+  return true;
+}
+
 // Rows (<= 64) of 16-bit activations on the matrix cores.  A workgroup takes 64 columns
 // where there are that many, so that an activation fragment is reused over 4 weight
 // fragments (every workgroup reads all the activations of its slice of K from L2: with 16
@@ -583,6 +772,11 @@ int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipSt
     // (variant bit 20 keeps the row-block kernels, for tests and tuning)
     const uint64_t need = q8_gemm_scratch_bytes(p0, T::dtype, mc);
     if (need != 0 && need <= mc.scratch_bytes && !((variant >> 20) & 1) && !(variant & 0xffff)) return launch_q8_gemm(p0, T::dtype, mc, stream, err);
+    // more than 32 rows (batched decode): the tile kernel (variant bit 21 forces it with bits 24+ slices, bit 22 keeps it off)
+    if (((p0.m > 32 && !(variant & 0xffff)) || ((variant >> 21) & 1)) && !((variant >> 22) & 1) && !((variant >> 17) & 1) && !((variant >> 18) & 1) &&
+        !((variant >> 19) & 1) && !((variant >> 20) & 1)) {
+      if (launch_tile_kernel<T>(p0, variant >> 24, mc, stream)) return 0;
+    }
     // From 3 rows on the matrix cores win: the GEMV kernels convert every weight and multiply it once per row on
     // the vector units (measured at K = 4096, N = 14336: 10.5, 16.4, 23.0, 23.4 us for 1 to 4 rows; the matrix
     // cores take 16 us for up to 8).  variant bit 17 forces the GEMV kernels (tests, tuning).
