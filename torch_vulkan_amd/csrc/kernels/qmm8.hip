@@ -25,6 +25,8 @@
 // Rows beyond the largest kernel's are served by the launcher in chunks (the weight stream
 // is then re-read per chunk).
 #include "common.h"
+#include <type_traits>
+
 #include "kernels.h"
 
 namespace vkt {
@@ -490,10 +492,10 @@ bool launch_staged(const Q8Params& p, int mt, int nt, int waves, uint32_t slices
 // 32 wm .. + 31 by columns 32 wn .. + 31 with V_MFMA_F32_16X16X32, the weights widened (exactly) as they leave LDS.
 // K is cut into slices across workgroups until the grid fills the machine; the slices' float32 tiles meet in the
 // runtime's workspace and qmm8_tile_finish adds them in slice order, scales and stores.
-constexpr uint32_t kTileStepK = 256;
+constexpr uint32_t kTileStepK = 128, kTileStages = 4;
 template <class T>
 __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_slice, uint64_t workspace) {
-  constexpr uint32_t A_BYTES = 64 * 512, B_BYTES = 128 * 256, STAGE = A_BYTES + B_BYTES;
+  constexpr uint32_t A_BYTES = 64 * 256, B_BYTES = 128 * 128, STAGE = A_BYTES + B_BYTES;
   extern __shared__ __attribute__((aligned(16))) uint8_t tile_lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
   const int wm = wave >> 2, wn = wave & 3;
@@ -501,31 +503,31 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
   const uint32_t steps = p.k / kTileStepK;
   const uint32_t s_begin = slice * steps_per_slice, s_end = s_begin + steps_per_slice < steps ? s_begin + steps_per_slice : steps;
 
-  // loads of one step: activations 32 wave-loads of 2 rows x 512 bytes, weights 32 of 4 rows x 256 bytes; a wave issues 4 + 4
-  uint64_t a_src[4], b_src[4];
-  uint32_t a_dst[4], b_dst[4];
+  // loads of one step: activations 16 wave-loads of 4 rows x 256 bytes, weights 16 of 8 rows x 128 bytes; a wave issues 2 + 2
+  uint64_t a_src[2], b_src[2];
+  uint32_t a_dst[2], b_dst[2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const uint32_t row = (wave * 4 + i) * 2 + (lane >> 5), slot = lane & 31u;
+  for (int i = 0; i < 2; ++i) {
+    const uint32_t row = (wave * 2 + i) * 4 + (lane >> 4), slot = lane & 15u;
     const uint32_t m = m0 + row < p.m ? m0 + row : p.m - 1;
     a_src[i] = p.a + uint64_t(int64_t(m) * p.a_sm * 2) + ((slot ^ (row & 15u)) * 16);
-    a_dst[i] = (wave * 4 + i) * 1024;  // (+ 16 * lane, by the hardware)
+    a_dst[i] = (wave * 2 + i) * 1024;  // (+ 16 * lane, by the hardware)
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const uint32_t row = (wave * 4 + i) * 4 + (lane >> 4), slot = lane & 15u;
+  for (int i = 0; i < 2; ++i) {
+    const uint32_t row = (wave * 2 + i) * 8 + (lane >> 3), slot = lane & 7u;
     const uint32_t n = n0 + row < p.n ? n0 + row : p.n - 1;
-    b_src[i] = p.b + uint64_t(n) * p.k + ((slot ^ (row & 15u)) * 16);
-    b_dst[i] = A_BYTES + (wave * 4 + i) * 1024;
+    b_src[i] = p.b + uint64_t(n) * p.k + ((slot ^ ((row >> 1) & 7u)) * 16);
+    b_dst[i] = A_BYTES + (wave * 2 + i) * 1024;
   }
-  auto request = [&](uint32_t step, uint32_t stage) {
-    uint8_t* base = tile_lds + stage * STAGE;
+  auto request = [&](uint32_t step) {
+    uint8_t* base = tile_lds + ((step - s_begin) % kTileStages) * STAGE;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 2; ++i)
       __builtin_amdgcn_global_load_lds(reinterpret_cast<const VKT_GLOBAL void*>(a_src[i] + uint64_t(step) * kTileStepK * 2),
                                        (__attribute__((address_space(3))) void*)(base + a_dst[i]), 16, 0, 0);
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 2; ++i)
       __builtin_amdgcn_global_load_lds(reinterpret_cast<const VKT_GLOBAL void*>(b_src[i] + uint64_t(step) * kTileStepK),
                                        (__attribute__((address_space(3))) void*)(base + b_dst[i]), 16, 0, 0);
   };
@@ -536,38 +538,67 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
 #pragma unroll
     for (int t = 0; t < 2; ++t) acc[mt][t] = V4F{0.0f, 0.0f, 0.0f, 0.0f};
 
-  if (s_begin < s_end) request(s_begin, 0);
-  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
-  __syncthreads();
-  for (uint32_t step = s_begin; step < s_end; ++step) {
-    const uint32_t stage = (step - s_begin) & 1u;
-    if (step + 1 < s_end) request(step + 1, stage ^ 1u);
-    const uint8_t* ta = tile_lds + stage * STAGE;
+  // Fragments of step s + 1 are read from LDS (12 reads per lane, into the other of two register sets) while step s is
+  // widened and multiplied, so the LDS, the vector units and the matrix cores work at the same time; two further steps
+  // are in flight from memory.  Loads land in the order issued: "at most 4 outstanding" (one step's worth per wave)
+  // means everything older has landed.
+  U4 fa0[2][2][2], fa1[2][2][2], fw[2][2][2];  // [register set][64-value half][tile]
+  auto read_fragments = [&](auto set, uint32_t step) {
+    constexpr int S = decltype(set)::value;
+    const uint8_t* ta = tile_lds + ((step - s_begin) % kTileStages) * STAGE;
     const uint8_t* tb = ta + A_BYTES;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {  // 64 values of k each
-      U4 a0[2], a1[2];
-#pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
-        const uint32_t row = 32 * wm + 16 * mt + c;
-        a0[mt] = *reinterpret_cast<const U4*>(ta + row * 512 + (((8 * j + 2 * g) ^ (row & 15u)) * 16));
-        a1[mt] = *reinterpret_cast<const U4*>(ta + row * 512 + (((8 * j + 2 * g + 1) ^ (row & 15u)) * 16));
-      }
+    for (int j = 0; j < 2; ++j) {
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
         const uint32_t row = 32 * wn + 16 * t + c;
-        const U4 wv = *reinterpret_cast<const U4*>(tb + row * 256 + (((4 * j + g) ^ (row & 15u)) * 16));
-        U4 wlo, whi;
-        widen16_to_operands<T>(wv, &wlo, &whi);
+        fw[S][j][t] = *reinterpret_cast<const U4*>(tb + row * 128 + (((4 * j + g) ^ ((row >> 1) & 7u)) * 16));
+      }
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
-          acc[mt][t] = mfma16<T>(wlo, a0[mt], acc[mt][t]);
-          acc[mt][t] = mfma16<T>(whi, a1[mt], acc[mt][t]);
-        }
+      for (int mt = 0; mt < 2; ++mt) {
+        const uint32_t row = 32 * wm + 16 * mt + c;
+        fa0[S][j][mt] = *reinterpret_cast<const U4*>(ta + row * 256 + (((8 * j + 2 * g) ^ (row & 15u)) * 16));
+        fa1[S][j][mt] = *reinterpret_cast<const U4*>(ta + row * 256 + (((8 * j + 2 * g + 1) ^ (row & 15u)) * 16));
       }
     }
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the next step's tiles have landed
-    __syncthreads();                      // ... for every wave, and every wave is done reading this step's
+  };
+  auto multiply = [&](auto set) {
+    constexpr int S = decltype(set)::value;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        U4 wlo, whi;
+        widen16_to_operands<T>(fw[S][j][t], &wlo, &whi);
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) acc[mt][t] = mfma16<T>(wlo, fa0[S][j][mt], acc[mt][t]);
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) acc[mt][t] = mfma16<T>(whi, fa1[S][j][mt], acc[mt][t]);
+      }
+  };
+  auto iteration = [&](auto set, uint32_t step) {
+    constexpr int S = decltype(set)::value;
+    // step + 1 must have landed (step + 2 may still be in flight), for every wave; and every wave must be done with
+    // the registers-from-LDS reads of step (issued an iteration ago, consumed below) before its stage is reused
+    if (step + 2 < s_end) __builtin_amdgcn_s_waitcnt(0x0f74);  // vmcnt(4)
+    else __builtin_amdgcn_s_waitcnt(0x0f70);                   // vmcnt(0)
+    __syncthreads();
+    if (step + 3 < s_end) request(step + 3);  // (into the stage that step - 1 was read from: all of its reads have returned)
+    if (step + 1 < s_end) read_fragments(std::integral_constant<int, S ^ 1>{}, step + 1);
+    __builtin_amdgcn_sched_barrier(0);  // (the scheduler would move each read down to its first use)
+    multiply(set);
+  };
+#pragma unroll
+  for (uint32_t ahead = 0; ahead < 3; ++ahead)
+    if (s_begin + ahead < s_end) request(s_begin + ahead);
+  if (s_begin + 2 < s_end) __builtin_amdgcn_s_waitcnt(0x0f78);       // vmcnt(8): the first of three steps has landed
+  else if (s_begin + 1 < s_end) __builtin_amdgcn_s_waitcnt(0x0f74);  // vmcnt(4)
+  else __builtin_amdgcn_s_waitcnt(0x0f70);                           // vmcnt(0)
+  __syncthreads();
+  if (s_begin < s_end) read_fragments(std::integral_constant<int, 0>{}, s_begin);
+  for (uint32_t step = s_begin; step < s_end; step += 2) {
+    iteration(std::integral_constant<int, 0>{}, step);
+    if (step + 1 < s_end) iteration(std::integral_constant<int, 1>{}, step + 1);
   }
 
   // lane (c, g) holds, per tile (mt, t), row 32 wm + 16 mt + c, columns 32 wn + 16 t + 4 g .. + 3
@@ -635,11 +666,11 @@ __global__ __launch_bounds__(256) void qmm8_tile_finish(Q8Params p, uint32_t sli
   }
 }
 
-// Whether the tile kernel takes the product (rows a multiple of ... any; k a multiple of 256; 16-byte aligned rows), and its launch.
+// Launches the tile kernel if it takes the product (k a multiple of its step, 16-byte aligned activation rows).
 template <class T>
 bool launch_tile_kernel(const Q8Params& p, uint32_t want_slices, const Machine& mc, hipStream_t stream) {
   if (p.k % kTileStepK != 0 || p.k == 0 || (int64_t(p.a_sm) * 2) % 16 != 0 || p.a_sm <= 0) return false;
-  constexpr uint32_t lds = 2 * (64 * 512 + 128 * 256);
+  constexpr uint32_t lds = kTileStages * (64 * 256 + 128 * 128);
   auto kernel = qmm8_tile<T>;
   static bool configured = false;  // guarded by the runtime's stream mutex
   if (!configured) {
@@ -653,7 +684,7 @@ bool launch_tile_kernel(const Q8Params& p, uint32_t want_slices, const Machine& 
   uint32_t slices = want_slices;
   if (slices == 0) {  // about one workgroup per compute unit (measured: more slices cost more than they fill), 2 steps per slice at least
     slices = (uint32_t(mc.compute_units) + gx * gy / 2) / (gx * gy);
-    const uint32_t most = steps / 2 ? steps / 2 : 1;
+    const uint32_t most = steps / 4 ? steps / 4 : 1;
     slices = slices > most ? most : slices;
     slices = slices < 1 ? 1 : slices;
   }
