@@ -643,12 +643,22 @@ __global__ __launch_bounds__(256) void qmm8_tile_finish(Q8Params p, uint32_t sli
   if (i >= total) return;
   const float* part = reinterpret_cast<const float*>(workspace);
   float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (uint32_t s = 0; s < slices; ++s) {
-    if (vec) {
-      const V4F t = *reinterpret_cast<const V4F*>(part + uint64_t(s) * total + i);
+  if (vec) {
+    // eight slices' loads are in flight together; the additions keep the slice order
+    for (uint32_t s0 = 0; s0 < slices; s0 += 8) {
+      V4F t[8];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) v[r] = s == 0 ? t[r] : v[r] + t[r];
-    } else {
+      for (uint32_t u = 0; u < 8; ++u)
+        if (s0 + u < slices) t[u] = *reinterpret_cast<const V4F*>(part + uint64_t(s0 + u) * total + i);
+#pragma unroll
+      for (uint32_t u = 0; u < 8; ++u)
+        if (s0 + u < slices) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) v[r] = s0 + u == 0 ? t[u][r] : v[r] + t[u][r];
+        }
+    }
+  } else {
+    for (uint32_t s = 0; s < slices; ++s) {
       const float t = part[uint64_t(s) * total + i];
       v[0] = s == 0 ? t : v[0] + t;
     }
