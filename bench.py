@@ -32,6 +32,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 FP8_PEAK_TFLOPS = 5000.0    # MI355X dense fp8 MFMA, published
 BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 / fp16 MFMA, published
+INT8_PEAK_TOPS = 5000.0     # MI355X dense int8 MFMA, published
 
 
 def _abi():
@@ -112,7 +113,7 @@ def wl_q8(abi, m, k, n, dtype, steps, warmup, seed=1020, prefill=False):
                 name=f"_weight_int8pack_mm {abi.SUFFIX[dtype]} M={m} K={k} N={n}", copies=len(copies))
 
 
-def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030):
+def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030, prefill=False):
     """_dyn_quant_matmul_4bit on the compact side-car: up to 4 rows the streaming layout with
     row quantisation fused into the launch, above that the matrix-core layout (two launches)."""
     import torch
@@ -147,6 +148,10 @@ def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030):
         fns.append(Launch(abi, "qmm4c_f32", [2, 1, layout], p))  # row quantisation + product
     wall, ev = time_steps(abi, fns, steps, warmup)
     work = n * k // 2 + 4 * n * (k // bs) + 4 * n + 4 * m * k + 4 * m * n
+    if prefill:  # many rows: the matrix cores' int8 rate is the published bound
+        return dict(kind="mfma", peak=INT8_PEAK_TOPS, metric="int4-weight prefill TOP/s (% of int8 MFMA peak)", work=2 * m * n * k,
+                    wall_ms=wall, event_ms=ev, bytes=work, inputs=None, copies=len(copies),
+                    name=f"_dyn_quant_matmul_4bit f32 M={m} K={k} N={n} bs={bs} (prefill)")
     return dict(kind="hbm", work=work, wall_ms=wall, event_ms=ev, flops=2 * m * n * k, inputs=(x, packed),
                 name=f"_dyn_quant_matmul_4bit f32 M={m} K={k} N={n} bs={bs} (compact side-car)", copies=len(copies),
                 reference_layout_bytes=int(packed.numel()) * 4 + 4 * m * k + 4 * m * n)
@@ -296,6 +301,8 @@ WORKLOADS = {
     "c1_f32_m1_k4096_n4096": lambda abi, s, w: wl_q8(abi, 1, 4096, 4096, abi.F32, s, w, seed=1010),
     "c3_int4_m1": lambda abi, s, w: wl_q4(abi, 1, 4096, 11008, 32, s, w),
     "c3_int4_m32": lambda abi, s, w: wl_q4(abi, 32, 4096, 11008, 32, max(s // 4, 5), w),
+    # many rows of the same operator (prefill; not a BASELINE configuration)
+    "c3_int4_prefill_m2048": lambda abi, s, w: wl_q4(abi, 2048, 4096, 11008, 32, max(s // 10, 5), w, prefill=True),
     "c4_fp8_8192": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 10, 5), max(w // 4, 3)),
     "c5_fp8_rowwise_70b": lambda abi, s, w: wl_fp8(abi, 4096, 8192, 28672, True, max(s // 10, 5), max(w // 4, 3),
                                                    seed=1050),

@@ -75,9 +75,10 @@ class CompactWeights:
         dp.free()
 
 
-def q4_compact(x, odt, cw, fused=True):
+def q4_compact(x, odt, cw, fused=True, flags=0):
     """_dyn_quant_matmul_4bit through the streaming path ("qmm4c_*"): one fused launch
-    (PHASE 2), or row quantisation (PHASE 0) then the product (PHASE 1)."""
+    (PHASE 2), or row quantisation (PHASE 0) then the product (PHASE 1).  flags (matrix-core layout): 16 keeps the
+    one-row-tile kernel, 32 forces the wave-per-tile kernel (| 64: one tile per wave, | 128: two, | 192: four)."""
     x = np.ascontiguousarray(x)
     m, n, k, bs = x.shape[0], cw.n, cw.k, cw.bs
     dx = abi.Buffer.from_numpy(x)
@@ -89,10 +90,10 @@ def q4_compact(x, odt, cw, fused=True):
     g = int(bs != k)
     name = "qmm4c_" + abi.SUFFIX[odt]
     if m and n and fused:
-        abi.dispatch(name, [2, g, cw.layout], p, ((n + 31) // 32, (m + 7) // 8))
+        abi.dispatch(name, [2 | flags, g, cw.layout], p, ((n + 31) // 32, (m + 7) // 8))
     elif m and n:
         abi.dispatch(name, [0, g, cw.layout], p, (m,))
-        abi.dispatch(name, [1, g, cw.layout], p, ((n + 31) // 32, (m + 7) // 8))
+        abi.dispatch(name, [1 | flags, g, cw.layout], p, ((n + 31) // 32, (m + 7) // 8))
     return do.to_numpy(_NP[odt], (m, n))
 
 

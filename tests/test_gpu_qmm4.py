@@ -17,7 +17,9 @@ EXTRA = [(2, 4096, 300, 32, True), (3, 14336, 20, 32, True), (9, 28672, 6, 128, 
          (6, 4160, 10, 4160, True), (1, 32, 1, 32, False), (5, 8, 3, 8, True),
          # more than 4 rows: the matrix-core layout's row tiles (16 rows each, 64 rows per launch)
          (70, 512, 40, 64, True), (33, 1056, 17, 32, False), (16, 4096, 64, 128, True), (20, 4160, 10, 4160, False),
-         (130, 96, 33, 32, True), (17, 2048, 16, 256, False)]
+         (130, 96, 33, 32, True), (17, 2048, 16, 256, False),
+         # many rows: a wave per tile that walks all of K, every block size of the matrix-core layout
+         (64, 4160, 40, 4160, True), (200, 1024, 48, 128, False), (100, 2048, 20, 256, True), (49, 640, 130, 64, False)]
 
 
 @pytest.mark.parametrize("m,k,n,bs,bias", Q4_CASES + EXTRA)
@@ -45,6 +47,11 @@ def test_q4_bit_exact(m, k, n, bs, bias, dtype):
         cm = _dev.CompactWeights(packed.numpy(), bs, k, n, layout=1)
         assert np.array_equal(_dev.q4_compact(bits(x), odt, cm, fused=True), want)
         assert np.array_equal(_dev.q4_compact(bits(x), odt, cm, fused=False), want)
+        if m > 4:  # both matrix-core kernels, whichever the row count selects
+            assert np.array_equal(_dev.q4_compact(bits(x), odt, cm, fused=False, flags=16), want)
+            assert np.array_equal(_dev.q4_compact(bits(x), odt, cm, fused=True, flags=32 | 64), want)
+            assert np.array_equal(_dev.q4_compact(bits(x), odt, cm, fused=False, flags=32 | 128), want)
+            assert np.array_equal(_dev.q4_compact(bits(x), odt, cm, fused=True, flags=32 | 192), want)
 
 
 @pytest.mark.parametrize("m", [1, 32])

@@ -888,6 +888,206 @@ __global__ __launch_bounds__(256) void qmm4m_tile(Q4CParams p, MatrixLayout L, u
   }
 }
 
+// Many rows: a wave per tile of RT x CT matrix-core tiles (16 rows x 16 columns each).  A workgroup is 4 waves
+// with the same rows and neighbouring column tiles (the activations, the larger operand, come from the vector cache
+// for three of them).  Each wave walks all of K by itself, so the block terms of its outputs come in block order and
+// are added in registers: no LDS, no barriers.  Operands are requested kRowsAhead quads ahead, always (past the end
+// the last quad again), so that the loop body is straight-line code.
+constexpr int kRowsAhead = 2;
+
+template <class T, int UPB, int RT, int CT>
+__global__ __launch_bounds__(256) void qmm4m_rows(Q4CParams p, MatrixLayout L, uint32_t m0) {
+  constexpr uint64_t item = sizeof(typename T::storage);
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t col = lane & 15, kg = lane >> 4;
+  const uint32_t tile0 = (blockIdx.x * 4 + wave) * CT;
+  const uint32_t row0 = m0 + blockIdx.y * (16 * RT);
+  if (row0 >= p.m || tile0 >= L.tiles) return;  // (a whole wave, and the kernel has no barrier)
+
+  V4I unit_const[RT];  // -256 nzp, for the rows this lane receives
+  int nzp_r[RT][4];
+  long nz_a[RT], nz_b[RT];
+  uint64_t qbase[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    const uint32_t rt = row0 + 16 * t < p.m ? row0 + 16 * t : row0;  // (a row tile past the end: the first again, not stored)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const uint32_t m = rt + kg * 4 + r < p.m ? rt + kg * 4 + r : p.m - 1;
+      nzp_r[t][r] = ldg<int32_t>(p.rows + 8ull * m + 4);
+      unit_const[t][r] = -256 * nzp_r[t][r];
+    }
+    const uint32_t m = rt + col < p.m ? rt + col : p.m - 1;
+    const int nzp = ldg<int32_t>(p.rows + 8ull * m + 4);
+    const int h1 = nzp >> 1, h2 = nzp - h1;
+    const uint32_t w1 = (uint32_t(h1) & 255u) * 0x01010101u, w2 = (uint32_t(h2) & 255u) * 0x01010101u;
+    nz_a[t] = long(uint64_t(w1) | uint64_t(w1) << 32);
+    nz_b[t] = long(uint64_t(w2) | uint64_t(w2) << 32);
+    qbase[t] = p.q + (uint64_t(rt >> 4) * L.quads * 128 + lane) * 16;
+  }
+  const long minus8 = long(0xf8f8f8f8f8f8f8f8ull);
+  const V4I minus8x4 = V4I{int(0xf8f8f8f8u), int(0xf8f8f8f8u), int(0xf8f8f8f8u), int(0xf8f8f8f8u)};
+  V4I nz_a4[RT], nz_b4[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    nz_a4[t] = V4I{int(nz_a[t]), int(nz_a[t]), int(nz_a[t]), int(nz_a[t])};
+    nz_b4[t] = V4I{int(nz_b[t]), int(nz_b[t]), int(nz_b[t]), int(nz_b[t])};
+  }
+  uint64_t wbase[CT], sbase[CT];
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    const uint32_t tile = tile0 + c < L.tiles ? tile0 + c : tile0;
+    wbase[c] = p.compact + (uint64_t(tile) * 64 + lane) * 16;
+    sbase[c] = p.compact + L.scale_off + (uint64_t(tile) * 16 + col) * 16;
+  }
+  const uint64_t wstep = uint64_t(L.tiles) * 1024, sstep = uint64_t(L.tiles) * 256;
+
+  struct Set {
+    U4 w[CT], q0[RT], q1[RT];
+    F4 s[CT];
+  };
+  Set sets[kRowsAhead];
+  auto request = [&](Set& set, uint32_t quad) {
+    quad = quad < L.quads ? quad : L.quads - 1;
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      set.q0[t] = ldg<U4>(qbase[t] + uint64_t(quad) * 2048);
+      set.q1[t] = ldg<U4>(qbase[t] + uint64_t(quad) * 2048 + 1024);
+    }
+#pragma unroll
+    for (int c = 0; c < CT; ++c) {
+      set.w[c] = ldg_stream<U4>(wbase[c] + quad * wstep);
+      if constexpr (UPB != 0) set.s[c] = ldg<F4>(sbase[c] + quad * sstep);
+    }
+  };
+#pragma unroll
+  for (int i = 0; i < kRowsAhead; ++i) request(sets[i], i);
+
+  float acc[RT][CT][4];
+  V4I d[RT][CT], d2[RT][CT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t)
+#pragma unroll
+    for (int c = 0; c < CT; ++c) {
+      d[t][c] = d2[t][c] = V4I{0, 0, 0, 0};
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[t][c][r] = -0.0f;
+    }
+  // (quads is a multiple of 16, so of kRowsAhead, and blocks of up to 8 units start at even quads)
+  for (uint32_t quad0 = 0; quad0 < L.quads; quad0 += kRowsAhead) {
+#pragma unroll
+    for (int i = 0; i < kRowsAhead; ++i) {
+      const Set cur = sets[i];
+      request(sets[i], quad0 + i + kRowsAhead);
+      constexpr int mask = UPB ? UPB - 1 : 0;
+      if constexpr (UPB == 1) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          long b[CT];
+#pragma unroll
+          for (int c = 0; c < CT; ++c) {
+            const uint32_t v = cur.w[c][j];
+            b[c] = long(uint64_t(v & 0x0f0f0f0fu) | uint64_t((v >> 4) & 0x0f0f0f0fu) << 32);
+          }
+#pragma unroll
+          for (int t = 0; t < RT; ++t) {
+            const U4& qq = j < 2 ? cur.q0[t] : cur.q1[t];
+            const long a = long(uint64_t(qq[(j & 1) * 2]) | uint64_t(qq[(j & 1) * 2 + 1]) << 32);
+#pragma unroll
+            for (int c = 0; c < CT; ++c) {
+              V4I x = unit_const[t];
+              x = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b[c], x, 0, 0, 0);
+              x = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, minus8, x, 0, 0, 0);
+              x = __builtin_amdgcn_mfma_i32_16x16x32_i8(nz_a[t], b[c], x, 0, 0, 0);
+              x = __builtin_amdgcn_mfma_i32_16x16x32_i8(nz_b[t], b[c], x, 0, 0, 0);
+#pragma unroll
+              for (int r = 0; r < 4; ++r) acc[t][c][r] = acc[t][c][r] + float(x[r]) * cur.s[c][j];  // in block order
+            }
+          }
+        }
+      } else {
+        // Blocks of two units and more: two units, 64 values of k, per matrix-core instruction (the full-rate form),
+        // and the zero-point products as a chain of their own (integers: any order).
+#pragma unroll
+        for (int j = 0; j < 4; j += 2) {
+          const int u = i * 4 + j;
+          const bool first = UPB != 0 && (u & mask) == 0, last = UPB != 0 && ((u + 1) & mask) == mask;
+          V4I b[CT];
+#pragma unroll
+          for (int c = 0; c < CT; ++c) {
+            const uint32_t v0 = cur.w[c][j], v1 = cur.w[c][j + 1];
+            b[c] = V4I{int(v0 & 0x0f0f0f0fu), int((v0 >> 4) & 0x0f0f0f0fu), int(v1 & 0x0f0f0f0fu), int((v1 >> 4) & 0x0f0f0f0fu)};
+          }
+#pragma unroll
+          for (int t = 0; t < RT; ++t) {
+            const U4& qq = j < 2 ? cur.q0[t] : cur.q1[t];
+            const V4I a = V4I{int(qq[0]), int(qq[1]), int(qq[2]), int(qq[3])};
+#pragma unroll
+            for (int c = 0; c < CT; ++c) {
+              V4I x = first ? unit_const[t] * (UPB ? UPB : 1) : d[t][c];
+              V4I y = first ? V4I{0, 0, 0, 0} : d2[t][c];
+              x = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[c], x, 0, 0, 0);
+              y = __builtin_amdgcn_mfma_i32_16x16x64_i8(nz_a4[t], b[c], y, 0, 0, 0);
+              x = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, minus8x4, x, 0, 0, 0);
+              y = __builtin_amdgcn_mfma_i32_16x16x64_i8(nz_b4[t], b[c], y, 0, 0, 0);
+              d2[t][c] = y;
+              if (last) {  // the block's term, added in block order
+                x = x + y;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[t][c][r] = acc[t][c][r] + float(x[r]) * cur.s[c][j + 1];
+              }
+              d[t][c] = x;
+            }
+          }
+        }
+      }
+    }
+    // The four matrix-core instructions of a unit are a dependent chain, 16 cycles apart: with one tile per wave the
+    // float32 work of the unit before it (4 conversions, 4 products, 4 sums, and the unpacking) is put in between,
+    // four instructions at a time.  (With more tiles per wave the chains of the tiles overlap by themselves, and
+    // prescribing the order made those kernels slower.)
+    if constexpr (UPB != 0 && RT * CT == 1) {
+#pragma unroll
+      for (int g = 0; g < kRowsAhead * 4 * 4; ++g) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    const uint32_t n = (tile0 + c) * kTileCols + col;
+    if (tile0 + c >= L.tiles || n >= p.n) continue;
+    const float bias = ldg<float>(p.compact + L.bias_off + n * 4ull);
+    float s = 0.0f;
+    if constexpr (UPB == 0) s = ldg<float>(p.compact + L.scale_off + n * 4ull);
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const uint32_t m = row0 + 16 * t + kg * 4 + r;
+        if (m >= p.m) continue;
+        float v = acc[t][c][r];
+        if constexpr (UPB == 0) v = float(d[t][c][r] + d2[t][c][r] - 256 * nzp_r[t][r] * int(L.quads * 4)) * s;
+        finish_store<T>(p.out + (uint64_t(m) * p.n + n) * item, v, bits_f32(ldg<uint32_t>(p.rows + 8ull * m)), p.has_bias != 0, bias);
+      }
+  }
+}
+
+template <class T, int RT, int CT>
+int launch_rows(const Q4CParams& p, const MatrixLayout& M, uint32_t m0, uint32_t rows, hipStream_t stream) {
+  const dim3 grid((M.tiles + 4 * CT - 1) / (4 * CT), (rows + 16 * RT - 1) / (16 * RT));
+  switch (M.upb) {
+    case 0: hipLaunchKernelGGL((qmm4m_rows<T, 0, RT, CT>), grid, dim3(256), 0, stream, p, M, m0); break;
+    case 1: hipLaunchKernelGGL((qmm4m_rows<T, 1, RT, CT>), grid, dim3(256), 0, stream, p, M, m0); break;
+    case 2: hipLaunchKernelGGL((qmm4m_rows<T, 2, RT, CT>), grid, dim3(256), 0, stream, p, M, m0); break;
+    case 4: hipLaunchKernelGGL((qmm4m_rows<T, 4, RT, CT>), grid, dim3(256), 0, stream, p, M, m0); break;
+    case 8: hipLaunchKernelGGL((qmm4m_rows<T, 8, RT, CT>), grid, dim3(256), 0, stream, p, M, m0); break;
+    default: return -1;
+  }
+  return 0;
+}
+
 bool check_q4_shape(uint32_t m, uint32_t n, uint32_t k, uint32_t bs, std::string* err) {
   if (bs == 0 || !(bs == k || (bs % 32 == 0 && k % bs == 0))) {
     *err = "qmm4: block size must equal k or be a multiple of 32 dividing k";
@@ -1040,8 +1240,9 @@ int launch_qmm4c_pack(const Q4PackParams& p, uint32_t layout, const Machine&, hi
 
 // The matrix-layout form of the product: phase 0, 1 or 2 (= 0 then 1).
 template <class T>
-int launch_matrix(const Q4CParams& p, uint32_t phase, uint32_t groupwise, hipStream_t stream, std::string* err) {
+int launch_matrix(const Q4CParams& p, uint32_t phase_and_flags, uint32_t groupwise, hipStream_t stream, std::string* err) {
   constexpr uint32_t item = sizeof(typename T::storage);
+  const uint32_t phase = phase_and_flags & 15u, flags = phase_and_flags & ~15u;
   MatrixLayout M;
   if (!matrix_layout(p.n, p.k, p.bs, &M)) {
     *err = "qmm4c: this shape has no compact form (groupwise block sizes: 32, 64, 128, 256)";
@@ -1065,7 +1266,26 @@ int launch_matrix(const Q4CParams& p, uint32_t phase, uint32_t groupwise, hipStr
       *err = "qmm4c: null or unaligned side-car address";
       return -1;
     }
-    for (uint32_t m0 = 0; m0 < p.m; m0 += 16 * 1024) {
+    // Enough row tiles x column tiles to give every SIMD two and a half waves: a wave per tile walks all of K; fewer: the
+    // one-row-tile kernel, whose four waves split K.  Phase values 1 | 2 with bit 4 (16) set keep the one-row-tile
+    // kernel, with bit 5 (32) force the wave-per-tile kernel (tests, tuning).
+    const bool rows_kernel = ((uint64_t((p.m + 15) / 16) * M.tiles >= 2560 && !(flags & 16)) || (flags & 32));
+    // (wave tiles of 2 x 2, 2 x 1 or 1 x 1 matrix-core tiles: the largest that leaves every SIMD two and a half
+    //  waves; flag bits 6-7 choose: 1 = 1 x 1, 2 = 2 x 1, 3 = 2 x 2)
+    for (uint32_t m0 = 0; rows_kernel && m0 < p.m; m0 += 16 * 1024) {
+      const uint32_t rows = p.m - m0 < 16 * 1024 ? p.m - m0 : 16 * 1024;
+      uint32_t shape = (flags >> 6) & 3u;
+      if (shape == 0)
+        shape = uint64_t((rows + 31) / 32) * ((M.tiles + 1) / 2) >= 2560 ? 3 : uint64_t((rows + 31) / 32) * M.tiles >= 2560 ? 2 : 1;
+      const int rc = shape == 3 ? launch_rows<T, 2, 2>(p, M, m0, rows, stream)
+                   : shape == 2 ? launch_rows<T, 2, 1>(p, M, m0, rows, stream)
+                                : launch_rows<T, 1, 1>(p, M, m0, rows, stream);
+      if (rc != 0) {
+        *err = "qmm4c: bad layout";
+        return -1;
+      }
+    }
+    for (uint32_t m0 = 0; !rows_kernel && m0 < p.m; m0 += 16 * 1024) {
       const uint32_t rows = p.m - m0 < 16 * 1024 ? p.m - m0 : 16 * 1024;
       const dim3 grid(M.tiles, (rows + 15) / 16);
       switch (M.upb) {
@@ -1095,8 +1315,8 @@ int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwi
       *err = "qmm4c: GROUPWISE must be 1 exactly when bs != k";
       return -1;
     }
-    if (!p.inp || !p.out || phase > 2) {
-      *err = phase > 2 ? "qmm4c: PHASE must be 0, 1 or 2" : "qmm4c: null or unaligned tensor address";
+    if (!p.inp || !p.out || (phase & 15u) > 2 || (phase & ~255u)) {
+      *err = (phase & 15u) > 2 || (phase & ~255u) ? "qmm4c: PHASE must be 0, 1 or 2" : "qmm4c: null or unaligned tensor address";
       return -1;
     }
     const int rc = dtype == VKT_F32 ? launch_matrix<f32_t>(p, phase, groupwise, stream, err)
