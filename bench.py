@@ -58,22 +58,45 @@ class Launch:
             self.abi.check(-1)
 
 
+class Timing(tuple):
+    """(wall ms per step, event ms per step); .median: the median over five equal parts of the timed loop of the
+    event time per step (the whole loop where it has fewer than 10 steps)."""
+    median = None
+
+
 def time_steps(abi, step_fns, steps, warmup):
-    """Runs step_fns[i % len] for `warmup` untimed and `steps` timed steps.
-    Returns (wall ms per step, event ms per step)."""
+    """Runs step_fns[i % len] for `warmup` untimed and `steps` timed steps, events at five equally spaced marks."""
     n = len(step_fns)
     for i in range(warmup):
         step_fns[i % n]()
     abi.synchronize()
-    e0, e1 = abi.Event(), abi.Event()
+    parts = 5 if steps >= 10 else 1
+    marks = [steps * j // parts for j in range(parts + 1)]
+    events = [abi.Event() for _ in marks]
     t0 = time.perf_counter()
-    e0.record()
+    events[0].record()
+    at = 1
     for i in range(steps):
         step_fns[i % n]()
-    e1.record()
+        if i + 1 == marks[at]:
+            events[at].record()
+            at += 1
     abi.synchronize()
     t1 = time.perf_counter()
-    return (t1 - t0) * 1e3 / steps, e0.elapsed_ms(e1) / steps
+    t = Timing(((t1 - t0) * 1e3 / steps, events[0].elapsed_ms(events[-1]) / steps))
+    per = sorted(events[j].elapsed_ms(events[j + 1]) / (marks[j + 1] - marks[j]) for j in range(parts))
+    t.median = per[len(per) // 2]
+    return t
+
+
+def timed(abi, fns, steps, warmup, resident=True):
+    """Timing fields of a workload result: the rotation over distinct weight copies (HBM), and where there is a
+    rotation also the same launch on one copy over and over (cache resident, labelled so)."""
+    t = time_steps(abi, fns, steps, warmup)
+    out = dict(wall_ms=t[0], event_ms=t[1], event_ms_median=t.median, copies=len(fns))
+    if len(fns) > 1 and resident:
+        out["cache_resident_ms"] = time_steps(abi, fns[:1], steps, warmup)[1]
+    return out
 
 
 def rotation(nbytes, floor_mib=512):
@@ -102,15 +125,14 @@ def wl_q8(abi, m, k, n, dtype, steps, warmup, seed=1020, prefill=False):
     fns = [Launch(abi, "qmm8_" + abi.SUFFIX[dtype], [0],
                   abi.Q8Params(a=dx.address, b=c.address, scales=ds.address, c=out.address, m=m, n=n, k=k, a_sm=k,
                                a_sk=1)) for c in copies]
-    wall, ev = time_steps(abi, fns, steps, warmup)
     work = n * k + item * (m * k + n + m * n)  # weights once + activations + scales + output
     keep = (x, w, s)
     if prefill:
         return dict(kind="mfma", peak=BF16_PEAK_TFLOPS, metric="int8-weight prefill TFLOP/s (% of bf16 MFMA peak)", work=2 * m * n * k,
-                    wall_ms=wall, event_ms=ev, bytes=work, inputs=None, copies=len(copies),
-                    name=f"_weight_int8pack_mm {abi.SUFFIX[dtype]} M={m} K={k} N={n} (prefill)")
-    return dict(kind="hbm", work=work, wall_ms=wall, event_ms=ev, flops=2 * m * n * k, inputs=keep,
-                name=f"_weight_int8pack_mm {abi.SUFFIX[dtype]} M={m} K={k} N={n}", copies=len(copies))
+                    bytes=work, inputs=None, name=f"_weight_int8pack_mm {abi.SUFFIX[dtype]} M={m} K={k} N={n} (prefill)",
+                    **timed(abi, fns, steps, max(warmup, len(fns)), resident=False))
+    return dict(kind="hbm", work=work, flops=2 * m * n * k, inputs=keep,
+                name=f"_weight_int8pack_mm {abi.SUFFIX[dtype]} M={m} K={k} N={n}", **timed(abi, fns, steps, warmup))
 
 
 def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030, prefill=False):
@@ -146,15 +168,14 @@ def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030, prefill=False):
         p = abi.Q4CParams(inp=dx.address, q=dq.address, rows=dr.address, compact=c.address, out=out.address, m=m, n=n,
                           k=k, bs=bs, has_bias=1)
         fns.append(Launch(abi, "qmm4c_f32", [2, 1, layout], p))  # row quantisation + product
-    wall, ev = time_steps(abi, fns, steps, warmup)
     work = n * k // 2 + 4 * n * (k // bs) + 4 * n + 4 * m * k + 4 * m * n
     if prefill:  # many rows: the matrix cores' int8 rate is the published bound
         return dict(kind="mfma", peak=INT8_PEAK_TOPS, metric="int4-weight prefill TOP/s (% of int8 MFMA peak)", work=2 * m * n * k,
-                    wall_ms=wall, event_ms=ev, bytes=work, inputs=None, copies=len(copies),
-                    name=f"_dyn_quant_matmul_4bit f32 M={m} K={k} N={n} bs={bs} (prefill)")
-    return dict(kind="hbm", work=work, wall_ms=wall, event_ms=ev, flops=2 * m * n * k, inputs=(x, packed),
-                name=f"_dyn_quant_matmul_4bit f32 M={m} K={k} N={n} bs={bs} (compact side-car)", copies=len(copies),
-                reference_layout_bytes=int(packed.numel()) * 4 + 4 * m * k + 4 * m * n)
+                    bytes=work, inputs=None, name=f"_dyn_quant_matmul_4bit f32 M={m} K={k} N={n} bs={bs} (prefill)",
+                    **timed(abi, fns, steps, max(warmup, len(fns)), resident=False))
+    return dict(kind="hbm", work=work, flops=2 * m * n * k, inputs=(x, packed),
+                name=f"_dyn_quant_matmul_4bit f32 M={m} K={k} N={n} bs={bs} (compact side-car)",
+                reference_layout_bytes=int(packed.numel()) * 4 + 4 * m * k + 4 * m * n, **timed(abi, fns, steps, warmup))
 
 
 def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False):
@@ -178,8 +199,8 @@ def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False)
     p = abi.F8Params(a=da.address, b=db.address, scale_a=dsa.address, scale_b=dsb.address, out=out.address, m=m, n=n,
                      k=k, lda=k, ldb=k, ldo=n, fmt_a=abi.E4M3, fmt_b=abi.E4M3, out_dtype=abi.BF16, rowwise=int(rowwise))
     fns = [Launch(abi, "fp8mm", [0], p)]
-    wall, ev = time_steps(abi, fns, steps, warmup)
-    return dict(kind="mfma", work=2 * m * n * k, wall_ms=wall, event_ms=ev, bytes=m * k + n * k + 2 * m * n,
+    tm = time_steps(abi, fns, steps, warmup)
+    return dict(kind="mfma", work=2 * m * n * k, wall_ms=tm[0], event_ms=tm[1], event_ms_median=tm.median, bytes=m * k + n * k + 2 * m * n,
                 inputs=(a, bt, sa, sb), copies=1,
                 name=f"_scaled_mm e4m3fn {'rowwise' if rowwise else 'per-tensor'} M={m} K={k} N={n} -> bf16"
                      + (" (all-zero operands)" if zero_operands else ""))
@@ -199,8 +220,8 @@ def wl_gemm16(abi, m, k, n, steps, warmup, seed=1090, layout="nt"):
         p.b_sk, p.b_sn = n, 1
     if layout == "tn":
         p.a_sm, p.a_sk = 1, m
-    wall, ev = time_steps(abi, [Launch(abi, "gemmcm_bf16", [0], p)], steps, warmup)
-    return dict(kind="mfma", peak=BF16_PEAK_TFLOPS, metric="bf16 mm TFLOP/s (% of MFMA peak)", work=2 * m * n * k, wall_ms=wall, event_ms=ev,
+    tm = time_steps(abi, [Launch(abi, "gemmcm_bf16", [0], p)], steps, warmup)
+    return dict(kind="mfma", peak=BF16_PEAK_TFLOPS, metric="bf16 mm TFLOP/s (% of MFMA peak)", work=2 * m * n * k, wall_ms=tm[0], event_ms=tm[1], event_ms_median=tm.median,
                 bytes=2 * (m * k + n * k + m * n), inputs=None, copies=1, name=f"mm bf16 M={m} K={k} N={n} ({layout}: " + {"nt": "x @ w.T, the Linear layout", "nn": "x @ w", "tn": "x.T @ w"}[layout] + ")")
 
 
@@ -212,8 +233,8 @@ def wl_cast(abi, n, steps, warmup, seed=1070):
     dx = abi.Buffer.from_numpy(x.view(torch.int16).numpy())
     out = abi.Buffer(n)
     p = abi.CastParams(src=dx.address, dst=out.address, n=n, src_dtype=abi.BF16, dst_dtype=abi.E4M3)
-    wall, ev = time_steps(abi, [Launch(abi, "cast_fp8", [], p)], steps, warmup)
-    return dict(kind="hbm", work=3 * n, wall_ms=wall, event_ms=ev, flops=0, inputs=None, copies=1,
+    tm = time_steps(abi, [Launch(abi, "cast_fp8", [], p)], steps, warmup)
+    return dict(kind="hbm", work=3 * n, wall_ms=tm[0], event_ms=tm[1], event_ms_median=tm.median, flops=0, inputs=None, copies=1,
                 name=f"cast bf16 -> e4m3fn, {n >> 20} Mi values")
 
 
@@ -226,8 +247,8 @@ def wl_quant(abi, m, k, steps, warmup, seed=1080):
     out, scales = abi.Buffer(m * k), abi.Buffer(m * 4)
     p = abi.F8QuantParams(src=dx.address, dst=out.address, scale=scales.address, m=m, k=k, lds=k, ldd=k,
                           src_dtype=abi.BF16, dst_fmt=abi.E4M3)
-    wall, ev = time_steps(abi, [Launch(abi, "fp8_quant", [1], p)], steps, warmup)
-    return dict(kind="hbm", work=3 * m * k + 4 * m, wall_ms=wall, event_ms=ev, flops=0, inputs=None, copies=1,
+    tm = time_steps(abi, [Launch(abi, "fp8_quant", [1], p)], steps, warmup)
+    return dict(kind="hbm", work=3 * m * k + 4 * m, wall_ms=tm[0], event_ms=tm[1], event_ms_median=tm.median, flops=0, inputs=None, copies=1,
                 name=f"fp8_quant rowwise bf16 -> e4m3fn M={m} K={k}")
 
 
@@ -246,9 +267,9 @@ def wl_move(abi, kind, steps, warmup, rows=16384, cols=16384):
     p.out = out.address
     for d in range(4):
         p.size[d], p.so[d], p.sa[d] = (sizes[d], so[d], sa[d]) if d < 2 else (1, 0, 0)
-    wall, ev = time_steps(abi, [Launch(abi, name, [abi.MOVE_COPY], p)], steps, warmup)
+    tm = time_steps(abi, [Launch(abi, name, [abi.MOVE_COPY], p)], steps, warmup)
     label = {"transpose": "x.t().contiguous()", "rows": "x[::2].contiguous()"}[kind]
-    return dict(kind="hbm", metric="strided copy GB/s (% of HBM peak)", work=work, wall_ms=wall, event_ms=ev, flops=0, inputs=None,
+    return dict(kind="hbm", metric="strided copy GB/s (% of HBM peak)", work=work, wall_ms=tm[0], event_ms=tm[1], event_ms_median=tm.median, flops=0, inputs=None,
                 copies=1, name=f"{name} {label}, bfloat16 [{rows}, {cols}]")
 
 
@@ -270,8 +291,8 @@ def wl_affine(abi, kind, n, steps, warmup, seed=1100):
         p = abi.QuantParams(src=src.address, dst=dst.address, mask=mask.address, n=n, scale_bits=scale_bits, zero_point=5, qmin=0,
                             qmax=255, dtype=abi.F32)
         name, spec, work = "fake_quant", [0, 0], 9 * n
-    wall, ev = time_steps(abi, [Launch(abi, name, spec, p)], steps, warmup)
-    return dict(kind="hbm", metric="affine quantisation GB/s (% of HBM peak)", work=work, wall_ms=wall, event_ms=ev, flops=0,
+    tm = time_steps(abi, [Launch(abi, name, spec, p)], steps, warmup)
+    return dict(kind="hbm", metric="affine quantisation GB/s (% of HBM peak)", work=work, wall_ms=tm[0], event_ms=tm[1], event_ms_median=tm.median, flops=0,
                 inputs=None, copies=1, name=f"{name} float32 / quint8 per tensor, {n >> 20} Mi values")
 
 
@@ -283,8 +304,8 @@ def wl_copy(abi, nbytes, steps, warmup):
 
     def step():
         abi.check(L.vkt_copy_on_device(dst.address, src.address, nbytes))
-    wall, ev = time_steps(abi, [step], steps, warmup)
-    return dict(kind="hbm", work=2 * nbytes, wall_ms=wall, event_ms=ev, flops=0, inputs=None, copies=1,
+    tm = time_steps(abi, [step], steps, warmup)
+    return dict(kind="hbm", work=2 * nbytes, wall_ms=tm[0], event_ms=tm[1], event_ms_median=tm.median, flops=0, inputs=None, copies=1,
                 name=f"device copy of {nbytes >> 20} MiB (read + write)")
 
 
@@ -339,8 +360,14 @@ def summarise(r):
     else:
         value, unit, peak = r["work"] / r["wall_ms"] / 1e9, "TFLOP/s", r.get("peak", FP8_PEAK_TFLOPS)
         achieved = r["work"] / r["event_ms"] / 1e9
-    return value, unit, dict(bound=r["kind"], achieved=round(achieved, 1), peak=peak, unit=unit,
-                             frac=round(achieved / peak, 4), traffic=None)
+    roof = dict(bound=r["kind"], achieved=round(achieved, 1), peak=peak, unit=unit, frac=round(achieved / peak, 4),
+                traffic=None)
+    if r.get("event_ms_median"):  # the same figure from the median fifth of the timed loop
+        roof["achieved_median_of_5"] = round(achieved * r["event_ms"] / r["event_ms_median"], 1)
+    if r.get("cache_resident_ms"):  # one weight copy over and over: L2 / Infinity Cache, not HBM (reported, not priced)
+        roof["cache_resident"] = dict(achieved=round(achieved * r["event_ms"] / r["cache_resident_ms"], 1), unit=unit,
+                                      kernel_ms=round(r["cache_resident_ms"], 5))
+    return value, unit, roof
 
 
 def cpu_baselines(abi, name, r):
@@ -376,6 +403,32 @@ def cpu_baselines(abi, name, r):
                             host_cpus=os.cpu_count(), kind="torch CPU kernel of the same op",
                             sample=f"median of 15 calls of torch._weight_int8pack_mm, {dt * 1e3:.2f} ms")
     return out
+
+
+def through_dispatcher(abi, name, r, calls=200):
+    """The same op called as torch._weight_int8pack_mm on device "vk" tensors (schema -> op layer -> C ABI -> kernel),
+    one weight tensor over and over: wall time per call with the queue kept full, beside the kernel's own time on
+    the same resident weights, so that the host's share shows."""
+    import torch
+    import torch_vulkan_amd.backend as tv
+    if not name.startswith(("c1", "c2")) or not r.get("inputs"):
+        return None
+    x, w, s = (t.to("vk") for t in r["inputs"])
+    before = tv.fallback_counts()
+    for _ in range(20):
+        torch._weight_int8pack_mm(x, w, s)
+    abi.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(calls):
+        torch._weight_int8pack_mm(x, w, s)
+    t_issue = time.perf_counter()
+    abi.synchronize()
+    t1 = time.perf_counter()
+    if tv.fallback_counts() != before:
+        raise RuntimeError("bench.py: torch._weight_int8pack_mm on device vk fell back to the CPU")
+    return dict(op="torch._weight_int8pack_mm on device vk", calls=calls, us_per_call=round((t1 - t0) * 1e6 / calls, 2),
+                host_issue_us_per_call=round((t_issue - t0) * 1e6 / calls, 2),
+                kernel_us_cache_resident=round(r["cache_resident_ms"] * 1e3, 2) if r.get("cache_resident_ms") else None)
 
 
 def load_traffic():
@@ -418,6 +471,7 @@ def main():
     }
     if not args.no_cpu:
         line.update(cpu_baselines(abi, args.workload, r))
+        line["through_dispatcher"] = through_dispatcher(abi, args.workload, r)
     if "cpu_baseline" not in line:
         line["cpu_baseline"] = None
     del r
