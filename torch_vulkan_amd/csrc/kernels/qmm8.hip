@@ -79,9 +79,9 @@ __global__ __launch_bounds__(256) void qmm8_gemv(Q8Params p) {
     U4 wv[COLS];
 #pragma unroll
     for (int c = 0; c < COLS; ++c) wv[c] = ldg_stream<U4>(brow[c] + k);
-    if constexpr (T::dtype != VKT_F32 && ROWS > 1) {
-      // 16-bit activations, several rows: the weights widen (exactly) to the activations' type once, and each row
-      // takes 8 two-element dot products per 16 weights, its activations as they are in memory
+    if constexpr (T::dtype != VKT_F32) {
+      // 16-bit activations: the weights widen (exactly) to the activations' type once, and each row takes 8
+      // two-element dot products per 16 weights, its activations as they are in memory (no conversions)
       U4 wlo[COLS], whi[COLS];
 #pragma unroll
       for (int c = 0; c < COLS; ++c) widen16_to_operands<T>(wv[c], &wlo[c], &whi[c]);
