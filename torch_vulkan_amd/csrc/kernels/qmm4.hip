@@ -836,16 +836,27 @@ __global__ __launch_bounds__(256) void qmm4m_tile(Q4CParams p, MatrixLayout L, u
           constexpr int mask = UPB ? UPB - 1 : 0;
           const int u = x * 4 + j;  // unit within the wave's step
           const bool first = UPB != 0 && (u & mask) == 0;
-          d = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, first ? unit_const * (UPB ? UPB : 1) : d, 0, 0, 0);
-          d = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, minus8, d, 0, 0, 0);
-          d = __builtin_amdgcn_mfma_i32_16x16x32_i8(nz_a, b, d, 0, 0, 0);
-          d = __builtin_amdgcn_mfma_i32_16x16x32_i8(nz_b, b, d, 0, 0, 0);
-          if constexpr (UPB != 0) {
-            if ((u & mask) == mask) {  // the block's last unit
-              // position r * 64 + lane for row 4 kg + r: a wave's 64 stores of one r fall on 64 banks
-              float* at = &terms[parity][wave * BW + u / UPB][lane];
+          if constexpr (UPB == 1) {
+            // a block per unit: a chain of its own, the constant as the first accumulator input (no copy)
+            V4I x = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, unit_const, 0, 0, 0);
+            x = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, minus8, x, 0, 0, 0);
+            x = __builtin_amdgcn_mfma_i32_16x16x32_i8(nz_a, b, x, 0, 0, 0);
+            x = __builtin_amdgcn_mfma_i32_16x16x32_i8(nz_b, b, x, 0, 0, 0);
+            float* at = &terms[parity][wave * BW + u][lane];
 #pragma unroll
-              for (int r = 0; r < 4; ++r) at[r * 64] = float(d[r]) * set.s[sl][j];
+            for (int r = 0; r < 4; ++r) at[r * 64] = float(x[r]) * set.s[sl][j];
+          } else {
+            d = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, first ? unit_const * (UPB ? UPB : 1) : d, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, minus8, d, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_i32_16x16x32_i8(nz_a, b, d, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_i32_16x16x32_i8(nz_b, b, d, 0, 0, 0);
+            if constexpr (UPB != 0) {
+              if ((u & mask) == mask) {  // the block's last unit
+                // position r * 64 + lane for row 4 kg + r: a wave's 64 stores of one r fall on 64 banks
+                float* at = &terms[parity][wave * BW + u / UPB][lane];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) at[r * 64] = float(d[r]) * set.s[sl][j];
+              }
             }
           }
         }
