@@ -96,7 +96,11 @@ uint64_t vkt_qmm4c_q_bytes(uint32_t m, uint32_t k);
 /* ---------------------------------------------------------------- parameter blocks */
 
 /* "qmm8_f32" | "qmm8_f16" | "qmm8_bf16", spec {ROWS}: C = A @ (B * scales).T
- * (quant.cpp:31-37, qmm8.slang:21-33).  56 bytes. */
+ * (quant.cpp:31-37, qmm8.slang:21-33).  56 bytes.  ROWS is 0 or m.  An optional second entry overrides the
+ * launcher's choice of kernel and shape (tests, tuning; 0 or absent: planned): bits 0-7 columns per wave or
+ * column tiles per workgroup, 8-15 waves that split K, 24+ slices of K over workgroups; bit 16 the any-shape
+ * kernel, 17 the vector-unit kernels, 18 / 19 the matrix-core kernel with / without staging through LDS, 20 no
+ * widened-weights product for many rows, 21 / 22 the 64 x 128 tile kernel forced / off. */
 typedef struct Q8Params {
   uint64_t a, b, scales, c; /* A [m,k] (row stride a_sm, a_sk must be 1), B int8 [n,k], scales [n], C [m,n] */
   uint32_t m, n, k;
@@ -138,7 +142,9 @@ typedef struct Q4PackParams {
  * (vkt_qmm4c_q_bytes; the arrangement differs per layout) and rows; PHASE 1 is the
  * product; PHASE 2 does both: with LAYOUT 0 in one launch per 4 rows where the rows can
  * be quantised from registers (k a multiple of 8, at most 16384), otherwise as PHASE 0
- * then 1.  Results are bit-identical to qmm4. */
+ * then 1.  Results are bit-identical to qmm4.  With LAYOUT 1, bits 4-7 of PHASE override the choice
+ * between the two product kernels, which give the same bits (tests, tuning): 16 keeps the kernel whose four waves
+ * split K, 32 forces the one whose waves each walk all of K (| 64, 128, 192: 1, 2, 4 tiles of 16 x 16 per wave). */
 typedef struct Q4CParams {
   uint64_t inp, q, rows, compact, out;
   uint32_t m, n, k, bs, has_bias, pad;
