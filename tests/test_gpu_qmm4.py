@@ -19,7 +19,9 @@ EXTRA = [(2, 4096, 300, 32, True), (3, 14336, 20, 32, True), (9, 28672, 6, 128, 
          (70, 512, 40, 64, True), (33, 1056, 17, 32, False), (16, 4096, 64, 128, True), (20, 4160, 10, 4160, False),
          (130, 96, 33, 32, True), (17, 2048, 16, 256, False),
          # many rows: a wave per tile that walks all of K, every block size of the matrix-core layout
-         (64, 4160, 40, 4160, True), (200, 1024, 48, 128, False), (100, 2048, 20, 256, True), (49, 640, 130, 64, False)]
+         (64, 4160, 40, 4160, True), (200, 1024, 48, 128, False), (100, 2048, 20, 256, True), (49, 640, 130, 64, False),
+         # more rows than one launch of the matrix-core kernels takes (16384)
+         (16400, 64, 20, 32, True)]
 
 
 @pytest.mark.parametrize("m,k,n,bs,bias", Q4_CASES + EXTRA)
