@@ -403,17 +403,23 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma_staged(Q8Params p, uint3
     for (int t = 0; t < NT; ++t) acc[mt][t] = V4F{0.0f, 0.0f, 0.0f, 0.0f};
 
   const U4 zero = {0, 0, 0, 0};
-  for (uint32_t q = q_begin + wave; q < q_end; q += WAVES) {
+  // The weights of a chunk are loaded into registers a chunk ahead (non-temporal 16-byte loads: this part streams
+  // from HBM ~1.5x as fast that way as straight into LDS with global_load_lds_dwordx4, measured with the loads alone)
+  // and written to the wave's region when their turn comes.
+  U4 wr[NT][4];
+  auto request = [&](uint32_t q) {
     const uint32_t k0 = q * 256;
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         // (bytes past k are fetched from the row's start instead: their activations are zeros below)
-        const uint64_t src = wsrc[t][i] + (k0 + wk[i] < p.k ? k0 + wk[i] : 0u);
-        __builtin_amdgcn_global_load_lds(reinterpret_cast<const VKT_GLOBAL void*>(src),
-                                         (__attribute__((address_space(3))) void*)(mine + (t * 16 + 4 * i) * 256), 16, 0, 0);
+        wr[t][i] = ldg_stream<U4>(wsrc[t][i] + (k0 + wk[i] < p.k ? k0 + wk[i] : 0u));
       }
+  };
+  if (q_begin + wave < q_end) request(q_begin + wave);
+  for (uint32_t q = q_begin + wave; q < q_end; q += WAVES) {
+    const uint32_t k0 = q * 256;
     U4 a0[MT][4], a1[MT][4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -426,11 +432,16 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma_staged(Q8Params p, uint3
         a1[mt][j] = real ? ldg<U4>(arow[mt] + (k0 + 64 * j) * item + 16) : zero;
       }
     }
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the chunk's weights are in LDS
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) *reinterpret_cast<U4*>(mine + (t * 16 + 4 * i) * 256 + lane * 16) = wr[t][i];
+    if (q + WAVES < q_end) request(q + WAVES);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
+        // (a wave's LDS operations execute in order: these reads see the writes above)
         const U4 wv = *reinterpret_cast<const U4*>(mine + (t * 16 + c) * 256 + (((4 * j + g) ^ c) & 15) * 16);
         U4 wlo, whi;
         widen16_to_operands<T>(wv, &wlo, &whi);
@@ -441,8 +452,6 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma_staged(Q8Params p, uint3
         }
       }
     }
-    // (the next chunk's loads overwrite the region: every read above has returned by then, as its value is used)
-    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
   }
 
   // the waves' partial tiles meet in wave 0 (through the staging memory, once every wave is done with it)
@@ -518,18 +527,19 @@ bool launch_staged(const Q8Params& p, int mt, int nt, int waves, uint32_t slices
 }
 
 // 33 to a few hundred rows (batched decode): a tile kernel.  A workgroup of 8 waves owns 64 rows x 128 columns and a
-// slice of K, walked in steps of 128 values through 4 LDS stages.  Both operand tiles of a step come straight into
-// LDS (global_load_lds_dwordx4; two steps in flight from memory while one is read and one multiplied): the
-// activations [64 rows][256 bytes] once per workgroup, the raw int8 weights [128 rows][128 bytes] in runs of 128
-// contiguous bytes per row.  16-byte chunks are swizzled by the row's low bits, so that the operand-shaped reads
-// (16 lanes = 16 rows at one logical chunk) are conflict free.  The waves split the step's K, not only its
-// columns: wave (kc, nh) multiplies all 64 rows by columns 64 nh .. + 63 over the 32 values 32 kc .. + 31 of each
-// step, so a step costs the LDS 48 KB of fragment reads (every wave reading its own 32 x 32 outputs' operands: 96 KB)
-// and every weight is widened once per workgroup.  After the loop the four k-parts of a column half meet through LDS,
-// added in a fixed order.  K is cut into slices across workgroups until the grid fills the machine; the slices'
-// float32 tiles meet in the runtime's workspace and qmm8_tile_finish adds them in slice order, scales and stores.
-constexpr uint32_t kTileStepK = 128, kTileStages = 4;
-constexpr uint32_t kTileLds = kTileStages * (64 * 256 + 128 * 128);
+// slice of K, walked in steps of 128 values.  Both operand tiles of a step are loaded into registers four steps
+// ahead and written to one of two LDS stages a step before they are multiplied: the activations [64 rows][256 bytes]
+// once per workgroup, the raw int8 weights [128 rows][128 bytes] in runs of 128 contiguous bytes per row.  16-byte
+// chunks are swizzled by the row's low bits (the lane fetches the chunk that belongs in its slot), so that the
+// operand-shaped reads (16 lanes = 16 rows at one logical chunk) are conflict free.  The waves split the step's K,
+// not only its columns: wave (kc, nh) multiplies all 64 rows by columns 64 nh .. + 63 over the 32 values 32 kc .. + 31
+// of each step, so a step costs the LDS 48 KB of fragment reads (every wave reading its own 32 x 32 outputs'
+// operands: 96 KB) and every weight is widened once per workgroup.  After the loop the four k-parts of a column half
+// meet through LDS, added in a fixed order.  K is cut into slices across workgroups until the grid fills the machine;
+// the slices' float32 tiles meet in the runtime's workspace and qmm8_tile_finish adds them in slice order, scales
+// and stores.
+constexpr uint32_t kTileStepK = 128, kTileAhead = 4;
+constexpr uint32_t kTileLds = 8 * 16 * 1024;  // the k-parts' meeting place; the two operand stages use its first half
 template <class T>
 __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_slice, uint64_t workspace) {
   constexpr uint32_t A_BYTES = 64 * 256, B_BYTES = 128 * 128, STAGE = A_BYTES + B_BYTES;
@@ -540,9 +550,10 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
   const uint32_t steps = p.k / kTileStepK;
   const uint32_t s_begin = slice * steps_per_slice, s_end = s_begin + steps_per_slice < steps ? s_begin + steps_per_slice : steps;
 
-  // loads of one step: activations 16 wave-loads of 4 rows x 256 bytes, weights 16 of 8 rows x 128 bytes; a wave issues 2 + 2
-  // (Giving the weights a ring of their own, 6 stages deep, issued by other waves than the activations so that the
-  // in-order return of a wave's loads does not tie the two depths together, made every shape slower.)
+  // Loads of one step: activations 16 wave-loads of 4 rows x 256 bytes, weights 16 of 8 rows x 128 bytes; a wave issues
+  // 2 + 2, into registers, kTileAhead steps ahead, and writes them to LDS (16 bytes per lane, lane after lane) one
+  // step before they are multiplied.  (Straight into LDS with global_load_lds_dwordx4 the same stream runs at 2.6
+  // TB/s from 112 compute units where this path gives 4.1-4.4: measured with the loads alone.)
   uint64_t a_src[2], b_src[2];
   uint32_t a_dst[2], b_dst[2];
 #pragma unroll
@@ -550,25 +561,31 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
     const uint32_t row = (wave * 2 + i) * 4 + (lane >> 4), slot = lane & 15u;
     const uint32_t m = m0 + row < p.m ? m0 + row : p.m - 1;
     a_src[i] = p.a + uint64_t(int64_t(m) * p.a_sm * 2) + ((slot ^ (row & 15u)) * 16);
-    a_dst[i] = (wave * 2 + i) * 1024;  // (+ 16 * lane, by the hardware)
+    a_dst[i] = (wave * 2 + i) * 1024 + lane * 16;
   }
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const uint32_t row = (wave * 2 + i) * 8 + (lane >> 3), slot = lane & 7u;
     const uint32_t n = n0 + row < p.n ? n0 + row : p.n - 1;
     b_src[i] = p.b + uint64_t(n) * p.k + ((slot ^ ((row >> 1) & 7u)) * 16);
-    b_dst[i] = A_BYTES + (wave * 2 + i) * 1024;
+    b_dst[i] = A_BYTES + (wave * 2 + i) * 1024 + lane * 16;
   }
-  auto request = [&](uint32_t step) {
-    uint8_t* base = tile_lds + ((step - s_begin) % kTileStages) * STAGE;
+  U4 ra[kTileAhead][2], rb[kTileAhead][2];
+  auto request = [&](auto set, uint32_t step) {
+    constexpr int R = decltype(set)::value;
+    const uint32_t st = step < s_end ? step : s_end - 1;  // (past the end the last step again, never published: the count of loads in flight stays the same)
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const VKT_GLOBAL void*>(a_src[i] + uint64_t(step) * kTileStepK * 2),
-                                       (__attribute__((address_space(3))) void*)(base + a_dst[i]), 16, 0, 0);
+    for (int i = 0; i < 2; ++i) ra[R][i] = ldg<U4>(a_src[i] + uint64_t(st) * kTileStepK * 2);
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const VKT_GLOBAL void*>(b_src[i] + uint64_t(step) * kTileStepK),
-                                       (__attribute__((address_space(3))) void*)(base + b_dst[i]), 16, 0, 0);
+    for (int i = 0; i < 2; ++i) rb[R][i] = ldg_stream<U4>(b_src[i] + uint64_t(st) * kTileStepK);
+  };
+  auto publish = [&](auto set, uint32_t step) {
+    constexpr int R = decltype(set)::value;
+    uint8_t* base = tile_lds + ((step - s_begin) & 1u) * STAGE;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) *reinterpret_cast<U4*>(base + a_dst[i]) = ra[R][i];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) *reinterpret_cast<U4*>(base + b_dst[i]) = rb[R][i];
   };
 
   V4F acc[4][4];  // [row tile][column tile of this half]
@@ -578,9 +595,9 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
     for (int t = 0; t < 4; ++t) acc[mt][t] = V4F{0.0f, 0.0f, 0.0f, 0.0f};
 
   // Fragments of step s + 1 are read from LDS (8 reads per lane, into the other of two register sets) while step s is
-  // widened and multiplied, so the LDS, the vector units and the matrix cores work at the same time; two further steps
-  // are in flight from memory.  Loads land in the order issued: "at most 4 outstanding" (one step's worth per wave)
-  // means everything older has landed.
+  // widened and multiplied, so the LDS, the vector units and the matrix cores work at the same time; three further
+  // steps are in flight from memory.  Loads land in the order issued: "at most 12 outstanding" (three steps' worth
+  // per wave) means everything older has landed.
   // lane (c, g): activations of row 16 mt + c, weights of column 64 nh + 16 t + c, both at k = 32 kc + 8 g .. + 7
   U4 fa[2][4];
   U2 fw[2][4];
@@ -597,7 +614,7 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
   }
   auto read_fragments = [&](auto set, uint32_t step) {
     constexpr int S = decltype(set)::value;
-    const uint8_t* ta = tile_lds + ((step - s_begin) % kTileStages) * STAGE;
+    const uint8_t* ta = tile_lds + ((step - s_begin) & 1u) * STAGE;
     const uint8_t* tb = ta + A_BYTES;
 #pragma unroll
     for (int t = 0; t < 4; ++t) fw[S][t] = *reinterpret_cast<const U2*>(tb + w_off[t]);
@@ -616,32 +633,45 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
       for (int mt = 0; mt < 4; ++mt) acc[mt][t + 1] = mfma16<T>(w1, fa[S][mt], acc[mt][t + 1]);
     }
   };
-  auto iteration = [&](auto set, uint32_t step) {
-    constexpr int S = decltype(set)::value;
-    // step + 1 must have landed (step + 2 may still be in flight), for every wave; and every wave must be done with
-    // the registers-from-LDS reads of step (issued an iteration ago, consumed below) before its stage is reused
-    if (step + 2 < s_end) __builtin_amdgcn_s_waitcnt(0x0f74);  // vmcnt(4)
-    else __builtin_amdgcn_s_waitcnt(0x0f70);                   // vmcnt(0)
+  auto iteration = [&](auto index, auto guarded, uint32_t step) {
+    constexpr int J = decltype(index)::value, S = J & 1, NEXT = (J + 1) % kTileAhead;  // J = (step - s_begin) % kTileAhead
+    constexpr bool GUARDED = decltype(guarded)::value;  // the last steps of the slice: step + 1 may be past the end
+    // the registers of step + 1 have landed; they go to the stage that step - 1 was read from (every wave's reads of
+    // it had returned before it passed the last barrier), and the register set takes the loads of step + 1 + kTileAhead
+    __builtin_amdgcn_s_waitcnt(0x0f7c);  // vmcnt(12)
+    if (!GUARDED || step + 1 < s_end) publish(std::integral_constant<int, NEXT>{}, step + 1);
+    request(std::integral_constant<int, NEXT>{}, step + 1 + kTileAhead);
     __syncthreads();
-    if (step + 3 < s_end) request(step + 3);  // (into the stage that step - 1 was read from: all of its reads have returned)
-    if (step + 1 < s_end) read_fragments(std::integral_constant<int, S ^ 1>{}, step + 1);
+    if (!GUARDED || step + 1 < s_end) read_fragments(std::integral_constant<int, S ^ 1>{}, step + 1);
     __builtin_amdgcn_sched_barrier(0);  // (the scheduler would move each read down to its first use)
-    multiply(set);
+    multiply(std::integral_constant<int, S>{});
   };
-#pragma unroll
-  for (uint32_t ahead = 0; ahead < 3; ++ahead)
-    if (s_begin + ahead < s_end) request(s_begin + ahead);
-  if (s_begin + 2 < s_end) __builtin_amdgcn_s_waitcnt(0x0f78);       // vmcnt(8): the first of three steps has landed
-  else if (s_begin + 1 < s_end) __builtin_amdgcn_s_waitcnt(0x0f74);  // vmcnt(4)
-  else __builtin_amdgcn_s_waitcnt(0x0f70);                           // vmcnt(0)
+  request(std::integral_constant<int, 0>{}, s_begin);
+  request(std::integral_constant<int, 1>{}, s_begin + 1);
+  request(std::integral_constant<int, 2>{}, s_begin + 2);
+  request(std::integral_constant<int, 3>{}, s_begin + 3);
+  __builtin_amdgcn_s_waitcnt(0x0f7c);  // vmcnt(12): the first of four steps has landed
+  publish(std::integral_constant<int, 0>{}, s_begin);
+  request(std::integral_constant<int, 0>{}, s_begin + kTileAhead);
   __syncthreads();
-  if (s_begin < s_end) read_fragments(std::integral_constant<int, 0>{}, s_begin);
-  for (uint32_t step = s_begin; step < s_end; step += 2) {
-    iteration(std::integral_constant<int, 0>{}, step);
-    if (step + 1 < s_end) iteration(std::integral_constant<int, 1>{}, step + 1);
+  read_fragments(std::integral_constant<int, 0>{}, s_begin);
+  // groups of four steps with a step after them: straight-line code; then the last one to four steps
+  uint32_t step = s_begin;
+  constexpr std::false_type plain{};
+  constexpr std::true_type guarded{};
+  for (; step + kTileAhead < s_end; step += kTileAhead) {
+    iteration(std::integral_constant<int, 0>{}, plain, step);
+    iteration(std::integral_constant<int, 1>{}, plain, step + 1);
+    iteration(std::integral_constant<int, 2>{}, plain, step + 2);
+    iteration(std::integral_constant<int, 3>{}, plain, step + 3);
   }
+  iteration(std::integral_constant<int, 0>{}, guarded, step);
+  if (step + 1 < s_end) iteration(std::integral_constant<int, 1>{}, guarded, step + 1);
+  if (step + 2 < s_end) iteration(std::integral_constant<int, 2>{}, guarded, step + 2);
+  if (step + 3 < s_end) iteration(std::integral_constant<int, 3>{}, guarded, step + 3);
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // (the re-reads of the last step, requested past the end)
 
-  // The four k-parts of a column half meet through LDS (8 waves x 16 tiles x 1 KiB = the 4 stages' 128 KiB): wave
+  // The four k-parts of a column half meet through LDS (8 waves x 16 tiles x 1 KiB = 128 KiB): wave
   // (kc, nh) adds up row tile kc, its own part and the three others in the order of kc.
   __syncthreads();  // (every wave is done reading fragments: the stages are free)
   V4F* const parts = reinterpret_cast<V4F*>(tile_lds);
@@ -805,6 +835,11 @@ void launch_mfma(const Q8Params& p, uint32_t variant, const Machine& mc, hipStre
   if (!(variant & 0xffff) && !((variant >> 19) & 1) && p.m <= 8 && p.k >= 2048 && p.n >= 64) {
     staged = true;
     nt = (p.k >= 16384 || (p.n >= 12288 && p.k <= 4096)) ? 2 : 1, waves = 8, slices = 1;  // (measured on the Llama shapes)
+  } else if (!(variant & 0xffff) && !((variant >> 19) & 1) && p.m <= 32 && p.k >= 2048 && p.k <= 8192 && p.n >= 8192) {
+    // 9 to 32 rows against many short weight rows: 64 columns per workgroup (K = 4096, N = 14336: 17.3 and 21.7 us
+    // at 16 and 32 rows against 18.6 and 23.3; with long rows and few columns the unstaged kernel stays ahead)
+    staged = true;
+    nt = 4, waves = 4, slices = 1;
   }
   if (staged) {  // chunks of 256 values of k
     const uint64_t sgroups = (p.n + 16 * nt - 1) / (16 * nt);
