@@ -47,8 +47,8 @@ def _q4_shapes():
             k = int(rng.choice([256, 512, 768, 1024, 2048])) if bs else int(rng.choice([96, 160, 1000, 1056, 2048]))
             n = int(rng.choice([1, 5, 16, 33, 100, 256, 700]))
             out.append((m, k, n, bs or k, bool(rng.integers(2))))
-    # row tiles x column tiles on both sides of 2560 (a wave per tile from there), and of the wave-tile sizes
-    out += [(640, 128, 1024, 32, True), (640, 128, 1008, 32, False), (1280, 64, 1024, 64, True), (2560, 256, 1030, 128, False),
+    # row tiles x column tiles on both sides of 2048 / 2560 (a wave per tile from there), and of the wave-tile sizes
+    out += [(512, 128, 1024, 32, True), (512, 128, 1008, 32, False), (640, 128, 1024, 32, True), (640, 128, 1008, 32, False), (640, 96, 1024, 96, False), (1280, 64, 1024, 64, True), (2560, 256, 1030, 128, False),
             (650, 96, 1024, 96, True), (1290, 64, 2048, 64, False)]
     return out
 

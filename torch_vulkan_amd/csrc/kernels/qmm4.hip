@@ -1277,10 +1277,10 @@ int launch_matrix(const Q4CParams& p, uint32_t phase_and_flags, uint32_t groupwi
       *err = "qmm4c: null or unaligned side-car address";
       return -1;
     }
-    // Enough row tiles x column tiles to give every SIMD two and a half waves: a wave per tile walks all of K; fewer: the
+    // Enough row tiles x column tiles to give every SIMD two waves (two and a half channelwise): a wave per tile walks all of K; fewer: the
     // one-row-tile kernel, whose four waves split K.  Phase values 1 | 2 with bit 4 (16) set keep the one-row-tile
     // kernel, with bit 5 (32) force the wave-per-tile kernel (tests, tuning).
-    const bool rows_kernel = ((uint64_t((p.m + 15) / 16) * M.tiles >= 2560 && !(flags & 16)) || (flags & 32));
+    const bool rows_kernel = ((uint64_t((p.m + 15) / 16) * M.tiles >= (M.upb ? 2048u : 2560u) && !(flags & 16)) || (flags & 32));
     // (wave tiles of 2 x 2, 2 x 1 or 1 x 1 matrix-core tiles: the largest that leaves every SIMD two and a half
     //  waves; flag bits 6-7 choose: 1 = 1 x 1, 2 = 2 x 1, 3 = 2 x 2)
     for (uint32_t m0 = 0; rows_kernel && m0 < p.m; m0 += 16 * 1024) {
