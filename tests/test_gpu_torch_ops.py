@@ -185,6 +185,25 @@ def test_scaled_mm_errors(tv):
         torch._scaled_mm(a, b, one, one, bias=torch.ones(5).to("vk"), out_dtype=torch.float32)
 
 
+def test_empty_inputs(tv):
+    """No rows: every op of the path returns an empty result of the right shape and type (and launches nothing wrong)."""
+    with on_gpu(tv):
+        b = torch.randint(-128, 128, (5, 64), dtype=torch.int8, generator=gen(1)).to("vk")
+        out = torch._weight_int8pack_mm(torch.zeros(0, 64, dtype=torch.bfloat16).to("vk"), b, torch.ones(5, dtype=torch.bfloat16).to("vk"))
+        assert out.shape == (0, 5) and out.dtype == torch.bfloat16
+        w, sc, bias = pack_case(6, 64, 32, 3, True)
+        packed = torch._dyn_quant_pack_4bit_weight(w, sc, bias, 32, 64, 6).to("vk")
+        out = torch._dyn_quant_matmul_4bit(torch.zeros(0, 64).to("vk"), packed, 32, 64, 6)
+        assert out.shape == (0, 6) and out.dtype == torch.float32
+        a8 = torch.zeros(0, 32).to(torch.float8_e4m3fn).to("vk")
+        b8 = torch.zeros(16, 32).to(torch.float8_e4m3fn).to("vk").t()
+        one = torch.ones(()).to("vk")
+        out = torch._scaled_mm(a8, b8, one, one, out_dtype=torch.bfloat16)
+        assert out.shape == (0, 16) and out.dtype == torch.bfloat16
+        out = torch.mm(torch.zeros(0, 8, dtype=torch.bfloat16).to("vk"), torch.zeros(8, 4, dtype=torch.bfloat16).to("vk"))
+        assert out.shape == (0, 4)
+
+
 def test_fallback_is_counted(tv):
     """An op without a vk kernel runs on the CPU and shows in fallback_counts (what on_gpu() watches)."""
     before = sum(tv.fallback_counts().values())
