@@ -164,3 +164,11 @@ def test_qmm8_empty_and_errors():
         abi.dispatch("qmm8_f32", [1], p, (0, 1, 1))
     with pytest.raises(abi.VktError, match="does not match"):
         abi.dispatch("qmm8_f32", [3], p)
+    # weights of 4 GiB and more are refused before anything is launched (32-bit indexing in the kernels)
+    p.n, p.k, p.a_sm = 70000, 65536, 65536
+    with pytest.raises(abi.VktError, match="too large"):
+        abi.dispatch("qmm8_f32", [1], p)
+    p.n, p.k, p.a_sm = 4, 16, 16
+    p.b = 0
+    with pytest.raises(abi.VktError, match="null tensor address"):
+        abi.dispatch("qmm8_f32", [1], p)
