@@ -146,6 +146,23 @@ def test_qmm8_golden_fixtures():
         assert (np.abs(oracle.to_f32(got, odt).astype(np.float64) - oracle.to_f32(g[key + "_out"], odt)) <= 2 * tol).all()
 
 
+@pytest.mark.parametrize("m", [1, 5, 40])
+def test_qmm8_vocabulary_sized_weights(m):
+    """A 1 GiB weight (N = 128256, K = 8192: byte offsets beyond 2^30) against the oracle on the last rows of the
+    weight, and against the same product of a slice of the weight on the first."""
+    import _dev
+    n, k = 128256, 8192
+    rng = np.random.default_rng(5)
+    b = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    a = torch.randn(m, k, generator=gen(6)).bfloat16()
+    s = (torch.rand(n, generator=gen(7)) / 50).bfloat16()
+    got = _dev.qmm8(bits(a), oracle.BF16, b, bits(s))
+    assert got.shape == (m, n)
+    for lo, hi in ((0, 300), (n - 300, n)):
+        bs_, ss_ = torch.from_numpy(b[lo:hi].copy()), s[lo:hi]
+        check_q8(np.ascontiguousarray(got[:, lo:hi]), a, bs_, ss_, torch.bfloat16)
+
+
 def test_qmm8_empty_and_errors():
     import _dev
     from torch_vulkan_amd import abi
