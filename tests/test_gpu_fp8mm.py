@@ -28,7 +28,7 @@ HW_WINDOW = 2.0**-13
 def on_matrix_cores(odt, variant, k):
     if variant in (6, 7, 255) or k % 16:
         return False
-    return variant in (1, 2, 3, 4, 5) or odt in (oracle.BF16, oracle.E4M3, oracle.E5M2)
+    return variant in (1, 2, 3, 4, 5, 8) or odt in (oracle.BF16, oracle.E4M3, oracle.E5M2)
 
 
 def run_case(m, k, n, fa, fb, out_dtype, rowwise, bias_dtype=None, scale_result=None, variant=0, seed=1, scale=1.0):
@@ -79,7 +79,7 @@ def test_scaled_mm_reference_cases(fa, fb, out_dtype, rowwise):
 
 @pytest.mark.parametrize("m,k,n", [(1, 16, 1), (130, 256, 70), (257, 384, 129), (64, 1040, 300), (300, 128, 520),
                                    (5, 100, 7), (33, 48, 17)])
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 255])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 255])
 @pytest.mark.parametrize("rowwise", [False, True])
 def test_scaled_mm_tile_edges(m, k, n, variant, rowwise):
     """Shapes that are not multiples of any tile, K tails (K % 128 != 0, K % 16 != 0 -> the

@@ -40,7 +40,7 @@ def test_gemm16_layouts(dtype, m, k, n):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 255])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 5, 255])
 @pytest.mark.parametrize("m,k,n", [(130, 256, 70), (257, 384, 129), (64, 1088, 300), (300, 128, 520)])
 def test_gemm16_tile_variants(dtype, variant, m, k, n):
     """The Linear layout (both operands contiguous along k) through every tile variant and the strided kernel."""
@@ -55,7 +55,7 @@ def test_gemm16_tile_variants(dtype, variant, m, k, n):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
-@pytest.mark.parametrize("variant", [0, 3, 4])
+@pytest.mark.parametrize("variant", [0, 3, 4, 5])
 @pytest.mark.parametrize("m,k,n", [(128, 64, 136), (264, 192, 520), (1032, 128, 1024), (8, 64, 8)])
 def test_gemm16_k_major_operands(dtype, variant, m, k, n):
     """Operands contiguous along m / n (x @ W with W row-major, x.t() @ y): the matrix-core tiles read them

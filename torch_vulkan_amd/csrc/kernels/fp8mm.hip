@@ -160,11 +160,13 @@ int launch_formats(const F8Params& p, uint32_t variant, int compute_units, hipSt
   // (tests, tuning): 1: 128x128 tiles (4 waves of 64x64, 16x16x128 MFMA); 2: 256x256 (4 waves of
   // 128x128, 16x16x128); 3: 256x128; 4: 256x256 with the 32x32x64 MFMA (measured ~10 % faster
   // than 16x16x128 at equal work); 5: as 4 with global-to-LDS direct loads when k is a
-  // multiple of 128 (else 4).  255: the one-thread-per-output kernel.
+  // multiple of 128 (else 4); 8: as 5 with 8 waves of 64x128 instead of 4 of 128x128 (two waves per SIMD cover each
+  // other's waits: 8192^3 2.34-2.42 -> 2.56-2.59 PFLOP/s; what large bfloat16 / float8 outputs get).  255: the
+  // one-thread-per-output kernel.
   // 6 / 7: the exact path (float8 widened to bfloat16 in registers, 32x32x16 bfloat16 MFMA) on
   // 256x256 / 128x128 tiles: what float32 and float16 outputs get.
   const bool big = uint64_t(p.m) * p.n >= (1ull << 20);
-  if (variant == 0) variant = (p.out_dtype == VKT_F32 || p.out_dtype == VKT_F16) ? (big ? 6 : 7) : (big ? 5 : 1);
+  if (variant == 0) variant = (p.out_dtype == VKT_F32 || p.out_dtype == VKT_F16) ? (big ? 6 : 7) : (big ? 8 : 1);
   switch (variant) {
     case 6:
       if (p.k % BK == 0) return launch_tile<2, 2, 8, 8, FA, FB, true, true, true>(p, compute_units, stream, err);
@@ -174,6 +176,12 @@ int launch_formats(const F8Params& p, uint32_t variant, int compute_units, hipSt
     case 2: return launch_tile<2, 2, 8, 8, FA, FB>(p, compute_units, stream, err);
     case 3: return launch_tile<2, 2, 8, 4, FA, FB>(p, compute_units, stream, err);
     case 4: return launch_tile<2, 2, 8, 8, FA, FB, true>(p, compute_units, stream, err);
+    case 9:  // as 6 with 8 waves of 64x128
+      if (p.k % BK == 0) return launch_tile<4, 2, 4, 8, FA, FB, true, true, true>(p, compute_units, stream, err);
+      return launch_tile<2, 2, 8, 4, FA, FB, true, false, true>(p, compute_units, stream, err);
+    case 8:  // 256x256 tiles over 8 waves of 64x128 (two waves per SIMD), direct loads
+      if (p.k % BK == 0) return launch_tile<4, 2, 4, 8, FA, FB, true, true>(p, compute_units, stream, err);
+      return launch_tile<2, 2, 8, 8, FA, FB, true>(p, compute_units, stream, err);
     case 5:
       if (p.k % BK == 0) return launch_tile<2, 2, 8, 8, FA, FB, true, true>(p, compute_units, stream, err);
       return launch_tile<2, 2, 8, 8, FA, FB, true>(p, compute_units, stream, err);

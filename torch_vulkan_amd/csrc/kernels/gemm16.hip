@@ -96,12 +96,15 @@ int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t
   g.alpha = bits_f32_host(uint32_t(p.alpha)), g.beta = bits_f32_host(uint32_t(p.beta));
   g.c_sm = p.c_sm, g.c_sb = p.c_sb, g.cin_sm = p.cin_sm, g.cin_sn = p.cin_sn, g.cin_sb = p.cin_sb;
   const bool direct_ok = g.k % BK == 0;
-  // variant 0: planned; 1: 128x128 tiles; 2: 256x128; 3: 256x256 with direct loads; 4: 128x128 with direct loads
+  // variant 0: planned; 1: 128x128 tiles; 2: 256x128; 3: 256x256 with direct loads; 4: 128x128 with direct loads;
+  // 5: 256x256 with direct loads over 8 waves
   // (direct loads: k a multiple of 64; k-major operands run on the direct forms only)
   if (variant == 0) {
     // 256 x 256 tiles where they give every compute unit one, else 128 x 128
     const bool large = uint64_t((p.m + 255) / 256) * ((p.n + 255) / 256) * batch >= uint64_t(mc.compute_units);
-    variant = large ? (direct_ok ? 3 : 2) : (TRA || TRB ? 4 : 1);
+    // (both operands k-major: 8 waves, whose transposing LDS reads cover each other: 8192^3 0.94 -> 1.11-1.13 PFLOP/s;
+    //  with k-contiguous operands the 8-wave form reads 1.5x the LDS bytes and is 3-5 % slower)
+    variant = large ? (direct_ok ? (TRA && TRB ? 5 : 3) : 2) : (TRA || TRB ? 4 : 1);
   }
   if constexpr (!TRA && !TRB) {
     if (variant == 1) return launch_mma_tile<2, 2, 4, 4, 0, 0, true, false, MATH>(g, mc.compute_units, stream, err, "gemmcm");
@@ -109,6 +112,8 @@ int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t
   }
   if (variant == 3 && direct_ok) return launch_mma_tile<2, 2, 8, 8, 0, 0, true, true, MATH>(g, mc.compute_units, stream, err, "gemmcm");
   if (variant == 4 && direct_ok) return launch_mma_tile<2, 2, 4, 4, 0, 0, true, true, MATH>(g, mc.compute_units, stream, err, "gemmcm");
+  // 5: 256x256 over 8 waves of 64x128 (two waves per SIMD), direct loads
+  if (variant == 5 && direct_ok) return launch_mma_tile<4, 2, 4, 8, 0, 0, true, true, MATH>(g, mc.compute_units, stream, err, "gemmcm");
   *err = "gemmcm: unknown variant " + std::to_string(variant) + " for this k and layout";
   return -1;
 }

@@ -296,8 +296,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void mma_tile(P p, uint32_t 
         if constexpr (TRB) return frag32_t(tb, BN, (wn * TN2 + j) * 32, kk);
         else return frag32(tb, (wn * TN2 + j) * 32 + l32, kk);
       };
+      // With two waves per SIMD (8 waves) the column fragments of the second half of k take the registers of the
+      // first half's, each right after its last use (256 registers per wave do not hold both halves next to the
+      // accumulators), and row fragments are asked for one group ahead: the other wave covers the LDS latency.
+      constexpr bool kLean = WAVES_M * WAVES_N > 4;
       V8I af = row_frag(0);
-      V8I bf[2][TN2];
+      V8I bf[kLean ? 1 : 2][TN2];
 #pragma unroll
       for (int j = 0; j < TN2; ++j) bf[0][j] = col_frag(j, 0);
       V8I next = row_frag(1 < 2 * TM2 ? 1 : 0);
@@ -306,9 +310,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void mma_tile(P p, uint32_t 
         const int kk = gi / TM2, i = gi % TM2;
         V8I next2 = next;
         if (gi + 2 < 2 * TM2) next2 = row_frag(gi + 2);
-        if (gi == 0) {
+        if (gi == 0 && !kLean) {
 #pragma unroll
-          for (int j = 0; j < TN2; ++j) bf[1][j] = col_frag(j, 1);
+          for (int j = 0; j < TN2; ++j) bf[kLean ? 0 : 1][j] = col_frag(j, 1);
         }
         V8BF af_wide[WIDE ? 4 : 1];
         if constexpr (WIDE) {
@@ -333,14 +337,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void mma_tile(P p, uint32_t 
           if constexpr (WIDE) {
 #pragma unroll
             for (int q = 0; q < 4; ++q)
-              acc32[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(widen_slice<FB>(bf[kk][j], q), af_wide[q], acc32[i][j], 0, 0, 0);
+              acc32[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(widen_slice<FB>(bf[kLean ? 0 : kk][j], q), af_wide[q], acc32[i][j], 0, 0, 0);
           } else if constexpr (MATH == kMathBf16 || MATH == kMathF16) {
             // 16-bit elements: a fragment's 32 bytes are two operands of 8 values
 #pragma unroll
-            for (int q = 0; q < 2; ++q) acc32[i][j] = mfma_16bit<MATH>(half_of(bf[kk][j], q), half_of(af, q), acc32[i][j]);
+            for (int q = 0; q < 2; ++q) acc32[i][j] = mfma_16bit<MATH>(half_of(bf[kLean ? 0 : kk][j], q), half_of(af, q), acc32[i][j]);
           } else {
-            acc32[i][j] = mfma_f8_32<FA, FB>(bf[kk][j], af, acc32[i][j]);
+            acc32[i][j] = mfma_f8_32<FA, FB>(bf[kLean ? 0 : kk][j], af, acc32[i][j]);
           }
+          if (kLean && gi == TM2 - 1) bf[0][j] = col_frag(j, 1);
         }
         __builtin_amdgcn_sched_barrier(0);
         af = next;
