@@ -258,6 +258,15 @@ typedef struct F8Params {
   uint32_t pad;
 } F8Params;
 
+/* "probe_read", spec {GEOMETRY} and "probe_mfma_f8", spec {OPERANDS}: calibration kernels for the rooflines (what
+ * a launch geometry can stream, what the fp8 matrix cores sustain on given operand bits); they read src [n, k] bytes
+ * (probe_read) or run `iters` iterations of 4 matrix-core instructions per wave, 4 waves on every compute unit
+ * (probe_mfma_f8), and write nothing (dst must be a valid address).  No counterpart in the reference.  32 bytes. */
+typedef struct ProbeParams {
+  uint64_t src, dst;
+  uint32_t n, k, iters, pad;
+} ProbeParams;
+
 enum { VKT_F32 = 0, VKT_F16 = 1, VKT_BF16 = 2, VKT_E4M3 = 3, VKT_E5M2 = 4 };
 
 #ifdef __cplusplus

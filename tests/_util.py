@@ -39,3 +39,32 @@ def unbits(a, dtype):
 def ref_tol(want_f32, mag, odt):
     """eps * |want| + 2^-20 * mag  (reference tests/python/test_quant.py:36-37)."""
     return EPS[odt] * np.abs(want_f32.astype(np.float64)) + 2.0**-20 * mag
+
+
+class no_fallback:
+    """with no_fallback(tv): ... fails if an op inside ran on the CPU instead of the device (the per-op fallback
+    counters of the backend moved), naming the ops.  The reference guards its device tests the same way."""
+
+    def __init__(self, backend):
+        self.backend = backend
+
+    def __enter__(self):
+        self.start = dict(self.backend.fallback_counts())
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        if exc_type is None:
+            moved = sorted(op for op, count in self.backend.fallback_counts().items() if count != self.start.get(op, 0))
+            assert not moved, "fell back to the CPU: " + ", ".join(moved)
+        return False
+
+
+def to_device(value, device="vk"):
+    """Tensors (also inside tuples, lists and dict values) moved to `device`; everything else as is."""
+    if isinstance(value, torch.Tensor):
+        return value.to(device)
+    if isinstance(value, (tuple, list)):
+        return type(value)(to_device(v, device) for v in value)
+    if isinstance(value, dict):
+        return {k: to_device(v, device) for k, v in value.items()}
+    return value

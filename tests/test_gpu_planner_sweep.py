@@ -10,7 +10,7 @@ import torch
 import oracle
 from _util import ODT, bits, gen
 from test_gpu_qmm8 import check_q8
-from test_oracle_pins import pack_case, q4_input, q8_case
+from _cases import int4_rows, int4_weights, int8_case
 
 pytestmark = pytest.mark.gpu
 
@@ -34,7 +34,7 @@ def test_qmm8_planner(dtype, m, k, n):
     import _dev
     if dtype != torch.bfloat16 and m * n * k > 1 << 27:
         pytest.skip("large case: bfloat16 only")
-    a, b, s = q8_case(dtype, m, k, n)
+    a, b, s = int8_case(dtype, m, k, n)
     check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s)), a, b, s, dtype)
 
 
@@ -57,12 +57,12 @@ def _q4_shapes():
 def test_qmm4_planner(m, k, n, bs, bias):
     import _dev
     from torch_vulkan_amd import abi
-    w, sc, bvec = pack_case(n, k, bs, 11, bias)
+    w, sc, bvec = int4_weights(n, k, bs, seed=11, bias=bias)
     packed = torch._dyn_quant_pack_4bit_weight(w, sc, bvec, bs, k, n).numpy()
     for dtype in (torch.float32, torch.bfloat16):
         if dtype == torch.bfloat16 and bs != k:
             continue
-        x = q4_input(m, k, dtype)
+        x = int4_rows(m, k, dtype)
         want = oracle.q4_matmul(bits(x), ODT[dtype], packed, bs, k, n)
         if not abi.lib().vkt_qmm4c_bytes(n, k, bs):
             assert np.array_equal(_dev.q4_reference_layout(bits(x), ODT[dtype], packed, bs, k, n), want)

@@ -9,7 +9,7 @@ import torch
 
 import oracle
 from _util import ODT, bits, gen
-from test_oracle_pins import Q4_CASES, pack_case, q4_input
+from _cases import INT4_SHAPES, int4_rows, int4_weights
 
 pytestmark = pytest.mark.gpu
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
@@ -24,15 +24,15 @@ EXTRA = [(2, 4096, 300, 32, True), (3, 14336, 20, 32, True), (9, 28672, 6, 128, 
          (16400, 64, 20, 32, True)]
 
 
-@pytest.mark.parametrize("m,k,n,bs,bias", Q4_CASES + EXTRA)
+@pytest.mark.parametrize("m,k,n,bs,bias", INT4_SHAPES + EXTRA)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_q4_bit_exact(m, k, n, bs, bias, dtype):
     import _dev
     from torch_vulkan_amd import abi
     if dtype == torch.bfloat16 and bs != k:
         pytest.skip("bfloat16 inputs are channelwise only (the CPU's check)")
-    w, sc, bvec = pack_case(n, k, bs, 7, bias)
-    x = q4_input(m, k, dtype)
+    w, sc, bvec = int4_weights(n, k, bs, bias=bias)
+    x = int4_rows(m, k, dtype)
     packed = torch._dyn_quant_pack_4bit_weight(w, sc, bvec, bs, k, n)
     want = bits(torch._dyn_quant_matmul_4bit(x, packed, bs, k, n))
     odt = ODT[dtype]
@@ -94,7 +94,7 @@ def test_q4_config3(m):
 def test_q4_golden_fixtures():
     import _dev
     g = np.load(os.path.join(GOLDEN, "q4.npz"))
-    for i in range(len(Q4_CASES)):
+    for i in range(len(INT4_SHAPES)):
         m, k, n, bs, bias = (int(v) for v in g[f"c{i}_shape"])
         for tag, odt in (("f32", oracle.F32), ("bf16", oracle.BF16)):
             key = f"c{i}_{tag}"

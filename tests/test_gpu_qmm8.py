@@ -9,7 +9,7 @@ import torch
 
 import oracle
 from _util import ODT, bits, gen, ref_tol, unbits
-from test_oracle_pins import Q8_SHAPES, q8_case
+from _cases import INT8_SHAPES, int8_case
 
 pytestmark = pytest.mark.gpu
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
@@ -27,11 +27,11 @@ def check_q8(got_bits, a, b, s, dtype, rows=slice(None)):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("m,k,n", Q8_SHAPES + [(1, 4096, 4096), (8, 4096, 640), (16, 2048, 130), (3, 1024, 7),
+@pytest.mark.parametrize("m,k,n", INT8_SHAPES + [(1, 4096, 4096), (8, 4096, 640), (16, 2048, 130), (3, 1024, 7),
                                                (17, 256, 33), (2, 16, 1), (1, 48, 5)])
 def test_qmm8_reference_shapes(dtype, m, k, n):
     import _dev
-    a, b, s = q8_case(dtype, m, k, n)
+    a, b, s = int8_case(dtype, m, k, n)
     got = _dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s))
     assert got.shape == (m, n)
     check_q8(got, a, b, s, dtype)
@@ -46,7 +46,7 @@ def test_qmm8_every_variant(variant, dtype):
     """Each (COLS, KSPLIT) instantiation and the generic kernel give results inside the band."""
     import _dev
     for m, k, n in [(1, 4096, 130), (4, 2064, 67)]:
-        a, b, s = q8_case(dtype, m, k, n)
+        a, b, s = int8_case(dtype, m, k, n)
         check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=variant), a, b, s, dtype)
 
 
@@ -61,7 +61,7 @@ def test_qmm8_matrix_core_variants(dtype, variant, m, k, n):
     library's workspace), the GEMV kernels forced on the same problem (bit 17), and the kernel that stages the
     weights through LDS (bit 18; up to 32 rows, otherwise the plain one runs)."""
     import _dev
-    a, b, s = q8_case(dtype, m, k, n)
+    a, b, s = int8_case(dtype, m, k, n)
     check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=variant), a, b, s, dtype)
     sliced_variant = variant if (m + 1) // 2 > 4 else 0  # (4 rows or fewer: the GEMV kernels plan themselves)
     check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=sliced_variant, row_step=2), a, b, s, dtype,
@@ -74,7 +74,7 @@ def test_qmm8_many_rows(dtype, m, k, n):
     """From 192 rows on (prefill) the weights are widened once into the library's scratch region and the product runs
     on the tile kernel; the row-block kernels (variant bit 20) give the same results to the test's bound."""
     import _dev
-    a, b, s = q8_case(dtype, m, k, n)
+    a, b, s = int8_case(dtype, m, k, n)
     got = _dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s))
     check_q8(got, a, b, s, dtype)
     check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=1 << 20), a, b, s, dtype)
@@ -88,7 +88,7 @@ def test_qmm8_tile_kernel(dtype, variant, m, k, n):
     """More than 32 rows with k a multiple of 256 run on the tile kernel (64 x 128 tiles, K sliced over workgroups,
     slices met in the workspace): planned, forced with 1 and 3 slices (bit 21; also with fewer rows), and switched off (bit 22)."""
     import _dev
-    a, b, s = q8_case(dtype, m, k, n)
+    a, b, s = int8_case(dtype, m, k, n)
     check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=variant), a, b, s, dtype)
     if m > 8:
         check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=variant, row_step=2), a, b, s, dtype, rows=slice(None, None, 2))

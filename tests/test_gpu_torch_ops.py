@@ -1,14 +1,22 @@
-"""The five quantised aten ops on device "vk", written as the reference's own tests are
-(tests/python/test_quant.py): each op on "vk" against PyTorch's CPU result, with the
-reference's `on_gpu()` assertion that nothing fell back to the CPU (tests/python/_util.py:28-35).
+"""The five quantised aten ops on device "vk": each op called on device tensors, with nothing allowed to fall back
+to the CPU, against the oracle (and PyTorch's CPU op where it has one), on the reference's parametrisations
+(tests/python/test_quant.py:20-21,61-63,101-103, kept as tables in _cases.py), on the frozen fixtures under
+tests/golden/, and on the op layer's own behaviour (side-car cache, inference tensors, empty products, errors).
 The C++ op layer (csrc/torch/quant.cpp) reaches the kernels through the C ABI."""
 import contextlib
+import os
 
+import numpy as np
 import pytest
 import torch
 
+import oracle
+from _cases import (FLOAT8, FLOAT8_OUT, FLOAT8_PAIRS, INT4_SHAPES, INT8_SHAPES, draw, float8_case, int4_rows, int4_weights,
+                    int8_case)
+from _util import ODT, bits, no_fallback as on_gpu, ref_tol, to_device, unbits
+
 pytestmark = pytest.mark.gpu
-FLOAT8 = [torch.float8_e4m3fn, torch.float8_e5m2]
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 # bfloat16 / float8 results come off the fp8 matrix cores, whose products are added in a
 # window ~14 bits below the largest (a hardware property); float32 / float16 results are exact sums
 HW_WINDOW = 2.0**-13
@@ -17,22 +25,28 @@ HW_WINDOW = 2.0**-13
 @pytest.fixture(scope="module")
 def tv():
     import torch_vulkan_amd.backend as tv
-    assert tv.is_available() and (tv.capabilities() & 12) == 12  # 8- and 16-bit storage (test_quant.py:12)
+    assert tv.is_available() and (tv.capabilities() & 12) == 12  # 8- and 16-bit storage
     return tv
-
-
-@contextlib.contextmanager
-def on_gpu(tv):
-    """Fails if anything inside falls back to the CPU."""
-    before = tv.fallback_counts()
-    yield
-    after = tv.fallback_counts()
-    new = {k: v - before.get(k, 0) for k, v in after.items() if v != before.get(k, 0)}
-    assert not new, f"ran on the CPU: {new}"
 
 
 def gen(seed):
     return torch.Generator().manual_seed(seed)
+
+
+def on_vk(tv, op, *args, **kwargs):
+    """op(*args, **kwargs) with every tensor moved to the device, nothing allowed to run on the CPU; the results
+    come back as host tensors (a tuple stays a tuple)."""
+    with on_gpu(tv):
+        out = op(*to_device(args), **to_device(kwargs))
+    assert all(t.device.type == "vk" for t in (out if isinstance(out, tuple) else (out,)))
+    return to_device(out, "cpu")
+
+
+def raises_each(table, call):
+    """table: (exception type, message pattern, arguments); call(*arguments) must raise that."""
+    for kind, pattern, arguments in table:
+        with pytest.raises(kind, match=pattern):
+            call(*arguments)
 
 
 def test_device_round_trip(tv):
@@ -50,139 +64,257 @@ def test_device_round_trip(tv):
     torch.vk.synchronize()
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("m,k,n", [(32, 64, 48), (1, 4096, 300), (5, 100, 17), (70, 33, 5), (65, 1, 66)])
-def test_weight_int8pack_mm(tv, dtype, m, k, n):
-    a = torch.randn(m, k, generator=gen(1)).to(dtype)
-    b = torch.randint(-128, 128, (n, k), dtype=torch.int8, generator=gen(2))
-    s = (torch.rand(n, generator=gen(3)) / 50).to(dtype)
-    want = (a.float() @ (b.float() * s.float()[:, None]).t()).to(dtype)
+# ------------------------------------------------------------------ _weight_int8pack_mm
+def within_int8_band(got, dtype, a, b, s, rows=slice(None)):
+    """|got - float64 sum| <= eps |sum| + 2^-20 sum|a||w| (the bound the reference's test states), from the oracle."""
+    _, c64, mag = oracle.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), want_f64=True)
+    assert got.dtype == dtype and got.shape == c64[rows].shape
+    excess = np.abs(got.double().numpy() - c64[rows]) - ref_tol(c64, mag, ODT[dtype])[rows]
+    assert (excess <= 0).all(), excess.max()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("shape", INT8_SHAPES, ids=str)
+def test_int8_weight_product(tv, dtype, shape):
+    case = int8_case(dtype, *shape)
+    within_int8_band(on_vk(tv, torch._weight_int8pack_mm, *case), dtype, *case)
+    # every other row of A, read in place through the row stride
     with on_gpu(tv):
-        got = torch._weight_int8pack_mm(a.to("vk"), b.to("vk"), s.to("vk"))
-        sliced = torch._weight_int8pack_mm(a.to("vk")[::2], b.to("vk"), s.to("vk"))
-    mag = a.float().abs() @ (b.float() * s.float()[:, None]).abs().t()
-    tol = torch.finfo(dtype).eps * want.float().abs() + 2**-20 * mag
-    assert got.dtype == want.dtype and got.shape == want.shape and got.device.type == "vk"
-    assert ((got.cpu().float() - want.float()).abs() <= tol).all()
-    assert ((sliced.cpu().float() - want[::2].float()).abs() <= tol[::2]).all()
+        a, b, s = to_device(tuple(case))
+        strided = torch._weight_int8pack_mm(a[::2], b, s).cpu()
+    within_int8_band(strided, dtype, *case, rows=slice(None, None, 2))
 
 
-def test_weight_int8pack_mm_errors(tv):
-    a, b, s = torch.randn(4, 8).to("vk"), torch.zeros(3, 8, dtype=torch.int8).to("vk"), torch.ones(3).to("vk")
-    with pytest.raises(RuntimeError, match="expect B to be int8 tensor"):
-        torch._weight_int8pack_mm(a, b.float(), s)
-    with pytest.raises(RuntimeError, match="expect scales to be 1d tensor with size 3"):
-        torch._weight_int8pack_mm(a, b, s[:2])
-    with pytest.raises(RuntimeError, match="A must be contiguous on the last dimension"):
-        torch._weight_int8pack_mm(a.t().contiguous().t(), b[:, :4], s)
+def test_int8_weight_product_fixtures(tv):
+    """The frozen CPU results (tests/golden/q8.npz): the device inside twice the band around them that the oracle's
+    float64 sum is held to (both sides are roundings of that sum)."""
+    g = np.load(os.path.join(GOLDEN, "q8.npz"))
+    for key in sorted(k[:-2] for k in g.files if k.endswith("_a")):
+        odt = int(g[key + "_odt"])
+        dtype = {v: k for k, v in ODT.items()}[odt]
+        a, s, b = unbits(g[key + "_a"], dtype), unbits(g[key + "_s"], dtype), torch.from_numpy(g[key + "_b"])
+        got = on_vk(tv, torch._weight_int8pack_mm, a, b, s)
+        _, c64, mag = oracle.qmm8(g[key + "_a"], odt, g[key + "_b"], g[key + "_s"], want_f64=True)
+        frozen = oracle.to_f32(g[key + "_out"], odt).astype(np.float64)
+        assert (np.abs(got.double().numpy() - frozen) <= 2 * ref_tol(c64, mag, odt)).all(), key
 
 
-def pack_case(n, k, bs, seed, bias):
-    w = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, generator=gen(seed))
-    nb = 1 if bs == k else k // bs
-    sc = torch.rand(n, nb, generator=gen(seed + 1)) / 10
-    sc = sc if bs == k else sc.to(torch.bfloat16)
-    return w, sc, (torch.randn(n, generator=gen(seed + 2)) if bias else None)
+def test_int8_weight_product_refusals(tv):
+    a, b, s = to_device((torch.randn(4, 8), torch.zeros(3, 8, dtype=torch.int8), torch.ones(3)))
+    raises_each([(RuntimeError, "expect B to be int8 tensor", (a, b.float(), s)),
+                 (RuntimeError, "expect scales to be 1d tensor with size 3", (a, b, s[:2])),
+                 (RuntimeError, "A must be contiguous on the last dimension", (a.t().contiguous().t(), b[:, :4], s))],
+                torch._weight_int8pack_mm)
 
 
-@pytest.mark.parametrize("m,k,n,bs,bias", [(1, 64, 4096, 32, False), (32, 128, 11008, 32, True), (5, 96, 70, 96, True),
-                                           (3, 100, 9, 100, False), (4, 256, 16, 64, True), (9, 64, 33, 64, False)])
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_dyn_quant_matmul_4bit_exact(tv, m, k, n, bs, bias, dtype):
-    if dtype == torch.bfloat16 and bs != k:
-        pytest.skip("bfloat16 inputs are channelwise only (the CPU's check)")
-    w, sc, bvec = pack_case(n, k, bs, 7, bias)
-    x = (torch.randn(m, k, generator=gen(11)) * 3).to(dtype)
-    x[0, : k // 2] = 0.0
-    if m > 1:
-        x[1] = -x[1].abs()
-    packed = torch._dyn_quant_pack_4bit_weight(w, sc, bvec, bs, k, n)
-    want = torch._dyn_quant_matmul_4bit(x, packed, bs, k, n)
+# ------------------------------------------------------------------ _dyn_quant_pack_4bit_weight / _dyn_quant_matmul_4bit
+INT4_DTYPES = [(torch.float32, True), (torch.bfloat16, False)]  # (activation type, also with groupwise blocks)
+
+
+@pytest.mark.parametrize("m,k,n,bs,bias", INT4_SHAPES)
+@pytest.mark.parametrize("dtype,groupwise_too", INT4_DTYPES, ids=["float32", "bfloat16"])
+def test_int4_product_bit_exact(tv, m, k, n, bs, bias, dtype, groupwise_too):
+    if bs != k and not groupwise_too:
+        pytest.skip("bfloat16 activations take one block per channel only (the CPU's check)")
+    weights = int4_weights(n, k, bs, bias=bias)
+    x = int4_rows(m, k, dtype)
+    # the expectation: the oracle's packed vector and product, which the CPU's ops must equal bit for bit too
+    packed = oracle.q4_pack(weights.nibble_bytes.numpy(), bits(weights.scales), ODT[weights.scales.dtype],
+                            None if weights.bias is None else weights.bias.numpy())
+    want = oracle.q4_matmul(bits(x), ODT[dtype], packed, bs, k, n)
+    assert np.array_equal(bits(torch._dyn_quant_matmul_4bit(x, torch.from_numpy(packed), bs, k, n)), want)
     with on_gpu(tv):
-        packed_vk = torch._dyn_quant_pack_4bit_weight(w.to("vk"), sc.to("vk"), None if bvec is None else bvec.to("vk"),
-                                                      bs, k, n)
-        got = torch._dyn_quant_matmul_4bit(x.to("vk"), packed_vk, bs, k, n)
-        again = torch._dyn_quant_matmul_4bit(x.to("vk"), packed_vk, bs, k, n)  # (the cached side-car)
-        got_cpu_packed = torch._dyn_quant_matmul_4bit(x.to("vk"), packed.to("vk"), bs, k, n)
-    assert torch.equal(packed_vk.cpu(), packed)
-    assert got.dtype == want.dtype
-    assert torch.equal(got.cpu(), want) and torch.equal(again.cpu(), want)
-    assert torch.equal(got_cpu_packed.cpu(), want)
+        packed_on_device = torch._dyn_quant_pack_4bit_weight(*to_device(tuple(weights)), bs, k, n)
+        x_vk = x.to("vk")
+        products = [torch._dyn_quant_matmul_4bit(x_vk, packed_on_device, bs, k, n),
+                    torch._dyn_quant_matmul_4bit(x_vk, packed_on_device, bs, k, n),  # (from the cached side-car)
+                    torch._dyn_quant_matmul_4bit(x_vk, torch.from_numpy(packed).to("vk"), bs, k, n)]  # (packed on the host)
+    assert np.array_equal(packed_on_device.cpu().numpy().view(np.uint32), packed.view(np.uint32))
+    for got in products:
+        assert got.dtype == dtype and np.array_equal(bits(got.cpu()), want)
 
 
-def test_dyn_quant_sidecar_follows_writes(tv):
-    """The cached side-car is keyed by the packed tensor's version: an in-place change of the
-    packed weights must show in the next product."""
-    w, sc, _ = pack_case(16, 64, 32, 3, False)
-    x = torch.randn(2, 64, generator=gen(5))
-    packed = torch._dyn_quant_pack_4bit_weight(w, sc, None, 32, 64, 16)
-    pv = packed.to("vk")
-    first = torch._dyn_quant_matmul_4bit(x.to("vk"), pv, 32, 64, 16).cpu()
-    packed2 = packed.clone()
-    packed2[: 16 * 32] = 255.0 - packed2[: 16 * 32]
-    pv.copy_(packed2)
-    second = torch._dyn_quant_matmul_4bit(x.to("vk"), pv, 32, 64, 16).cpu()
-    assert torch.equal(first, torch._dyn_quant_matmul_4bit(x, packed, 32, 64, 16))
-    assert torch.equal(second, torch._dyn_quant_matmul_4bit(x, packed2, 32, 64, 16))
+def test_int4_product_fixtures(tv):
+    """The frozen CPU results (tests/golden/q4.npz), bit for bit."""
+    g = np.load(os.path.join(GOLDEN, "q4.npz"))
+    for i in range(len(INT4_SHAPES)):
+        m, k, n, bs, _ = (int(v) for v in g[f"c{i}_shape"])
+        for tag, dtype in (("f32", torch.float32), ("bf16", torch.bfloat16)):
+            if f"c{i}_{tag}_out" not in g:
+                continue
+            got = on_vk(tv, torch._dyn_quant_matmul_4bit, unbits(g[f"c{i}_{tag}_x"], dtype), torch.from_numpy(g[f"c{i}_packed"]), bs, k, n)
+            assert np.array_equal(bits(got), g[f"c{i}_{tag}_out"]), (i, tag)
 
 
-def test_dyn_quant_errors(tv):
-    x = torch.randn(2, 64).to("vk")
-    w, sc, _ = pack_case(8, 64, 32, 3, False)
-    with pytest.raises(RuntimeError, match="Group size should be multiple of 32"):
-        torch._dyn_quant_pack_4bit_weight(w.to("vk"), sc.to("vk"), None, 48, 64, 8)
-    with pytest.raises(RuntimeError, match="expect weight to be kByte"):
-        torch._dyn_quant_pack_4bit_weight(w.to(torch.int8).to("vk"), sc.to("vk"), None, 32, 64, 8)
-    packed = torch._dyn_quant_pack_4bit_weight(w.to("vk"), sc.to("vk"), None, 32, 64, 8)
-    with pytest.raises(RuntimeError, match="expect input to be float32 or bfloat16 tensor"):
-        torch._dyn_quant_matmul_4bit(x.cpu().bfloat16().to("vk"), packed, 32, 64, 8)
-    with pytest.raises(RuntimeError, match="Invalid packed weight tensor size"):
-        torch._dyn_quant_matmul_4bit(x, packed[:100], 32, 64, 8)
+def test_int4_under_inference_mode(tv):
+    """Inference tensors carry no version counter: packing and multiplying under torch.inference_mode() (and
+    no_grad) must work and agree with the CPU."""
+    n, k, bs = 24, 128, 32
+    weights = int4_weights(n, k, bs, seed=31, bias=True)
+    x = int4_rows(5, k, torch.float32, seed=32)
+    want = torch._dyn_quant_matmul_4bit(x, torch._dyn_quant_pack_4bit_weight(*weights, bs, k, n), bs, k, n)
+    for mode in (torch.inference_mode, torch.no_grad):
+        with mode(), on_gpu(tv):
+            packed = torch._dyn_quant_pack_4bit_weight(*to_device(tuple(weights)), bs, k, n)
+            first = torch._dyn_quant_matmul_4bit(x.to("vk"), packed, bs, k, n)
+            one_row = torch._dyn_quant_matmul_4bit(x[:1].to("vk"), packed, bs, k, n)  # (the other side-car layout)
+            again = torch._dyn_quant_matmul_4bit(x.to("vk"), packed, bs, k, n)
+        assert torch.equal(first.cpu(), want) and torch.equal(again.cpu(), want) and torch.equal(one_row.cpu(), want[:1])
 
 
-@pytest.mark.parametrize("fa,fb", [(FLOAT8[0], FLOAT8[0]), (FLOAT8[1], FLOAT8[0]), (FLOAT8[0], FLOAT8[1])])
-@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32, torch.float16, torch.float8_e4m3fn, None])
-@pytest.mark.parametrize("rowwise", [False, True])
-def test_scaled_mm(tv, fa, fb, out_dtype, rowwise):
-    a = torch.randn(16, 32, generator=gen(1)).to(fa)
-    b = torch.randn(48, 32, generator=gen(2)).to(fb).t()
-    sa = torch.rand(16, 1, generator=gen(3)) + 0.5 if rowwise else torch.tensor(1.25)
-    sb = torch.rand(1, 48, generator=gen(4)) + 0.5 if rowwise else torch.tensor(0.75)
-    bias = torch.randn(48, generator=gen(5)).to(torch.bfloat16) if out_dtype == torch.bfloat16 else None
-    scale_result = torch.tensor(2.0) if out_dtype == torch.float8_e4m3fn else None
-    kw = dict(bias=bias, out_dtype=out_dtype, scale_result=scale_result)
-    res_dtype = out_dtype or fa
-    if rowwise:  # torch 2.10's CPU kernel takes per-tensor scales only: the closed form it emulates
-        want = (a.float() * sa) @ (b.float() * sb)
-        want = want + bias.float() if bias is not None else want
-        want = (want * 0.5 if scale_result is not None else want).to(res_dtype)
-    else:
-        want = torch._scaled_mm(a, b, sa, sb, **kw)
-    vkw = {k: (v.to("vk") if isinstance(v, torch.Tensor) else v) for k, v in kw.items()}
+def test_int4_sidecar_follows_writes(tv):
+    """A side-car belongs to one version of the packed tensor: writing into the packed weights must show in the
+    next product."""
+    n, k, bs = 16, 64, 32
+    weights = int4_weights(n, k, bs, seed=3)
+    x = draw(("normal", (2, k)), 5)
+    packed = torch._dyn_quant_pack_4bit_weight(*weights, bs, k, n)
+    flipped = packed.clone()
+    flipped[: n * k // 2] = 255.0 - flipped[: n * k // 2]
+    on_device = packed.to("vk")
+    before = torch._dyn_quant_matmul_4bit(x.to("vk"), on_device, bs, k, n).cpu()
+    on_device.copy_(flipped)
+    after = torch._dyn_quant_matmul_4bit(x.to("vk"), on_device, bs, k, n).cpu()
+    assert torch.equal(before, torch._dyn_quant_matmul_4bit(x, packed, bs, k, n))
+    assert torch.equal(after, torch._dyn_quant_matmul_4bit(x, flipped, bs, k, n))
+
+
+def test_int4_sidecars_of_a_whole_model(tv):
+    """300 live packed weights (more linear layers than Llama-3-8B has), decoded twice: the second pass must find
+    every side-car (no "qmm4c_pack": one dispatch per product), results unchanged; a dead weight's side-car goes."""
+    n, k, bs, layers = 16, 64, 32, 300
+    torch.ops.vk.sidecar_cache(True)
+    x = draw(("normal", (1, k)), 40).to("vk")
+    base = int4_weights(n, k, bs, seed=41, bias=True)
+    packed = []
+    for layer in range(layers):
+        nibble_bytes = base.nibble_bytes.roll(layer, 1)  # a different weight per layer, cheaply
+        packed.append(torch._dyn_quant_pack_4bit_weight(nibble_bytes, base.scales, base.bias, bs, k, n).to("vk"))
     with on_gpu(tv):
-        got = torch._scaled_mm(a.to("vk"), b.to("vk"), sa.to("vk"), sb.to("vk"), **vkw)
-        out = torch.empty(0, dtype=want.dtype).to("vk")
-        torch._scaled_mm(a.to("vk"), b.to("vk"), sa.to("vk"), sb.to("vk"), **vkw, out=out)
-    assert got.dtype == want.dtype and got.shape == want.shape
-    mag = (a.float() * sa).abs() @ (b.float() * sb).abs() / (2.0 if scale_result is not None else 1.0)
-    eps = torch.finfo(want.dtype).eps
-    tol = eps * want.float().abs() + 2**-20 * mag
-    if want.dtype not in (torch.float32, torch.float16):
+        start = tv.dispatch_count()
+        first = [torch._dyn_quant_matmul_4bit(x, w, bs, k, n) for w in packed]
+        middle = tv.dispatch_count()
+        second = [torch._dyn_quant_matmul_4bit(x, w, bs, k, n) for w in packed]
+        end = tv.dispatch_count()
+    assert middle - start == 2 * layers and end - middle == layers
+    entries, held = torch.ops.vk.sidecar_cache()
+    assert entries == layers and held >= layers * n * k // 2
+    for layer in (0, 1, 150, 299):
+        want = torch._dyn_quant_matmul_4bit(x.cpu(), packed[layer].cpu(), bs, k, n)
+        assert torch.equal(first[layer].cpu(), want) and torch.equal(second[layer].cpu(), want)
+    del packed[:100]
+    assert torch.ops.vk.sidecar_cache()[0] == layers - 100
+    assert torch.ops.vk.sidecar_cache(True) == (0, 0)
+
+
+def test_int4_refusals(tv):
+    n, k = 8, 64
+    weights = int4_weights(n, k, 32, seed=3)
+    w, sc = weights.nibble_bytes.to("vk"), weights.scales.to("vk")
+    raises_each([(RuntimeError, "Group size should be multiple of 32", (w, sc, None, 48, k, n)),
+                 (RuntimeError, "expect weight to be kByte", (w.cpu().to(torch.int8).to("vk"), sc, None, 32, k, n))],
+                torch._dyn_quant_pack_4bit_weight)
+    packed = torch._dyn_quant_pack_4bit_weight(w, sc, None, 32, k, n)
+    x = torch.randn(2, k).to("vk")
+    raises_each([(RuntimeError, "expect input to be float32 or bfloat16 tensor", (x.cpu().bfloat16().to("vk"), packed, 32, k, n)),
+                 (RuntimeError, "Invalid packed weight tensor size", (x, packed[:100], 32, k, n))],
+                torch._dyn_quant_matmul_4bit)
+
+
+# ------------------------------------------------------------------ _scaled_mm
+def scaled_mm_expectation(case):
+    """(expected values as float64 in the result type's precision, allowed error) from the oracle: its float64-accurate
+    sum rounded once, the reference's bound eps |want| + 2^-20 sum|a||b| and, for results that come off the fp8
+    matrix cores, their summation window."""
+    a, b, sa, sb, bias, sr, res_dtype = case
+    want, mag = oracle.scaled_mm(bits(a), ODT[a.dtype], bits(b.t()), ODT[b.dtype], sa.numpy(), sb.numpy(), sa.numel() > 1,
+                                 None if bias is None else bits(bias), oracle.BF16, None if sr is None else float(sr),
+                                 ODT[res_dtype], want_mag=True)
+    want = oracle.to_f32(want, ODT[res_dtype]).astype(np.float64)
+    mag = mag / (float(sr) if sr is not None else 1.0)
+    tol = ref_tol(want, mag, ODT[res_dtype])
+    if res_dtype not in (torch.float32, torch.float16):
         tol = tol + HW_WINDOW * mag
-    for res in (got, out):
-        assert ((res.cpu().float() - want.float()).abs() <= tol).all()
+    return want, tol
 
 
-def test_scaled_mm_errors(tv):
+@pytest.mark.parametrize("fa,fb", FLOAT8_PAIRS, ids=str)
+@pytest.mark.parametrize("out_dtype", FLOAT8_OUT, ids=str)
+@pytest.mark.parametrize("rowwise", [False, True], ids=["per_tensor", "per_row"])
+def test_scaled_mm(tv, fa, fb, out_dtype, rowwise):
+    case = float8_case(fa, fb, out_dtype, rowwise)
+    want, tol = scaled_mm_expectation(case)
+    options = dict(bias=case.bias, scale_result=case.scale_result, out_dtype=out_dtype)
+    functional = on_vk(tv, torch._scaled_mm, case.a, case.b, case.scale_a, case.scale_b, **options)
+    with on_gpu(tv):
+        into = torch.empty(0, dtype=case.result_dtype).to("vk")
+        torch._scaled_mm(*to_device((case.a, case.b, case.scale_a, case.scale_b)), **to_device(options), out=into)
+    for got in (functional, into.cpu()):
+        assert got.dtype == case.result_dtype and got.shape == want.shape
+        assert (np.abs(got.double().numpy() - want) <= tol).all()
+
+
+def test_scaled_mm_fixtures(tv):
+    """The frozen CPU results (tests/golden/f8.npz, per-tensor scales)."""
+    g = np.load(os.path.join(GOLDEN, "f8.npz"))
+    torch_type = {v: k for k, v in ODT.items()}
+    for key in sorted(k[:-2] for k in g.files if k.endswith("_a")):
+        fa, fb, odt = (int(v) for v in g[key + "_fmt"])
+        sr = float(g[key + "_sr"]) if key + "_sr" in g else None
+        bias = unbits(g[key + "_bias"], torch.bfloat16) if key + "_bias" in g else None
+        _, mag = oracle.scaled_mm(g[key + "_a"], fa, g[key + "_bt"], fb, g[key + "_sa"], g[key + "_sb"], False,
+                                  None if bias is None else bits(bias), oracle.BF16, sr, odt, want_mag=True)
+        mag = mag / (sr or 1.0)
+        frozen = oracle.to_f32(g[key + "_out"], odt).astype(np.float64)
+        asked = None if key.endswith("_None") else torch_type[odt]
+        got = on_vk(tv, torch._scaled_mm, unbits(g[key + "_a"], torch_type[fa]), unbits(g[key + "_bt"], torch_type[fb]).t(),
+                    torch.tensor(float(g[key + "_sa"][0])), torch.tensor(float(g[key + "_sb"][0])), bias=bias,
+                    scale_result=None if sr is None else torch.tensor(sr), out_dtype=asked)
+        tol = ref_tol(frozen, mag, odt) + (0 if torch_type[odt] in (torch.float32, torch.float16) else HW_WINDOW * mag)
+        assert got.dtype == torch_type[odt] and (np.abs(got.double().numpy() - frozen) <= tol).all(), key
+
+
+def test_scaled_mm_result_scale_needs_a_float8_out_dtype(tv):
+    """scale_result applies when out_dtype asks for float8; without out_dtype the functional form returns the
+    operands' float8 type unscaled, as the CPU's op does."""
+    case = float8_case(FLOAT8[0], FLOAT8[0], None, False)
+    sr = torch.tensor(4.0)
+    plain = torch._scaled_mm(case.a, case.b, case.scale_a, case.scale_b)
+    assert torch.equal(torch._scaled_mm(case.a, case.b, case.scale_a, case.scale_b, scale_result=sr).view(torch.uint8),
+                       plain.view(torch.uint8))  # (the CPU ignores it here)
+    unscaled = on_vk(tv, torch._scaled_mm, case.a, case.b, case.scale_a, case.scale_b, scale_result=sr)
+    without = on_vk(tv, torch._scaled_mm, case.a, case.b, case.scale_a, case.scale_b)
+    scaled = on_vk(tv, torch._scaled_mm, case.a, case.b, case.scale_a, case.scale_b, scale_result=sr, out_dtype=FLOAT8[0])
+    assert unscaled.dtype == FLOAT8[0] and torch.equal(unscaled.view(torch.uint8), without.view(torch.uint8))
+    want, tol = scaled_mm_expectation(case)
+    assert (np.abs(unscaled.double().numpy() - want) <= tol).all()
+    assert (np.abs(scaled.double().numpy() * 4.0 - want) <= 4.0 * tol + 2.0**-3 * np.abs(want)).all()
+    assert not torch.equal(scaled.view(torch.uint8), unscaled.view(torch.uint8))
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32, torch.float8_e4m3fn], ids=str)
+def test_scaled_mm_of_no_columns_of_k(tv, out_dtype):
+    """K = 0: the product is zeros, the bias and the cast still apply, and it runs on the device."""
+    a = torch.zeros(5, 0).to(FLOAT8[0])
+    b = torch.zeros(7, 0).to(FLOAT8[0]).t()
+    bias = draw(("normal", (7,)), 8).bfloat16()
+    one = torch.tensor(1.0)
+    got = on_vk(tv, torch._scaled_mm, a, b, one, one, bias=bias, out_dtype=out_dtype)
+    assert got.shape == (5, 7) and got.dtype == out_dtype
+    assert torch.equal(got.float(), bias.float().to(out_dtype).float().expand(5, 7))
+    rows = on_vk(tv, torch._scaled_mm, a, b, torch.ones(5, 1), torch.ones(1, 7), out_dtype=out_dtype)
+    assert (rows.float() == 0).all()
+
+
+def test_scaled_mm_refusals(tv):
     a = torch.randn(4, 8).to(FLOAT8[0]).to("vk")
     b = torch.randn(6, 8).to(FLOAT8[0]).to("vk").t()
     one = torch.tensor(1.0).to("vk")
-    with pytest.raises(ValueError, match="Invalid scaling configuration"):
-        torch._scaled_mm(a, b, torch.ones(3).to("vk"), one)
-    with pytest.raises(ValueError, match="out_dtype must match output matrix type"):
-        torch._scaled_mm(a, b, one, one, out_dtype=torch.float32, out=torch.empty(0, dtype=torch.half).to("vk"))
-    with pytest.raises(RuntimeError, match="Bias must be size 6"):
-        torch._scaled_mm(a, b, one, one, bias=torch.ones(5).to("vk"), out_dtype=torch.float32)
+    raises_each([(ValueError, "Invalid scaling configuration", ((a, b, torch.ones(3).to("vk"), one), {})),
+                 (ValueError, "out_dtype must match output matrix type",
+                  ((a, b, one, one), dict(out_dtype=torch.float32, out=torch.empty(0, dtype=torch.half).to("vk")))),
+                 (RuntimeError, "Bias must be size 6", ((a, b, one, one), dict(bias=torch.ones(5).to("vk"), out_dtype=torch.float32)))],
+                lambda args, kwargs: torch._scaled_mm(*args, **kwargs))
 
 
 def test_empty_inputs(tv):
@@ -191,8 +323,7 @@ def test_empty_inputs(tv):
         b = torch.randint(-128, 128, (5, 64), dtype=torch.int8, generator=gen(1)).to("vk")
         out = torch._weight_int8pack_mm(torch.zeros(0, 64, dtype=torch.bfloat16).to("vk"), b, torch.ones(5, dtype=torch.bfloat16).to("vk"))
         assert out.shape == (0, 5) and out.dtype == torch.bfloat16
-        w, sc, bias = pack_case(6, 64, 32, 3, True)
-        packed = torch._dyn_quant_pack_4bit_weight(w, sc, bias, 32, 64, 6).to("vk")
+        packed = torch._dyn_quant_pack_4bit_weight(*int4_weights(6, 64, 32, seed=3, bias=True), 32, 64, 6).to("vk")
         out = torch._dyn_quant_matmul_4bit(torch.zeros(0, 64).to("vk"), packed, 32, 64, 6)
         assert out.shape == (0, 6) and out.dtype == torch.float32
         a8 = torch.zeros(0, 32).to(torch.float8_e4m3fn).to("vk")

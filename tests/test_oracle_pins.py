@@ -14,10 +14,10 @@ import pytest
 import torch
 
 import oracle
+from _cases import FLOAT8, FLOAT8_OUT, FLOAT8_PAIRS, INT4_SHAPES, INT8_SHAPES, float8_case, int4_rows, int4_weights, int8_case
 from _util import ODT, bits, gen, ref_tol, unbits
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
-FLOAT8 = [torch.float8_e4m3fn, torch.float8_e5m2]
 
 
 # ------------------------------------------------------------------ casts
@@ -67,20 +67,10 @@ def test_f16_bf16_encode_matches_torch():
 
 
 # ------------------------------------------------------------------ int8
-Q8_SHAPES = [(32, 64, 48), (1, 4096, 300), (5, 100, 17), (70, 33, 5), (65, 1, 66)]  # test_quant.py:21
-
-
-def q8_case(dtype, m, k, n):
-    a = torch.randn(m, k, generator=gen(1)).to(dtype)
-    b = torch.randint(-128, 128, (n, k), dtype=torch.int8, generator=gen(2))
-    s = (torch.rand(n, generator=gen(3)) / 50).to(dtype)
-    return a, b, s
-
-
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("m,k,n", Q8_SHAPES)
+@pytest.mark.parametrize("m,k,n", INT8_SHAPES)
 def test_qmm8_vs_closed_form_and_torch(dtype, m, k, n):
-    a, b, s = q8_case(dtype, m, k, n)
+    a, b, s = int8_case(dtype, m, k, n)
     odt = ODT[dtype]
     c, c64, mag = oracle.qmm8(bits(a), odt, b.numpy(), bits(s), want_f64=True)
     # closed form of the reference's test (test_quant.py:32): float64 here
@@ -118,33 +108,13 @@ def test_qmm8_brute_force_tiny():
 
 
 # ------------------------------------------------------------------ int4
-Q4_CASES = [(1, 64, 4096, 32, False), (32, 128, 11008, 32, True), (5, 96, 70, 96, True), (3, 100, 9, 100, False),
-            (4, 256, 16, 64, True), (9, 64, 33, 64, False)]  # test_quant.py:61-62
-
-
-def pack_case(n, k, bs, seed, bias):  # test_quant.py:53-58
-    w = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, generator=gen(seed))
-    nb = 1 if bs == k else k // bs
-    sc = torch.rand(n, nb, generator=gen(seed + 1)) / 10
-    sc = sc if bs == k else sc.to(torch.bfloat16)
-    return w, sc, (torch.randn(n, generator=gen(seed + 2)) if bias else None)
-
-
-def q4_input(m, k, dtype):  # test_quant.py:72-75
-    x = (torch.randn(m, k, generator=gen(11)) * 3).to(dtype)
-    x[0, : k // 2] = 0.0
-    if m > 1:
-        x[1] = -x[1].abs()
-    return x
-
-
-@pytest.mark.parametrize("m,k,n,bs,bias", Q4_CASES)
+@pytest.mark.parametrize("m,k,n,bs,bias", INT4_SHAPES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_q4_bit_exact_vs_torch_cpu(m, k, n, bs, bias, dtype):
     if dtype == torch.bfloat16 and bs != k:
         pytest.skip("bfloat16 inputs are channelwise only (the CPU's check)")
-    w, sc, bvec = pack_case(n, k, bs, 7, bias)
-    x = q4_input(m, k, dtype)
+    w, sc, bvec = int4_weights(n, k, bs, bias=bias)
+    x = int4_rows(m, k, dtype)
     packed = torch._dyn_quant_pack_4bit_weight(w, sc, bvec, bs, k, n)
     want = torch._dyn_quant_matmul_4bit(x, packed, bs, k, n)
     mine = oracle.q4_pack(w.numpy(), bits(sc), ODT[sc.dtype], None if bvec is None else bvec.numpy())
@@ -206,18 +176,12 @@ def test_q4_nibble_order_and_block_scales():
 
 
 # ------------------------------------------------------------------ float8
-@pytest.mark.parametrize("fa,fb", [(FLOAT8[0], FLOAT8[0]), (FLOAT8[1], FLOAT8[0]), (FLOAT8[0], FLOAT8[1])])
-@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32, torch.float16, torch.float8_e4m3fn, None])
+@pytest.mark.parametrize("fa,fb", FLOAT8_PAIRS)
+@pytest.mark.parametrize("out_dtype", FLOAT8_OUT)
 @pytest.mark.parametrize("rowwise", [False, True])
 def test_scaled_mm_vs_torch_cpu(fa, fb, out_dtype, rowwise):
-    # test_quant.py:101-128 (the CPU op of torch 2.10 rejects rowwise scales: closed form there)
-    a = torch.randn(16, 32, generator=gen(1)).to(fa)
-    b = torch.randn(48, 32, generator=gen(2)).to(fb).t()
-    sa = torch.rand(16, 1, generator=gen(3)) + 0.5 if rowwise else torch.tensor(1.25)
-    sb = torch.rand(1, 48, generator=gen(4)) + 0.5 if rowwise else torch.tensor(0.75)
-    bias = torch.randn(48, generator=gen(5)).to(torch.bfloat16) if out_dtype == torch.bfloat16 else None
-    scale_result = torch.tensor(2.0) if out_dtype == torch.float8_e4m3fn else None
-    res_dtype = out_dtype or fa
+    # the reference's parametrisation (test_quant.py:101-128); the CPU op of torch 2.10 rejects rowwise scales: closed form there
+    a, b, sa, sb, bias, scale_result, res_dtype = float8_case(fa, fb, out_dtype, rowwise)
     got, mag = oracle.scaled_mm(bits(a), ODT[fa], bits(b.t()), ODT[fb], sa.numpy(), sb.numpy(), rowwise,
                                 None if bias is None else bits(bias), oracle.BF16,
                                 None if scale_result is None else 2.0, ODT[res_dtype], want_mag=True)
@@ -265,7 +229,7 @@ def test_golden_fixtures():
     ops on the reference's parametrisations; the oracle must reproduce them (bit-exact for
     the int4 op, packed layout and fp8 codes; within the reference's band otherwise)."""
     g = np.load(os.path.join(GOLDEN, "q4.npz"))
-    for i in range(len(Q4_CASES)):
+    for i in range(len(INT4_SHAPES)):
         m, k, n, bs, bias = (int(v) for v in g[f"c{i}_shape"])  # (large-N cases frozen at 64 features)
         for tag, odt in (("f32", oracle.F32), ("bf16", oracle.BF16)):
             key = f"c{i}_{tag}"

@@ -101,6 +101,11 @@ class F8QuantParams(ctypes.Structure):
                 ("src_dtype", u32), ("dst_fmt", u32)]
 
 
+class ProbeParams(ctypes.Structure):
+    _fields_ = [("src", u64), ("dst", u64), ("n", u32), ("k", u32), ("iters", u32), ("pad", u32)]
+
+
+assert ctypes.sizeof(ProbeParams) == 32
 assert ctypes.sizeof(Q8Params) == 56 and ctypes.sizeof(Q4Params) == 64 and ctypes.sizeof(F8Params) == 104
 assert ctypes.sizeof(CastParams) == 32 and ctypes.sizeof(F8QuantParams) == 48 and ctypes.sizeof(GemmParams) == 112
 assert ctypes.sizeof(StridedParams) == 128 and ctypes.sizeof(Copy8Params) == 128 and ctypes.sizeof(QuantParams) == 88 and ctypes.sizeof(MinMaxParams) == 40

@@ -34,6 +34,7 @@ SOURCES = {
     # (the CPU's quantisation arithmetic, operation by operation)
     "kernels/quantize.hip": ["-ffp-contract=off"],
     "kernels/util.hip": [],
+    "kernels/probe.hip": [],
 }
 
 

@@ -53,10 +53,14 @@ struct HipSource {
   void unmap(uint64_t address) { (void)hipFree(reinterpret_cast<void*>(address)); }
 };
 
+constexpr uint64_t kWorkspaceBytes = 32ull << 20;
+// The widened-weights region of many-row int8 products is capped: larger weights run on the row-block kernels.
+constexpr uint64_t kMaxWidenedBytes = 2ull << 30;
+
 struct Runtime {
   int device = 0;
   hipDeviceProp_t props{};
-  Machine machine;
+  Machine machine;  // what the launchers see through vkt_dispatch
   hipStream_t stream = nullptr;
   std::mutex pool_mutex;  // lock order: pool, then stream (vkcore/src/lib.rs:33-50)
   std::mutex stream_mutex;
@@ -64,29 +68,46 @@ struct Runtime {
   std::atomic<uint64_t> dispatches{0};
   bool trace = false;
   uint64_t generation = 0;
-  void* workspace_base = nullptr;
-  void* scratch_base = nullptr;
+  // The kernels' own memory, both pool allocations (so they show in vkt_memory_stats and go back with
+  // vkt_empty_cache): the workspace of products split over workgroups, taken at the first vkt_dispatch, and the
+  // widened-weights region, grown on demand.  Guarded by pool_mutex (the Machine fields also by stream_mutex).
+  Allocation workspace_alloc{}, widened_alloc{};
+  std::atomic<uint64_t> workspace_ready{0}, widened_ready{0};  // bytes of each that dispatches may count on
 
-  // Grows the scratch region to at least `bytes` (never shrinks before vkt_empty_cache / shutdown).  hipFree waits
-  // for the device, so a region still in use by queued kernels is not pulled away.  Caller holds stream_mutex.
-  bool ensure_scratch(uint64_t bytes, std::string* err) {
-    if (bytes <= machine.scratch_bytes) return true;
-    if (scratch_base) (void)hipFree(scratch_base);
-    scratch_base = nullptr, machine.scratch = 0, machine.scratch_bytes = 0;
-    const uint64_t want = (bytes + (uint64_t(64) << 20) - 1) >> 26 << 26;  // whole 64 MiB
-    void* base = nullptr;
-    const hipError_t e = hipMalloc(&base, want);
-    if (e != hipSuccess) {
-      (void)hipGetLastError();
-      *err = hip_message("scratch allocation", e);
-      return false;
+  // Makes sure the workspace exists and the widened-weights region holds `widened` bytes.  Called by vkt_dispatch
+  // before it takes the stream: a new pool block is a hipMalloc, which may wait for the device.  Pool memory is
+  // reused in stream order, so giving the old region back while queued kernels still read it is safe.
+  bool ensure_kernel_memory(uint64_t widened, std::string* err) {
+    std::lock_guard<std::mutex> lock(pool_mutex);
+    if (workspace_alloc.size == 0) {
+      Allocation a;
+      if (!pool->alloc(kWorkspaceBytes, &a, err)) return false;
+      std::lock_guard<std::mutex> stream_lock(stream_mutex);
+      workspace_alloc = a;
+      machine.workspace = a.address, machine.workspace_bytes = kWorkspaceBytes;
+      workspace_ready.store(kWorkspaceBytes, std::memory_order_release);
     }
-    scratch_base = base, machine.scratch = reinterpret_cast<uint64_t>(base), machine.scratch_bytes = want;
+    if (widened > widened_alloc.size && widened <= kMaxWidenedBytes) {
+      Allocation a;
+      std::string ignored;  // (without memory for it the row-block kernels run)
+      if (pool->alloc(widened, &a, &ignored)) {
+        std::lock_guard<std::mutex> stream_lock(stream_mutex);
+        if (widened_alloc.size) pool->free(widened_alloc);
+        widened_alloc = a;
+        machine.scratch = a.address, machine.scratch_bytes = a.size;
+        widened_ready.store(a.size, std::memory_order_release);
+      }
+    }
     return true;
   }
-  void drop_scratch() {
-    if (scratch_base) (void)hipFree(scratch_base);
-    scratch_base = nullptr, machine.scratch = 0, machine.scratch_bytes = 0;
+  // Gives the kernels' memory back to the pool (vkt_empty_cache).  Caller holds pool_mutex.
+  void drop_kernel_memory() {
+    std::lock_guard<std::mutex> stream_lock(stream_mutex);
+    if (workspace_alloc.size) pool->free(workspace_alloc);
+    if (widened_alloc.size) pool->free(widened_alloc);
+    workspace_alloc = widened_alloc = Allocation{};
+    machine.workspace = machine.workspace_bytes = machine.scratch = machine.scratch_bytes = 0;
+    workspace_ready.store(0, std::memory_order_release), widened_ready.store(0, std::memory_order_release);
   }
 
   ~Runtime() {
@@ -94,8 +115,6 @@ struct Runtime {
       (void)hipStreamSynchronize(stream);
     }
     pool.reset();
-    if (workspace_base) (void)hipFree(workspace_base);
-    if (scratch_base) (void)hipFree(scratch_base);
     if (stream) (void)hipStreamDestroy(stream);
   }
 };
@@ -143,21 +162,6 @@ std::shared_ptr<Runtime> runtime(std::string* err) {
     return nullptr;
   }
   rt->machine.compute_units = rt->props.multiProcessorCount;
-  // The kernels' own workspace (partial tiles of products that are split over workgroups).
-  // Held outside the pool until shutdown: it is not the caller's memory and does not show
-  // in vkt_memory_stats.  Every use is queued on the runtime's one stream, so uses do not
-  // overlap.
-  {
-    constexpr uint64_t kWorkspaceBytes = 32ull << 20;
-    void* base = nullptr;
-    if ((e = hipMalloc(&base, kWorkspaceBytes)) != hipSuccess) {
-      *err = hip_message("workspace allocation", e);
-      return nullptr;
-    }
-    rt->workspace_base = base;
-    rt->machine.workspace = reinterpret_cast<uint64_t>(base);
-    rt->machine.workspace_bytes = kWorkspaceBytes;
-  }
   rt->pool = std::make_unique<Pool<HipSource>>(HipSource{});
   rt->pool->set_idle_hook(&idle_hook, rt.get());
   const char* tr = std::getenv("TORCH_VK_TRACE");  // reference ffi.rs:144-148
@@ -179,126 +183,137 @@ int dtype_of_suffix(const char* suffix) {
   return -1;
 }
 
-template <class P>
-bool read_push(const uint8_t* push, size_t npush, P* out, const char* name, std::string* err) {
-  if (npush != sizeof(P)) {
-    *err = std::string("kernel ") + name + " takes a parameter block of " + std::to_string(sizeof(P)) + " bytes, got " +
-           std::to_string(npush);
-    return false;
-  }
-  std::memcpy(out, push, sizeof(P));
-  return true;
+// One dispatch as the launchers see it.
+struct Call {
+  const char* name;
+  const char* rest;  // the name after the table entry's key (a dtype or size label), "" for exact names
+  const uint32_t* spec;
+  size_t nspec;
+  uint32_t gz;
+  const Machine& machine;
+  hipStream_t stream;
+  std::string* err;
+  uint32_t spec_at(size_t i) const { return i < nspec ? spec[i] : 0u; }
+};
+
+int unknown_kernel(const Call& c) {
+  *c.err = std::string("unknown kernel ") + c.name;
+  return -1;
 }
 
-// name + specialisation constants -> launcher (the role of kernels.rs:72-140 KernelCache::get).
-int dispatch_named(Runtime& rt, const char* name, const uint32_t* spec, size_t nspec, const uint8_t* push, size_t npush,
-                   uint32_t gz, std::string* err) {
-  auto spec_at = [&](size_t i) { return i < nspec ? spec[i] : 0u; };
-  if (!std::strncmp(name, "qmm8_", 5)) {
-    int dt = dtype_of_suffix(name + 5);
-    Q8Params p;
-    if (dt < 0) goto unknown;
-    if (!read_push(push, npush, &p, name, err)) return -1;
-    // spec[0] is the reference's ROWS constant (0: tile path, 1..8: GEMV); the row count
-    // that matters is p.m, so it is checked for consistency only.
-    if (spec_at(0) != 0 && spec_at(0) != p.m) {
-      *err = "qmm8: specialisation ROWS=" + std::to_string(spec_at(0)) + " does not match m=" + std::to_string(p.m);
-      return -1;
+int call_qmm8(const Q8Params& p, const Call& c) {
+  const int dt = dtype_of_suffix(c.rest);
+  if (dt < 0) return unknown_kernel(c);
+  // spec[0] is the reference's ROWS constant (0: tile path, 1..8: GEMV); the row count
+  // that matters is p.m, so it is checked for consistency only.
+  if (c.spec_at(0) != 0 && c.spec_at(0) != p.m) {
+    *c.err = "qmm8: specialisation ROWS=" + std::to_string(c.spec_at(0)) + " does not match m=" + std::to_string(p.m);
+    return -1;
+  }
+  return launch_qmm8(p, dt, c.spec_at(1), c.machine, c.stream, c.err);
+}
+int call_qmm4(const Q4Params& p, const Call& c) {
+  const int dt = dtype_of_suffix(c.rest);
+  if (dt != VKT_F32 && dt != VKT_BF16) return unknown_kernel(c);
+  return launch_qmm4(p, dt, c.spec_at(0), c.spec_at(1), c.machine, c.stream, c.err);
+}
+int call_qmm4c(const Q4CParams& p, const Call& c) {
+  const int dt = dtype_of_suffix(c.rest);
+  if (dt != VKT_F32 && dt != VKT_BF16) return unknown_kernel(c);
+  return launch_qmm4c(p, dt, c.spec_at(0), c.spec_at(1), c.spec_at(2), c.machine, c.stream, c.err);
+}
+int call_gemmcm(const GemmParams& p, const Call& c) {
+  const int dt = dtype_of_suffix(c.rest);
+  if (dt != VKT_BF16 && dt != VKT_F16) return unknown_kernel(c);
+  return launch_gemm16(p, dt, c.spec_at(0), c.gz, c.spec_at(3), c.machine, c.stream, c.err);
+}
+int call_cast_strided(const StridedParams& p, const Call& c) {  // "cast_<src>_<dst>"
+  const char* second = std::strchr(c.rest, '_');
+  if (!second) return unknown_kernel(c);
+  const int sdt = dtype_of_suffix(std::string(c.rest, second).c_str()), ddt = dtype_of_suffix(second + 1);
+  if (sdt < 0 || ddt < 0 || sdt == ddt) return unknown_kernel(c);
+  return launch_cast_strided(p, sdt, ddt, c.machine, c.stream, c.err);
+}
+int call_packvec(const Q4VecParams& p, const Call& c) { return launch_qmm4_packvec(p, c.stream, c.err); }
+int call_qmm4c_pack(const Q4PackParams& p, const Call& c) { return launch_qmm4c_pack(p, c.spec_at(0), c.machine, c.stream, c.err); }
+int call_move(const StridedParams& p, const Call& c) { return launch_move(p, c.rest, c.spec_at(0), c.spec_at(2), c.machine, c.stream, c.err); }
+int call_copy8(const Copy8Params& p, const Call& c) { return launch_copy8(p, c.rest, c.spec_at(0), c.machine, c.stream, c.err); }
+int call_cast_fp8(const CastParams& p, const Call& c) { return launch_cast_fp8(p, c.machine, c.stream, c.err); }
+int call_quantize(const QuantParams& p, const Call& c) { return launch_quantize_affine(p, c.spec_at(0), false, c.machine, c.stream, c.err); }
+int call_dequantize(const QuantParams& p, const Call& c) { return launch_quantize_affine(p, c.spec_at(0), true, c.machine, c.stream, c.err); }
+int call_fake_quant(const QuantParams& p, const Call& c) { return launch_fake_quant(p, c.spec_at(0), c.spec_at(1), c.machine, c.stream, c.err); }
+int call_aminmax(const MinMaxParams& p, const Call& c) { return launch_aminmax(p, c.machine, c.stream, c.err); }
+int call_fp8_quant(const F8QuantParams& p, const Call& c) { return launch_fp8_quant(p, c.spec_at(0), c.machine, c.stream, c.err); }
+int call_probe_read(const ProbeParams& p, const Call& c) { return launch_probe_read(p, c.spec_at(0), c.machine, c.stream, c.err); }
+int call_probe_mfma(const ProbeParams& p, const Call& c) { return launch_probe_mfma(p, c.spec_at(0), c.machine, c.stream, c.err); }
+int call_fp8mm(const F8Params& p, const Call& c) { return launch_fp8mm(p, c.spec_at(0), c.machine, c.stream, c.err); }
+
+// name -> parameter block type + launcher (the role of kernels.rs:72-140 KernelCache::get).  An entry ties a
+// launcher to the one block type it takes, so a name cannot reach a launcher with another kernel's block.
+struct KernelEntry {
+  const char* key;
+  bool prefix;  // the key is followed by a dtype / size label
+  size_t param_bytes;
+  int (*run)(const uint8_t* push, const Call& c);
+};
+template <class P, int (*F)(const P&, const Call&)>
+int with_block(const uint8_t* push, const Call& c) {
+  P p;
+  std::memcpy(&p, push, sizeof(P));
+  return F(p, c);
+}
+template <class P, int (*F)(const P&, const Call&)>
+constexpr KernelEntry entry(const char* key, bool prefix) {
+  return KernelEntry{key, prefix, sizeof(P), &with_block<P, F>};
+}
+// exact names first, so that "qmm4_packvec", "qmm4c_pack" and "cast_fp8" are not read as a prefix plus a label
+const KernelEntry kKernels[] = {
+    entry<Q4VecParams, call_packvec>("qmm4_packvec", false),
+    entry<Q4PackParams, call_qmm4c_pack>("qmm4c_pack", false),
+    entry<CastParams, call_cast_fp8>("cast_fp8", false),
+    entry<QuantParams, call_quantize>("quantize_affine", false),
+    entry<QuantParams, call_dequantize>("dequantize_affine", false),
+    entry<QuantParams, call_fake_quant>("fake_quant", false),
+    entry<MinMaxParams, call_aminmax>("aminmax", false),
+    entry<F8QuantParams, call_fp8_quant>("fp8_quant", false),
+    entry<F8Params, call_fp8mm>("fp8mm", false),
+    entry<ProbeParams, call_probe_read>("probe_read", false),
+    entry<ProbeParams, call_probe_mfma>("probe_mfma_f8", false),
+    entry<Q8Params, call_qmm8>("qmm8_", true),
+    entry<Q4CParams, call_qmm4c>("qmm4c_", true),
+    entry<Q4Params, call_qmm4>("qmm4_", true),
+    entry<GemmParams, call_gemmcm>("gemmcm_", true),
+    entry<StridedParams, call_move>("move_", true),
+    entry<Copy8Params, call_copy8>("copy8_", true),
+    entry<StridedParams, call_cast_strided>("cast_", true),
+};
+
+const KernelEntry* find_kernel(const char* name, const char** rest) {
+  for (const KernelEntry& e : kKernels) {
+    const size_t len = std::strlen(e.key);
+    if (e.prefix ? std::strncmp(name, e.key, len) == 0 && name[len] != '\0' : std::strcmp(name, e.key) == 0) {
+      *rest = name + (e.prefix ? len : std::strlen(name));
+      return &e;
     }
-    // (many rows: the weights are widened into the scratch region first; without memory for it the row-block kernels run)
-    if (const uint64_t need = q8_gemm_scratch_bytes(p, dt, rt.machine); need != 0 && !((spec_at(1) >> 20) & 1)) {
-      std::string ignored;
-      (void)rt.ensure_scratch(need, &ignored);
-    }
-    return launch_qmm8(p, dt, spec_at(1), rt.machine, rt.stream, err);
   }
-  if (!std::strcmp(name, "qmm4_packvec")) {
-    Q4VecParams p;
-    if (!read_push(push, npush, &p, name, err)) return -1;
-    return launch_qmm4_packvec(p, rt.stream, err);
+  return nullptr;
+}
+
+int dispatch_named(const Machine& machine, hipStream_t stream, const char* name, const uint32_t* spec, size_t nspec,
+                   const uint8_t* push, size_t npush, uint32_t gz, std::string* err) {
+  const char* rest = nullptr;
+  const KernelEntry* e = find_kernel(name, &rest);
+  if (!e) {
+    *err = std::string("unknown kernel ") + name;
+    return -1;
   }
-  if (!std::strncmp(name, "qmm4_", 5)) {
-    int dt = dtype_of_suffix(name + 5);
-    Q4Params p;
-    if (dt != VKT_F32 && dt != VKT_BF16) goto unknown;
-    if (!read_push(push, npush, &p, name, err)) return -1;
-    return launch_qmm4(p, dt, spec_at(0), spec_at(1), rt.machine, rt.stream, err);
+  if (npush != e->param_bytes) {
+    *err = std::string("kernel ") + name + " takes a parameter block of " + std::to_string(e->param_bytes) + " bytes, got " +
+           std::to_string(npush);
+    return -1;
   }
-  if (!std::strcmp(name, "qmm4c_pack")) {
-    Q4PackParams p;
-    if (!read_push(push, npush, &p, name, err)) return -1;
-    return launch_qmm4c_pack(p, spec_at(0), rt.machine, rt.stream, err);
-  }
-  if (!std::strncmp(name, "qmm4c_", 6)) {
-    int dt = dtype_of_suffix(name + 6);
-    Q4CParams p;
-    if (dt != VKT_F32 && dt != VKT_BF16) goto unknown;
-    if (!read_push(push, npush, &p, name, err)) return -1;
-    return launch_qmm4c(p, dt, spec_at(0), spec_at(1), spec_at(2), rt.machine, rt.stream, err);
-  }
-  if (!std::strncmp(name, "gemmcm_", 7)) {
-    int dt = dtype_of_suffix(name + 7);
-    GemmParams p;
-    if (dt != VKT_BF16 && dt != VKT_F16) goto unknown;
-    if (!read_push(push, npush, &p, name, err)) return -1;
-    return launch_gemm16(p, dt, spec_at(0), gz, spec_at(3), rt.machine, rt.stream, err);
-  }
-  if (!std::strncmp(name, "move_", 5)) {
-    StridedParams p;
-    if (!read_push(push, npush, &p, name, err)) return -1;
-    return launch_move(p, name + 5, spec_at(0), spec_at(2), rt.machine, rt.stream, err);
-  }
-  if (!std::strncmp(name, "copy8_", 6)) {
-    Copy8Params p;
-    if (!read_push(push, npush, &p, name, err)) return -1;
-    return launch_copy8(p, name + 6, spec_at(0), rt.machine, rt.stream, err);
-  }
-  if (!std::strncmp(name, "cast_", 5) && std::strcmp(name, "cast_fp8")) {
-    // "cast_<src>_<dst>"
-    const char* second = std::strchr(name + 5, '_');
-    if (!second) goto unknown;
-    const std::string from(name + 5, second);
-    const int sdt = dtype_of_suffix(from.c_str()), ddt = dtype_of_suffix(second + 1);
-    StridedParams p;
-    if (sdt < 0 || ddt < 0 || sdt == ddt) goto unknown;
-    if (!read_push(push, npush, &p, name, err)) return -1;
-    return launch_cast_strided(p, sdt, ddt, rt.machine, rt.stream, err);
-  }
-  if (!std::strcmp(name, "cast_fp8")) {
-    CastParams p;
-    if (!read_push(push, npush, &p, name, err)) return -1;
-    return launch_cast_fp8(p, rt.machine, rt.stream, err);
-  }
-  if (!std::strcmp(name, "quantize_affine") || !std::strcmp(name, "dequantize_affine")) {
-    QuantParams p;
-    if (!read_push(push, npush, &p, name, err)) return -1;
-    return launch_quantize_affine(p, spec_at(0), name[0] == 'd', rt.machine, rt.stream, err);
-  }
-  if (!std::strcmp(name, "aminmax")) {
-    MinMaxParams p;
-    if (!read_push(push, npush, &p, name, err)) return -1;
-    return launch_aminmax(p, rt.machine, rt.stream, err);
-  }
-  if (!std::strcmp(name, "fake_quant") || !std::strcmp(name, "aminmax")) {
-    QuantParams p;
-    if (!read_push(push, npush, &p, name, err)) return -1;
-    return launch_fake_quant(p, spec_at(0), spec_at(1), rt.machine, rt.stream, err);
-  }
-  if (!std::strcmp(name, "fp8_quant") || !std::strncmp(name, "move_", 5) || !std::strncmp(name, "copy8_", 6) ||
-          !std::strncmp(name, "cast_", 5) || !std::strcmp(name, "quantize_affine") || !std::strcmp(name, "dequantize_affine") ||
-          !std::strcmp(name, "fake_quant") || !std::strcmp(name, "aminmax")) {
-    F8QuantParams p;
-    if (!read_push(push, npush, &p, name, err)) return -1;
-    return launch_fp8_quant(p, spec_at(0), rt.machine, rt.stream, err);
-  }
-  if (!std::strcmp(name, "fp8mm")) {
-    F8Params p;
-    if (!read_push(push, npush, &p, name, err)) return -1;
-    return launch_fp8mm(p, spec_at(0), rt.machine, rt.stream, err);
-  }
-unknown:
-  *err = std::string("unknown kernel ") + name;
-  return -1;
+  const Call c{name, rest, spec, nspec, gz, machine, stream, err};
+  return e->run(push, c);
 }
 
 struct Handle {
@@ -355,11 +370,8 @@ int vkt_empty_cache(void) {
   if (!rt) return 0;
   int rc = vkt_synchronize();
   std::lock_guard<std::mutex> lock(rt->pool_mutex);
+  rt->drop_kernel_memory();  // (the next vkt_dispatch takes the workspace again)
   rt->pool->trim();
-  {
-    std::lock_guard<std::mutex> stream_lock(rt->stream_mutex);
-    rt->drop_scratch();
-  }
   return rc;
 }
 
@@ -375,29 +387,57 @@ void vkt_memory_stats(uint64_t* allocated, uint64_t* reserved) {
   if (reserved) *reserved = r;
 }
 
-int vkt_dispatch(const char* name, const uint32_t* spec, size_t nspec, const uint8_t* push, size_t npush, uint32_t gx,
-                 uint32_t gy, uint32_t gz) {
+namespace {
+
+// Queue `name` on the runtime's stream against `machine`.
+int queue_kernel(Runtime& rt, const Machine& machine, const char* name, const uint32_t* spec, size_t nspec,
+                 const uint8_t* push, size_t npush, uint32_t gx, uint32_t gy, uint32_t gz) {
   std::string err;
-  auto rt = runtime(&err);
-  if (!rt) return fail(err);
-  if (!name) return fail("kernel name is null");
-  if (npush > 128) return fail("parameter blocks are limited to 128 bytes");
-  if (npush != 0 && !push) return fail("parameter block is null");
-  if (gx == 0 || gy == 0 || gz == 0) return fail("empty grid");
-  std::lock_guard<std::mutex> lock(rt->stream_mutex);
-  if (dispatch_named(*rt, name, spec, nspec, push, npush, gz, &err) != 0) return fail(err);
-  rt->dispatches.fetch_add(1, std::memory_order_relaxed);
-  if (rt->trace) {
+  if (dispatch_named(machine, rt.stream, name, spec, nspec, push, npush, gz, &err) != 0) return fail(err);
+  rt.dispatches.fetch_add(1, std::memory_order_relaxed);
+  if (rt.trace) {
     // each kernel runs to completion before the next is queued, so a kernel that
     // faults is the last one printed (ffi.rs:135-142)
     std::fprintf(stderr, "[vkt] %s [", name);
     for (size_t i = 0; i < nspec; ++i) std::fprintf(stderr, i ? ", %u" : "%u", spec[i]);
     std::fprintf(stderr, "] grid %ux%ux%u\n", gx, gy, gz);
     std::fflush(stderr);
-    hipError_t e = hipStreamSynchronize(rt->stream);
+    hipError_t e = hipStreamSynchronize(rt.stream);
     if (e != hipSuccess) return fail(hip_message(name, e));
   }
   return 0;
+}
+
+int check_dispatch_arguments(const char* name, const uint8_t* push, size_t npush, uint32_t gx, uint32_t gy, uint32_t gz) {
+  if (!name) return fail("kernel name is null");
+  if (npush > 128) return fail("parameter blocks are limited to 128 bytes");
+  if (npush != 0 && !push) return fail("parameter block is null");
+  if (gx == 0 || gy == 0 || gz == 0) return fail("empty grid");
+  return 0;
+}
+
+}  // namespace
+
+int vkt_dispatch(const char* name, const uint32_t* spec, size_t nspec, const uint8_t* push, size_t npush, uint32_t gx,
+                 uint32_t gy, uint32_t gz) {
+  std::string err;
+  auto rt = runtime(&err);
+  if (!rt) return fail(err);
+  if (check_dispatch_arguments(name, push, npush, gx, gy, gz) != 0) return -1;
+  // The kernels' own memory comes from the pool, before the stream is taken (a new pool block is a hipMalloc, which
+  // may wait for the device): the workspace at the first dispatch and after vkt_empty_cache; the widened-weights
+  // region when a many-row int8 product first needs more of it than there is.
+  uint64_t widened = 0;
+  if (!std::strncmp(name, "qmm8_", 5) && npush == sizeof(Q8Params) && !((nspec > 1 ? spec[1] : 0u) >> 20 & 1)) {
+    Q8Params p;
+    std::memcpy(&p, push, sizeof(p));
+    widened = q8_gemm_scratch_bytes(p, dtype_of_suffix(name + 5), rt->machine);
+  }
+  if ((rt->workspace_ready.load(std::memory_order_acquire) == 0 || widened > rt->widened_ready.load(std::memory_order_acquire)) &&
+      !rt->ensure_kernel_memory(widened, &err))
+    return fail(err);
+  std::lock_guard<std::mutex> lock(rt->stream_mutex);
+  return queue_kernel(*rt, rt->machine, name, spec, nspec, push, npush, gx, gy, gz);
 }
 
 int vkt_grid_1d(uint64_t n, uint32_t* groups, uint32_t* stride) {
@@ -434,12 +474,8 @@ uint32_t vkt_kernel_subgroup_size(const char* name) {
   if (!name) return 0;
   std::string err;
   if (!runtime(&err)) return 0;
-  return (!std::strncmp(name, "qmm", 3) || !std::strcmp(name, "fp8mm") || !std::strcmp(name, "cast_fp8") || !std::strncmp(name, "gemmcm_", 7) ||
-          !std::strcmp(name, "fp8_quant") || !std::strncmp(name, "move_", 5) || !std::strncmp(name, "copy8_", 6) ||
-          !std::strncmp(name, "cast_", 5) || !std::strcmp(name, "quantize_affine") || !std::strcmp(name, "dequantize_affine") ||
-          !std::strcmp(name, "fake_quant") || !std::strcmp(name, "aminmax"))
-             ? 64u
-             : 0u;
+  const char* rest = nullptr;
+  return find_kernel(name, &rest) ? 64u : 0u;
 }
 
 int vkt_copy_to_device(uint64_t dst, const void* src, uint64_t nbytes) {
@@ -472,6 +508,7 @@ int vkt_copy_on_device(uint64_t dst, uint64_t src, uint64_t nbytes) {
   if (!rt) return fail(err);
   if (nbytes == 0) return 0;
   if (!dst || !src) return fail("vkt_copy_on_device: null address");
+  if (dst == src) return 0;  // a copy onto itself changes nothing (as on the CPU)
   std::lock_guard<std::mutex> lock(rt->stream_mutex);
   // a kernel on the stream (not a DMA engine): it is ordered like every other dispatch, can
   // be recorded into a HIP graph, and shows up in kernel traces and counters

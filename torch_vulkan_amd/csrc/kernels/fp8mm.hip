@@ -203,7 +203,8 @@ int launch_fp8mm(const F8Params& p, uint32_t variant, const Machine& mc, hipStre
     *err = "fp8mm: unsupported output or bias dtype";
     return -1;
   }
-  if (!p.a || !p.b || !p.scale_a || !p.scale_b || !p.out) {
+  // (k == 0: an empty product, zeros through the epilogue; the operands are then empty and may have no address)
+  if ((p.k != 0 && (!p.a || !p.b)) || !p.scale_a || !p.scale_b || !p.out) {
     *err = "fp8mm: null tensor address";
     return -1;
   }
