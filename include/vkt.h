@@ -84,6 +84,23 @@ int vkt_event_record(void* event);
 int vkt_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop` */
 void vkt_event_destroy(void* event);
 
+/* vkt_dispatch for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid it).  No counterpart in the reference.  Same arguments, same kernels, same results; the
+ * difference is where the kernels' own workspace lives (the partial sums of a product that is split over
+ * workgroups, e.g. "qmm8_bf16" at 64 rows): here it is a fixed array of VKT_STATIC_SCRATCH_BYTES in the library's
+ * code object, one per device, held until the process ends, and the call makes no hipMalloc / hipFree (vkt_dispatch
+ * takes its workspace from the pool at its first call and grows a second region for many-row int8 products).
+ *   - The runtime must be running: call any other function (e.g. vkt_device_info) once at start-up.
+ *   - A product whose planned split needs more workspace than the array holds returns -1 with a message that
+ *     names both sizes; it is never re-planned with fewer slices.  Many-row int8 products do not widen their
+ *     weights here: they run on the row-block kernels.
+ *   - Calls are queued on the runtime's one in-order stream like every other dispatch, so two calls never overlap on
+ *     the device; the array keeps the last call's partial sums, and every kernel writes what it later reads (nothing
+ *     has to start at zero). */
+#define VKT_STATIC_SCRATCH_BYTES (16u << 20)
+int vkt_dispatch_static(const char* name, const uint32_t* spec, size_t nspec, const uint8_t* push, size_t npush,
+                        uint32_t gx, uint32_t gy, uint32_t gz);
+
 uint64_t vkt_dispatch_count(void); /* kernels queued so far (reference pyvk/src/lib.rs:112-116) */
 void vkt_shutdown(void);           /* releases the device; later vkt_free calls are no-ops */
 

@@ -12,9 +12,9 @@ _NP = {oracle.F32: np.float32, oracle.F16: np.uint16, oracle.BF16: np.uint16, or
        oracle.E5M2: np.uint8}
 
 
-def qmm8(a, odt, b, s, variant=0, row_step=1):
+def qmm8(a, odt, b, s, variant=0, row_step=1, static=False):
     """_weight_int8pack_mm.  a: storage array [M_total,K]; rows taken every `row_step`
-    (a strided A as in a[::2]); returns the storage array [M,N]."""
+    (a strided A as in a[::2]); returns the storage array [M,N].  static: through vkt_dispatch_static."""
     a = np.ascontiguousarray(a)
     b = np.ascontiguousarray(b, dtype=np.int8)
     s = np.ascontiguousarray(s)
@@ -28,7 +28,7 @@ def qmm8(a, odt, b, s, variant=0, row_step=1):
     spec = [m if m <= 8 else 0, variant]
     grid = ((n + 7) // 8,) if m <= 8 else ((n + 63) // 64, (m + 63) // 64)
     if m and n:
-        abi.dispatch("qmm8_" + abi.SUFFIX[odt], spec, p, grid)
+        abi.dispatch("qmm8_" + abi.SUFFIX[odt], spec, p, grid, static=static)
     return dc.to_numpy(_NP[odt], (m, n))
 
 

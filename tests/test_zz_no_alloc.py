@@ -1,0 +1,51 @@
+"""vkt_dispatch_static, the dispatch entry point that allocates nothing: the kernels' workspace is a fixed array in
+the library instead of pool memory.  Its results are compared with vkt_dispatch's on products that are split over
+workgroups (so that the workspace is really used), on calls in a row of decreasing size (the array keeps the last
+call's contents), and a product whose split needs more than the array holds must be refused."""
+import numpy as np
+import pytest
+import torch
+
+import _dev
+import oracle
+from _util import bits, gen, ref_tol
+from torch_vulkan_amd import abi
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(m, k, n, seed):
+    a = torch.randn(m, k, generator=gen(seed)).bfloat16()
+    b = torch.randint(-128, 128, (n, k), dtype=torch.int8, generator=gen(seed + 1))
+    s = torch.empty(n).uniform_(0.005, 0.02, generator=gen(seed + 2)).bfloat16()
+    return bits(a), b.numpy(), bits(s)
+
+
+def test_static_dispatch_matches_dispatch():
+    abi.device_info()  # starts the runtime: the static entry point does not
+    # 64 rows x 8 slices of K (tile kernel + finish: 8.4 MB of partial sums), then smaller products: 40 rows on the
+    # same kernels, and 16 rows on the kernel whose workgroups write whole matrix-core tiles to the workspace
+    for i, (m, k, n) in enumerate([(64, 14336, 4096), (40, 4096, 1024), (16, 14336, 4096)]):
+        a, b, s = _case(m, k, n, 100 + 10 * i)
+        want = _dev.qmm8(a, oracle.BF16, b, s)
+        got = _dev.qmm8(a, oracle.BF16, b, s, static=True)
+        assert np.array_equal(got, want), (m, k, n)
+        if m == 40:  # against the oracle too
+            _, c64, mag = oracle.qmm8(a, oracle.BF16, b, s, want_f64=True)
+            assert (np.abs(oracle.bf16_to_f32(got) - c64) <= ref_tol(c64, mag, oracle.BF16)).all()
+
+
+def test_static_dispatch_refuses_more_than_the_array_holds():
+    abi.device_info()
+    a, b, s = _case(64, 4096, 4096, 200)
+    forced = (1 << 21) | (32 << 24)  # the tile kernel with 32 slices of K: 32 x 64 x 4096 x 4 bytes of partial sums
+    assert 32 * 64 * 4096 * 4 > abi.STATIC_SCRATCH_BYTES
+    with pytest.raises(abi.VktError, match="fixed workspace holds"):
+        _dev.qmm8(a, oracle.BF16, b, s, variant=forced, static=True)
+    # the same call through vkt_dispatch runs (with as many slices as its workspace holds), and the static entry
+    # point still works afterwards
+    want = _dev.qmm8(a, oracle.BF16, b, s, variant=forced)
+    got = _dev.qmm8(a, oracle.BF16, b, s, static=True)
+    _, c64, mag = oracle.qmm8(a, oracle.BF16, b, s, want_f64=True)
+    for out in (want, got):
+        assert (np.abs(oracle.bf16_to_f32(out) - c64) <= ref_tol(c64, mag, oracle.BF16)).all()

@@ -115,7 +115,7 @@ SYMBOLS = ["vkt_last_error", "vkt_alloc", "vkt_free", "vkt_synchronize", "vkt_em
            "vkt_dispatch", "vkt_grid_1d", "vkt_has_float64", "vkt_vendor_id", "vkt_capabilities",
            "vkt_kernel_subgroup_size", "vkt_copy_to_device", "vkt_copy_to_host", "vkt_copy_on_device", "vkt_fill",
            "vkt_device_info", "vkt_event_create", "vkt_event_record", "vkt_event_elapsed_ms", "vkt_event_destroy",
-           "vkt_dispatch_count", "vkt_shutdown", "vkt_qmm4c_bytes", "vkt_qmm4c_q_bytes"]
+           "vkt_dispatch_count", "vkt_dispatch_static", "vkt_shutdown", "vkt_qmm4c_bytes", "vkt_qmm4c_q_bytes"]
 
 _lib = None
 
@@ -135,6 +135,7 @@ def lib():
         L.vkt_memory_stats.restype = None
         L.vkt_dispatch.argtypes = [ctypes.c_char_p, ctypes.POINTER(u32), ctypes.c_size_t, ctypes.c_void_p,
                                    ctypes.c_size_t, u32, u32, u32]
+        L.vkt_dispatch_static.argtypes = L.vkt_dispatch.argtypes
         L.vkt_grid_1d.argtypes = [u64, ctypes.POINTER(u32), ctypes.POINTER(u32)]
         L.vkt_vendor_id.restype = u32
         L.vkt_capabilities.restype = u32
@@ -208,11 +209,16 @@ class Buffer:
             pass
 
 
-def dispatch(name, spec, params, grid=(1, 1, 1)):
-    """vkt_dispatch: kernel `name`, specialisation constants `spec`, parameter block `params`."""
+STATIC_SCRATCH_BYTES = 16 << 20  # VKT_STATIC_SCRATCH_BYTES
+
+
+def dispatch(name, spec, params, grid=(1, 1, 1), static=False):
+    """vkt_dispatch: kernel `name`, specialisation constants `spec`, parameter block `params`.
+    static: through vkt_dispatch_static (the kernels' workspace is the library's fixed array; no allocation)."""
     arr = (u32 * max(len(spec), 1))(*spec)
     gx, gy, gz = (list(grid) + [1, 1])[:3]
-    check(lib().vkt_dispatch(name.encode(), arr, len(spec), ctypes.byref(params), ctypes.sizeof(params), gx, gy, gz))
+    fn = lib().vkt_dispatch_static if static else lib().vkt_dispatch
+    check(fn(name.encode(), arr, len(spec), ctypes.byref(params), ctypes.sizeof(params), gx, gy, gz))
 
 
 def synchronize():

@@ -53,6 +53,12 @@ struct HipSource {
   void unmap(uint64_t address) { (void)hipFree(reinterpret_cast<void*>(address)); }
 };
 
+// The no-allocation entry point's workspace (vkt_dispatch_static): a fixed array in the code object, one copy per
+// device, held from the time the library's code is loaded until the process ends.  Host code never uses this name
+// as an address: the runtime asks for the device address once (hipGetSymbolAddress, in runtime()) and passes that.
+constexpr uint64_t kStaticScratchBytes = VKT_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 constexpr uint64_t kWorkspaceBytes = 32ull << 20;
 // The widened-weights region of many-row int8 products is capped: larger weights run on the row-block kernels.
 constexpr uint64_t kMaxWidenedBytes = 2ull << 30;
@@ -73,6 +79,7 @@ struct Runtime {
   // widened-weights region, grown on demand.  Guarded by pool_mutex (the Machine fields also by stream_mutex).
   Allocation workspace_alloc{}, widened_alloc{};
   std::atomic<uint64_t> workspace_ready{0}, widened_ready{0};  // bytes of each that dispatches may count on
+  uint64_t static_scratch = 0;  // device address of `scratch` on this runtime's device
 
   // Makes sure the workspace exists and the widened-weights region holds `widened` bytes.  Called by vkt_dispatch
   // before it takes the stream: a new pool block is a hipMalloc, which may wait for the device.  Pool memory is
@@ -162,6 +169,16 @@ std::shared_ptr<Runtime> runtime(std::string* err) {
     return nullptr;
   }
   rt->machine.compute_units = rt->props.multiProcessorCount;
+  // the device address of this device's copy of the fixed workspace (the array's name is not an address on the host)
+  {
+    void* at = nullptr;
+    if ((e = hipGetSymbolAddress(&at, HIP_SYMBOL(scratch))) != hipSuccess || at == nullptr) {
+      (void)hipGetLastError();
+      *err = hip_message("hipGetSymbolAddress(scratch)", e);
+      return nullptr;
+    }
+    rt->static_scratch = reinterpret_cast<uint64_t>(at);
+  }
   rt->pool = std::make_unique<Pool<HipSource>>(HipSource{});
   rt->pool->set_idle_hook(&idle_hook, rt.get());
   const char* tr = std::getenv("TORCH_VK_TRACE");  // reference ffi.rs:144-148
@@ -389,7 +406,7 @@ void vkt_memory_stats(uint64_t* allocated, uint64_t* reserved) {
 
 namespace {
 
-// Queue `name` on the runtime's stream against `machine`.
+// The common part of vkt_dispatch and vkt_dispatch_static: queue `name` on the runtime's stream against `machine`.
 int queue_kernel(Runtime& rt, const Machine& machine, const char* name, const uint32_t* spec, size_t nspec,
                  const uint8_t* push, size_t npush, uint32_t gx, uint32_t gy, uint32_t gz) {
   std::string err;
@@ -438,6 +455,23 @@ int vkt_dispatch(const char* name, const uint32_t* spec, size_t nspec, const uin
     return fail(err);
   std::lock_guard<std::mutex> lock(rt->stream_mutex);
   return queue_kernel(*rt, rt->machine, name, spec, nspec, push, npush, gx, gy, gz);
+}
+
+int vkt_dispatch_static(const char* name, const uint32_t* spec, size_t nspec, const uint8_t* push, size_t npush,
+                        uint32_t gx, uint32_t gy, uint32_t gz) {
+  auto rt = running();
+  if (!rt) return fail("vkt_dispatch_static: the runtime is not running (start it with any other call, e.g. vkt_device_info)");
+  if (check_dispatch_arguments(name, push, npush, gx, gy, gz) != 0) return -1;
+  // the same launchers against a machine whose only kernel memory is the fixed array: a product that would need more
+  // of it than kStaticScratchBytes is refused by its launcher (workspace_fixed), never shrunk or re-planned, and
+  // nothing is widened into a second region
+  Machine fixed;
+  fixed.compute_units = rt->machine.compute_units;
+  fixed.workspace = rt->static_scratch;
+  fixed.workspace_bytes = kStaticScratchBytes;
+  fixed.workspace_fixed = true;
+  std::lock_guard<std::mutex> lock(rt->stream_mutex);
+  return queue_kernel(*rt, fixed, name, spec, nspec, push, npush, gx, gy, gz);
 }
 
 int vkt_grid_1d(uint64_t n, uint32_t* groups, uint32_t* stride) {

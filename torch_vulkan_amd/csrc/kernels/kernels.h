@@ -16,6 +16,9 @@ struct Machine {
   // device memory the runtime owns for kernels that split one product over several
   // workgroups: partial results between a kernel and the one that adds them up
   uint64_t workspace = 0, workspace_bytes = 0;
+  // the workspace cannot be traded for a different plan: a product whose planned split needs more of it than
+  // workspace_bytes is an error, not a product with fewer slices (the no-allocation entry point)
+  bool workspace_fixed = false;
   // a second region that the runtime grows on demand, for whole operands rewritten before a product
   // (the int8 weights of a many-row product widened to 16 bits); queued uses are ordered by the one stream
   uint64_t scratch = 0, scratch_bytes = 0;

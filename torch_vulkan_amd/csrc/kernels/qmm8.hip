@@ -769,17 +769,27 @@ __global__ __launch_bounds__(256) void qmm8_tile_finish(Q8Params p, uint32_t sli
   }
 }
 
-// Launches the tile kernel if it takes the product (k a multiple of its step, 16-byte aligned activation rows).
+// A product whose planned split over workgroups needs `need` bytes of workspace, on a machine whose workspace
+// cannot be traded for another plan: an error that names both sizes.
+bool workspace_refused(const Machine& mc, uint64_t need, std::string* err) {
+  if (!mc.workspace_fixed || need <= mc.workspace_bytes) return false;
+  *err = "qmm8: this product's partial sums need " + std::to_string(need) + " bytes of workspace, the fixed workspace holds " +
+         std::to_string(mc.workspace_bytes);
+  return true;
+}
+
+// Launches the tile kernel if it takes the product (k a multiple of its step, 16-byte aligned activation rows):
+// 1 launched, 0 not this kernel's shape, -1 refused (*err set).
 template <class T>
-bool launch_tile_kernel(const Q8Params& p, uint32_t want_slices, const Machine& mc, hipStream_t stream) {
-  if (p.k % kTileStepK != 0 || p.k == 0 || (int64_t(p.a_sm) * 2) % 16 != 0 || p.a_sm <= 0) return false;
+int launch_tile_kernel(const Q8Params& p, uint32_t want_slices, const Machine& mc, hipStream_t stream, std::string* err) {
+  if (p.k % kTileStepK != 0 || p.k == 0 || (int64_t(p.a_sm) * 2) % 16 != 0 || p.a_sm <= 0) return 0;
   constexpr uint32_t lds = kTileLds;
   auto kernel = qmm8_tile<T>;
   static bool configured = false;  // guarded by the runtime's stream mutex
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
       (void)hipGetLastError();
-      return false;
+      return 0;
     }
     configured = true;
   }
@@ -791,17 +801,18 @@ bool launch_tile_kernel(const Q8Params& p, uint32_t want_slices, const Machine& 
     slices = slices > most ? most : slices;
     slices = slices < 1 ? 1 : slices;
   }
+  if (slices > 1 && workspace_refused(mc, uint64_t(slices) * p.m * p.n * 4, err)) return -1;
   while (slices > 1 && uint64_t(slices) * p.m * p.n * 4 > mc.workspace_bytes) --slices;
   uint32_t per_slice = (steps + slices - 1) / slices;
   slices = (steps + per_slice - 1) / per_slice;
-  if (gy > 65535 || slices > 65535) return false;
+  if (gy > 65535 || slices > 65535) return 0;
   hipLaunchKernelGGL(kernel, dim3(gx, gy, slices), dim3(512), lds, stream, p, per_slice, mc.workspace);
   if (slices > 1) {
     const uint32_t vec = (p.n & 3u) == 0;
     const uint64_t threads = (uint64_t(p.m) * p.n + (vec ? 3 : 0)) / (vec ? 4 : 1);
     hipLaunchKernelGGL(qmm8_tile_finish<T>, dim3(uint32_t((threads + 255) / 256)), dim3(256), 0, stream, p, slices, mc.workspace, vec);
   }
-  return true;
+  return 1;
 }
 
 // Rows (<= 64) of 16-bit activations on the matrix cores.  A workgroup takes 64 columns
@@ -811,7 +822,7 @@ bool launch_tile_kernel(const Q8Params& p, uint32_t want_slices, const Machine& 
 // and K is cut into slices across workgroups until the grid covers the machine about
 // twice.  variant = NT | WAVES << 8 | SLICES << 24 overrides the plan (tuning, tests).
 template <class T>
-void launch_mfma(const Q8Params& p, uint32_t variant, const Machine& mc, hipStream_t stream) {
+int launch_mfma(const Q8Params& p, uint32_t variant, const Machine& mc, hipStream_t stream, std::string* err) {
   const int mt = p.m <= 16 ? 1 : p.m <= 32 ? 2 : 4;
   int nt = p.n >= 64 ? 4 : 1, waves = p.m > 32 ? 4 : 8;  // (measured: K = 4096 and 14336, N = 14336 and 4096)
   uint32_t slices = 1;
@@ -844,22 +855,28 @@ void launch_mfma(const Q8Params& p, uint32_t variant, const Machine& mc, hipStre
   if (staged) {  // chunks of 256 values of k
     const uint64_t sgroups = (p.n + 16 * nt - 1) / (16 * nt);
     const uint32_t schunks = (p.k + 255) / 256;
+    if (slices > 1 && workspace_refused(mc, sgroups * slices * mt * nt * 1024, err)) return -1;
     while (slices > 1 && (sgroups * slices * mt * nt * 1024 > mc.workspace_bytes || (schunks + slices - 1) / slices * (slices - 1) >= schunks)) --slices;
-    if (mt <= 2 && launch_staged<T>(p, mt, nt, waves, slices, mc, stream)) return;
+    if (mt <= 2 && launch_staged<T>(p, mt, nt, waves, slices, mc, stream)) return 0;
   }
   // the workspace holds groups * slices tiles of MT * NT KiB
   const uint64_t groups = (p.n + 16 * nt - 1) / (16 * nt);
+  if (slices > 1 && workspace_refused(mc, groups * slices * mt * nt * 1024, err)) return -1;
   while (slices > 1 && groups * slices * mt * nt * 1024 > mc.workspace_bytes) --slices;
   const uint32_t chunks = (p.k + 63) / 64;
   while (slices > 1 && (chunks + slices - 1) / slices * (slices - 1) >= chunks) --slices;  // no empty slice
-#define VKT_MFMA_CASE(MT_, NT_) \
-  if (mt == MT_ && nt == NT_) return launch_mfma_waves<T, MT_, NT_>(p, waves, slices, mc, stream);
+#define VKT_MFMA_CASE(MT_, NT_)                                           \
+  if (mt == MT_ && nt == NT_) {                                           \
+    launch_mfma_waves<T, MT_, NT_>(p, waves, slices, mc, stream);         \
+    return 0;                                                             \
+  }
   VKT_MFMA_CASE(1, 1) VKT_MFMA_CASE(1, 2) VKT_MFMA_CASE(1, 4)
   VKT_MFMA_CASE(2, 1) VKT_MFMA_CASE(2, 2) VKT_MFMA_CASE(2, 4)
   VKT_MFMA_CASE(4, 1) VKT_MFMA_CASE(4, 2) VKT_MFMA_CASE(4, 4)
   VKT_MFMA_CASE(1, 8) VKT_MFMA_CASE(2, 8) VKT_MFMA_CASE(4, 8)
 #undef VKT_MFMA_CASE
   launch_mfma_waves<T, 4, 1>(p, waves, slices, mc, stream);
+  return 0;
 }
 
 
@@ -917,7 +934,8 @@ int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipSt
     // more than 32 rows (batched decode): the tile kernel (variant bit 21 forces it with bits 24+ slices, bit 22 keeps it off)
     if (((p0.m > 32 && !(variant & 0xffff)) || ((variant >> 21) & 1)) && !((variant >> 22) & 1) && !((variant >> 17) & 1) && !((variant >> 18) & 1) &&
         !((variant >> 19) & 1) && !((variant >> 20) & 1)) {
-      if (launch_tile_kernel<T>(p0, variant >> 24, mc, stream)) return 0;
+      const int rc = launch_tile_kernel<T>(p0, variant >> 24, mc, stream, err);
+      if (rc != 0) return rc < 0 ? -1 : 0;
     }
     // From 3 rows on the matrix cores win: the GEMV kernels convert every weight and multiply it once per row on
     // the vector units (measured at K = 4096, N = 14336: 10.5, 16.4, 23.0, 23.4 us for 1 to 4 rows; the matrix
@@ -928,7 +946,7 @@ int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipSt
         p.m = p0.m - r0 < 64 ? p0.m - r0 : 64;
         p.a = p0.a + uint64_t(int64_t(r0) * p0.a_sm * int64_t(item));
         p.c = p0.c + uint64_t(r0) * p0.n * item;
-        launch_mfma<T>(p, variant, mc, stream);
+        if (launch_mfma<T>(p, variant, mc, stream, err) != 0) return -1;
       }
       return 0;
     }
