@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-matmul path on one MI355X, through the C ABI.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all] [--no-extra] [--no-cpu] [--verbose]
 
 A "step" is one pass of the hot path over one batch of seeded synthetic input: one
 `_weight_int8pack_mm` / `_dyn_quant_matmul_4bit` / `_scaled_mm` call's kernels, queued through
@@ -13,9 +13,15 @@ copies so that the figure is HBM bandwidth and not the 256 MB last-level cache.
 Prints ONE JSON line.  `value` is algorithmic bytes (or flops) per step / wall time per step
 over exactly K timed steps bracketed by device synchronisation; `roofline.achieved` is the
 same work / the kernel's average duration from HIP events recorded on the stream the
-kernels run on; `cpu_baseline` times the CPU oracle (a scalar C port of the reference's
-arithmetic, one core) on a bounded sample of the same workload, and `cpu_torch` PyTorch's own
-CPU kernel for the op on all host cores.  `extra` carries the other BASELINE configurations.
+kernels run on.  `cpu_baseline` is PyTorch's own CPU kernel for the same op on all host cores
+(the CPU path the reference quotes its numbers against), `cpu_oracle_port` the scalar C
+restatement under oracle/ on one core, both on a bounded sample that `sample` describes.
+`extra` carries the other BASELINE configurations, one short entry each (key, value, unit,
+frac of the published peak, kernel time, CPU figure), the configurations the targets are
+stated on last; `ceilings` what bare loads and a register-only matrix-core loop sustain in
+the same run.  --all adds the workloads beside the BASELINE configurations (prefill shapes,
+the float8 producer, 16-bit products, strided copies, affine quantisation); --verbose keeps
+every entry's full roofline object.
 """
 import argparse
 import ctypes
@@ -64,25 +70,46 @@ class Timing(tuple):
     median = None
 
 
+_DELAY = {}
+
+
+def queue_delay(abi, microseconds):
+    """Queues the one-wave kernel that waits `microseconds` ("probe_delay"): what follows it on the stream is queued by
+    the host while the device waits, so the device then runs it back to back."""
+    if "launch" not in _DELAY:
+        _DELAY["params"] = abi.ProbeParams()
+        _DELAY["launch"] = Launch(abi, "probe_delay", [], _DELAY["params"])
+    _DELAY["params"].iters = int(min(max(microseconds, 1), 100000))
+    _DELAY["launch"]()
+
+
 def time_steps(abi, step_fns, steps, warmup):
-    """Runs step_fns[i % len] for `warmup` untimed and `steps` timed steps, events at five equally spaced marks."""
+    """Runs step_fns[i % len] for `warmup` untimed and `steps` timed steps: wall time per step between two device
+    synchronisations (the host queues a step as soon as the one before is queued).  Then the same `steps` steps once
+    more behind a queued delay, with events at five equally spaced marks: the device's own time per step, with every
+    launch already in its queue (the host needs 3-5 us to queue a launch, as long as the shortest kernels here run)."""
     n = len(step_fns)
-    for i in range(warmup):
-        step_fns[i % n]()
+    seq = [step_fns[i % n] for i in range(max(steps, warmup))]
+    for f in seq[:warmup]:
+        f()
     abi.synchronize()
+    t0 = time.perf_counter()
+    for f in seq[:steps]:
+        f()
+    abi.synchronize()
+    t1 = time.perf_counter()
     parts = 5 if steps >= 10 else 1
     marks = [steps * j // parts for j in range(parts + 1)]
     events = [abi.Event() for _ in marks]
-    t0 = time.perf_counter()
+    queue_delay(abi, 8 * steps + 200)
     events[0].record()
     at = 1
-    for i in range(steps):
-        step_fns[i % n]()
+    for i, f in enumerate(seq[:steps]):
+        f()
         if i + 1 == marks[at]:
             events[at].record()
             at += 1
     abi.synchronize()
-    t1 = time.perf_counter()
     t = Timing(((t1 - t0) * 1e3 / steps, events[0].elapsed_ms(events[-1]) / steps))
     per = sorted(events[j].elapsed_ms(events[j + 1]) / (marks[j + 1] - marks[j]) for j in range(parts))
     t.median = per[len(per) // 2]
@@ -175,7 +202,7 @@ def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030, prefill=False):
                     **timed(abi, fns, steps, max(warmup, len(fns)), resident=False))
     return dict(kind="hbm", work=work, flops=2 * m * n * k, inputs=(x, packed),
                 name=f"_dyn_quant_matmul_4bit f32 M={m} K={k} N={n} bs={bs} (compact side-car)",
-                reference_layout_bytes=int(packed.numel()) * 4 + 4 * m * k + 4 * m * n, **timed(abi, fns, steps, warmup))
+                shape=(n, bs), reference_layout_bytes=int(packed.numel()) * 4 + 4 * m * k + 4 * m * n, **timed(abi, fns, steps, warmup))
 
 
 def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False):
@@ -309,46 +336,87 @@ def wl_copy(abi, nbytes, steps, warmup):
                 name=f"device copy of {nbytes >> 20} MiB (read + write)")
 
 
-WORKLOADS = {
-    # BASELINE.json configs[1]: the configuration the metric is quoted on
+def wl_probe_read(abi, n, k, geometry, steps, warmup, label):
+    """Bare 16-byte non-temporal loads of n * k bytes in a product kernel's launch geometry (kernel "probe_read"),
+    rotated through more than 512 MiB like the product itself: what that geometry can stream at all."""
+    nbytes = n * k if geometry != 2 else abi.lib().vkt_qmm4c_bytes(n, k, 32)
+    sink = abi.Buffer(256)
+    copies = [abi.Buffer(nbytes) for _ in range(rotation(nbytes))]
+    for c in copies:
+        abi.check(abi.lib().vkt_fill(c.address, 1, nbytes))
+    fns = [Launch(abi, "probe_read", [geometry], abi.ProbeParams(src=c.address, dst=sink.address, n=n, k=k)) for c in copies]
+    work = n * k if geometry != 2 else n * k // 2 + 4 * n * (k // 32)
+    tm = time_steps(abi, fns, steps, warmup)
+    return dict(kind="hbm", metric="bare read GB/s (% of HBM peak)", work=work, wall_ms=tm[0], event_ms=tm[1], event_ms_median=tm.median,
+                flops=0, inputs=None, copies=len(fns), name=f"probe_read {label}: {work} bytes")
+
+
+def wl_probe_mfma(abi, operands, steps, warmup, iters=4096):
+    """A register-only loop of fp8 32x32x64 matrix-core instructions on every compute unit (kernel "probe_mfma_f8"):
+    operands 0 all zero, 1 random bits held in registers, 2 fresh bits for every instruction."""
+    sink = abi.Buffer(256)
+    info = abi.device_info()
+    fns = [Launch(abi, "probe_mfma_f8", [operands], abi.ProbeParams(dst=sink.address, iters=iters))]
+    tm = time_steps(abi, fns, steps, warmup)
+    work = info.compute_units * 4 * iters * 4 * 2 * 32 * 32 * 64
+    label = {0: "all-zero operands", 1: "random operands held in registers", 2: "fresh random operands per instruction"}[operands]
+    return dict(kind="mfma", metric="fp8 MFMA loop TFLOP/s (% of MFMA peak)", work=work, wall_ms=tm[0], event_ms=tm[1], event_ms_median=tm.median,
+                bytes=0, inputs=None, copies=1, name=f"probe_mfma_f8, {label}")
+
+
+# The BASELINE.json configurations.  Order of the extras in the output: the configurations the targets are stated on
+# come last (a stored tail of the line keeps them).
+BASELINE = {
+    # configs[1]: the configuration the metric is quoted on
     "c2_m1_k4096_n14336": lambda abi, s, w: wl_q8(abi, 1, 4096, 14336, abi.BF16, s, w),
-    "c2_m1_k14336_n4096": lambda abi, s, w: wl_q8(abi, 1, 14336, 4096, abi.BF16, s, w),
     "c2_m8_k4096_n14336": lambda abi, s, w: wl_q8(abi, 8, 4096, 14336, abi.BF16, s, w),
     "c2_m8_k14336_n4096": lambda abi, s, w: wl_q8(abi, 8, 14336, 4096, abi.BF16, s, w),
     "c2_m64_k4096_n14336": lambda abi, s, w: wl_q8(abi, 64, 4096, 14336, abi.BF16, s, w),
     "c2_m64_k14336_n4096": lambda abi, s, w: wl_q8(abi, 64, 14336, 4096, abi.BF16, s, w),
-    # many rows of the same operator (prefill; not a BASELINE configuration)
-    "c2_prefill_m4096_k4096_n14336": lambda abi, s, w: wl_q8(abi, 4096, 4096, 14336, abi.BF16, max(s // 20, 5), max(w // 4, 3), prefill=True),
+    "c3_int4_m32": lambda abi, s, w: wl_q4(abi, 32, 4096, 11008, 32, max(s // 4, 5), w),
+    "c2_m1_k14336_n4096": lambda abi, s, w: wl_q8(abi, 1, 14336, 4096, abi.BF16, s, w),
+    "c5_fp8_rowwise_70b": lambda abi, s, w: wl_fp8(abi, 4096, 8192, 28672, True, max(s // 10, 5), max(w // 4, 3), seed=1050),
     "c1_f32_m1_k4096_n4096": lambda abi, s, w: wl_q8(abi, 1, 4096, 4096, abi.F32, s, w, seed=1010),
     "c3_int4_m1": lambda abi, s, w: wl_q4(abi, 1, 4096, 11008, 32, s, w),
-    "c3_int4_m32": lambda abi, s, w: wl_q4(abi, 32, 4096, 11008, 32, max(s // 4, 5), w),
-    # many rows of the same operator (prefill; not a BASELINE configuration)
-    "c3_int4_prefill_m2048": lambda abi, s, w: wl_q4(abi, 2048, 4096, 11008, 32, max(s // 10, 5), w, prefill=True),
     "c4_fp8_8192": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 10, 5), max(w // 4, 3)),
-    "c5_fp8_rowwise_70b": lambda abi, s, w: wl_fp8(abi, 4096, 8192, 28672, True, max(s // 10, 5), max(w // 4, 3),
-                                                   seed=1050),
-    # the float8 steps in front of _scaled_mm (not BASELINE configurations: the next rows of the path),
-    # at the size of config 4's A operand and beyond the L2 / MALL capacity
+}
+# Beside the BASELINE configurations (--all, or by name): many rows of the same operators, the steps either side of
+# the path, the planner off the Llama grid, config 4's launch on all-zero operands.
+OTHER = {
+    "c2_prefill_m4096_k4096_n14336": lambda abi, s, w: wl_q8(abi, 4096, 4096, 14336, abi.BF16, max(s // 20, 5), max(w // 4, 3), prefill=True),
+    "c3_int4_prefill_m2048": lambda abi, s, w: wl_q4(abi, 2048, 4096, 11008, 32, max(s // 10, 5), w, prefill=True),
+    "q8_m1_k5120_n13824": lambda abi, s, w: wl_q8(abi, 1, 5120, 13824, abi.BF16, s, w, seed=1110),
+    "q8_m1_k8192_n8192": lambda abi, s, w: wl_q8(abi, 1, 8192, 8192, abi.BF16, s, w, seed=1120),
+    "q8_m8_k5120_n13824": lambda abi, s, w: wl_q8(abi, 8, 5120, 13824, abi.BF16, s, w, seed=1110),
+    "q8_m64_k8192_n8192": lambda abi, s, w: wl_q8(abi, 64, 8192, 8192, abi.BF16, s, w, seed=1120),
     "f8_cast_bf16_e4m3_256mi": lambda abi, s, w: wl_cast(abi, 1 << 28, max(s // 10, 5), max(w // 4, 3)),
     "f8_quant_rowwise_bf16_16384x16384": lambda abi, s, w: wl_quant(abi, 16384, 16384, max(s // 10, 5), max(w // 4, 3)),
-    # the unquantised 16-bit product beside the path (not a BASELINE configuration), at the reference's own shape
     "mm_bf16_8192": lambda abi, s, w: wl_gemm16(abi, 8192, 8192, 8192, max(s // 10, 5), max(w // 4, 3)),
     "mm_bf16_8192_nn": lambda abi, s, w: wl_gemm16(abi, 8192, 8192, 8192, max(s // 10, 5), max(w // 4, 3), layout="nn"),
     "mm_bf16_8192_tn": lambda abi, s, w: wl_gemm16(abi, 8192, 8192, 8192, max(s // 10, 5), max(w // 4, 3), layout="tn"),
-    # strided device copies either side of the path (not BASELINE configurations)
     "move_transpose_bf16_16384": lambda abi, s, w: wl_move(abi, "transpose", max(s // 10, 5), max(w // 4, 3)),
     "move_rows_bf16_16384": lambda abi, s, w: wl_move(abi, "rows", max(s // 10, 5), max(w // 4, 3)),
-    # per-tensor affine quantised tensors and fake quantisation (not BASELINE configurations)
     "affine_quantize_256mi": lambda abi, s, w: wl_affine(abi, "quantize", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
     "affine_dequantize_256mi": lambda abi, s, w: wl_affine(abi, "dequantize", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
     "affine_fake_quant_256mi": lambda abi, s, w: wl_affine(abi, "fake_quant", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
-    # config 4's launch on all-zero operands (not a BASELINE configuration: it shows how much of the
-    # distance to the published peak is the data's, not the kernel's)
-    "c4_fp8_8192_zero_operands": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 10, 5),
-                                                          max(w // 4, 3), zero_operands=True),
+    "c4_fp8_8192_zero_operands": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 10, 5), max(w // 4, 3), zero_operands=True),
 }
-# not a BASELINE configuration: selected by name only (counter calibration)
-CALIBRATION = {"copy_256mib": lambda abi, s, w: wl_copy(abi, 256 << 20, max(s // 4, 5), w)}
+# Ceilings measured in the same run (`ceilings` of the output line; also selectable by name): bare 16-byte loads of
+# each GEMV configuration's weight bytes in its kernel's launch geometry, a persistent-grid read, a device copy of known
+# size (calibrates the traffic counters), and the register-only fp8 matrix-core loop on three kinds of operand bits.
+CALIBRATION = {
+    "probe_read_c1_16mb": lambda abi, s, w: wl_probe_read(abi, 4096, 4096, 0, s, w, "config 1 (4096 x 4096 int8, GEMV geometry)"),
+    "probe_read_c3_28mb": lambda abi, s, w: wl_probe_read(abi, 11008, 4096, 2, s, w, "config 3 (int4 side-car, streaming geometry)"),
+    "probe_read_c2_58mb": lambda abi, s, w: wl_probe_read(abi, 14336, 4096, 0, s, w, "config 2 (14336 x 4096 int8, GEMV geometry)"),
+    "probe_read_c2_58mb_k14336": lambda abi, s, w: wl_probe_read(abi, 4096, 14336, 1, s, w, "config 2 (4096 x 14336 int8, GEMV geometry)"),
+    "probe_read_persistent_58mb": lambda abi, s, w: wl_probe_read(abi, 14336, 4096, 3, s, w, "58 MB, persistent grid"),
+    "probe_read_persistent_16mb": lambda abi, s, w: wl_probe_read(abi, 4096, 4096, 3, s, w, "16 MB, persistent grid"),
+    "probe_mfma_f8_zero": lambda abi, s, w: wl_probe_mfma(abi, 0, max(s // 10, 5), max(w // 4, 3)),
+    "probe_mfma_f8_held": lambda abi, s, w: wl_probe_mfma(abi, 1, max(s // 10, 5), max(w // 4, 3)),
+    "probe_mfma_f8_fresh": lambda abi, s, w: wl_probe_mfma(abi, 2, max(s // 10, 5), max(w // 4, 3)),
+    "copy_256mib": lambda abi, s, w: wl_copy(abi, 256 << 20, max(s // 4, 5), w),
+}
+WORKLOADS = {**BASELINE, **OTHER}
 HEADLINE = "c2_m1_k4096_n14336"
 
 
@@ -370,38 +438,77 @@ def summarise(r):
     return value, unit, roof
 
 
-def cpu_baselines(abi, name, r):
-    """The oracle (scalar C port, one core) on a bounded sample, and PyTorch's CPU op on all cores."""
-    import torch
-    import oracle
-    out = {}
-    if not name.startswith(("c1", "c2")):
-        return out
-    x, w, s = r["inputs"]
-    m, k = x.shape
-    n = w.shape[0]
-    odt = {torch.float32: oracle.F32, torch.bfloat16: oracle.BF16, torch.float16: oracle.F16}[x.dtype]
-    xb = x.numpy() if odt == oracle.F32 else x.view(torch.int16).numpy().view(np.uint16)
-    sb = s.numpy() if odt == oracle.F32 else s.view(torch.int16).numpy().view(np.uint16)
-    oracle.qmm8(xb, odt, w.numpy()[:64], sb[:64])  # load + warm
-    reps, t0 = 0, time.perf_counter()
-    while time.perf_counter() - t0 < 10.0 and reps < 200:
-        oracle.qmm8(xb, odt, w.numpy(), sb)
-        reps += 1
-    dt = (time.perf_counter() - t0) / reps
-    out["cpu_baseline"] = dict(value=round(r["work"] / dt / 1e9, 3), unit="GB/s", cores=1, kind="port",
-                               sample=f"{reps} full passes of the same workload through oracle/qmm_oracle.c "
-                                      f"(scalar C restatement), {dt * 1e3:.1f} ms each")
-    torch._weight_int8pack_mm(x, w, s)
+def _median_time(fn, reps, warm=1):
+    for _ in range(warm):
+        fn()
     ts = []
-    for _ in range(15):
+    for _ in range(reps):
         t0 = time.perf_counter()
-        torch._weight_int8pack_mm(x, w, s)
+        fn()
         ts.append(time.perf_counter() - t0)
-    dt = sorted(ts)[len(ts) // 2]
-    out["cpu_torch"] = dict(value=round(r["work"] / dt / 1e9, 3), unit="GB/s", cores=torch.get_num_threads(),
-                            host_cpus=os.cpu_count(), kind="torch CPU kernel of the same op",
-                            sample=f"median of 15 calls of torch._weight_int8pack_mm, {dt * 1e3:.2f} ms")
+    return sorted(ts)[len(ts) // 2]
+
+
+def cpu_baselines(abi, name, r, port=False):
+    """The CPU beside the GPU figure, on the same seeded inputs: `cpu_baseline` = PyTorch's CPU kernel of the op on all
+    host cores (what the reference's own numbers are quoted against), on a bounded sample; port=True adds
+    `cpu_oracle_port`, the scalar C restatement on one core."""
+    import torch
+    out = {}
+    cores = torch.get_num_threads()
+    if not r.get("inputs"):
+        return out
+    if name.startswith(("c1", "c2", "q8_")):
+        x, w, s = r["inputs"]
+        reps = 15 if x.shape[0] <= 8 else 5
+        dt = _median_time(lambda: torch._weight_int8pack_mm(x, w, s), reps)
+        out["cpu_baseline"] = dict(value=round(r["work"] / dt / 1e9, 3), unit="GB/s", cores=cores, kind="reference",
+                                   sample=f"torch._weight_int8pack_mm on CPU tensors (PyTorch's own kernel of the op: the CPU path the reference "
+                                          f"is quoted against), full workload, median of {reps} calls, {dt * 1e3:.2f} ms; host has {os.cpu_count()} CPUs")
+        if port:
+            import oracle
+            odt = {torch.float32: oracle.F32, torch.bfloat16: oracle.BF16, torch.float16: oracle.F16}[x.dtype]
+            xb = x.numpy() if odt == oracle.F32 else x.view(torch.int16).numpy().view(np.uint16)
+            sb = s.numpy() if odt == oracle.F32 else s.view(torch.int16).numpy().view(np.uint16)
+            oracle.qmm8(xb, odt, w.numpy()[:64], sb[:64])  # load + warm
+            reps, t0 = 0, time.perf_counter()
+            while time.perf_counter() - t0 < 3.0 and reps < 100:
+                oracle.qmm8(xb, odt, w.numpy(), sb)
+                reps += 1
+            dt = (time.perf_counter() - t0) / reps
+            out["cpu_oracle_port"] = dict(value=round(r["work"] / dt / 1e9, 3), unit="GB/s", cores=1, kind="port",
+                                          sample=f"{reps} full passes through oracle/qmm_oracle.c (scalar C restatement), {dt * 1e3:.1f} ms each")
+    elif name.startswith("c3"):
+        x, packed = r["inputs"]
+        m, k = x.shape
+        n, bs = r["shape"]
+        reps = 3
+        dt = _median_time(lambda: torch._dyn_quant_matmul_4bit(x, packed, bs, k, n), reps)
+        out["cpu_baseline"] = dict(value=round(r["work"] / dt / 1e9, 3), unit="GB/s", cores=cores, kind="reference",
+                                   sample=f"torch._dyn_quant_matmul_4bit on CPU tensors (float32-expanded packed vector), full workload, "
+                                          f"median of {reps} calls, {dt * 1e3:.1f} ms; priced on the same algorithmic bytes as the GPU figure")
+    elif name.startswith(("c4", "c5")):
+        a, bt, sa, sb = r["inputs"]
+        m, k = a.shape
+        n = bt.shape[0]
+        rowwise = sa.numel() > 1
+        rows = min(m, 1024)  # a bounded sample: the first rows of A against all of B
+        a_s, sa_s = a[:rows], (sa[:rows].reshape(rows, 1) if rowwise else sa)
+        sb_s = sb.reshape(1, n) if rowwise else sb
+
+        def closed_form():
+            return ((a_s.float() * sa_s) @ (bt.float() * sb_s.reshape(-1, 1) if rowwise else bt.float() * sb_s).t()).bfloat16()
+        dt = _median_time(closed_form, 1, warm=0)
+        out["cpu_baseline"] = dict(value=round(2.0 * rows * n * k / dt / 1e12, 4), unit="TFLOP/s", cores=cores, kind="reference",
+                                   sample=f"the emulated closed form ((A.float()*sa) @ (B.float()*sb)).bfloat16() in PyTorch on the CPU (what the "
+                                          f"reference's composite computes; torch's CPU _scaled_mm kernel " + ("rejects rowwise scales" if rowwise else "is a scalar loop, timed below") +
+                                          f"), first {rows} of {m} rows of A against all of B, one call, {dt:.2f} s")
+        if not rowwise:
+            e = 768  # torch's CPU _scaled_mm itself, at a reduced size (a scalar reference kernel: cubic extrapolation)
+            dt = _median_time(lambda: torch._scaled_mm(a[:e, :e].contiguous(), bt[:e, :e].contiguous().t(), sa.reshape(()), sb.reshape(()), out_dtype=torch.bfloat16), 1, warm=0)
+            out["cpu_scaled_mm_op"] = dict(value=round(2.0 * e ** 3 / dt / 1e12, 6), unit="TFLOP/s", cores=cores, kind="reference",
+                                           sample=f"torch._scaled_mm on CPU tensors at {e}^3 (one call, {dt:.2f} s); at this rate {m}x{k}x{n} would take "
+                                                  f"{dt * (m * k * n) / e ** 3 / 60:.0f} min")
     return out
 
 
@@ -411,7 +518,7 @@ def through_dispatcher(abi, name, r, calls=200):
     the same resident weights, so that the host's share shows."""
     import torch
     import torch_vulkan_amd.backend as tv
-    if not name.startswith(("c1", "c2")) or not r.get("inputs"):
+    if not name.startswith(("c1", "c2", "q8_")) or not r.get("inputs"):
         return None
     x, w, s = (t.to("vk") for t in r["inputs"])
     before = tv.fallback_counts()
@@ -440,14 +547,29 @@ def load_traffic():
         return {}
 
 
+def compact(key, rr, v, u, rf, cpu):
+    """One short entry of `extra`."""
+    e = {"key": key, "value": round(v, 1), "unit": u, "frac": rf["frac"], "kernel_ms": round(rr["event_ms"], 5)}
+    if "cache_resident" in rf:
+        e["resident_ms"] = rf["cache_resident"]["kernel_ms"]
+    if rf.get("traffic"):
+        e["traffic"] = rf["traffic"]
+    if cpu.get("cpu_baseline"):
+        c = cpu["cpu_baseline"]
+        e["cpu"] = {"value": c["value"], "unit": c["unit"], "cores": c["cores"]}
+    return e
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS) + sorted(CALIBRATION))
+    ap.add_argument("--all", action="store_true", help="also the workloads beside the BASELINE configurations")
     ap.add_argument("--no-extra", action="store_true", help="only the selected workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--verbose", action="store_true", help="full roofline objects and CPU samples for every entry")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is a one-GPU path (no collectives, no sharding); run with --gpus 1")
@@ -458,39 +580,57 @@ def main():
     r = {**WORKLOADS, **CALIBRATION}[args.workload](abi, args.steps, args.warmup)
     value, unit, roof = summarise(r)
     roof["traffic"] = traffic.get(args.workload)
+    if r["kind"] == "hbm":
+        metric, dtype = "M=1 int8 GEMV GB/s (% of HBM peak)", "f32 accumulate (bf16 activations, int8 weights)"
+    else:
+        metric, dtype = "fp8 _scaled_mm TFLOP/s (% of MFMA peak)", "f32 accumulate (fp8 e4m3 operands)"
+    if args.workload.startswith("c1"):
+        dtype = "f32"
+    elif args.workload.startswith("c3"):
+        metric, dtype = "M=1 int4 GEMV GB/s (% of HBM peak)", "int32 block sums, f32 accumulate (int4 weights, int8 activations)"
     line = {
-        "metric": r.get("metric") or ("M=1 int8 GEMV GB/s (% of HBM peak)" if r["kind"] == "hbm"
-                                      else "fp8 _scaled_mm TFLOP/s (% of MFMA peak)"),
+        "metric": r.get("metric") or metric,
         "value": round(value, 1), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(r["wall_ms"], 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32 accumulate (bf16 activations, int8 weights)" if args.workload.startswith("c2") else "see workload",
-        "data": "synthetic (seeded)",
+        "dtype": dtype, "data": "synthetic (seeded)",
         "config": {"workload": r["name"], "key": args.workload, "weight_copies_rotated": r["copies"],
                    "device": info.name.decode(), "compute_units": info.compute_units},
         "roofline": roof,
     }
     if not args.no_cpu:
-        line.update(cpu_baselines(abi, args.workload, r))
+        line.update(cpu_baselines(abi, args.workload, r, port=True))
         line["through_dispatcher"] = through_dispatcher(abi, args.workload, r)
     if "cpu_baseline" not in line:
         line["cpu_baseline"] = None
     del r
     if not args.no_extra:
+        # what bare loads and a register-only matrix-core loop sustain, in this run on this box (GB/s, TFLOP/s)
+        ceilings = {}
+        for key, fn in CALIBRATION.items():
+            if key == args.workload or key == "copy_256mib":
+                continue
+            rr = fn(abi, args.steps, args.warmup)
+            v, u, rf = summarise(rr)
+            ceilings[key] = {"achieved": rf["achieved"], "unit": u, "kernel_ms": round(rr["event_ms"], 5)}
+            del rr
+        line["ceilings"] = ceilings
         extra = []
-        for name, fn in WORKLOADS.items():
+        for name, fn in ({**OTHER, **BASELINE} if args.all else BASELINE).items():
             if name == args.workload:
                 continue
             rr = fn(abi, args.steps, args.warmup)
             v, u, rf = summarise(rr)
             rf["traffic"] = traffic.get(name)
-            e = {"key": name, "workload": rr["name"], "value": round(v, 1), "unit": u,
-                 "ms_per_step": round(rr["wall_ms"], 5), "kernel_ms": round(rr["event_ms"], 5), "roofline": rf}
-            if rr["kind"] == "hbm":
-                e["tflops"] = round(rr["flops"] / rr["event_ms"] / 1e9, 2)
-            else:
-                e["hbm_gbps_algorithmic"] = round(rr["bytes"] / rr["event_ms"] / 1e6, 1)
-            if "reference_layout_bytes" in rr:
-                e["reference_layout_bytes"] = rr["reference_layout_bytes"]
+            cpu = {} if args.no_cpu or name not in BASELINE else cpu_baselines(abi, name, rr)
+            e = compact(name, rr, v, u, rf, cpu)
+            if args.verbose:
+                e.update(workload=rr["name"], ms_per_step=round(rr["wall_ms"], 5), roofline=rf, **cpu)
+                if rr["kind"] == "hbm":
+                    e["tflops"] = round(rr["flops"] / rr["event_ms"] / 1e9, 2)
+                else:
+                    e["hbm_gbps_algorithmic"] = round(rr["bytes"] / rr["event_ms"] / 1e6, 1)
+                if "reference_layout_bytes" in rr:
+                    e["reference_layout_bytes"] = rr["reference_layout_bytes"]
             extra.append(e)
             del rr
         line["extra"] = extra

@@ -117,7 +117,9 @@ uint64_t vkt_qmm4c_q_bytes(uint32_t m, uint32_t k);
  * launcher's choice of kernel and shape (tests, tuning; 0 or absent: planned): bits 0-7 columns per wave or
  * column tiles per workgroup, 8-15 waves that split K, 24+ slices of K over workgroups; bit 16 the any-shape
  * kernel, 17 the vector-unit kernels, 18 / 19 the matrix-core kernel with / without staging through LDS, 20 no
- * widened-weights product for many rows, 21 / 22 the 64 x 128 tile kernel forced / off. */
+ * widened-weights product for many rows, 21 / 22 the 64 x 128 tile kernel forced / off; one row: bit 23 keeps the
+ * kernel with a workgroup per pair of columns, bits 8-11 / 12-15 (bits 0-7 clear) ask for the persistent streaming
+ * kernel with that many workgroups per compute unit / rows per iteration. */
 typedef struct Q8Params {
   uint64_t a, b, scales, c; /* A [m,k] (row stride a_sm, a_sk must be 1), B int8 [n,k], scales [n], C [m,n] */
   uint32_t m, n, k;
@@ -278,7 +280,9 @@ typedef struct F8Params {
 /* "probe_read", spec {GEOMETRY} and "probe_mfma_f8", spec {OPERANDS}: calibration kernels for the rooflines (what
  * a launch geometry can stream, what the fp8 matrix cores sustain on given operand bits); they read src [n, k] bytes
  * (probe_read) or run `iters` iterations of 4 matrix-core instructions per wave, 4 waves on every compute unit
- * (probe_mfma_f8), and write nothing (dst must be a valid address).  No counterpart in the reference.  32 bytes. */
+ * (probe_mfma_f8), and write nothing (dst must be a valid address).  "probe_delay", spec {}: one wave that waits
+ * `iters` microseconds (at most 100000) and exits; a timing loop queues it in front of its launches so that the host
+ * has queued them all before the device starts on them.  No counterpart in the reference.  32 bytes. */
 typedef struct ProbeParams {
   uint64_t src, dst;
   uint32_t n, k, iters, pad;

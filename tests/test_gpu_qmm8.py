@@ -50,6 +50,24 @@ def test_qmm8_every_variant(variant, dtype):
         check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=variant), a, b, s, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("k", [16, 1008, 1024, 2048, 2064, 3072, 4096, 4112, 6144, 8192, 8208, 12288, 14336, 16384])
+def test_qmm8_one_row_streaming_kernel(dtype, k):
+    """One activation row through the persistent streaming kernel: every split of a row over a workgroup's waves
+    (1 to 4 chunks of 1 KiB per wave, 1, 2 or 4 waves per row), rows that end inside a chunk, fewer rows than a
+    workgroup takes per iteration, more iterations than one, and the rows-per-iteration forms the planner picks from."""
+    import _dev
+    for n in (1, 7, 300):
+        a, b, s = int8_case(dtype, 1, k, n)
+        for variant in (2 << 8, 1 << 8 | 1 << 12, 3 << 8 | 2 << 12):
+            if (variant >> 12) == 2 and k <= 1024 or (variant >> 12) == 1 and k <= 2048:
+                continue  # (forms that are not built: short rows take 8 or 4 rows per iteration)
+            check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=variant), a, b, s, dtype)
+    # enough rows for several iterations per wave on a full grid
+    a, b, s = int8_case(dtype, 1, k, 9000 if k <= 4096 else 3000)
+    check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=1 << 8), a, b, s, dtype)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("variant", [0, 1 | 4 << 8, 2 | 8 << 8, 4 | 16 << 8, 4 | 8 << 8 | 3 << 24, 1 | 4 << 8 | 16 << 24,
                                      1 << 17, 1 << 18, 1 | 4 << 8 | 1 << 18, 2 | 8 << 8 | 1 << 18, 4 | 4 << 8 | 1 << 18,

@@ -263,6 +263,7 @@ int call_aminmax(const MinMaxParams& p, const Call& c) { return launch_aminmax(p
 int call_fp8_quant(const F8QuantParams& p, const Call& c) { return launch_fp8_quant(p, c.spec_at(0), c.machine, c.stream, c.err); }
 int call_probe_read(const ProbeParams& p, const Call& c) { return launch_probe_read(p, c.spec_at(0), c.machine, c.stream, c.err); }
 int call_probe_mfma(const ProbeParams& p, const Call& c) { return launch_probe_mfma(p, c.spec_at(0), c.machine, c.stream, c.err); }
+int call_probe_delay(const ProbeParams& p, const Call& c) { return launch_probe_delay(p, c.stream, c.err); }
 int call_fp8mm(const F8Params& p, const Call& c) { return launch_fp8mm(p, c.spec_at(0), c.machine, c.stream, c.err); }
 
 // name -> parameter block type + launcher (the role of kernels.rs:72-140 KernelCache::get).  An entry ties a
@@ -296,6 +297,7 @@ const KernelEntry kKernels[] = {
     entry<F8Params, call_fp8mm>("fp8mm", false),
     entry<ProbeParams, call_probe_read>("probe_read", false),
     entry<ProbeParams, call_probe_mfma>("probe_mfma_f8", false),
+    entry<ProbeParams, call_probe_delay>("probe_delay", false),
     entry<Q8Params, call_qmm8>("qmm8_", true),
     entry<Q4CParams, call_qmm4c>("qmm4c_", true),
     entry<Q4Params, call_qmm4>("qmm4_", true),

@@ -60,6 +60,7 @@ int launch_fake_quant(const QuantParams& p, uint32_t per_channel, uint32_t zp_fl
 int launch_fp8_quant(const F8QuantParams& p, uint32_t rowwise, const Machine& mc, hipStream_t stream, std::string* err);
 int launch_probe_read(const ProbeParams& p, uint32_t geometry, const Machine& mc, hipStream_t stream, std::string* err);
 int launch_probe_mfma(const ProbeParams& p, uint32_t operands, const Machine& mc, hipStream_t stream, std::string* err);
+int launch_probe_delay(const ProbeParams& p, hipStream_t stream, std::string* err);
 int launch_fill(uint64_t dst, uint8_t value, uint64_t nbytes, hipStream_t stream, std::string* err);
 int launch_copy(uint64_t dst, uint64_t src, uint64_t nbytes, hipStream_t stream, std::string* err);
 

@@ -11,11 +11,20 @@
 //                                       accumulator tiles per wave): 0 all-zero operands, 1 random bits held in the same
 //                                       registers throughout, 2 fresh operands for every instruction (made by vector
 //                                       operations, no memory at all)
+//   "probe_delay", spec {}              one wave that waits `iters` microseconds on the constant-rate clock and exits: a
+//                                       timing loop queues it first so that the launches behind it are all queued by the
+//                                       time the device reaches them (the device, not the host, then sets the pace)
 #include "common.h"
 #include "kernels.h"
 
 namespace vkt {
 namespace {
+
+__global__ __launch_bounds__(64) void probe_delay(uint64_t ticks) {
+  const uint64_t start = wall_clock64();
+  // (bounded by construction: the clock advances whatever else happens)
+  while (wall_clock64() - start < ticks) __builtin_amdgcn_s_sleep(32);
+}
 
 __device__ __forceinline__ void sink(uint64_t dst, const U4& acc) {
   // (never true for the buffers bench.py passes; keeps the loads alive)
@@ -97,11 +106,13 @@ __global__ __launch_bounds__(256) void probe_mfma_f8(ProbeParams p) {
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         if constexpr (OPERANDS == 2) {
-          // a fresh pair of fragments for this instruction: one multiply-add per register
+          // fresh bits for this instruction: about half the bits of half of each fragment's registers flip (one
+          // exclusive-or per register, 8 vector operations per matrix-core instruction: more would make the loop
+          // wait for the vector unit; the masks keep the lowest mantissa bit of every byte clear: no NaN code appears)
 #pragma unroll
-          for (int r = 0; r < 8; ++r) {
-            a[i][r] = int((uint32_t(a[i][r]) * 1664525u + 1013904223u) & 0xfefefefeu);
-            b[j][r] = int((uint32_t(b[j][r]) * 22695477u + 1u) & 0xfefefefeu);
+          for (int r = 0; r < 4; ++r) {
+            a[i][2 * r + (j & 1)] ^= int(0x5ac6963au + 0x02040810u * uint32_t(r) + 0x20406080u * uint32_t(j)) & int(0xfefefefeu);
+            b[j][2 * r + (i & 1)] ^= int(0xc6a4d2b8u + 0x04081020u * uint32_t(r) + 0x10204080u * uint32_t(i)) & int(0xfefefefeu);
           }
         }
         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b[j], a[i], acc[i][j], 0, 0, 0, 0, 0, 0);
@@ -133,6 +144,23 @@ int launch_probe_read(const ProbeParams& p, uint32_t geometry, const Machine& mc
   }
   if (hipGetLastError() != hipSuccess) {
     *err = "probe_read: kernel launch failed";
+    return -1;
+  }
+  return 0;
+}
+
+int launch_probe_delay(const ProbeParams& p, hipStream_t stream, std::string* err) {
+  if (p.iters > 100000) {
+    *err = "probe_delay: at most 100000 microseconds";
+    return -1;
+  }
+  int rate_khz = 100000;  // the constant-rate clock: 100 MHz unless the device says otherwise
+  int dev = 0;
+  if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&rate_khz, hipDeviceAttributeWallClockRate, dev);
+  if (rate_khz <= 0) rate_khz = 100000;
+  hipLaunchKernelGGL(probe_delay, dim3(1), dim3(64), 0, stream, uint64_t(p.iters) * uint64_t(rate_khz) / 1000);
+  if (hipGetLastError() != hipSuccess) {
+    *err = "probe_delay: kernel launch failed";
     return -1;
   }
   return 0;

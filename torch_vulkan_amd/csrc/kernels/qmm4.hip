@@ -329,12 +329,13 @@ __global__ __launch_bounds__(256) void qmm4c_rowquant(Q4CParams p, uint32_t grou
 }
 
 // The streaming kernel.  UPB = units per scale block (1, 2, 4, 8), or 0 for channelwise (one
-// block spanning K).  FUSED: the workgroup quantises its MR activation rows itself (phase 0
+// block spanning K).  XG != 0 (fused): the workgroup quantises its MR activation rows itself (phase 0
 // folded in: no second launch, no scratch round trip); otherwise it stages the planes that
 // phase 0 left in global memory.  The inner loop reads activations from LDS and weights
 // straight from HBM.
-template <class T, int MR, int UPB, bool FUSED>
+template <class T, int MR, int UPB, int XG>
 __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L, uint32_t m0, uint32_t groupwise) {
+  constexpr bool FUSED = XG != 0;  // XG: groups of 8 activations a thread quantises (k <= 2048 * XG)
   constexpr uint64_t item = sizeof(typename T::storage);
   constexpr int BPL = UPB ? kUnitsPerLane / UPB : 1;  // blocks per lane per round
   constexpr int UN = UPB ? UPB : kUnitsPerLane;       // units of a block within a lane
@@ -347,6 +348,9 @@ __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L
   float* const carry = reinterpret_cast<float*>(q_lds + MR * qs);      // [MR][16]
   int* const itotal = reinterpret_cast<int*>(carry);                    // (channelwise: integer totals)
   float* const terms = carry + MR * kTileCols + 16;                     // [MR][16][kTermPitch]: a round's block terms
+
+  // (every thread: a load without a branch around it; asked for first, so that it is there long before the sums are)
+  const float bias = ldg<float>(p.compact + L.bias_off + (n < p.n ? n : p.n - 1) * 4ull);
 
   // Loads return in the order they were issued.  The first row's activations are asked for first (they come
   // from L2 and the row quantisation waits for them alone), then the first round's weights and scales: the
@@ -382,32 +386,32 @@ __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L
     const uint32_t m = m0 + r < p.m ? m0 + r : p.m - 1;
     if constexpr (FUSED) {
       const uint64_t row = p.inp + uint64_t(m) * p.k * item;
-      // A thread owns the groups of 8 values g = tid + 256 i, i < kFusedGroups: all loads are
-      // in flight together, the row's range is reduced from registers and the values are
-      // quantised from registers.  (The launcher fuses only when k is a multiple of 8, rows
-      // are 16-byte aligned and k <= 2048 * kFusedGroups; otherwise it runs phase 0 itself.)
+      // A thread owns the groups of 8 values g = tid + 256 i, i < XG: all loads are in flight together, the row's
+      // range is reduced from registers and the values are quantised from registers.  (The launcher fuses only
+      // when k is a multiple of 8, rows are 16-byte aligned and k <= 2048 * XG; otherwise it runs phase 0 itself.)
+      // No branch goes around a load (groups past the row read its first group again): the compiler then knows how
+      // many younger loads there are and waits for the row alone, not for the weights requested after it.
       const uint32_t groups = p.k / 8;
-      float x[kFusedGroups][8];
+      float x[XG ? XG : 1][8];
       float mn = 3.40282347e38f, mx = -3.40282347e38f;
 #pragma unroll
-      for (int i = 0; i < kFusedGroups; ++i) {
+      for (int i = 0; i < XG; ++i) {
         const uint32_t g = tid + 256 * i;
-        if (g < groups) load8_f32<T>(row + g * 8 * item, x[i]);
+        load8_f32<T>(row + uint64_t(g < groups ? g : 0) * 8 * item, x[i]);
       }
       if (r == 0) request_round(0);
 #pragma unroll
-      for (int i = 0; i < kFusedGroups; ++i) {
-        if (uint32_t(tid + 256 * i) < groups) {
+      for (int i = 0; i < XG; ++i) {
+        const bool inside = uint32_t(tid + 256 * i) < groups;
 #pragma unroll
-          for (int e = 0; e < 8; ++e) mn = fminf(mn, x[i][e]), mx = fmaxf(mx, x[i][e]);
-        }
+        for (int e = 0; e < 8; ++e) mn = fminf(mn, inside ? x[i][e] : mn), mx = fmaxf(mx, inside ? x[i][e] : mx);
       }
       block_range(&mn, &mx);
       const RowQuant rq = row_quant(mn, mx, groupwise != 0);
       nzp8[r] = 8 - rq.izp;
       recip[r] = rq.recip;
 #pragma unroll
-      for (int i = 0; i < kFusedGroups; ++i) {
+      for (int i = 0; i < XG; ++i) {
         const uint32_t g = tid + 256 * i;
         if (g < L.kpad / 8) {
           uint32_t hi = 0, lo = 0x88888888u;  // beyond k: value 0 = planes (0, 0 - 8)
@@ -443,6 +447,21 @@ __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L
     const uint32_t unit0 = round * kRoundUnits + part * kUnitsPerLane;
     const uint8_t* qbase = q_lds + unit0 * kUnit + unit0 / 8 * 16;
 
+    // With one row the round's activation planes are read from LDS into registers before the first weight is
+    // touched: the reads then wait under the weights' flight time, not between the products (measured per workgroup at
+    // one row: products 0.75 us after the weights' arrival with a pair of reads in front of every unit's products).
+    constexpr bool PRELOAD = MR == 1;
+    U4 qreg[PRELOAD ? MR : 1][kUnitsPerLane][2];
+    if constexpr (PRELOAD) {
+#pragma unroll
+      for (int r = 0; r < MR; ++r)
+#pragma unroll
+        for (int j = 0; j < kUnitsPerLane; ++j) {
+          qreg[r][j][0] = *reinterpret_cast<const U4*>(qbase + r * qs + j * kUnit);
+          qreg[r][j][1] = *reinterpret_cast<const U4*>(qbase + r * qs + j * kUnit + 16);
+        }
+      __builtin_amdgcn_sched_barrier(0);  // (the scheduler would move each read down to its first use)
+    }
     float t[MR][BPL];
 #pragma unroll
     for (int jb = 0; jb < BPL; ++jb) {
@@ -460,8 +479,8 @@ __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L
         }
 #pragma unroll
         for (int r = 0; r < MR; ++r) {
-          const U4 qh = *reinterpret_cast<const U4*>(qbase + r * qs + j * kUnit);
-          const U4 ql = *reinterpret_cast<const U4*>(qbase + r * qs + j * kUnit + 16);
+          const U4 qh = PRELOAD ? qreg[PRELOAD ? r : 0][j][0] : *reinterpret_cast<const U4*>(qbase + r * qs + j * kUnit);
+          const U4 ql = PRELOAD ? qreg[PRELOAD ? r : 0][j][1] : *reinterpret_cast<const U4*>(qbase + r * qs + j * kUnit + 16);
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
             da[r] = __builtin_amdgcn_sdot8(int(qh[d]), int(ws[d]), da[r], false);
@@ -505,13 +524,24 @@ __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L
         // (thread (grp, col) of the first wave owns row grp, column col; its sum lives in acc[0])
         const float* from = terms + (grp * kTileCols + col) * kTermPitch;
         float a = round == 0 ? -0.0f : acc[0];
+        // The terms are read 16 reads at a time, all before the first addition of their batch: the additions are a
+        // chain of dependent operations, and with a read in front of every few of them the chain waits for LDS at
+        // every step (0.75 us per round; batches keep the kernel at three waves per SIMD).
+        constexpr int BATCH = 4 * BPL < 16 ? 4 * BPL : 16;
 #pragma unroll
-        for (int b = 0; b < 16 * BPL; b += 4) {
-          const F4 v = *reinterpret_cast<const F4*>(from + b);
-          a = a + v.x;
-          a = a + v.y;
-          a = a + v.z;
-          a = a + v.w;
+        for (int b0 = 0; b0 < 4 * BPL; b0 += BATCH) {
+          F4 v[BATCH];
+#pragma unroll
+          for (int b = 0; b < BATCH; ++b) v[b] = *reinterpret_cast<const F4*>(from + 4 * (b0 + b));
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int b = 0; b < BATCH; ++b) {
+            a = a + v[b].x;
+            a = a + v[b].y;
+            a = a + v[b].z;
+            a = a + v[b].w;
+          }
+          __builtin_amdgcn_sched_barrier(0);
         }
         acc[0] = a;
       }
@@ -531,14 +561,12 @@ __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L
   }
   if constexpr (UPB != 0) {
     if (wave == 0 && grp < MR && n < p.n && m0 + grp < p.m) {
-      const float bias = ldg<float>(p.compact + L.bias_off + n * 4ull);
       float rc = recip[0];
 #pragma unroll
       for (int r = 1; r < MR; ++r) rc = grp == r ? recip[r] : rc;
       finish_store<T>(p.out + (uint64_t(m0 + grp) * p.n + n) * item, acc[0], rc, p.has_bias != 0, bias);
     }
   } else if (part == 15 && n < p.n) {
-    const float bias = ldg<float>(p.compact + L.bias_off + n * 4ull);
 #pragma unroll
     for (int r = 0; r < MR; ++r)
       if (m0 + r < p.m) finish_store<T>(p.out + (uint64_t(m0 + r) * p.n + n) * item, acc[r], recip[r], p.has_bias != 0, bias);
@@ -1111,10 +1139,10 @@ bool check_q4_shape(uint32_t m, uint32_t n, uint32_t k, uint32_t bs, std::string
   return true;
 }
 
-template <class T, int MR, int UPB, bool FUSED>
+template <class T, int MR, int UPB, int XG>
 int launch_stream_one(const Q4CParams& p, const CompactLayout& L, uint32_t m0, uint32_t groupwise, hipStream_t stream,
                       std::string* err) {
-  auto kernel = qmm4c_stream<T, MR, UPB, FUSED>;
+  auto kernel = qmm4c_stream<T, MR, UPB, XG>;
   const uint32_t lds = q_lds_bytes(MR, L.kpad);
   static uint32_t reserved = 48 * 1024;  // guarded by the runtime's stream mutex
   if (lds > reserved) {
@@ -1130,22 +1158,22 @@ int launch_stream_one(const Q4CParams& p, const CompactLayout& L, uint32_t m0, u
   return 0;
 }
 
-template <class T, int MR, bool FUSED>
+template <class T, int MR, int XG>
 int launch_stream_upb(const Q4CParams& p, const CompactLayout& L, uint32_t m0, uint32_t groupwise, hipStream_t stream,
                       std::string* err) {
   switch (L.upb) {
-    case 0: return launch_stream_one<T, MR, 0, FUSED>(p, L, m0, groupwise, stream, err);
-    case 1: return launch_stream_one<T, MR, 1, FUSED>(p, L, m0, groupwise, stream, err);
-    case 2: return launch_stream_one<T, MR, 2, FUSED>(p, L, m0, groupwise, stream, err);
-    case 4: return launch_stream_one<T, MR, 4, FUSED>(p, L, m0, groupwise, stream, err);
-    case 8: return launch_stream_one<T, MR, 8, FUSED>(p, L, m0, groupwise, stream, err);
+    case 0: return launch_stream_one<T, MR, 0, XG>(p, L, m0, groupwise, stream, err);
+    case 1: return launch_stream_one<T, MR, 1, XG>(p, L, m0, groupwise, stream, err);
+    case 2: return launch_stream_one<T, MR, 2, XG>(p, L, m0, groupwise, stream, err);
+    case 4: return launch_stream_one<T, MR, 4, XG>(p, L, m0, groupwise, stream, err);
+    case 8: return launch_stream_one<T, MR, 8, XG>(p, L, m0, groupwise, stream, err);
   }
   *err = "qmm4c: bad layout";
   return -1;
 }
 
 // Rows in groups of at most 4 (fewer when the activations of 4 rows would not fit in LDS).
-template <class T, bool FUSED>
+template <class T, int XG>
 int launch_stream_rows(const Q4CParams& p, const CompactLayout& L, uint32_t groupwise, hipStream_t stream,
                        std::string* err) {
   uint32_t per = 4;
@@ -1157,10 +1185,10 @@ int launch_stream_rows(const Q4CParams& p, const CompactLayout& L, uint32_t grou
   for (uint32_t m0 = 0; m0 < p.m; m0 += per) {
     const uint32_t rows = p.m - m0 < per ? p.m - m0 : per;
     int rc;
-    if (rows >= 4) rc = launch_stream_upb<T, 4, FUSED>(p, L, m0, groupwise, stream, err);
-    else if (rows == 3) rc = launch_stream_upb<T, 3, FUSED>(p, L, m0, groupwise, stream, err);
-    else if (rows == 2) rc = launch_stream_upb<T, 2, FUSED>(p, L, m0, groupwise, stream, err);
-    else rc = launch_stream_upb<T, 1, FUSED>(p, L, m0, groupwise, stream, err);
+    if (rows >= 4) rc = launch_stream_upb<T, 4, XG>(p, L, m0, groupwise, stream, err);
+    else if (rows == 3) rc = launch_stream_upb<T, 3, XG>(p, L, m0, groupwise, stream, err);
+    else if (rows == 2) rc = launch_stream_upb<T, 2, XG>(p, L, m0, groupwise, stream, err);
+    else rc = launch_stream_upb<T, 1, XG>(p, L, m0, groupwise, stream, err);
     if (rc != 0) return rc;
   }
   return 0;
@@ -1365,8 +1393,8 @@ int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwi
       *err = "qmm4c: null or unaligned side-car address";
       return -1;
     }
-    const int rc = dtype == VKT_F32 ? launch_stream_rows<f32_t, false>(p, L, groupwise, stream, err)
-                                    : launch_stream_rows<bf16_t, false>(p, L, groupwise, stream, err);
+    const int rc = dtype == VKT_F32 ? launch_stream_rows<f32_t, 0>(p, L, groupwise, stream, err)
+                                    : launch_stream_rows<bf16_t, 0>(p, L, groupwise, stream, err);
     if (rc != 0) return rc;
   } else if (phase == 2) {
     // both phases in one launch per group of rows when the rows can be quantised from
@@ -1382,8 +1410,12 @@ int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwi
       if (rc == 0) rc = launch_qmm4c(p, dtype, 1, groupwise, 0, mc, stream, err);
       return rc;
     }
-    const int rc = dtype == VKT_F32 ? launch_stream_rows<f32_t, true>(p, L, groupwise, stream, err)
-                                    : launch_stream_rows<bf16_t, true>(p, L, groupwise, stream, err);
+    // (a thread quantises 2 groups of 8 activations where that covers the row, else up to kFusedGroups)
+    const bool few = p.k <= 4096;
+    const int rc = dtype == VKT_F32 ? (few ? launch_stream_rows<f32_t, 2>(p, L, groupwise, stream, err)
+                                           : launch_stream_rows<f32_t, kFusedGroups>(p, L, groupwise, stream, err))
+                                    : (few ? launch_stream_rows<bf16_t, 2>(p, L, groupwise, stream, err)
+                                           : launch_stream_rows<bf16_t, kFusedGroups>(p, L, groupwise, stream, err));
     if (rc != 0) return rc;
   } else {
     *err = "qmm4c: PHASE must be 0, 1 or 2";

@@ -151,6 +151,196 @@ __global__ __launch_bounds__(256) void qmm8_gemv(Q8Params p) {
   }
 }
 
+// One activation row (the decode case): a persistent grid streams the weights.  A few workgroups per compute unit are
+// launched (sixteen waves per unit, each with 4-8 KiB of weight loads in flight, saturate the memory system; thousands
+// of short-lived workgroups pay for their launch, their ramp and their epilogue's dependent loads one after the other),
+// and the waves walk through the weight rows in a fixed round-robin order.  A row is cut into chunks of 1 KiB (a
+// wave's 16-byte load); KS waves of a workgroup (a team) share a row, wave ks taking chunks ks, ks + KS, ..., at most
+// CH of them, and a team handles R rows per iteration.  What a lane needs of the activation row (CH x 16 values) stays
+// in its registers for the whole kernel: the row is staged once per workgroup through LDS, requested before the first
+// weights.  With KS > 1 the waves' sums meet in LDS (one barrier per iteration; all waves of a workgroup make the same
+// number of iterations).
+template <class T, int CH, int KS, int R>
+__global__ __launch_bounds__(256) void qmm8_stream(Q8Params p) {
+  constexpr int TEAMS = 4 / KS;
+  constexpr bool F32 = T::dtype == VKT_F32;
+  constexpr uint32_t item = sizeof(typename T::storage);
+  extern __shared__ __attribute__((aligned(16))) uint8_t x_lds[];
+  __shared__ float part[2][4][R];
+  // (the wave's number as a scalar: row numbers and row addresses are then scalars too, and the loads take a scalar
+  // base plus the lane's offset instead of per-lane 64-bit address arithmetic)
+  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t team = wave / KS, ks = wave % KS;
+  const uint32_t chunks = (p.k + 1023) / 1024;
+  // Row groups of R rows; a workgroup takes TEAMS neighbouring groups at a time (one per team), round-robin over the
+  // grid, so that all its waves make the same number of iterations (the barriers below match).
+  const uint32_t groups = (p.n + R - 1) / R, supers = (groups + TEAMS - 1) / TEAMS;
+  if (blockIdx.x >= supers) return;  // (the whole workgroup, before any barrier)
+  const uint32_t mine = (supers - blockIdx.x + gridDim.x - 1) / gridDim.x;
+  auto group_of = [&](uint32_t i) { return (blockIdx.x + i * gridDim.x) * TEAMS + team; };
+
+  // the activation row: global -> LDS (once per workgroup) -> this lane's CH x 16 values.  Requested before the
+  // first weights (loads return in the order issued, and the row, which comes from L2, is needed first).
+  const uint32_t x_pieces = p.k * item / 16;  // (k is a multiple of 16: whole pieces)
+  constexpr int XP = (CH * KS * int(item) + 3) / 4;  // pieces per thread: k <= CH * KS * 1024
+  U4 staged[XP];
+#pragma unroll
+  for (int i = 0; i < XP; ++i) {
+    // (no branch around a load: the compiler would wait for it on the spot; pieces past the row read its start)
+    const uint32_t piece = tid + 256 * i;
+    staged[i] = ldg<U4>(p.a + uint64_t(piece < x_pieces ? piece : 0) * 16);
+  }
+  __builtin_amdgcn_sched_barrier(0);  // (the scheduler would put the weights' loads first)
+
+  uint32_t chunk_at[CH];  // byte offset of this lane's 16 bytes within a weight row, per chunk (0 past k)
+  bool chunk_ok[CH];
+#pragma unroll
+  for (int j = 0; j < CH; ++j) {
+    const uint32_t c = ks + KS * j, at = c * 1024 + lane * 16;
+    chunk_ok[j] = c < chunks && at < p.k;
+    chunk_at[j] = chunk_ok[j] ? at : 0;
+  }
+  // (rows past n: the last row again, not stored)
+  auto request = [&](U4 (&w)[R][CH], float* scale, uint32_t g) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const uint32_t n = g * R + r < p.n ? g * R + r : p.n - 1;
+      const VKT_GLOBAL uint8_t* row = reinterpret_cast<const VKT_GLOBAL uint8_t*>(p.b + uint64_t(n) * p.k);
+#pragma unroll
+      for (int j = 0; j < CH; ++j) w[r][j] = __builtin_nontemporal_load(reinterpret_cast<const VKT_GLOBAL U4*>(row + chunk_at[j]));
+    }
+    // lane r of the team's first wave finishes row r: its scale comes with the weights, not after the sums
+    const uint32_t n = g * R + (lane < uint32_t(R) ? lane : 0);
+    *scale = load_f32<T>(p.scales + uint64_t(n < p.n ? n : p.n - 1) * item);
+  };
+  U4 cur[R][CH];
+  float cur_scale;
+  request(cur, &cur_scale, group_of(0));
+
+#pragma unroll
+  for (int i = 0; i < XP; ++i) {
+    const uint32_t piece = tid + 256 * i;
+    if (piece < x_pieces) *reinterpret_cast<U4*>(x_lds + piece * 16) = staged[i];
+  }
+  __syncthreads();
+  // values of k beyond the row are zeros (their weights are read from the row's start)
+  float xf[F32 ? CH : 1][16];
+  U4 xh[F32 ? 1 : CH][2];
+#pragma unroll
+  for (int j = 0; j < CH; ++j) {
+    const uint32_t at = (ks + KS * j) * 1024 + lane * 16;  // first value of k
+    if constexpr (F32) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const F4 v = chunk_ok[j] ? *reinterpret_cast<const F4*>(x_lds + (at + 4 * q) * 4) : F4{0.0f, 0.0f, 0.0f, 0.0f};
+        xf[j][4 * q] = v.x, xf[j][4 * q + 1] = v.y, xf[j][4 * q + 2] = v.z, xf[j][4 * q + 3] = v.w;
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < 2; ++q) xh[j][q] = chunk_ok[j] ? *reinterpret_cast<const U4*>(x_lds + (at + 8 * q) * 2) : U4{0, 0, 0, 0};
+    }
+  }
+
+  // one group: products, sums over the wave, over the team's waves, scale, store
+  auto finish = [&](const U4 (&w)[R][CH], float scale, uint32_t g, uint32_t i) {
+    float sum[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      // (two chains of dependent multiply-adds per chunk: one chain leaves the vector unit waiting for its own results)
+      float acc[CH][2];
+#pragma unroll
+      for (int j = 0; j < CH; ++j) {
+        acc[j][0] = acc[j][1] = 0.0f;
+        if constexpr (F32) {
+          float v[16];
+          widen16_i8(w[r][j], v);
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[j][e & 1] = fmaf(xf[j][e], v[e], acc[j][e & 1]);
+        } else {
+          U4 lo, hi;
+          widen16_to_operands<T>(w[r][j], &lo, &hi);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[j][0] = dot2<T>(xh[j][0][e], lo[e], acc[j][0]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[j][1] = dot2<T>(xh[j][1][e], hi[e], acc[j][1]);
+        }
+      }
+      float row = 0.0f;
+#pragma unroll
+      for (int j = 0; j < CH; ++j) row += acc[j][0] + acc[j][1];
+      sum[r] = wave_sum(row);
+    }
+    float total = 0.0f;
+    if constexpr (KS > 1) {
+      if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) part[i & 1][wave][r] = sum[r];
+      }
+      __syncthreads();  // (one per iteration: the next iteration writes the other half of `part`)
+      if (ks == 0 && lane < uint32_t(R)) {
+        total = part[i & 1][wave][lane];
+#pragma unroll
+        for (int q = 1; q < KS; ++q) total += part[i & 1][wave + q][lane];
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < R; ++r) total = lane == uint32_t(r) ? sum[r] : total;
+    }
+    const uint32_t n = g * R + lane;
+    if (ks == 0 && lane < uint32_t(R) && n < p.n) store_f32<T>(p.c + uint64_t(n) * item, total * scale);
+  };
+
+  // No software prefetch: the waves of a SIMD, each with its own group's loads in flight, cover each other's waits.
+  // (A second register set filled an iteration ahead was tried in three forms: the compiler's waits for it came out as
+  // waits for everything in flight.  So was one more pass through the products' code on zeros while the first loads
+  // are on their way: a launch starts with a cold instruction cache, and a wave's first run through straight-line code
+  // is held up at every 64-byte line of it, measured at ~40 ns a line; the register copies that form needed made it
+  // wait for the loads all the same.)
+  // (one copy of the products' code: every line of it that a launch runs through for the first time costs it time)
+#pragma clang loop unroll(disable)
+  for (uint32_t i = 0; i < mine; ++i) {
+    if (i != 0) request(cur, &cur_scale, group_of(i));
+    finish(cur, cur_scale, group_of(i), i);
+  }
+}
+
+// One row through qmm8_stream where it applies (k up to 16384, 16-byte aligned rows).  variant bits 8-11 override
+// the workgroups per compute unit, bits 12-15 the rows per iteration (tuning).  False: not this kernel's shape.
+template <class T>
+bool launch_stream(const Q8Params& p, uint32_t variant, const Machine& mc, hipStream_t stream) {
+  const uint32_t chunks = (p.k + 1023) / 1024;
+  if (p.m != 1 || chunks > 16 || p.k == 0) return false;
+  const int ks = chunks <= 4 ? 1 : chunks <= 8 ? 2 : 4, ch = int((chunks + ks - 1) / ks);
+  // rows per team and iteration: 8 KiB of weights in flight per wave (6 KiB with three chunks per row)
+  const uint32_t teams = 4 / ks, per_cu = (variant >> 8) & 0xf ? (variant >> 8) & 0xf : 2;
+  uint32_t rows_per = ch == 1 ? 8 : ch == 2 ? 4 : 2;
+  if ((variant >> 12) & 0xf) rows_per = (variant >> 12) & 0xf;  // (tuning)
+  const uint32_t groups = (p.n + rows_per - 1) / rows_per;
+  uint32_t grid = uint32_t(mc.compute_units) * per_cu;
+  if (grid * teams > groups) grid = (groups + teams - 1) / teams;
+  const uint32_t lds = (p.k * sizeof(typename T::storage) + 15) / 16 * 16;
+#define VKT_STREAM_CASE(CH_, KS_, R_)                                                                          \
+  if (ch == CH_ && ks == KS_ && rows_per == R_) {                                                              \
+    auto kernel = qmm8_stream<T, CH_, KS_, R_>;                                                                \
+    static bool configured = false; /* guarded by the runtime's stream mutex */                                \
+    if (!configured) {                                                                                         \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024) != hipSuccess) { \
+        (void)hipGetLastError();                                                                               \
+        return false;                                                                                          \
+      }                                                                                                        \
+      configured = true;                                                                                       \
+    }                                                                                                          \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds, stream, p);                                         \
+    return true;                                                                                               \
+  }
+  VKT_STREAM_CASE(1, 1, 8) VKT_STREAM_CASE(2, 1, 4) VKT_STREAM_CASE(3, 1, 2) VKT_STREAM_CASE(4, 1, 2)
+  VKT_STREAM_CASE(1, 1, 4) VKT_STREAM_CASE(2, 1, 2) VKT_STREAM_CASE(3, 1, 1) VKT_STREAM_CASE(4, 1, 1)
+  VKT_STREAM_CASE(3, 2, 2) VKT_STREAM_CASE(4, 2, 2) VKT_STREAM_CASE(3, 4, 2) VKT_STREAM_CASE(4, 4, 2)
+  VKT_STREAM_CASE(3, 2, 1) VKT_STREAM_CASE(4, 2, 1) VKT_STREAM_CASE(3, 4, 1) VKT_STREAM_CASE(4, 4, 1)
+#undef VKT_STREAM_CASE
+  return false;
+}
+
 // Any shape: a wave per output column, lanes strided along k with element loads, rows of
 // A in chunks of 8.
 template <class T>
@@ -951,6 +1141,13 @@ int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipSt
       return 0;
     }
   }
+  // One row of float32 activations: the persistent streaming kernel (measured at K = N = 4096: 4.85 us against 5.8; a
+  // workgroup of the other kernel reads 4 KiB of activations per 2 KiB of weights).  With 16-bit activations the two
+  // are level at every shape tried (K = 4096 ... 14336, N = 4096 ... 14336) and the other one stays.  variant bit 23
+  // keeps the other kernel; bits 8-15 (with bits 0-7 clear) ask for this one whatever the type (tests, tuning).
+  if (p0.m == 1 && !(variant & 0xff) && !((variant >> 23) & 1) && !((variant >> 17) & 1) &&
+      (T::dtype == VKT_F32 || ((variant >> 8) & 0xff)) && launch_stream<T>(p0, variant, mc, stream))
+    return 0;
   for (uint32_t r0 = 0; r0 < p0.m; r0 += 16) {
     Q8Params p = p0;
     p.m = p0.m - r0 < 16 ? p0.m - r0 : 16;
