@@ -111,33 +111,75 @@ def test_scaled_mm_golden_fixtures():
         assert (np.abs(oracle.to_f32(got, odt) - want) <= tol).all(), key
 
 
-def _sampled_check(a, bt, sa, sb, got, rows, cols, rowwise):
-    """Float64 closed form on a sample of output rows and columns."""
-    af = oracle.fp8_table(oracle.E4M3)[a[rows]].astype(np.float64)
-    bf = oracle.fp8_table(oracle.E4M3)[bt[cols]].astype(np.float64)
-    sa_ = sa.reshape(-1)[rows][:, None] if rowwise else float(sa)
-    sb_ = sb.reshape(-1)[cols][None, :] if rowwise else float(sb)
-    truth = (af @ bf.T) * sa_ * sb_
-    mag = (np.abs(af) @ np.abs(bf).T) * sa_ * sb_
-    sub = oracle.bf16_to_f32(got[np.ix_(rows, cols)]).astype(np.float64)
-    assert (np.abs(sub - truth) <= ref_tol(truth, mag, oracle.BF16) + HW_WINDOW * mag).all()
-    assert np.allclose(sub, truth, rtol=1e-2, atol=1e-2)  # the stated bar for bfloat16 outputs
+def _closed_form(a_rows, bt_rows, sa_rows, sb_cols):
+    """(float64 sum, magnitude sum) of rows of A against rows of B^T, scaled."""
+    af = oracle.fp8_table(oracle.E4M3)[a_rows].astype(np.float64)
+    bf = oracle.fp8_table(oracle.E4M3)[bt_rows].astype(np.float64)
+    scale = np.asarray(sa_rows, np.float64).reshape(-1, 1) * np.asarray(sb_cols, np.float64).reshape(1, -1)
+    return (af @ bf.T) * scale, (np.abs(af) @ np.abs(bf).T) * scale
+
+
+def _stripes_check(a, bt, sa, sb, got, rows, cols, rowwise):
+    """Whole output rows `rows` (every column) and whole output columns `cols` (every row) against the float64
+    closed form: stripes that cross every tile, wave and epilogue-pass boundary of the kernel, so that a tile, wave
+    or pass written to the wrong place cannot hide between sampled points."""
+    m, n = a.shape[0], bt.shape[0]
+    sa_all = sa.reshape(-1) if rowwise else np.full(m, float(sa))
+    sb_all = sb.reshape(-1) if rowwise else np.full(n, float(sb))
+
+    def check(sub, truth, mag):
+        sub = oracle.bf16_to_f32(sub).astype(np.float64)
+        assert (np.abs(sub - truth) <= ref_tol(truth, mag, oracle.BF16) + HW_WINDOW * mag).all()
+        assert np.allclose(sub, truth, rtol=1e-2, atol=1e-2)  # the stated bar for bfloat16 outputs
+
+    for c0 in range(0, n, 4096):  # (columns in pieces: the float64 operand of a piece is 256 MB)
+        truth, mag = _closed_form(a[rows], bt[c0:c0 + 4096], sa_all[rows], sb_all[c0:c0 + 4096])
+        check(got[rows][:, c0:c0 + 4096], truth, mag)
+    for r0 in range(0, m, 4096):
+        truth, mag = _closed_form(a[r0:r0 + 4096], bt[cols], sa_all[r0:r0 + 4096], sb_all[cols])
+        check(got[r0:r0 + 4096][:, cols], truth, mag)
+
+
+# rows / columns either side of every boundary of the 256 x 256 tile kernel: its waves' 64 x 128 sub-tiles, the
+# matrix-core tiles of 32, the epilogue's passes of 64 columns, tile edges, panel edges (8 tile rows), the last ones
+BOUNDARY_ROWS = [0, 31, 32, 63, 64, 255, 256, 2047, 2048]
+BOUNDARY_COLS = [0, 3, 4, 63, 64, 127, 128, 255, 256, 1023]
 
 
 def test_scaled_mm_config4_8192_cubed():
-    """BASELINE config 4: e4m3fn 8192^3, per-tensor scales 0.5 / 0.5, bf16 out.  A full CPU
-    product takes an hour, so: sampled rows/columns against the float64 closed form, and
-    exactness properties (scaling an operand by 2 doubles every output bit for bit)."""
+    """BASELINE config 4: e4m3fn 8192^3, per-tensor scales 0.5 / 0.5, bf16 out.  A full CPU product takes an hour,
+    so: whole rows and whole columns across every kernel boundary against the float64 closed form, and an exactness
+    property over the whole output (scaling an operand by 2 doubles every output bit for bit)."""
     import _dev
     m = n = k = 8192
     a = torch.randn(m, k, generator=gen(1040)).clamp(-448, 448).to(torch.float8_e4m3fn)
     bt = torch.randn(n, k, generator=gen(1041)).clamp(-448, 448).to(torch.float8_e4m3fn)
     got = _dev.scaled_mm(bits(a), oracle.E4M3, bits(bt), oracle.E4M3, [0.5], [0.5], False, out_dtype=oracle.BF16)
-    rows = np.array([0, 1, 17, 255, 256, 4095, 4096, 8191])
-    cols = np.array([0, 3, 64, 127, 128, 5000, 8190, 8191])
-    _sampled_check(bits(a), bits(bt), np.float32(0.5), np.float32(0.5), got, rows, cols, False)
+    _stripes_check(bits(a), bits(bt), np.float32(0.5), np.float32(0.5), got, np.array(BOUNDARY_ROWS + [4095, 4096, m - 1]),
+                   np.array(BOUNDARY_COLS + [5000, n - 2, n - 1]), False)
     got2 = _dev.scaled_mm(bits(a), oracle.E4M3, bits(bt), oracle.E4M3, [1.0], [0.5], False, out_dtype=oracle.BF16)
     assert np.array_equal(oracle.bf16_to_f32(got2), oracle.bf16_to_f32(got) * 2)
+
+
+@pytest.mark.parametrize("variant,out_dtype", [(8, oracle.BF16), (5, oracle.BF16), (9, oracle.F32), (6, oracle.F32)])
+def test_scaled_mm_large_tile_kernels_on_ragged_shapes(variant, out_dtype):
+    """The 256 x 256 tile kernels (8 waves of 64 x 128 and 4 waves of 128 x 128; fp8 matrix cores and the widened,
+    exact form) forced at a shape whose rows and columns are no multiple of any tile, wave or pass size: every output
+    against the oracle."""
+    import _dev
+    m, k, n = 300, 1024, 520
+    a = torch.randn(m, k, generator=gen(1070)).to(torch.float8_e4m3fn)
+    bt = torch.randn(n, k, generator=gen(1071)).to(torch.float8_e4m3fn)
+    sa = torch.empty(m, 1).uniform_(0.5, 2, generator=gen(1072)).numpy()
+    sb = torch.empty(1, n).uniform_(0.5, 2, generator=gen(1073)).numpy()
+    bias = torch.randn(n, generator=gen(1074)).numpy()
+    got = _dev.scaled_mm(bits(a), oracle.E4M3, bits(bt), oracle.E4M3, sa, sb, True, bias=bias, bias_dtype=oracle.F32,
+                         out_dtype=out_dtype, variant=variant)
+    want, mag = oracle.scaled_mm(bits(a), oracle.E4M3, bits(bt), oracle.E4M3, sa, sb, True, bias, oracle.F32, None, out_dtype,
+                                 want_mag=True)
+    want = oracle.to_f32(want, out_dtype).astype(np.float64)
+    tol = ref_tol(want, mag, out_dtype) + (HW_WINDOW * mag if out_dtype == oracle.BF16 else 0)
+    assert got.shape == (m, n) and (np.abs(oracle.to_f32(got, out_dtype) - want) <= tol).all()
 
 
 @pytest.mark.parametrize("fa,fb", [(FLOAT8[0], FLOAT8[0]), (FLOAT8[1], FLOAT8[0]), (FLOAT8[1], FLOAT8[1])])
@@ -171,9 +213,8 @@ def test_scaled_mm_config5_rowwise_70b():
     sa = torch.empty(m, 1).uniform_(0.5, 2, generator=gen(1052)).numpy()
     sb = torch.empty(1, n).uniform_(0.5, 2, generator=gen(1053)).numpy()
     got = _dev.scaled_mm(bits(a), oracle.E4M3, bits(bt), oracle.E4M3, sa, sb, True, out_dtype=oracle.BF16)
-    rows = np.array([0, 255, 256, 2047, 4095])
-    cols = np.array([0, 127, 128, 14336, 28671, 28670])
-    _sampled_check(bits(a), bits(bt), sa, sb, got, rows, cols, True)
+    _stripes_check(bits(a), bits(bt), sa, sb, got, np.array(BOUNDARY_ROWS + [m - 1]),
+                   np.array(BOUNDARY_COLS + [14335, 14336, n - 256, n - 1]), True)
 
 
 def test_scaled_mm_errors():

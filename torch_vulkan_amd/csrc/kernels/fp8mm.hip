@@ -118,6 +118,28 @@ struct F8Problem : F8Params {
         if (col + r < n) store_out(*this, index + r, v[r]);
     }
   }
+  // the epilogue that stores straight from the accumulators: bfloat16 outputs, 16-byte aligned rows
+  static constexpr bool kRegisterEpilogue = true;
+  __device__ __forceinline__ bool register_epilogue(const Whole&) const {
+    return out_dtype == VKT_BF16 && (ldo & 7u) == 0 && (out & 15u) == 0;
+  }
+  __device__ __forceinline__ float row_scale(uint32_t row, const Whole& w) const {
+    return rowwise ? ldg<float>(scale_a + 4ull * row) : w.sa_all;
+  }
+  // scale and bias of columns col .. col + 3 (all inside n)
+  __device__ __forceinline__ void column_terms(uint32_t col, const Whole& w, float (&s)[4], float (&b)[4]) const {
+    if (rowwise) {
+      const F4 v = ldg<F4>(scale_b + 4ull * col);
+      s[0] = v.x, s[1] = v.y, s[2] = v.z, s[3] = v.w;
+    } else {
+      s[0] = s[1] = s[2] = s[3] = w.sb_all;
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) b[r] = bias ? load_any_f32(bias, col + r, bias_dtype) : 0.0f;
+  }
+  __device__ __forceinline__ void store_bf16x8(uint32_t, uint32_t row, uint32_t col, const U4& v) const {
+    stg<U4>(out + (uint64_t(row) * ldo + col) * 2, v);
+  }
   template <class F>
   __device__ __forceinline__ void for_output_type(bool full, const Whole& w, F&& f) const {
     if (w.vec_ok && full) {

@@ -23,6 +23,7 @@ __device__ __forceinline__ float slot_float(uint64_t slot) { return bits_f32(uin
 template <class T, bool TRA = false, bool TRB = false>
 struct GemmProblem {
   static constexpr bool kTransA = TRA, kTransB = TRB;
+  static constexpr bool kRegisterEpilogue = false;
   // operands as the tile kernel takes them (bytes)
   uint64_t a, b;
   uint32_t m, n, k, lda, ldb, batches;
@@ -153,6 +154,7 @@ int launch_gemm16_t(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint3
 template <class T>
 struct Q8GemmProblem {
   static constexpr bool kTransA = false, kTransB = false;
+  static constexpr bool kRegisterEpilogue = false;
   uint64_t a, b;
   uint32_t m, n, k, lda, ldb, batches;
   uint64_t a_batch, b_batch;

@@ -9,6 +9,9 @@
 //   columns(batch, n, whole)             per-lane constants of columns n .. n + 3
 //   store<DT>(batch, m, n, t, cols, whole)   finish and store 4 outputs of row m
 //   for_output_type(full, whole, f)      call f(integral_constant<int, DT>) for the output type
+//   kRegisterEpilogue                    the problem also offers the epilogue that stores straight from the accumulators:
+//     register_epilogue(whole)             whether this launch takes it (bfloat16 output, aligned)
+//     row_scale(m, whole), column_terms(n, whole, scale[4], bias[4])   what an output needs: acc * row_scale * scale[c] + bias[c]
 //   kTransA, kTransB                     16-bit operands only: the operand is stored k-major, i.e.
 //                                        as [k, m] (or [k, n]) rows lda (ldb) bytes apart, contiguous
 //                                        along m (n); m (n) a multiple of 8, k of 64 values
@@ -403,7 +406,52 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void mma_tile(P p, uint32_t 
     for (; s < steps; ++s) step(s, std::false_type{});
   }
 
-  // Epilogue.  A lane holds out[m = .. + l16][n = .. + 4 g + r], r = 0..3, for each of its
+  const auto whole = p.whole();  // what the epilogue needs once per launch
+  const uint32_t wm0 = m0 + wm * TM * 16, wn0 = n0 + wn * TN * 16;
+  // Epilogue from the registers (bfloat16 outputs of whole tiles): no LDS, no barrier, so nothing holds a wave back
+  // once its last matrix-core instruction has gone, and the next tile's first loads may land in LDS meanwhile.  A 32 x 32
+  // matrix-core tile leaves lane l with row l % 32 and, for q = 0..3, columns 8 q + 4 (l / 32) .. + 3: two lanes 32
+  // apart hold the two halves of 8 consecutive outputs.  v_permlane32_swap puts them together (lanes below 32 take
+  // chunk q = 0 or 2 of their row, lanes from 32 chunk 1 or 3), and every lane stores 16 bytes; a store instruction
+  // of a wave writes 32 rows x 32 consecutive bytes.
+  bool from_registers = false;
+  if constexpr (MF32 && P::kRegisterEpilogue) {
+    from_registers = p.register_epilogue(whole) && n0 + BN <= p.n;  // (the same for every wave of the workgroup)
+    if (from_registers) {
+      const uint32_t l32 = lane & 31, h = lane >> 5;
+#pragma unroll
+      for (int j = 0; j < TN2; ++j) {
+        float scale[4][4], bias[4][4];  // of this lane's columns wn0 + 32 j + 8 q + 4 h + r
+#pragma unroll
+        for (int q = 0; q < 4; ++q) p.column_terms(wn0 + 32 * j + 8 * q + 4 * h, whole, scale[q], bias[q]);
+#pragma unroll
+        for (int i = 0; i < TM2; ++i) {
+          const uint32_t m = wm0 + 32 * i + l32;
+          const float rs = p.row_scale(m < p.m ? m : p.m - 1, whole);
+          const V16F& t = acc32[i][j];
+#pragma unroll
+          for (int qp = 0; qp < 2; ++qp) {
+            uint32_t lo[2], hi[2];  // chunks 2 qp and 2 qp + 1 as two bfloat16 pairs each
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+              const int q0 = 2 * qp, q1 = 2 * qp + 1;
+              lo[e] = pack_bf16(t[4 * q0 + 2 * e] * (rs * scale[q0][2 * e]) + bias[q0][2 * e],
+                                t[4 * q0 + 2 * e + 1] * (rs * scale[q0][2 * e + 1]) + bias[q0][2 * e + 1]);
+              hi[e] = pack_bf16(t[4 * q1 + 2 * e] * (rs * scale[q1][2 * e]) + bias[q1][2 * e],
+                                t[4 * q1 + 2 * e + 1] * (rs * scale[q1][2 * e + 1]) + bias[q1][2 * e + 1]);
+            }
+            // lanes 32.. of `lo` change places with lanes ..31 of `hi`
+            const auto s0 = __builtin_amdgcn_permlane32_swap(lo[0], hi[0], false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(lo[1], hi[1], false, false);
+            const uint32_t n = wn0 + 32 * j + 8 * (2 * qp + h);
+            if (m < p.m) p.store_bf16x8(batch, m, n, U4{s0[0], s1[0], s0[1], s1[1]});
+          }
+        }
+      }
+    }
+  }
+  if (!from_registers) {
+  // Epilogue through LDS.  A lane holds out[m = .. + l16][n = .. + 4 g + r], r = 0..3, for each of its
   // TM x TN tiles.  Each wave transposes its sub-tile through its own slice of LDS (the
   // operand buffers are dead by now), 64 columns at a time, so that the scale / bias / cast
   // code exists once (a loop, not TM*TN unrolled copies) and every store instruction of a
@@ -411,8 +459,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void mma_tile(P p, uint32_t 
   constexpr uint32_t EP_ROW = 256;                    // bytes: 64 float32 columns
   constexpr uint32_t EP_WAVE = TM * 16 * EP_ROW;      // bytes of LDS per wave
   float* ep = reinterpret_cast<float*>(lds + wave * EP_WAVE);
-  const auto whole = p.whole();  // what the epilogue needs once per launch
-  const uint32_t wm0 = m0 + wm * TM * 16, wn0 = n0 + wn * TN * 16;
 #pragma unroll
   for (int pass = 0; pass < TN / 4; ++pass) {
     // (the first pass may start only when every wave is done reading operands; later ones
@@ -465,6 +511,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void mma_tile(P p, uint32_t 
     p.for_output_type(n + 3 < p.n, whole, rows);
   }
   __syncthreads();  // the next tile's operands overwrite the LDS the epilogue has just read
+  }  // (epilogue through LDS)
   }  // (tile loop)
 }
 
