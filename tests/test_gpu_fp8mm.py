@@ -28,7 +28,7 @@ HW_WINDOW = 2.0**-13
 def on_matrix_cores(odt, variant, k):
     if variant in (6, 7, 255) or k % 16:
         return False
-    return variant in (1, 2, 3, 4, 5, 8) or odt in (oracle.BF16, oracle.E4M3, oracle.E5M2)
+    return variant in (1, 2, 3, 4, 5, 8, 11) or odt in (oracle.BF16, oracle.E4M3, oracle.E5M2)
 
 
 def run_case(m, k, n, fa, fb, out_dtype, rowwise, bias_dtype=None, scale_result=None, variant=0, seed=1, scale=1.0):
@@ -79,7 +79,7 @@ def test_scaled_mm_reference_cases(fa, fb, out_dtype, rowwise):
 
 @pytest.mark.parametrize("m,k,n", [(1, 16, 1), (130, 256, 70), (257, 384, 129), (64, 1040, 300), (300, 128, 520),
                                    (5, 100, 7), (33, 48, 17)])
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 255])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 11, 255])
 @pytest.mark.parametrize("rowwise", [False, True])
 def test_scaled_mm_tile_edges(m, k, n, variant, rowwise):
     """Shapes that are not multiples of any tile, K tails (K % 128 != 0, K % 16 != 0 -> the
@@ -161,7 +161,7 @@ def test_scaled_mm_config4_8192_cubed():
     assert np.array_equal(oracle.bf16_to_f32(got2), oracle.bf16_to_f32(got) * 2)
 
 
-@pytest.mark.parametrize("variant,out_dtype", [(8, oracle.BF16), (5, oracle.BF16), (9, oracle.F32), (6, oracle.F32)])
+@pytest.mark.parametrize("variant,out_dtype", [(8, oracle.BF16), (11, oracle.BF16), (5, oracle.BF16), (9, oracle.F32), (6, oracle.F32)])
 def test_scaled_mm_large_tile_kernels_on_ragged_shapes(variant, out_dtype):
     """The 256 x 256 tile kernels (8 waves of 64 x 128 and 4 waves of 128 x 128; fp8 matrix cores and the widened,
     exact form) forced at a shape whose rows and columns are no multiple of any tile, wave or pass size: every output
@@ -180,6 +180,35 @@ def test_scaled_mm_large_tile_kernels_on_ragged_shapes(variant, out_dtype):
     want = oracle.to_f32(want, out_dtype).astype(np.float64)
     tol = ref_tol(want, mag, out_dtype) + (HW_WINDOW * mag if out_dtype == oracle.BF16 else 0)
     assert got.shape == (m, n) and (np.abs(oracle.to_f32(got, out_dtype) - want) <= tol).all()
+
+
+@pytest.mark.parametrize("m,k,n,rowwise,with_bias,fb", [
+    (257, 256, 264, False, True, 0),     # the fewest steps it takes; one row and 8 columns beyond a tile
+    (1, 512, 8, False, False, 0),        # one row, 8 columns
+    (515, 640, 1032, True, True, 1),     # e5m2 second operand
+    (4352, 384, 4360, True, False, 0),   # 306 tiles: more than there are workgroups, so streams that run through two tiles
+])
+def test_scaled_mm_stream_kernel(m, k, n, rowwise, with_bias, fb):
+    """The stream kernel (variant 11: loads that run ahead across tiles, barrier in the middle of a step) forced at
+    shapes it serves: every output against the oracle, and bit for bit the tile kernel's (same products, same order)."""
+    import _dev
+    a = torch.randn(m, k, generator=gen(1080)).to(FLOAT8[0])
+    bt = torch.randn(n, k, generator=gen(1081)).to(FLOAT8[fb])
+    if rowwise:
+        sa = torch.empty(m, 1).uniform_(0.5, 2, generator=gen(1082)).numpy()
+        sb = torch.empty(1, n).uniform_(0.5, 2, generator=gen(1083)).numpy()
+    else:
+        sa, sb = np.array([0.75], dtype=np.float32), np.array([1.5], dtype=np.float32)
+    bias = torch.randn(n, generator=gen(1084)).numpy() if with_bias else None
+    kw = dict(bias=bias, bias_dtype=oracle.F32) if with_bias else {}
+    got = {v: _dev.scaled_mm(bits(a), oracle.E4M3, bits(bt), ODT[FLOAT8[fb]], sa, sb, rowwise, out_dtype=oracle.BF16, variant=v, **kw)
+           for v in (11, 8)}
+    assert got[11].shape == (m, n) and np.array_equal(got[11], got[8])
+    if m * n <= 1 << 20:
+        want, mag = oracle.scaled_mm(bits(a), oracle.E4M3, bits(bt), ODT[FLOAT8[fb]], sa, sb, rowwise, bias, oracle.F32, None, oracle.BF16,
+                                     want_mag=True)
+        want = oracle.to_f32(want, oracle.BF16).astype(np.float64)
+        assert (np.abs(oracle.to_f32(got[11], oracle.BF16) - want) <= ref_tol(want, mag, oracle.BF16) + HW_WINDOW * mag).all()
 
 
 @pytest.mark.parametrize("fa,fb", [(FLOAT8[0], FLOAT8[0]), (FLOAT8[1], FLOAT8[0]), (FLOAT8[1], FLOAT8[1])])

@@ -31,6 +31,7 @@
 //                  ends up with 4 consecutive output columns of one row (vector stores).
 //   fp8mm_generic  any shape / alignment: one thread per output, float32 FMA.
 #include "kernels.h"
+#include "mma_stream.h"
 #include "mma_tile.h"
 
 namespace vkt {
@@ -176,6 +177,15 @@ int launch_tile(const F8Params& p, int compute_units, hipStream_t stream, std::s
       problem, compute_units, stream, err, "fp8mm");
 }
 
+// The stream kernel, where it serves the problem (bfloat16 output in aligned rows); -2: it does not.
+template <int FA, int FB>
+int launch_stream(const F8Params& p, int compute_units, hipStream_t stream, std::string* err) {
+  F8Problem problem;
+  static_cast<F8Params&>(problem) = p;
+  if (p.out_dtype != VKT_BF16 || p.ldo % 8 || p.out % 16 || !mma_stream_serves(problem)) return -2;
+  return launch_mma_stream<FA, FB>(problem, compute_units, stream, err, "fp8mm");
+}
+
 template <int FA, int FB>
 int launch_formats(const F8Params& p, uint32_t variant, int compute_units, hipStream_t stream, std::string* err) {
   // variant 0: planned.  Explicit variants run the MFMA kernel whatever the output dtype
@@ -183,12 +193,12 @@ int launch_formats(const F8Params& p, uint32_t variant, int compute_units, hipSt
   // 128x128, 16x16x128); 3: 256x128; 4: 256x256 with the 32x32x64 MFMA (measured ~10 % faster
   // than 16x16x128 at equal work); 5: as 4 with global-to-LDS direct loads when k is a
   // multiple of 128 (else 4); 8: as 5 with 8 waves of 64x128 instead of 4 of 128x128 (two waves per SIMD cover each
-  // other's waits: 8192^3 2.34-2.42 -> 2.56-2.59 PFLOP/s; what large bfloat16 / float8 outputs get).  255: the
-  // one-thread-per-output kernel.
+  // other's waits: 8192^3 2.34-2.42 -> 2.56-2.59 PFLOP/s; what large float8 outputs get).  11: the stream kernel of
+  // mma_stream.h where it serves the problem (large bfloat16 outputs get it), else 8.  255: the one-thread-per-output kernel.
   // 6 / 7: the exact path (float8 widened to bfloat16 in registers, 32x32x16 bfloat16 MFMA) on
   // 256x256 / 128x128 tiles: what float32 and float16 outputs get.
   const bool big = uint64_t(p.m) * p.n >= (1ull << 20);
-  if (variant == 0) variant = (p.out_dtype == VKT_F32 || p.out_dtype == VKT_F16) ? (big ? 6 : 7) : (big ? 8 : 1);
+  if (variant == 0) variant = (p.out_dtype == VKT_F32 || p.out_dtype == VKT_F16) ? (big ? 6 : 7) : (big ? 11 : 1);
   switch (variant) {
     case 6:
       if (p.k % BK == 0) return launch_tile<2, 2, 8, 8, FA, FB, true, true, true>(p, compute_units, stream, err);
@@ -201,6 +211,11 @@ int launch_formats(const F8Params& p, uint32_t variant, int compute_units, hipSt
     case 9:  // as 6 with 8 waves of 64x128
       if (p.k % BK == 0) return launch_tile<4, 2, 4, 8, FA, FB, true, true, true>(p, compute_units, stream, err);
       return launch_tile<2, 2, 8, 4, FA, FB, true, false, true>(p, compute_units, stream, err);
+    case 11: {  // the stream kernel (mma_stream.h), else 8
+      const int rc = launch_stream<FA, FB>(p, compute_units, stream, err);
+      if (rc != -2) return rc;
+    }
+      [[fallthrough]];
     case 8:  // 256x256 tiles over 8 waves of 64x128 (two waves per SIMD), direct loads
       if (p.k % BK == 0) return launch_tile<4, 2, 4, 8, FA, FB, true, true>(p, compute_units, stream, err);
       return launch_tile<2, 2, 8, 8, FA, FB, true>(p, compute_units, stream, err);
