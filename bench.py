@@ -131,7 +131,7 @@ def rotation(nbytes, floor_mib=512):
 
 
 # ------------------------------------------------------------------ workloads
-def wl_q8(abi, m, k, n, dtype, steps, warmup, seed=1020, prefill=False):
+def wl_q8(abi, m, k, n, dtype, steps, warmup, seed=1020, prefill=False, variant=0):
     """_weight_int8pack_mm: x ~N(0,1) [m,k]; w int8 uniform [n,k]; scales ~U(0.005,0.02) [n].  prefill: many rows,
     priced against the matrix cores' bf16 rate (the weights are widened once, then one tile-kernel product)."""
     import torch
@@ -149,7 +149,7 @@ def wl_q8(abi, m, k, n, dtype, steps, warmup, seed=1020, prefill=False):
         abi.check(abi.lib().vkt_copy_on_device(b.address, copies[0].address, n * k))
         copies.append(b)
     out = abi.Buffer(m * n * item)
-    fns = [Launch(abi, "qmm8_" + abi.SUFFIX[dtype], [0],
+    fns = [Launch(abi, "qmm8_" + abi.SUFFIX[dtype], [0, variant],
                   abi.Q8Params(a=dx.address, b=c.address, scales=ds.address, c=out.address, m=m, n=n, k=k, a_sm=k,
                                a_sk=1)) for c in copies]
     work = n * k + item * (m * k + n + m * n)  # weights once + activations + scales + output
@@ -159,7 +159,8 @@ def wl_q8(abi, m, k, n, dtype, steps, warmup, seed=1020, prefill=False):
                     bytes=work, inputs=None, name=f"_weight_int8pack_mm {abi.SUFFIX[dtype]} M={m} K={k} N={n} (prefill)",
                     **timed(abi, fns, steps, max(warmup, len(fns)), resident=False))
     return dict(kind="hbm", work=work, flops=2 * m * n * k, inputs=keep,
-                name=f"_weight_int8pack_mm {abi.SUFFIX[dtype]} M={m} K={k} N={n}", **timed(abi, fns, steps, warmup))
+                name=f"_weight_int8pack_mm {abi.SUFFIX[dtype]} M={m} K={k} N={n}" + (f" (variant {variant:#x})" if variant else ""),
+                **timed(abi, fns, steps, warmup))
 
 
 def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030, prefill=False):
@@ -385,6 +386,9 @@ BASELINE = {
 OTHER = {
     "c2_prefill_m4096_k4096_n14336": lambda abi, s, w: wl_q8(abi, 4096, 4096, 14336, abi.BF16, max(s // 20, 5), max(w // 4, 3), prefill=True),
     "c3_int4_prefill_m2048": lambda abi, s, w: wl_q4(abi, 2048, 4096, 11008, 32, max(s // 10, 5), w, prefill=True),
+    "q8_f32_m64_k4096_n4096": lambda abi, s, w: wl_q8(abi, 64, 4096, 4096, abi.F32, s, w, seed=1010),
+    "q8_f32_m64_k4096_n4096_row_kernels": lambda abi, s, w: wl_q8(abi, 64, 4096, 4096, abi.F32, max(s // 4, 5), w, seed=1010, variant=1 << 22),
+    "q8_f32_m64_k14336_n4096": lambda abi, s, w: wl_q8(abi, 64, 14336, 4096, abi.F32, s, w),
     "q8_m1_k5120_n13824": lambda abi, s, w: wl_q8(abi, 1, 5120, 13824, abi.BF16, s, w, seed=1110),
     "q8_m1_k8192_n8192": lambda abi, s, w: wl_q8(abi, 1, 8192, 8192, abi.BF16, s, w, seed=1120),
     "q8_m8_k5120_n13824": lambda abi, s, w: wl_q8(abi, 8, 5120, 13824, abi.BF16, s, w, seed=1110),

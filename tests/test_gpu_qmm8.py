@@ -112,6 +112,45 @@ def test_qmm8_tile_kernel(dtype, variant, m, k, n):
         check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=variant, row_step=2), a, b, s, dtype, rows=slice(None, None, 2))
 
 
+@pytest.mark.parametrize("variant", [0, 1 << 21 | 1 << 24, 1 << 21 | 3 << 24, 1 << 22])
+@pytest.mark.parametrize("m,k,n", [(17, 256, 128), (32, 1024, 200), (64, 2048, 130), (70, 512, 257), (130, 768, 96), (200, 4096, 520)])
+def test_qmm8_float32_rows_on_tile_kernel(variant, m, k, n):
+    """More than 16 rows of float32 activations with k a multiple of 128 run on the tile kernel, the activations split
+    into three bfloat16 parts that add up to them exactly (one pass over the weights per 64 rows): planned, forced with
+    1 and 3 slices, and switched off (bit 22: the one-row kernels, a pass per 16 rows); strided rows as well."""
+    import _dev
+    a, b, s = int8_case(torch.float32, m, k, n)
+    check_q8(_dev.qmm8(bits(a), ODT[torch.float32], b.numpy(), bits(s), variant=variant), a, b, s, torch.float32)
+    check_q8(_dev.qmm8(bits(a), ODT[torch.float32], b.numpy(), bits(s), variant=variant, row_step=2), a, b, s, torch.float32,
+             rows=slice(None, None, 2))
+
+
+def test_qmm8_float32_rows_special_values():
+    """Infinities, NaNs (also one whose payload sits in the low mantissa bits), zeros, subnormal and huge finite values
+    among float32 activations on the tile kernel: each output is what float64 arithmetic on the same operands gives
+    (an infinity or NaN where that is one, else within the bound)."""
+    import _dev
+    m, k, n = 40, 256, 64
+    a, b, s = int8_case(torch.float32, m, k, n)
+    a = a.clone()
+    a[1, 5] = float("inf")
+    a[2, 7] = float("-inf")
+    a[3, 9] = float("nan")
+    a[4, 11] = torch.tensor(0x7f800001, dtype=torch.int32).view(torch.float32)
+    a[5, :] = 0.0
+    a[6, 3] = 1e-41
+    a[7, 2] = 3.0e38
+    b = b.clone()
+    b[:, 2] = 1  # (keeps row 7 finite)
+    got = unbits(_dev.qmm8(bits(a), ODT[torch.float32], b.numpy(), bits(s)), torch.float32).numpy().astype(np.float64)
+    want = (a.double() @ b.double().t() * s.double()).numpy()
+    nan, inf = np.isnan(want), np.isinf(want)
+    assert np.array_equal(np.isnan(got), nan) and np.array_equal(got[inf], want[inf])
+    fin = ~(nan | inf)
+    mag = (a.double().abs() @ b.double().abs().t() * s.double().abs()).numpy()
+    assert (np.abs(got - want)[fin] <= (2.0 ** -23 * np.abs(want) + 2.0 ** -20 * mag)[fin]).all()
+
+
 def test_qmm8_config1_vs_torch_cpu():
     """BASELINE config 1: fp32, M=1, K=N=4096, within rtol/atol 1e-4 of PyTorch's CPU op."""
     import _dev

@@ -383,7 +383,7 @@ __device__ __forceinline__ void widen16_to_operands(const U4& v, U4* lo, U4* hi)
   for (int i = 0; i < 4; ++i) {
     const float f0 = float(int(int8_t(v[i]))), f1 = float(int(int8_t(v[i] >> 8)));
     const float f2 = float(int(int8_t(v[i] >> 16))), f3 = float(int(int8_t(v[i] >> 24)));
-    if constexpr (T::dtype == VKT_BF16) {
+    if constexpr (T::dtype == VKT_BF16 || T::dtype == VKT_F32) {  // (float32 activations go to the bfloat16 matrix core in three parts)
       // an integer of magnitude <= 128 is its float32's upper 16 bits
       out[2 * i] = __builtin_amdgcn_perm(f32_bits(f1), f32_bits(f0), 0x07060302u);
       out[2 * i + 1] = __builtin_amdgcn_perm(f32_bits(f3), f32_bits(f2), 0x07060302u);
@@ -398,7 +398,7 @@ __device__ __forceinline__ void widen16_to_operands(const U4& v, U4* lo, U4* hi)
 
 template <class T>
 __device__ __forceinline__ V4F mfma16(const U4& w, const U4& a, const V4F& acc) {
-  if constexpr (T::dtype == VKT_BF16)
+  if constexpr (T::dtype == VKT_BF16 || T::dtype == VKT_F32)
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(V8BF, w), __builtin_bit_cast(V8BF, a), acc, 0, 0, 0);
   else
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(V8H, w), __builtin_bit_cast(V8H, a), acc, 0, 0, 0);
@@ -729,10 +729,41 @@ bool launch_staged(const Q8Params& p, int mt, int nt, int waves, uint32_t slices
 // the slices' float32 tiles meet in the runtime's workspace and qmm8_tile_finish adds them in slice order, scales
 // and stores.
 constexpr uint32_t kTileStepK = 128, kTileAhead = 4;
-constexpr uint32_t kTileLds = 8 * 16 * 1024;  // the k-parts' meeting place; the two operand stages use its first half
+constexpr uint32_t kTileLds = 8 * 16 * 1024;  // the k-parts' meeting place; the two operand stages use its first half (float32 activations: all of it)
+constexpr int vmcnt_only(int n) { return 0x0f70 | (n & 15) | ((n >> 4) << 14); }  // s_waitcnt vmcnt(n), nothing else
+
+// Eight float32 values as three bfloat16 operands whose sum they are, exactly: the upper 16 bits of the value, of what
+// that leaves, and of what that leaves (8 + 8 + 8 significant bits; every subtraction is exact).  Infinities and NaNs
+// stay in the first part alone.
+__device__ __forceinline__ void split_f32x8(const U4& x0, const U4& x1, U4* hi, U4* mid, U4* lo) {
+  uint32_t h[8], m[8], l[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const uint32_t bits = i < 4 ? x0[i] : x1[i - 4];
+    const bool special = (bits & 0x7f800000u) == 0x7f800000u;
+    h[i] = (special && (bits & 0x007fffffu) ? bits | 0x00400000u : bits) & 0xffff0000u;
+    const float r1 = special ? 0.0f : __builtin_bit_cast(float, bits) - __builtin_bit_cast(float, h[i]);
+    m[i] = f32_bits(r1) & 0xffff0000u;
+    const float r2 = r1 - __builtin_bit_cast(float, m[i]);
+    l[i] = f32_bits(r2) & 0xffff0000u;
+  }
+  auto pack = [](const uint32_t (&v)[8]) {
+    return U4{v[0] >> 16 | v[1], v[2] >> 16 | v[3], v[4] >> 16 | v[5], v[6] >> 16 | v[7]};
+  };
+  *hi = pack(h), *mid = pack(m), *lo = pack(l);
+}
+
 template <class T>
 __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_slice, uint64_t workspace) {
-  constexpr uint32_t A_BYTES = 64 * 256, B_BYTES = 128 * 128, STAGE = A_BYTES + B_BYTES;
+  // float32 activations: split into three bfloat16 parts when they are written to LDS (three planes of the 16-bit
+  // layout), and every weight fragment multiplies the three planes' fragments one after the other, so the product is
+  // that of the float32 values, added up in float32 (the matrix core's products of bfloat16 values are exact)
+  constexpr bool F32 = T::dtype == VKT_F32;
+  constexpr int PLANES = F32 ? 3 : 1, A_LOADS = F32 ? 2 : 1;
+  constexpr uint32_t PLANE = 64 * 256, A_BYTES = PLANES * PLANE, B_BYTES = 128 * 128, STAGE = A_BYTES + B_BYTES;
+  constexpr uint32_t ITEM = F32 ? 4 : 2, OUT_ITEM = ITEM;
+  constexpr int PER_STEP = 2 * A_LOADS + 2;  // loads per lane and step
+  static_assert(2 * STAGE <= kTileLds, "two stages");
   extern __shared__ __attribute__((aligned(16))) uint8_t tile_lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
   const int kc = wave & 3, nh = wave >> 2;
@@ -740,17 +771,18 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
   const uint32_t steps = p.k / kTileStepK;
   const uint32_t s_begin = slice * steps_per_slice, s_end = s_begin + steps_per_slice < steps ? s_begin + steps_per_slice : steps;
 
-  // Loads of one step: activations 16 wave-loads of 4 rows x 256 bytes, weights 16 of 8 rows x 128 bytes; a wave issues
-  // 2 + 2, into registers, kTileAhead steps ahead, and writes them to LDS (16 bytes per lane, lane after lane) one
-  // step before they are multiplied.  (Straight into LDS with global_load_lds_dwordx4 the same stream runs at 2.6
-  // TB/s from 112 compute units where this path gives 4.1-4.4: measured with the loads alone.)
+  // Loads of one step: activations 16 wave-loads of 4 rows x 128 values (8 values per lane), weights 16 of 8 rows x 128
+  // bytes; a wave issues 2 + 2 (float32: 4 + 2), into registers, kTileAhead steps ahead, and writes them to LDS (16
+  // bytes per lane and plane, lane after lane) one step before they are multiplied.  (Straight into LDS with
+  // global_load_lds_dwordx4 the same stream runs at 2.6 TB/s from 112 compute units where this path gives 4.1-4.4:
+  // measured with the loads alone.)
   uint64_t a_src[2], b_src[2];
   uint32_t a_dst[2], b_dst[2];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const uint32_t row = (wave * 2 + i) * 4 + (lane >> 4), slot = lane & 15u;
     const uint32_t m = m0 + row < p.m ? m0 + row : p.m - 1;
-    a_src[i] = p.a + uint64_t(int64_t(m) * p.a_sm * 2) + ((slot ^ (row & 15u)) * 16);
+    a_src[i] = p.a + uint64_t(int64_t(m) * p.a_sm * int64_t(ITEM)) + ((slot ^ (row & 15u)) * 8 * ITEM);
     a_dst[i] = (wave * 2 + i) * 1024 + lane * 16;
   }
 #pragma unroll
@@ -760,12 +792,14 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
     b_src[i] = p.b + uint64_t(n) * p.k + ((slot ^ ((row >> 1) & 7u)) * 16);
     b_dst[i] = A_BYTES + (wave * 2 + i) * 1024 + lane * 16;
   }
-  U4 ra[kTileAhead][2], rb[kTileAhead][2];
+  U4 ra[kTileAhead][2][A_LOADS], rb[kTileAhead][2];
   auto request = [&](auto set, uint32_t step) {
     constexpr int R = decltype(set)::value;
     const uint32_t st = step < s_end ? step : s_end - 1;  // (past the end the last step again, never published: the count of loads in flight stays the same)
 #pragma unroll
-    for (int i = 0; i < 2; ++i) ra[R][i] = ldg<U4>(a_src[i] + uint64_t(st) * kTileStepK * 2);
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int h = 0; h < A_LOADS; ++h) ra[R][i][h] = ldg<U4>(a_src[i] + uint64_t(st) * kTileStepK * ITEM + 16 * h);
 #pragma unroll
     for (int i = 0; i < 2; ++i) rb[R][i] = ldg_stream<U4>(b_src[i] + uint64_t(st) * kTileStepK);
   };
@@ -773,7 +807,16 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
     constexpr int R = decltype(set)::value;
     uint8_t* base = tile_lds + ((step - s_begin) & 1u) * STAGE;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) *reinterpret_cast<U4*>(base + a_dst[i]) = ra[R][i];
+    for (int i = 0; i < 2; ++i) {
+      if constexpr (F32) {
+        U4 part[3];
+        split_f32x8(ra[R][i][0], ra[R][i][A_LOADS - 1], &part[0], &part[1], &part[2]);
+#pragma unroll
+        for (int q = 0; q < 3; ++q) *reinterpret_cast<U4*>(base + q * PLANE + a_dst[i]) = part[q];
+      } else {
+        *reinterpret_cast<U4*>(base + a_dst[i]) = ra[R][i][0];
+      }
+    }
 #pragma unroll
     for (int i = 0; i < 2; ++i) *reinterpret_cast<U4*>(base + b_dst[i]) = rb[R][i];
   };
@@ -786,8 +829,8 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
 
   // Fragments of step s + 1 are read from LDS (8 reads per lane, into the other of two register sets) while step s is
   // widened and multiplied, so the LDS, the vector units and the matrix cores work at the same time; three further
-  // steps are in flight from memory.  Loads land in the order issued: "at most 12 outstanding" (three steps' worth
-  // per wave) means everything older has landed.
+  // steps are in flight from memory.  Loads land in the order issued: "at most three steps' worth outstanding" means
+  // everything older has landed.
   // lane (c, g): activations of row 16 mt + c, weights of column 64 nh + 16 t + c, both at k = 32 kc + 8 g .. + 7
   U4 fa[2][4];
   U2 fw[2][4];
@@ -802,49 +845,71 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
     const uint32_t row = 64 * nh + 16 * t + c;
     w_off[t] = row * 128 + (((2 * kc + (g >> 1)) ^ ((row >> 1) & 7u)) * 16) + 8 * (g & 1);
   }
-  auto read_fragments = [&](auto set, uint32_t step) {
+  auto read_weights = [&](auto set, uint32_t step) {
     constexpr int S = decltype(set)::value;
-    const uint8_t* ta = tile_lds + ((step - s_begin) & 1u) * STAGE;
-    const uint8_t* tb = ta + A_BYTES;
+    const uint8_t* tb = tile_lds + ((step - s_begin) & 1u) * STAGE + A_BYTES;
 #pragma unroll
     for (int t = 0; t < 4; ++t) fw[S][t] = *reinterpret_cast<const U2*>(tb + w_off[t]);
+  };
+  auto read_activations = [&](auto set, uint32_t step, uint32_t plane) {
+    constexpr int S = decltype(set)::value;
+    const uint8_t* ta = tile_lds + ((step - s_begin) & 1u) * STAGE + plane * PLANE;
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) fa[S][mt] = *reinterpret_cast<const U4*>(ta + a_off[mt]);
   };
-  auto multiply = [&](auto set) {
-    constexpr int S = decltype(set)::value;
+  auto multiply = [&](auto aset, auto wset) {
+    constexpr int S = decltype(aset)::value, W = decltype(wset)::value;
 #pragma unroll
     for (int t = 0; t < 4; t += 2) {
       U4 w0, w1;
-      widen16_to_operands<T>(U4{fw[S][t][0], fw[S][t][1], fw[S][t + 1][0], fw[S][t + 1][1]}, &w0, &w1);
+      widen16_to_operands<T>(U4{fw[W][t][0], fw[W][t][1], fw[W][t + 1][0], fw[W][t + 1][1]}, &w0, &w1);
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt) acc[mt][t] = mfma16<T>(w0, fa[S][mt], acc[mt][t]);
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt) acc[mt][t + 1] = mfma16<T>(w1, fa[S][mt], acc[mt][t + 1]);
     }
   };
+  // J = (step - s_begin) % kTileAhead.  The weights' register set is the step's parity; the activations' set changes
+  // with every plane: sub-step (step, plane) uses set (PLANES * J + plane) % 2.
   auto iteration = [&](auto index, auto guarded, uint32_t step) {
-    constexpr int J = decltype(index)::value, S = J & 1, NEXT = (J + 1) % kTileAhead;  // J = (step - s_begin) % kTileAhead
+    constexpr int J = decltype(index)::value, NEXT = (J + 1) % kTileAhead;
     constexpr bool GUARDED = decltype(guarded)::value;  // the last steps of the slice: step + 1 may be past the end
-    // the registers of step + 1 have landed; they go to the stage that step - 1 was read from (every wave's reads of
-    // it had returned before it passed the last barrier), and the register set takes the loads of step + 1 + kTileAhead
-    __builtin_amdgcn_s_waitcnt(0x0f7c);  // vmcnt(12)
+    // the registers of step + 1 have landed; they go to the stage that step - 1 was read from, and the register set
+    // takes the loads of step + 1 + kTileAhead.  16-bit activations: every wave's reads of that stage had returned
+    // before it passed the last barrier.  float32: a wave reads planes 1 and 2 of a step during the step itself, so
+    // a barrier of its own comes first.
+    if constexpr (F32) __syncthreads();
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(3 * PER_STEP));
     if (!GUARDED || step + 1 < s_end) publish(std::integral_constant<int, NEXT>{}, step + 1);
     request(std::integral_constant<int, NEXT>{}, step + 1 + kTileAhead);
     __syncthreads();
-    if (!GUARDED || step + 1 < s_end) read_fragments(std::integral_constant<int, S ^ 1>{}, step + 1);
-    __builtin_amdgcn_sched_barrier(0);  // (the scheduler would move each read down to its first use)
-    multiply(std::integral_constant<int, S>{});
+#pragma unroll
+    for (int plane = 0; plane < PLANES; ++plane) {
+      const int set = (PLANES * J + plane) & 1;
+      // the fragments of the next sub-step: the next plane of this step, or plane 0 (and the weights) of step + 1
+      if (plane + 1 < PLANES) {
+        if (set) read_activations(std::integral_constant<int, 0>{}, step, plane + 1);
+        else read_activations(std::integral_constant<int, 1>{}, step, plane + 1);
+      } else if (!GUARDED || step + 1 < s_end) {
+        if (set) read_activations(std::integral_constant<int, 0>{}, step + 1, 0);
+        else read_activations(std::integral_constant<int, 1>{}, step + 1, 0);
+        read_weights(std::integral_constant<int, (J + 1) & 1>{}, step + 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // (the scheduler would move each read down to its first use)
+      if (set) multiply(std::integral_constant<int, 1>{}, std::integral_constant<int, J & 1>{});
+      else multiply(std::integral_constant<int, 0>{}, std::integral_constant<int, J & 1>{});
+    }
   };
   request(std::integral_constant<int, 0>{}, s_begin);
   request(std::integral_constant<int, 1>{}, s_begin + 1);
   request(std::integral_constant<int, 2>{}, s_begin + 2);
   request(std::integral_constant<int, 3>{}, s_begin + 3);
-  __builtin_amdgcn_s_waitcnt(0x0f7c);  // vmcnt(12): the first of four steps has landed
+  __builtin_amdgcn_s_waitcnt(vmcnt_only(3 * PER_STEP));  // the first of four steps has landed
   publish(std::integral_constant<int, 0>{}, s_begin);
   request(std::integral_constant<int, 0>{}, s_begin + kTileAhead);
   __syncthreads();
-  read_fragments(std::integral_constant<int, 0>{}, s_begin);
+  read_activations(std::integral_constant<int, 0>{}, s_begin, 0);
+  read_weights(std::integral_constant<int, 0>{}, s_begin);
   // groups of four steps with a step after them: straight-line code; then the last one to four steps
   uint32_t step = s_begin;
   constexpr std::false_type plain{};
@@ -901,18 +966,27 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
           if (n + r < p.n) out[r] = sum[t][r];
       }
     } else {
-      uint32_t h[4];
+      float v[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float v = sum[t][r] * load_f32<T>(p.scales + uint64_t(n + r < p.n ? n + r : p.n - 1) * 2);
-        h[r] = T::dtype == VKT_BF16 ? f32_to_bf16(v) : f32_to_f16(v);
-      }
-      const uint64_t at = p.c + (uint64_t(m) * p.n + n) * 2;
-      if ((p.n & 3u) == 0 && (p.c & 7u) == 0) stg<U2>(at, U2{h[0] | h[1] << 16, h[2] | h[3] << 16});
-      else {
+      for (int r = 0; r < 4; ++r) v[r] = sum[t][r] * load_f32<T>(p.scales + uint64_t(n + r < p.n ? n + r : p.n - 1) * ITEM);
+      const uint64_t at = p.c + (uint64_t(m) * p.n + n) * OUT_ITEM;
+      if constexpr (F32) {
+        if ((p.n & 3u) == 0 && (p.c & 15u) == 0) stg<F4>(at, F4{v[0], v[1], v[2], v[3]});
+        else {
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (n + r < p.n) stg<uint16_t>(at + 2 * r, uint16_t(h[r]));
+          for (int r = 0; r < 4; ++r)
+            if (n + r < p.n) stg<float>(at + 4 * r, v[r]);
+        }
+      } else {
+        uint32_t h[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) h[r] = T::dtype == VKT_BF16 ? f32_to_bf16(v[r]) : f32_to_f16(v[r]);
+        if ((p.n & 3u) == 0 && (p.c & 7u) == 0) stg<U2>(at, U2{h[0] | h[1] << 16, h[2] | h[3] << 16});
+        else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (n + r < p.n) stg<uint16_t>(at + 2 * r, uint16_t(h[r]));
+        }
       }
     }
   }
@@ -947,15 +1021,23 @@ __global__ __launch_bounds__(256) void qmm8_tile_finish(Q8Params p, uint32_t sli
     }
   }
   const uint32_t n = uint32_t(i % p.n);
-  uint32_t h[4];
+  constexpr uint32_t ITEM = T::dtype == VKT_F32 ? 4 : 2;
+  float y[4];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const float y = v[r] * load_f32<T>(p.scales + uint64_t(n + r < p.n ? n + r : p.n - 1) * 2);
-    h[r] = T::dtype == VKT_BF16 ? f32_to_bf16(y) : f32_to_f16(y);
-  }
-  if (vec && (p.c & 7u) == 0) stg<U2>(p.c + i * 2, U2{h[0] | h[1] << 16, h[2] | h[3] << 16});
-  else {
-    for (uint32_t r = 0; r < per; ++r) stg<uint16_t>(p.c + (i + r) * 2, uint16_t(h[r]));
+  for (int r = 0; r < 4; ++r) y[r] = v[r] * load_f32<T>(p.scales + uint64_t(n + r < p.n ? n + r : p.n - 1) * ITEM);
+  if constexpr (T::dtype == VKT_F32) {
+    if (vec && (p.c & 15u) == 0) stg<F4>(p.c + i * 4, F4{y[0], y[1], y[2], y[3]});
+    else {
+      for (uint32_t r = 0; r < per; ++r) stg<float>(p.c + (i + r) * 4, y[r]);
+    }
+  } else {
+    uint32_t h[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) h[r] = T::dtype == VKT_BF16 ? f32_to_bf16(y[r]) : f32_to_f16(y[r]);
+    if (vec && (p.c & 7u) == 0) stg<U2>(p.c + i * 2, U2{h[0] | h[1] << 16, h[2] | h[3] << 16});
+    else {
+      for (uint32_t r = 0; r < per; ++r) stg<uint16_t>(p.c + (i + r) * 2, uint16_t(h[r]));
+    }
   }
 }
 
@@ -972,7 +1054,7 @@ bool workspace_refused(const Machine& mc, uint64_t need, std::string* err) {
 // 1 launched, 0 not this kernel's shape, -1 refused (*err set).
 template <class T>
 int launch_tile_kernel(const Q8Params& p, uint32_t want_slices, const Machine& mc, hipStream_t stream, std::string* err) {
-  if (p.k % kTileStepK != 0 || p.k == 0 || (int64_t(p.a_sm) * 2) % 16 != 0 || p.a_sm <= 0) return 0;
+  if (p.k % kTileStepK != 0 || p.k == 0 || (int64_t(p.a_sm) * int64_t(sizeof(typename T::storage))) % 16 != 0 || p.a_sm <= 0) return 0;
   constexpr uint32_t lds = kTileLds;
   auto kernel = qmm8_tile<T>;
   static bool configured = false;  // guarded by the runtime's stream mutex
@@ -1139,6 +1221,15 @@ int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipSt
         if (launch_mfma<T>(p, variant, mc, stream, err) != 0) return -1;
       }
       return 0;
+    }
+  }
+  if constexpr (T::dtype == VKT_F32) {
+    // More than 16 rows of float32 activations: the tile kernel on the activations' three bfloat16 parts, one pass
+    // over the weights per 64 rows (the one-row kernels below read them once per 16).  variant bit 21 forces it
+    // (bits 24+ slices), bit 22 keeps it off.
+    if (((p0.m > 16 && !(variant & 0xffff)) || ((variant >> 21) & 1)) && !((variant >> 22) & 1) && !((variant >> 17) & 1)) {
+      const int rc = launch_tile_kernel<T>(p0, variant >> 24, mc, stream, err);
+      if (rc != 0) return rc < 0 ? -1 : 0;
     }
   }
   // One row of float32 activations: the persistent streaming kernel (measured at K = N = 4096: 4.85 us against 5.8; a
