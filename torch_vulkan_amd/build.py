@@ -82,9 +82,9 @@ def build(force=False, verbose=True):
         cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs + ["-Wl,--no-undefined"]
         subprocess.check_call(cmd)
     # host-only test shim for the allocator policy (no HIP)
-    shim = os.path.join(CSRC, "core", "hosttest.cpp")
-    if force or _stale(HOSTTEST, [shim] + headers):
-        subprocess.check_call(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-o", HOSTTEST, shim])
+    shim = os.path.join(os.path.dirname(HERE), "tests", "pool_shim.cpp")
+    if os.path.exists(shim) and (force or _stale(HOSTTEST, [shim] + headers)):
+        subprocess.check_call(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-I", os.path.join(CSRC, "core"), "-o", HOSTTEST, shim])
     return LIB
 
 
