@@ -360,9 +360,12 @@ def wl_probe_mfma(abi, operands, steps, warmup, iters=4096):
     fns = [Launch(abi, "probe_mfma_f8", [operands], abi.ProbeParams(dst=sink.address, iters=iters))]
     tm = time_steps(abi, fns, steps, warmup)
     work = info.compute_units * 4 * iters * 4 * 2 * 32 * 32 * 64
+    import numpy as np
+    cycles, ticks = (int(v) for v in sink.to_numpy(np.uint64, (32,))[8:10])
     label = {0: "all-zero operands", 1: "random operands held in registers", 2: "fresh random operands per instruction"}[operands]
     return dict(kind="mfma", metric="fp8 MFMA loop TFLOP/s (% of MFMA peak)", work=work, wall_ms=tm[0], event_ms=tm[1], event_ms_median=tm.median,
-                bytes=0, inputs=None, copies=1, name=f"probe_mfma_f8, {label}")
+                bytes=0, inputs=None, copies=1, clock_ghz=round(cycles / (10.0 * ticks), 3) if ticks else None,
+                name=f"probe_mfma_f8, {label}")
 
 
 # The BASELINE.json configurations.  Order of the extras in the output: the configurations the targets are stated on
@@ -601,6 +604,8 @@ def main():
                    "device": info.name.decode(), "compute_units": info.compute_units},
         "roofline": roof,
     }
+    if r.get("clock_ghz"):
+        line["config"]["clock_ghz"] = r["clock_ghz"]
     if not args.no_cpu:
         line.update(cpu_baselines(abi, args.workload, r, port=True))
         line["through_dispatcher"] = through_dispatcher(abi, args.workload, r)
@@ -616,6 +621,8 @@ def main():
             rr = fn(abi, args.steps, args.warmup)
             v, u, rf = summarise(rr)
             ceilings[key] = {"achieved": rf["achieved"], "unit": u, "kernel_ms": round(rr["event_ms"], 5)}
+            if rr.get("clock_ghz"):
+                ceilings[key]["clock_ghz"] = rr["clock_ghz"]  # (shader cycles per tick of the constant clock, read in the kernel)
             del rr
         line["ceilings"] = ceilings
         extra = []

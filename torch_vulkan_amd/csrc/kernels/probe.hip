@@ -10,7 +10,8 @@
 //   "probe_mfma_f8", spec {OPERANDS}   a register-only loop of V_MFMA_F32_32X32X64_F8F6F4 (4 waves per workgroup, 4
 //                                       accumulator tiles per wave): 0 all-zero operands, 1 random bits held in the same
 //                                       registers throughout, 2 fresh operands for every instruction (made by vector
-//                                       operations, no memory at all)
+//                                       operations, no memory at all); dst + 64 / + 72 receive the loop's shader cycles
+//                                       and its ticks of the 100 MHz clock (the clock the part held)
 //   "probe_delay", spec {}              one wave that waits `iters` microseconds on the constant-rate clock and exits: a
 //                                       timing loop queues it first so that the launches behind it are all queued by the
 //                                       time the device reaches them (the device, not the host, then sets the pace)
@@ -100,6 +101,7 @@ __global__ __launch_bounds__(256) void probe_mfma_f8(ProbeParams p) {
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  const uint64_t cycles0 = clock64(), ticks0 = wall_clock64();
   for (uint32_t it = 0; it < p.iters; ++it) {
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -126,6 +128,11 @@ __global__ __launch_bounds__(256) void probe_mfma_f8(ProbeParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) s += acc[i][j][r];
   if (s == 1.2345e-30f) stg<float>(p.dst, s);
+  // the clock the loop ran at: shader cycles and ticks of the constant 100 MHz clock, first wave of the first workgroup
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    stg<uint64_t>(p.dst + 64, clock64() - cycles0);
+    stg<uint64_t>(p.dst + 72, wall_clock64() - ticks0);
+  }
 }
 
 }  // namespace
