@@ -40,8 +40,8 @@ def test_gemm16_layouts(dtype, m, k, n):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 5, 255])
-@pytest.mark.parametrize("m,k,n", [(130, 256, 70), (257, 384, 129), (64, 1088, 300), (300, 128, 520)])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 5, 6, 255])
+@pytest.mark.parametrize("m,k,n", [(130, 256, 70), (257, 384, 129), (64, 1088, 300), (300, 128, 520), (300, 320, 520), (1, 128, 8)])
 def test_gemm16_tile_variants(dtype, variant, m, k, n):
     """The Linear layout (both operands contiguous along k) through every tile variant and the strided kernel."""
     import _dev
@@ -52,6 +52,23 @@ def test_gemm16_tile_variants(dtype, variant, m, k, n):
     bias = bits(torch.randn(n, generator=gen(5)).to(dtype))
     want2, mag2 = oracle.gemm16(a, w.T, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, want_mag=True)
     close(_dev.gemm16(a, w.T, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, variant=variant), want2, mag2, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_gemm16_stream_kernel(dtype):
+    """The stream kernel (variant 6; what large products in the Linear layout get): more tiles than workgroups, so
+    streams that run through two tiles; batches; a broadcast bias; rows and columns past the last whole tile.  Every
+    output against the oracle, and bit for bit the tile kernel's (same products, same order)."""
+    import _dev
+    for batch, m, k, n in [(1, 4352, 192, 4360), (3, 515, 256, 1032)]:
+        a = bits((torch.randn(batch, m, k, generator=gen(13)) * 0.5).to(dtype))
+        w = bits((torch.randn(batch, n, k, generator=gen(14)) * 0.5).to(dtype))
+        bias = bits(torch.randn(n, generator=gen(15)).to(dtype))
+        got = {v: _dev.gemm16(a, w.transpose(0, 2, 1), ODT[dtype], cin=bias, alpha=2.0, beta=0.5, variant=v) for v in (6, 3)}
+        assert np.array_equal(got[6], got[3])
+        if m * n <= 1 << 20:
+            want, mag = oracle.gemm16(a, w.transpose(0, 2, 1), ODT[dtype], cin=bias, alpha=2.0, beta=0.5, want_mag=True)
+            close(got[6], want, mag, dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)

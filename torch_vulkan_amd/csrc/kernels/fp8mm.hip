@@ -141,6 +141,27 @@ struct F8Problem : F8Params {
   __device__ __forceinline__ void store_bf16x8(uint32_t, uint32_t row, uint32_t col, const U4& v) const {
     stg<U4>(out + (uint64_t(row) * ldo + col) * 2, v);
   }
+  // the stream kernel's epilogue: 8 consecutive bfloat16 outputs of a row
+  struct Columns8 {
+    float scale[8], bias[8];
+  };
+  __device__ __forceinline__ Columns8 columns8(uint32_t, uint32_t col, const Whole& w) const {
+    Columns8 c;
+    float s0[4], s1[4], b0[4], b1[4];
+    column_terms(col, w, s0, b0);
+    column_terms(col + 4, w, s1, b1);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) c.scale[r] = s0[r], c.scale[4 + r] = s1[r], c.bias[r] = b0[r], c.bias[4 + r] = b1[r];
+    return c;
+  }
+  __device__ __forceinline__ void finish8(uint32_t batch, uint32_t row, uint32_t col, const float (&t)[8], const Columns8& c, const Whole& w) const {
+    const float rs = row_scale(row, w);
+    uint32_t packed[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      packed[e] = pack_bf16(t[2 * e] * (rs * c.scale[2 * e]) + c.bias[2 * e], t[2 * e + 1] * (rs * c.scale[2 * e + 1]) + c.bias[2 * e + 1]);
+    store_bf16x8(batch, row, col, U4{packed[0], packed[1], packed[2], packed[3]});
+  }
   template <class F>
   __device__ __forceinline__ void for_output_type(bool full, const Whole& w, F&& f) const {
     if (w.vec_ok && full) {
@@ -183,7 +204,7 @@ int launch_stream(const F8Params& p, int compute_units, hipStream_t stream, std:
   F8Problem problem;
   static_cast<F8Params&>(problem) = p;
   if (p.out_dtype != VKT_BF16 || p.ldo % 8 || p.out % 16 || !mma_stream_serves(problem)) return -2;
-  return launch_mma_stream<FA, FB>(problem, compute_units, stream, err, "fp8mm");
+  return launch_mma_stream<FA, FB, kMathFp8>(problem, compute_units, stream, err, "fp8mm");
 }
 
 template <int FA, int FB>

@@ -13,6 +13,7 @@
 //   - everything else (strided views, odd sizes): one thread per output over the strides as
 //     given.  Correct for any strides, and slow.
 #include "kernels.h"
+#include "mma_stream.h"
 #include "mma_tile.h"
 
 namespace vkt {
@@ -66,6 +67,25 @@ struct GemmProblem {
     if (w.vec_ok && full) f(std::integral_constant<int, T::dtype>{});
     else f(std::integral_constant<int, -1>{});
   }
+  // the stream kernel's epilogue: 8 consecutive outputs of a row, one 16-byte store (C rows and batches 16-byte aligned)
+  struct Columns8 {};
+  __device__ __forceinline__ Columns8 columns8(uint32_t, uint32_t, const Whole&) const { return Columns8{}; }
+  __device__ __forceinline__ void finish8(uint32_t batch, uint32_t row, uint32_t col, const float (&t)[8], const Columns8&, const Whole&) const {
+    float v[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      v[r] = alpha * t[r];
+      if (cin != 0) {  // beta == 0 never reads Cin (it may hold NaN): then cin is 0
+        const int64_t at = int64_t(batch) * cin_sb + int64_t(row) * cin_sm + int64_t(col + r) * cin_sn;
+        v[r] += beta * load_f32<T>(cin + uint64_t(at * 2));
+      }
+    }
+    uint32_t packed[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      packed[e] = T::dtype == VKT_BF16 ? pack_bf16(v[2 * e], v[2 * e + 1]) : uint32_t(f32_to_f16(v[2 * e])) | uint32_t(f32_to_f16(v[2 * e + 1])) << 16;
+    stg<U4>(c + uint64_t((int64_t(batch) * c_sb + int64_t(row) * c_sm + int64_t(col)) * 2), U4{packed[0], packed[1], packed[2], packed[3]});
+  }
 };
 
 // Any strides: one thread per output, float32 accumulation.
@@ -98,7 +118,7 @@ int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t
   g.c_sm = p.c_sm, g.c_sb = p.c_sb, g.cin_sm = p.cin_sm, g.cin_sn = p.cin_sn, g.cin_sb = p.cin_sb;
   const bool direct_ok = g.k % BK == 0;
   // variant 0: planned; 1: 128x128 tiles; 2: 256x128; 3: 256x256 with direct loads; 4: 128x128 with direct loads;
-  // 5: 256x256 with direct loads over 8 waves
+  // 5: 256x256 with direct loads over 8 waves; 6: the stream kernel (mma_stream.h; else 3)
   // (direct loads: k a multiple of 64; k-major operands run on the direct forms only)
   if (variant == 0) {
     // 256 x 256 tiles where they give every compute unit one, else 128 x 128
@@ -106,8 +126,14 @@ int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t
     // (both operands k-major: 8 waves, whose transposing LDS reads cover each other: 8192^3 0.94 -> 1.11-1.13 PFLOP/s;
     //  with k-contiguous operands the 8-wave form reads 1.5x the LDS bytes and is 3-5 % slower)
     variant = large ? (direct_ok ? (TRA && TRB ? 5 : 3) : 2) : (TRA || TRB ? 4 : 1);
+    // both operands contiguous along k (x @ w.T): the stream kernel where it serves (8192^3: 0.94-1.00 -> 0.89 ms)
+    if (!TRA && !TRB && variant == 3) variant = 6;
   }
+  const bool stream_ok = direct_ok && g.k >= 2 * BK && p.n % 8 == 0 && p.c_sm % 8 == 0 && p.c_sb % 8 == 0 && p.c % 16 == 0;
+  if (variant == 6 && !stream_ok) variant = 3;
   if constexpr (!TRA && !TRB) {
+    // 6: the stream kernel (mma_stream.h) where it serves the problem: k a multiple of 64 values and at least 128, n a multiple of 8, C in 16-byte aligned rows
+    if (variant == 6) return launch_mma_stream<0, 0, MATH>(g, mc.compute_units, stream, err, "gemmcm");
     if (variant == 1) return launch_mma_tile<2, 2, 4, 4, 0, 0, true, false, MATH>(g, mc.compute_units, stream, err, "gemmcm");
     if (variant == 2) return launch_mma_tile<2, 2, 8, 4, 0, 0, true, false, MATH>(g, mc.compute_units, stream, err, "gemmcm");
   }
@@ -193,6 +219,29 @@ struct Q8GemmProblem {
     if (w.vec_ok && full) f(std::integral_constant<int, T::dtype>{});
     else f(std::integral_constant<int, -1>{});
   }
+  // the stream kernel's epilogue: 8 consecutive outputs of a row (n a multiple of 8, C 16-byte aligned)
+  struct Columns8 {
+    float s[8];
+  };
+  __device__ __forceinline__ Columns8 columns8(uint32_t, uint32_t col, const Whole&) const {
+    Columns8 cs;
+    const U4 raw = ldg<U4>(scales + uint64_t(col) * 2);  // (col a multiple of 8; the scales' address is checked by the launcher)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if constexpr (T::dtype == VKT_BF16) cs.s[2 * e] = bits_f32(raw[e] << 16), cs.s[2 * e + 1] = bits_f32(raw[e] & 0xffff0000u);
+      else cs.s[2 * e] = f16_to_f32(uint16_t(raw[e])), cs.s[2 * e + 1] = f16_to_f32(uint16_t(raw[e] >> 16));
+    }
+    return cs;
+  }
+  __device__ __forceinline__ void finish8(uint32_t, uint32_t row, uint32_t col, const float (&t)[8], const Columns8& cs, const Whole&) const {
+    uint32_t packed[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float v0 = t[2 * e] * cs.s[2 * e], v1 = t[2 * e + 1] * cs.s[2 * e + 1];
+      packed[e] = T::dtype == VKT_BF16 ? pack_bf16(v0, v1) : uint32_t(f32_to_f16(v0)) | uint32_t(f32_to_f16(v1)) << 16;
+    }
+    stg<U4>(c + (uint64_t(row) * n + col) * 2, U4{packed[0], packed[1], packed[2], packed[3]});
+  }
 };
 
 // 16 int8 values per thread -> 16 values of T (integers of magnitude <= 128 are exact in both 16-bit types).
@@ -229,6 +278,8 @@ int launch_q8_gemm_t(const Q8Params& p, const Machine& mc, hipStream_t stream, s
   g.batches = 1, g.a_batch = 0, g.b_batch = 0, g.c = p.c, g.scales = p.scales;
   const bool large = uint64_t((p.m + 255) / 256) * ((p.n + 255) / 256) >= uint64_t(mc.compute_units);
   if (g.k % BK == 0) {
+    if (large && g.k >= 2 * BK && p.n % 8 == 0 && p.c % 16 == 0 && p.scales % 16 == 0)
+      return launch_mma_stream<0, 0, MATH>(g, mc.compute_units, stream, err, "qmm8");
     if (large) return launch_mma_tile<2, 2, 8, 8, 0, 0, true, true, MATH>(g, mc.compute_units, stream, err, "qmm8");
     return launch_mma_tile<2, 2, 4, 4, 0, 0, true, true, MATH>(g, mc.compute_units, stream, err, "qmm8");
   }

@@ -19,8 +19,16 @@
 //     instruction makes it wait for ALL outstanding LDS reads before every use of any of them.
 //     The compiler therefore does not know these loads: the kernel waits for them itself (s_waitcnt vmcnt) and the
 //     compiler's own waits, which count only what it knows, can only be longer than needed.
-// The problem type P is mma_tile's, restricted to what the epilogue from the registers serves (P::kRegisterEpilogue):
-// bfloat16 outputs, rows 16-byte aligned, n a multiple of 8; k a multiple of 128 and at least 256.
+// (4 waves of 128 x 128, one per SIMD with the accumulators in the second half of the register file, would read two
+// thirds of the fragment bytes per instruction.  Tried: correct, but the compiler keeps fragments in the
+// accumulators' half of the file and spills both inside the loop, 860 bytes of scratch and ten times slower.)
+// The problem type P supplies the operands as mma_tile's does (a, b, lda, ldb in bytes, m, n, k in bytes, batches,
+// a_batch, b_batch) and the epilogue of 8 consecutive outputs of a row, which one lane holds after the accumulators'
+// halves have changed lanes (v_permlane32_swap, as float32: the epilogue's arithmetic comes after):
+//   whole()                                       per-launch constants
+//   columns8(batch, n, whole)                     per-lane constants of columns n .. n + 7
+//   finish8(batch, m, n, sums[8], columns, whole) finish and store them (16-bit outputs: one 16-byte store)
+// k a multiple of 128 bytes and at least 256, n a multiple of 8, 16-byte aligned operand rows.
 #pragma once
 
 #include "mma_tile.h"
@@ -35,12 +43,15 @@ __device__ __forceinline__ void load_to_lds(uint32_t offset, uint64_t base, uint
                : "memory", "m0");
 }
 
-template <int FA, int FB, class P>
+template <int FA, int FB, int MATH, class P>
 __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_t tiles_n) {
-  static_assert(P::kRegisterEpilogue && !P::kTransA && !P::kTransB, "float8-style operands, epilogue from the registers");
+  static_assert(!P::kTransA && !P::kTransB, "operands contiguous along k");
+  constexpr int WM = 4;  // waves along m: 8 waves of 64 x 128
   constexpr uint32_t BM = 256, BN = 256, STAGE = (BM + BN) * BK, B_AT = BM * BK;
-  constexpr int TM2 = 2, TN2 = 4;  // a wave's 64 x 128 as 32 x 32 matrix-core tiles
-  constexpr uint32_t BIAS = 3072;  // keeps the per-lane offsets non-negative (they carry -1024 i for load i of 4)
+  constexpr int WAVES = WM * 2, TM2 = 8 / WM, TN2 = 4;  // a wave's (256 / WM) x 128 as 32 x 32 matrix-core tiles
+  constexpr int ROWS = 256 / WAVES, PER = ROWS / 8;    // rows of each operand tile a wave brings; loads per operand and step
+  constexpr int NM = TM2 * TN2, FR = TM2 + TN2;        // matrix-core tiles and fragments per half step
+  constexpr uint32_t BIAS = 3072;  // keeps the per-lane offsets non-negative (they carry -1024 (i % 4) for load i)
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)(lds)));
 
@@ -65,36 +76,35 @@ __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_
     return Tile{batch, (panel * PANEL + in_panel % rows_here) * BM, (in_panel / rows_here) * BN};
   };
 
-  // The load stream: step load_s of tile load_tile is the next to be asked for.  Wave w brings rows 32 w .. 32 w + 31 of
-  // both operand tiles, 8 rows (1 KiB of LDS, in lane order) per instruction; a lane fetches the logical chunk that the
-  // swizzle keeps in its slot.
+  // The load stream: step load_s of tile load_tile is the next to be asked for.  Wave w brings rows ROWS w .. + ROWS - 1
+  // of both operand tiles, 8 rows (1 KiB of LDS, in lane order) per instruction; a lane fetches the logical chunk that
+  // the swizzle keeps in its slot.
   uint32_t load_tile = 0, load_s = 0;
   uint64_t load_a = 0, load_b = 0;  // uniform: the tile's first row, less BIAS
-  uint32_t off_a[4], off_b[4];
+  uint32_t off_a[PER], off_b[PER];
   auto load_setup = [&](uint32_t index) {
     const Tile t = tile_at(index);
     load_a = p.a + uint64_t(t.batch) * p.a_batch + uint64_t(t.m0) * p.lda - BIAS;
     load_b = p.b + uint64_t(t.batch) * p.b_batch + uint64_t(t.n0) * p.ldb - BIAS;
 #pragma unroll
-    for (uint32_t i = 0; i < 4; ++i) {
-      const uint32_t r = wave * 32 + 8 * i + (lane >> 3), c = (lane & 7u) ^ ((r >> 1) & 7u);
+    for (uint32_t i = 0; i < uint32_t(PER); ++i) {
+      const uint32_t r = wave * ROWS + 8 * i + (lane >> 3), c = (lane & 7u) ^ ((r >> 1) & 7u);
       const uint32_t ra = t.m0 + r < p.m ? r : p.m - 1 - t.m0, rb = t.n0 + r < p.n ? r : p.n - 1 - t.n0;  // rows past the end repeat the last one
-      off_a[i] = ra * p.lda + c * 16 + BIAS - 1024 * i;
-      off_b[i] = rb * p.ldb + c * 16 + BIAS - 1024 * i;
+      off_a[i] = ra * p.lda + c * 16 + BIAS - 1024 * (i & 3u);
+      off_b[i] = rb * p.ldb + c * 16 + BIAS - 1024 * (i & 3u);
     }
   };
-  auto load_piece = [&](int piece, uint32_t stage) {
-    const uint64_t a = load_a + uint64_t(load_s) * BK, b = load_b + uint64_t(load_s) * BK;
-    const uint32_t at = lds0 + stage * STAGE + wave * 4096;
-    switch (piece) {
-      case 0: load_to_lds<0>(off_a[0], a, at); break;
-      case 1: load_to_lds<1024>(off_a[1], a, at); break;
-      case 2: load_to_lds<2048>(off_a[2], a, at); break;
-      case 3: load_to_lds<3072>(off_a[3], a, at); break;
-      case 4: load_to_lds<0>(off_b[0], b, at + B_AT); break;
-      case 5: load_to_lds<1024>(off_b[1], b, at + B_AT); break;
-      case 6: load_to_lds<2048>(off_b[2], b, at + B_AT); break;
-      default: load_to_lds<3072>(off_b[3], b, at + B_AT); break;
+  auto load_piece = [&](int piece, uint32_t stage) {  // pieces 0 .. PER - 1: the first operand's, PER .. 2 PER - 1: the second's
+    const bool second = piece >= PER;
+    const int i = second ? piece - PER : piece;
+    const uint64_t base = (second ? load_b : load_a) + uint64_t(load_s) * BK;
+    const uint32_t at = lds0 + stage * STAGE + (second ? B_AT : 0u) + wave * (ROWS * BK) + uint32_t(i >> 2) * 4096;
+    const uint32_t offset = second ? off_b[i < PER ? i : 0] : off_a[i < PER ? i : 0];
+    switch (i & 3) {
+      case 0: load_to_lds<0>(offset, base, at); break;
+      case 1: load_to_lds<1024>(offset, base, at); break;
+      case 2: load_to_lds<2048>(offset, base, at); break;
+      default: load_to_lds<3072>(offset, base, at); break;
     }
   };
   auto load_advance = [&]() {
@@ -113,13 +123,20 @@ __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
       const uint32_t x = x0 ^ (kk * 64) ^ (c * 16);
-      at_a[kk][c] = x + wm * (64 * BK);
+      at_a[kk][c] = x + wm * (TM2 * 32 * BK);
       at_b[kk][c] = x + B_AT + wn * (128 * BK);
     }
   auto fragment = [&](const uint32_t (&at)[2], uint32_t block, uint32_t stage) {
     const V4I lo = *reinterpret_cast<const V4I*>(lds + stage * STAGE + at[0] + block * (32 * BK));
     const V4I hi = *reinterpret_cast<const V4I*>(lds + stage * STAGE + at[1] + block * (32 * BK));
     return V8I{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  };
+  auto multiply = [&](const V8I& b, const V8I& a, const V16F& c) {
+    if constexpr (MATH == kMathFp8) {
+      return mfma_f8_32<FA, FB>(b, a, c);
+    } else {  // 16-bit values: a fragment's 32 bytes are two operands of 8 values
+      return mfma_16bit<MATH>(half_of(b, 1), half_of(a, 1), mfma_16bit<MATH>(half_of(b, 0), half_of(a, 0), c));
+    }
   };
 
   V16F acc[TM2][TN2];
@@ -134,38 +151,29 @@ __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_
   clear();
   const auto whole = p.whole();
 
-  // The epilogue of mma_tile's register path, for this wave's 64 x 128 of tile t.
+  // The epilogue, straight from the accumulators.  A 32 x 32 matrix-core tile leaves lane l with row l % 32 and, for
+  // q = 0..3, columns 8 q + 4 (l / 32) .. + 3: two lanes 32 apart hold the two halves of 8 consecutive outputs;
+  // v_permlane32_swap puts them together (lanes below 32 take chunk q = 0 or 2 of their row, lanes from 32 chunk 1 or 3).
   auto epilogue = [&](const Tile& t) {
-    const uint32_t wm0 = t.m0 + wm * 64, wn0 = t.n0 + wn * 128;
+    const uint32_t wm0 = t.m0 + wm * (TM2 * 32), wn0 = t.n0 + wn * 128;
 #pragma unroll
     for (int j = 0; j < TN2; ++j) {
-      float scale[4][4], bias[4][4];  // of this lane's columns wn0 + 32 j + 8 q + 4 h + r
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const uint32_t n = wn0 + 32 * j + 8 * q + 4 * h;
-        p.column_terms(n + 4 <= p.n ? n : p.n - 4, whole, scale[q], bias[q]);
-      }
+      for (int qp = 0; qp < 2; ++qp) {
+        const uint32_t n = wn0 + 32 * j + 8 * (2 * qp + h);
+        const bool inside = n + 8 <= p.n;
+        const auto columns = p.columns8(t.batch, inside ? n : p.n - 8, whole);
 #pragma unroll
-      for (int i = 0; i < TM2; ++i) {
-        const uint32_t m = wm0 + 32 * i + l32;
-        const float rs = p.row_scale(m < p.m ? m : p.m - 1, whole);
-        const V16F& v = acc[i][j];
+        for (int i = 0; i < TM2; ++i) {
+          const uint32_t m = wm0 + 32 * i + l32;
+          const V16F& v = acc[i][j];
+          float sums[8];
 #pragma unroll
-        for (int qp = 0; qp < 2; ++qp) {
-          uint32_t lo[2], hi[2];  // chunks 2 qp and 2 qp + 1 as two bfloat16 pairs each
-#pragma unroll
-          for (int e = 0; e < 2; ++e) {
-            const int q0 = 2 * qp, q1 = 2 * qp + 1;
-            lo[e] = pack_bf16(v[4 * q0 + 2 * e] * (rs * scale[q0][2 * e]) + bias[q0][2 * e],
-                              v[4 * q0 + 2 * e + 1] * (rs * scale[q0][2 * e + 1]) + bias[q0][2 * e + 1]);
-            hi[e] = pack_bf16(v[4 * q1 + 2 * e] * (rs * scale[q1][2 * e]) + bias[q1][2 * e],
-                              v[4 * q1 + 2 * e + 1] * (rs * scale[q1][2 * e + 1]) + bias[q1][2 * e + 1]);
+          for (int r = 0; r < 4; ++r) {
+            const auto swapped = __builtin_amdgcn_permlane32_swap(f32_bits(v[8 * qp + r]), f32_bits(v[8 * qp + 4 + r]), false, false);
+            sums[r] = bits_f32(swapped[0]), sums[4 + r] = bits_f32(swapped[1]);
           }
-          // lanes 32.. of `lo` change places with lanes ..31 of `hi`: a lane then holds 8 consecutive outputs of its row
-          const auto s0 = __builtin_amdgcn_permlane32_swap(lo[0], hi[0], false, false);
-          const auto s1 = __builtin_amdgcn_permlane32_swap(lo[1], hi[1], false, false);
-          const uint32_t n = wn0 + 32 * j + 8 * (2 * qp + h);
-          if (m < p.m && n + 8 <= p.n) p.store_bf16x8(t.batch, m, n, U4{s0[0], s1[0], s0[1], s1[1]});
+          if (m < p.m && inside) p.finish8(t.batch, m, n, sums, columns, whole);
         }
       }
     }
@@ -175,36 +183,33 @@ __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_
   const uint32_t stream = mine * steps;
   load_setup(0);
 #pragma unroll
-  for (int c = 0; c < 8; ++c) load_piece(c, 0);
+  for (int c = 0; c < 2 * PER; ++c) load_piece(c, 0);
   load_advance();
 #pragma unroll
-  for (int c = 0; c < 8; ++c) load_piece(c, 1);  // (steps >= 2: a second step always exists)
+  for (int c = 0; c < 2 * PER; ++c) load_piece(c, 1);  // (steps >= 2: a second step always exists)
   load_advance();
-  __builtin_amdgcn_s_waitcnt(0x0f70 | 8);  // vmcnt(8): stage 0 has landed
+  __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * PER));  // vmcnt(2 PER): stage 0 has landed
   __syncthreads();
-  V8I a_first[2], a_second[2], b_first[TN2], b_second[TN2];  // of the first / second half of k (kk = 0 / 1)
+  V8I a_first[TM2], a_second[TM2], b_first[TN2], b_second[TN2];  // of the first / second half of k (kk = 0 / 1)
+  // fragment f of a half step, in the order the matrix-core instructions need them: row block 0, the column blocks, the other row blocks
+  auto read_fragment = [&](int f, V8I (&a)[TM2], V8I (&b)[TN2], int kk, uint32_t stage) {
+    if (f == 0) a[0] = fragment(at_a[kk], 0, stage);
+    else if (f <= TN2) b[f - 1 < TN2 ? f - 1 : 0] = fragment(at_b[kk], f - 1, stage);
+    else a[f - TN2 < TM2 ? f - TN2 : 0] = fragment(at_a[kk], f - TN2, stage);
+  };
 #pragma unroll
-  for (int j = 0; j < TN2; ++j) {
-    if (j < 2) a_first[j] = fragment(at_a[0], j, 0);
-    b_first[j] = fragment(at_b[0], j, 0);
-  }
+  for (int f = 0; f < FR; ++f) read_fragment(f, a_first, b_first, 0, 0);
 
   uint32_t tile = 0, s = 0;
   for (uint32_t t = 0; t < stream; ++t) {
     const uint32_t stage = t & 1u;
-    // First half of k: 8 matrix-core instructions, with the reads of the second half's fragments between them.
+    // First half of k, with the reads of the second half's fragments between the matrix-core instructions.
 #pragma unroll
-    for (int i = 0; i < TM2; ++i) {
-#pragma unroll
-      for (int j = 0; j < TN2; ++j) {
-        acc[i][j] = mfma_f8_32<FA, FB>(b_first[j], a_first[i], acc[i][j]);
-        if (i == 0) {
-          if (j == 0) a_second[0] = fragment(at_a[1], 0, stage);
-          b_second[j] = fragment(at_b[1], j, stage);
-          if (j == TN2 - 1) a_second[1] = fragment(at_a[1], 1, stage);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
+    for (int n = 0; n < NM; ++n) {
+      const int i = n / TN2, j = n % TN2;
+      acc[i][j] = multiply(b_first[j], a_first[i], acc[i][j]);
+      if (n < FR) read_fragment(n, a_second, b_second, 1, stage);
+      __builtin_amdgcn_sched_barrier(0);
     }
     // Every fragment of this stage is in registers, and this wave's loads of the next stage have landed.
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) and lgkmcnt(0)
@@ -212,21 +217,15 @@ __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_
     // Second half: the stage just read takes the loads of step t + 2; the other stage gives step t + 1's first fragments.
     const bool more = t + 2 < stream;
 #pragma unroll
-    for (int i = 0; i < TM2; ++i) {
-#pragma unroll
-      for (int j = 0; j < TN2; ++j) {
-        acc[i][j] = mfma_f8_32<FA, FB>(b_second[j], a_second[i], acc[i][j]);
-        if (i == 0) {
-          if (more) {
-            load_piece(2 * j, stage);
-            load_piece(2 * j + 1, stage);
-          }
-          if (j == 0) a_first[0] = fragment(at_a[0], 0, stage ^ 1u);
-          b_first[j] = fragment(at_b[0], j, stage ^ 1u);
-          if (j == TN2 - 1) a_first[1] = fragment(at_a[0], 1, stage ^ 1u);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+    for (int n = 0; n < NM; ++n) {
+      const int i = n / TN2, j = n % TN2;
+      acc[i][j] = multiply(b_second[j], a_second[i], acc[i][j]);
+      if (n < PER && more) {
+        load_piece(2 * n, stage);
+        load_piece(2 * n + 1, stage);
       }
+      if (n < FR) read_fragment(n, a_first, b_first, 0, stage ^ 1u);
+      __builtin_amdgcn_sched_barrier(0);
     }
     if (more) load_advance();
     if (++s == steps) {
@@ -244,10 +243,10 @@ bool mma_stream_serves(const P& p) {
   return p.k % BK == 0 && p.k >= 2 * BK && p.n % 8 == 0 && p.n >= 8 && p.m >= 1;
 }
 
-template <int FA, int FB, class P>
+template <int FA, int FB, int MATH, class P>
 int launch_mma_stream(const P& p, int compute_units, hipStream_t stream, std::string* err, const char* who) {
   constexpr uint32_t lds_bytes = 2 * (256 + 256) * BK;
-  auto kernel = mma_stream<FA, FB, P>;
+  auto kernel = mma_stream<FA, FB, MATH, P>;
   static bool configured = false;  // guarded by the runtime's stream mutex
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess) {
