@@ -1,5 +1,6 @@
-// The matrix-core kernel for large products with bfloat16 output: 256 x 256 tiles of A [m, k] x B [n, k]^T (rows of k
-// contiguous bytes, as in mma_tile.h) on 8 waves of 64 x 128, K in steps of 128 bytes through two LDS stages of 64 KiB.
+// The matrix-core kernel for large products with 16-bit outputs (float8 operands for _scaled_mm, 16-bit operands for
+// the matrix product and the many-row int8 product): 256 x 256 tiles of A [m, k] x B [n, k]^T (rows of k contiguous
+// bytes, as in mma_tile.h) on 8 waves of 64 x 128, K in steps of 128 bytes through two LDS stages of 64 KiB.
 // It differs from mma_tile in how a workgroup's time is laid out, after measuring where mma_tile's goes (one wave's
 // clock read at four points of every step): the matrix cores were busy 58-66 % of the cycles; the rest was the wave
 // issuing address arithmetic for its LDS-direct loads (380 cycles a step) and all eight waves starting every step
