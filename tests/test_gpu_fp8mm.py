@@ -209,6 +209,36 @@ def test_scaled_mm_stream_kernel(m, k, n, rowwise, with_bias, fb):
                                      want_mag=True)
         want = oracle.to_f32(want, oracle.BF16).astype(np.float64)
         assert (np.abs(oracle.to_f32(got[11], oracle.BF16) - want) <= ref_tol(want, mag, oracle.BF16) + HW_WINDOW * mag).all()
+    # float8 outputs with an output scale: 8 codes per store
+    for odt in (oracle.E4M3, oracle.E5M2):
+        out8 = {v: _dev.scaled_mm(bits(a), oracle.E4M3, bits(bt), ODT[FLOAT8[fb]], sa, sb, rowwise, out_dtype=odt, scale_result=16.0, variant=v, **kw)
+                for v in (11, 8)}
+        assert np.array_equal(out8[11], out8[8])
+        if m * n <= 1 << 20:
+            want, mag = oracle.scaled_mm(bits(a), oracle.E4M3, bits(bt), ODT[FLOAT8[fb]], sa, sb, rowwise, bias, oracle.F32, 16.0, odt, want_mag=True)
+            want = oracle.to_f32(want, odt).astype(np.float64)
+            fin = np.isfinite(want)
+            err = np.abs(oracle.to_f32(out8[11], odt).astype(np.float64) - want)
+            # (one step of the output format where the sums' small differences cross a rounding boundary: below the
+            #  smallest normal value a step is a fixed 2^-9 / 2^-16, not a fraction of the value)
+            step = 2.0 ** -9 if odt == oracle.E4M3 else 2.0 ** -16
+            assert (err[fin] <= (ref_tol(want, mag / 16.0, odt) + HW_WINDOW * mag / 16.0 + step)[fin]).all()
+
+
+def test_scaled_mm_zero_sums_keep_their_sign():
+    """A negative scale turns a zero sum into -0.0; without a bias it must stay -0.0 in the output (the kernels add the
+    bias from registers: an absent bias is -0.0f, whose addition changes nothing), with a bias of +0.0 it becomes +0.0."""
+    import _dev
+    m, k, n = 256, 256, 256
+    a = np.zeros((m, k), dtype=np.uint8)
+    bt = bits(torch.randn(n, k, generator=gen(1090)).to(FLOAT8[0]))
+    for variant in (11, 8, 1):
+        got = _dev.scaled_mm(a, oracle.E4M3, bt, oracle.E4M3, np.array([-1.0], np.float32), np.array([1.0], np.float32), False,
+                             out_dtype=oracle.BF16, variant=variant)
+        assert (got == 0x8000).all(), variant
+        got = _dev.scaled_mm(a, oracle.E4M3, bt, oracle.E4M3, np.array([-1.0], np.float32), np.array([1.0], np.float32), False,
+                             bias=np.zeros(n, np.float32), bias_dtype=oracle.F32, out_dtype=oracle.BF16, variant=variant)
+        assert (got == 0).all(), variant
 
 
 @pytest.mark.parametrize("fa,fb", [(FLOAT8[0], FLOAT8[0]), (FLOAT8[1], FLOAT8[0]), (FLOAT8[1], FLOAT8[1])])

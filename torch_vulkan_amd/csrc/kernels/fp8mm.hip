@@ -136,7 +136,7 @@ struct F8Problem : F8Params {
       s[0] = s[1] = s[2] = s[3] = w.sb_all;
     }
 #pragma unroll
-    for (int r = 0; r < 4; ++r) b[r] = bias ? load_any_f32(bias, col + r, bias_dtype) : 0.0f;
+    for (int r = 0; r < 4; ++r) b[r] = bias ? load_any_f32(bias, col + r, bias_dtype) : -0.0f;  // (adding -0.0f changes nothing, a zero's sign included)
   }
   __device__ __forceinline__ void store_bf16x8(uint32_t, uint32_t row, uint32_t col, const U4& v) const {
     stg<U4>(out + (uint64_t(row) * ldo + col) * 2, v);
@@ -156,11 +156,24 @@ struct F8Problem : F8Params {
   }
   __device__ __forceinline__ void finish8(uint32_t batch, uint32_t row, uint32_t col, const float (&t)[8], const Columns8& c, const Whole& w) const {
     const float rs = row_scale(row, w);
-    uint32_t packed[4];
+    float v[8];
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
-      packed[e] = pack_bf16(t[2 * e] * (rs * c.scale[2 * e]) + c.bias[2 * e], t[2 * e + 1] * (rs * c.scale[2 * e + 1]) + c.bias[2 * e + 1]);
-    store_bf16x8(batch, row, col, U4{packed[0], packed[1], packed[2], packed[3]});
+    for (int r = 0; r < 8; ++r) v[r] = t[r] * (rs * c.scale[r]) + c.bias[r];
+    if (out_dtype == VKT_BF16) {
+      store_bf16x8(batch, row, col, U4{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7])});
+    } else {  // float8 outputs: the output scale, 8 codes in one 8-byte store
+#pragma unroll
+      for (int r = 0; r < 8; ++r) v[r] *= w.inv;
+      uint32_t lo, hi;
+      if (out_dtype == VKT_E4M3) {
+        lo = pack2_fp8<VKT_E4M3>(v[0], v[1]) | pack2_fp8<VKT_E4M3>(v[2], v[3]) << 16;
+        hi = pack2_fp8<VKT_E4M3>(v[4], v[5]) | pack2_fp8<VKT_E4M3>(v[6], v[7]) << 16;
+      } else {
+        lo = pack2_fp8<VKT_E5M2>(v[0], v[1]) | pack2_fp8<VKT_E5M2>(v[2], v[3]) << 16;
+        hi = pack2_fp8<VKT_E5M2>(v[4], v[5]) | pack2_fp8<VKT_E5M2>(v[6], v[7]) << 16;
+      }
+      stg<U2>(out + uint64_t(row) * ldo + col, U2{lo, hi});
+    }
   }
   template <class F>
   __device__ __forceinline__ void for_output_type(bool full, const Whole& w, F&& f) const {
@@ -198,12 +211,13 @@ int launch_tile(const F8Params& p, int compute_units, hipStream_t stream, std::s
       problem, compute_units, stream, err, "fp8mm");
 }
 
-// The stream kernel, where it serves the problem (bfloat16 output in aligned rows); -2: it does not.
+// The stream kernel, where it serves the problem (bfloat16 or float8 output in aligned rows); -2: it does not.
 template <int FA, int FB>
 int launch_stream(const F8Params& p, int compute_units, hipStream_t stream, std::string* err) {
   F8Problem problem;
   static_cast<F8Params&>(problem) = p;
-  if (p.out_dtype != VKT_BF16 || p.ldo % 8 || p.out % 16 || !mma_stream_serves(problem)) return -2;
+  const bool float8_out = p.out_dtype == VKT_E4M3 || p.out_dtype == VKT_E5M2;
+  if (!(p.out_dtype == VKT_BF16 || float8_out) || p.ldo % 8 || p.out % (float8_out ? 8 : 16) || !mma_stream_serves(problem)) return -2;
   return launch_mma_stream<FA, FB, kMathFp8>(problem, compute_units, stream, err, "fp8mm");
 }
 
@@ -214,8 +228,8 @@ int launch_formats(const F8Params& p, uint32_t variant, int compute_units, hipSt
   // 128x128, 16x16x128); 3: 256x128; 4: 256x256 with the 32x32x64 MFMA (measured ~10 % faster
   // than 16x16x128 at equal work); 5: as 4 with global-to-LDS direct loads when k is a
   // multiple of 128 (else 4); 8: as 5 with 8 waves of 64x128 instead of 4 of 128x128 (two waves per SIMD cover each
-  // other's waits: 8192^3 2.34-2.42 -> 2.56-2.59 PFLOP/s; what large float8 outputs get).  11: the stream kernel of
-  // mma_stream.h where it serves the problem (large bfloat16 outputs get it), else 8.  255: the one-thread-per-output kernel.
+  // other's waits: 8192^3 2.34-2.42 -> 2.56-2.59 PFLOP/s; what they get where the stream kernel does not serve).  11: the stream kernel of
+  // mma_stream.h where it serves the problem (large bfloat16 and float8 outputs get it), else 8.  255: the one-thread-per-output kernel.
   // 6 / 7: the exact path (float8 widened to bfloat16 in registers, 32x32x16 bfloat16 MFMA) on
   // 256x256 / 128x128 tiles: what float32 and float16 outputs get.
   const bool big = uint64_t(p.m) * p.n >= (1ull << 20);
