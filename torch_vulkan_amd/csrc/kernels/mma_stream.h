@@ -38,10 +38,12 @@ namespace vkt {
 namespace {
 
 // One LDS-direct load of 16 bytes per lane: global address `base` + `offset` + OFF, LDS address `lds_at` + OFF + 16 * lane.
+// (M0 is written in every statement that uses it and by nothing else in this kernel: no other instruction the compiler
+// emits here reads it, and a clobber of a reserved register is not something the compiler honours anyway.)
 template <int OFF>
 __device__ __forceinline__ void load_to_lds(uint32_t offset, uint64_t base, uint32_t lds_at) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3" ::"v"(offset), "s"(base), "s"(lds_at), "i"(OFF)
-               : "memory", "m0");
+               : "memory");
 }
 
 template <int FA, int FB, int MATH, class P>
