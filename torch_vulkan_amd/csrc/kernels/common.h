@@ -201,6 +201,30 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   return __builtin_bit_cast(uint32_t, V2{static_cast<__bf16>(a), static_cast<__bf16>(b)});
 }
 
+// Four float32 -> four bfloat16 in two words, as pack_bf16 writes them.  NaN is rare: one comparison per pair of values
+// and one branch of the whole wave decide whether any lane has to look at its values one by one.
+__device__ __forceinline__ void pack_bf16x4(const float (&v)[4], uint32_t (&packed)[2]) {
+  using V2 = __bf16 __attribute__((ext_vector_type(2)));
+  const bool odd = __builtin_isunordered(v[0], v[1]) | __builtin_isunordered(v[2], v[3]);
+  if (__builtin_amdgcn_ballot_w64(odd) != 0) {
+    packed[0] = pack_bf16(v[0], v[1]), packed[1] = pack_bf16(v[2], v[3]);
+  } else {
+    packed[0] = __builtin_bit_cast(uint32_t, V2{static_cast<__bf16>(v[0]), static_cast<__bf16>(v[1])});
+    packed[1] = __builtin_bit_cast(uint32_t, V2{static_cast<__bf16>(v[2]), static_cast<__bf16>(v[3])});
+  }
+}
+
+// Four float32 -> four values of the 16-bit type T in two words.
+template <class T>
+__device__ __forceinline__ void pack_16bit_x4(const float (&v)[4], uint32_t (&packed)[2]) {
+  if constexpr (T::dtype == VKT_BF16) {
+    pack_bf16x4(v, packed);
+  } else {
+    packed[0] = uint32_t(f32_to_f16(v[0])) | uint32_t(f32_to_f16(v[1])) << 16;
+    packed[1] = uint32_t(f32_to_f16(v[2])) | uint32_t(f32_to_f16(v[3])) << 16;
+  }
+}
+
 // ---- wave64 reductions through DPP (no LDS traffic) ----
 template <int CTRL, int ROW_MASK = 0xf>
 __device__ __forceinline__ float dpp_f32(float v) {

@@ -141,39 +141,40 @@ struct F8Problem : F8Params {
   __device__ __forceinline__ void store_bf16x8(uint32_t, uint32_t row, uint32_t col, const U4& v) const {
     stg<U4>(out + (uint64_t(row) * ldo + col) * 2, v);
   }
-  // the stream kernel's epilogue: 8 consecutive bfloat16 outputs of a row
-  struct Columns8 {
-    float scale[8], bias[8];
+  // the stream kernel's epilogue (bfloat16 or float8 outputs)
+  struct Rows {
+    float scale;
   };
-  __device__ __forceinline__ Columns8 columns8(uint32_t, uint32_t col, const Whole& w) const {
-    Columns8 c;
-    float s0[4], s1[4], b0[4], b1[4];
-    column_terms(col, w, s0, b0);
-    column_terms(col + 4, w, s1, b1);
-#pragma unroll
-    for (int r = 0; r < 4; ++r) c.scale[r] = s0[r], c.scale[4 + r] = s1[r], c.bias[r] = b0[r], c.bias[4 + r] = b1[r];
+  struct Columns4 {
+    float scale[4], bias[4];
+  };
+  __device__ __forceinline__ Rows rows(uint32_t, uint32_t row, const Whole& w) const { return Rows{row_scale(row, w)}; }
+  __device__ __forceinline__ Columns4 columns4(uint32_t, uint32_t col, const Whole& w) const {
+    Columns4 c;
+    column_terms(col, w, c.scale, c.bias);
     return c;
   }
-  __device__ __forceinline__ void finish8(uint32_t batch, uint32_t row, uint32_t col, const float (&t)[8], const Columns8& c, const Whole& w) const {
-    const float rs = row_scale(row, w);
-    float v[8];
+  __device__ __forceinline__ bool narrow(const Whole&) const { return out_dtype != VKT_BF16; }
+  __device__ __forceinline__ void finish4(uint32_t, uint32_t, uint32_t, const float (&t)[4], const Rows& r, const Columns4& c, const Whole&,
+                                          float (&v)[4]) const {
 #pragma unroll
-    for (int r = 0; r < 8; ++r) v[r] = t[r] * (rs * c.scale[r]) + c.bias[r];
+    for (int e = 0; e < 4; ++e) v[e] = t[e] * (r.scale * c.scale[e]) + c.bias[e];
+  }
+  __device__ __forceinline__ void pack4(const float (&f)[4], const Whole& w, uint32_t (&packed)[2]) const {
     if (out_dtype == VKT_BF16) {
-      store_bf16x8(batch, row, col, U4{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7])});
-    } else {  // float8 outputs: the output scale, 8 codes in one 8-byte store
-#pragma unroll
-      for (int r = 0; r < 8; ++r) v[r] *= w.inv;
-      uint32_t lo, hi;
-      if (out_dtype == VKT_E4M3) {
-        lo = pack2_fp8<VKT_E4M3>(v[0], v[1]) | pack2_fp8<VKT_E4M3>(v[2], v[3]) << 16;
-        hi = pack2_fp8<VKT_E4M3>(v[4], v[5]) | pack2_fp8<VKT_E4M3>(v[6], v[7]) << 16;
-      } else {
-        lo = pack2_fp8<VKT_E5M2>(v[0], v[1]) | pack2_fp8<VKT_E5M2>(v[2], v[3]) << 16;
-        hi = pack2_fp8<VKT_E5M2>(v[4], v[5]) | pack2_fp8<VKT_E5M2>(v[6], v[7]) << 16;
-      }
-      stg<U2>(out + uint64_t(row) * ldo + col, U2{lo, hi});
+      pack_bf16x4(f, packed);
+    } else {  // float8 outputs: the output scale
+      const float v[4] = {f[0] * w.inv, f[1] * w.inv, f[2] * w.inv, f[3] * w.inv};
+      packed[0] = out_dtype == VKT_E4M3 ? pack2_fp8<VKT_E4M3>(v[0], v[1]) | pack2_fp8<VKT_E4M3>(v[2], v[3]) << 16
+                                        : pack2_fp8<VKT_E5M2>(v[0], v[1]) | pack2_fp8<VKT_E5M2>(v[2], v[3]) << 16;
+      packed[1] = 0;
     }
+  }
+  __device__ __forceinline__ void store8(uint32_t, uint32_t row, uint32_t col, const U4& v) const {
+    stg<U4>(out + (uint64_t(row) * ldo + col) * 2, v);
+  }
+  __device__ __forceinline__ void store8_narrow(uint32_t, uint32_t row, uint32_t col, const U2& v) const {
+    stg<U2>(out + uint64_t(row) * ldo + col, v);
   }
   template <class F>
   __device__ __forceinline__ void for_output_type(bool full, const Whole& w, F&& f) const {

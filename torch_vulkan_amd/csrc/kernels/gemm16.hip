@@ -67,25 +67,28 @@ struct GemmProblem {
     if (w.vec_ok && full) f(std::integral_constant<int, T::dtype>{});
     else f(std::integral_constant<int, -1>{});
   }
-  // the stream kernel's epilogue: 8 consecutive outputs of a row, one 16-byte store (C rows and batches 16-byte aligned)
-  struct Columns8 {};
-  __device__ __forceinline__ Columns8 columns8(uint32_t, uint32_t, const Whole&) const { return Columns8{}; }
-  __device__ __forceinline__ void finish8(uint32_t batch, uint32_t row, uint32_t col, const float (&t)[8], const Columns8&, const Whole&) const {
-    float v[8];
+  // the stream kernel's epilogue (C rows and batches 16-byte aligned)
+  struct Rows {};
+  struct Columns4 {};
+  __device__ __forceinline__ Rows rows(uint32_t, uint32_t, const Whole&) const { return Rows{}; }
+  __device__ __forceinline__ Columns4 columns4(uint32_t, uint32_t, const Whole&) const { return Columns4{}; }
+  __device__ __forceinline__ bool narrow(const Whole&) const { return false; }
+  __device__ __forceinline__ void finish4(uint32_t batch, uint32_t row, uint32_t col, const float (&t)[4], const Rows&, const Columns4&, const Whole&,
+                                          float (&v)[4]) const {
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
+    for (int r = 0; r < 4; ++r) {
       v[r] = alpha * t[r];
       if (cin != 0) {  // beta == 0 never reads Cin (it may hold NaN): then cin is 0
         const int64_t at = int64_t(batch) * cin_sb + int64_t(row) * cin_sm + int64_t(col + r) * cin_sn;
         v[r] += beta * load_f32<T>(cin + uint64_t(at * 2));
       }
     }
-    uint32_t packed[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e)
-      packed[e] = T::dtype == VKT_BF16 ? pack_bf16(v[2 * e], v[2 * e + 1]) : uint32_t(f32_to_f16(v[2 * e])) | uint32_t(f32_to_f16(v[2 * e + 1])) << 16;
-    stg<U4>(c + uint64_t((int64_t(batch) * c_sb + int64_t(row) * c_sm + int64_t(col)) * 2), U4{packed[0], packed[1], packed[2], packed[3]});
   }
+  __device__ __forceinline__ void pack4(const float (&v)[4], const Whole&, uint32_t (&packed)[2]) const { pack_16bit_x4<T>(v, packed); }
+  __device__ __forceinline__ void store8(uint32_t batch, uint32_t row, uint32_t col, const U4& v) const {
+    stg<U4>(c + uint64_t((int64_t(batch) * c_sb + int64_t(row) * c_sm + int64_t(col)) * 2), v);
+  }
+  __device__ __forceinline__ void store8_narrow(uint32_t, uint32_t, uint32_t, const U2&) const {}
 };
 
 // Any strides: one thread per output, float32 accumulation.
@@ -219,29 +222,31 @@ struct Q8GemmProblem {
     if (w.vec_ok && full) f(std::integral_constant<int, T::dtype>{});
     else f(std::integral_constant<int, -1>{});
   }
-  // the stream kernel's epilogue: 8 consecutive outputs of a row (n a multiple of 8, C 16-byte aligned)
-  struct Columns8 {
-    float s[8];
+  // the stream kernel's epilogue (n a multiple of 8, C and the scales 16-byte aligned)
+  struct Rows {};
+  struct Columns4 {
+    float s[4];
   };
-  __device__ __forceinline__ Columns8 columns8(uint32_t, uint32_t col, const Whole&) const {
-    Columns8 cs;
-    const U4 raw = ldg<U4>(scales + uint64_t(col) * 2);  // (col a multiple of 8; the scales' address is checked by the launcher)
+  __device__ __forceinline__ Rows rows(uint32_t, uint32_t, const Whole&) const { return Rows{}; }
+  __device__ __forceinline__ Columns4 columns4(uint32_t, uint32_t col, const Whole&) const {
+    Columns4 cs;
+    const U2 raw = ldg<U2>(scales + uint64_t(col) * 2);  // (col a multiple of 4)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
+    for (int e = 0; e < 2; ++e) {
       if constexpr (T::dtype == VKT_BF16) cs.s[2 * e] = bits_f32(raw[e] << 16), cs.s[2 * e + 1] = bits_f32(raw[e] & 0xffff0000u);
       else cs.s[2 * e] = f16_to_f32(uint16_t(raw[e])), cs.s[2 * e + 1] = f16_to_f32(uint16_t(raw[e] >> 16));
     }
     return cs;
   }
-  __device__ __forceinline__ void finish8(uint32_t, uint32_t row, uint32_t col, const float (&t)[8], const Columns8& cs, const Whole&) const {
-    uint32_t packed[4];
+  __device__ __forceinline__ bool narrow(const Whole&) const { return false; }
+  __device__ __forceinline__ void finish4(uint32_t, uint32_t, uint32_t, const float (&t)[4], const Rows&, const Columns4& cs, const Whole&,
+                                          float (&v)[4]) const {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float v0 = t[2 * e] * cs.s[2 * e], v1 = t[2 * e + 1] * cs.s[2 * e + 1];
-      packed[e] = T::dtype == VKT_BF16 ? pack_bf16(v0, v1) : uint32_t(f32_to_f16(v0)) | uint32_t(f32_to_f16(v1)) << 16;
-    }
-    stg<U4>(c + (uint64_t(row) * n + col) * 2, U4{packed[0], packed[1], packed[2], packed[3]});
+    for (int r = 0; r < 4; ++r) v[r] = t[r] * cs.s[r];
   }
+  __device__ __forceinline__ void pack4(const float (&v)[4], const Whole&, uint32_t (&packed)[2]) const { pack_16bit_x4<T>(v, packed); }
+  __device__ __forceinline__ void store8(uint32_t, uint32_t row, uint32_t col, const U4& v) const { stg<U4>(c + (uint64_t(row) * n + col) * 2, v); }
+  __device__ __forceinline__ void store8_narrow(uint32_t, uint32_t, uint32_t, const U2&) const {}
 };
 
 // 16 int8 values per thread -> 16 values of T (integers of magnitude <= 128 are exact in both 16-bit types).

@@ -24,11 +24,14 @@
 // thirds of the fragment bytes per instruction.  Tried: correct, but the compiler keeps fragments in the
 // accumulators' half of the file and spills both inside the loop, 860 bytes of scratch and ten times slower.)
 // The problem type P supplies the operands as mma_tile's does (a, b, lda, ldb in bytes, m, n, k in bytes, batches,
-// a_batch, b_batch) and the epilogue of 8 consecutive outputs of a row, which one lane holds after the accumulators'
-// halves have changed lanes (v_permlane32_swap, as float32: the epilogue's arithmetic comes after):
-//   whole()                                       per-launch constants
-//   columns8(batch, n, whole)                     per-lane constants of columns n .. n + 7
-//   finish8(batch, m, n, sums[8], columns, whole) finish and store them (16-bit outputs: one 16-byte store)
+// a_batch, b_batch) and the epilogue of 4 consecutive outputs of a row, as one lane holds them in its accumulators:
+//   whole()                                            per-launch constants
+//   rows(batch, m, whole)                              per-lane constants of row m
+//   columns4(batch, n, whole)                          per-lane constants of columns n .. n + 3
+//   finish4(batch, m, n, sums[4], rows, columns4, whole, values[4])   the outputs as float32
+//   pack4(values[4], whole, out[2])                    converted: two words of 16-bit outputs, or one of 8-bit
+//   narrow(whole)                                      whether outputs are 8-bit
+//   store8(batch, m, n, U4) / store8_narrow(batch, m, n, U2)     8 consecutive outputs of a row
 // k a multiple of 128 bytes and at least 256, n a multiple of 8, 16-byte aligned operand rows.
 #pragma once
 
@@ -53,7 +56,7 @@ __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_
   constexpr uint32_t BM = 256, BN = 256, STAGE = (BM + BN) * BK, B_AT = BM * BK;
   constexpr int WAVES = WM * 2, TM2 = 8 / WM, TN2 = 4;  // a wave's (256 / WM) x 128 as 32 x 32 matrix-core tiles
   constexpr int ROWS = 256 / WAVES, PER = ROWS / 8;    // rows of each operand tile a wave brings; loads per operand and step
-  constexpr int NM = TM2 * TN2, FR = TM2 + TN2;        // matrix-core tiles and fragments per half step
+  constexpr int NM = TM2 * TN2;                        // matrix-core tiles per half step
   constexpr uint32_t BIAS = 3072;  // keeps the per-lane offsets non-negative (they carry -1024 (i % 4) for load i)
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)(lds)));
@@ -110,30 +113,37 @@ __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_
       default: load_to_lds<3072>(offset, base, at); break;
     }
   };
+  // (The rare paths of the loop, a new tile for the loads and the epilogue, end by waiting for what they have asked
+  // for themselves.  Scalar and LDS results share a counter: with scalar loads possibly pending where the paths meet
+  // again the compiler would wait for EVERY fragment read before the next step's first matrix-core instruction.  The
+  // epilogue waits for its vector loads and stores as well, which the middle of the next step would do anyway: a
+  // vector load that the compiler believes pending there costs a wait at the head of every step, for the loads into
+  // LDS that still have half a step to land.)
   auto load_advance = [&]() {
     if (++load_s == steps) {
       load_s = 0;
       if (++load_tile < mine) load_setup(load_tile);
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
     }
   };
 
   // Fragment addresses.  Lane: row l32 of a 32-row block, 32 bytes of k at chunks 4 kk + 2 h and + 1; the swizzle key of
   // the row depends on l32 alone, so one base serves every block (immediate offsets) and the chunk variants are XORs.
   const uint32_t key = (l32 >> 1) & 7u, x0 = l32 * BK + (((2 * h) ^ key) << 4);
-  uint32_t at_a[2][2], at_b[2][2];  // [kk][low / high chunk], of stage 0
+  // (The second operand's addresses differ from the first's by the same amount in every lane: one set of registers.)
+  uint32_t at[2][2];  // [kk][low / high chunk]: the first operand's, of stage 0
 #pragma unroll
   for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      const uint32_t x = x0 ^ (kk * 64) ^ (c * 16);
-      at_a[kk][c] = x + wm * (TM2 * 32 * BK);
-      at_b[kk][c] = x + B_AT + wn * (128 * BK);
-    }
-  auto fragment = [&](const uint32_t (&at)[2], uint32_t block, uint32_t stage) {
-    const V4I lo = *reinterpret_cast<const V4I*>(lds + stage * STAGE + at[0] + block * (32 * BK));
-    const V4I hi = *reinterpret_cast<const V4I*>(lds + stage * STAGE + at[1] + block * (32 * BK));
+    for (int c = 0; c < 2; ++c) at[kk][c] = (x0 ^ (kk * 64) ^ (c * 16)) + wm * (TM2 * 32 * BK);
+  const uint32_t a_to_b = B_AT + wn * (128 * BK) - wm * (TM2 * 32 * BK);
+  auto fragment = [&](const uint32_t (&at)[2], uint32_t uniform) {
+    const V4I lo = *reinterpret_cast<const V4I*>(lds + uniform + at[0]);
+    const V4I hi = *reinterpret_cast<const V4I*>(lds + uniform + at[1]);
     return V8I{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
+  auto fragment_a = [&](int kk, uint32_t block, uint32_t stage) { return fragment(at[kk], stage * STAGE + block * (32 * BK)); };
+  auto fragment_b = [&](int kk, uint32_t block, uint32_t stage) { return fragment(at[kk], stage * STAGE + a_to_b + block * (32 * BK)); };
   auto multiply = [&](const V8I& b, const V8I& a, const V16F& c) {
     if constexpr (MATH == kMathFp8) {
       return mfma_f8_32<FA, FB>(b, a, c);
@@ -155,28 +165,58 @@ __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_
   const auto whole = p.whole();
 
   // The epilogue, straight from the accumulators.  A 32 x 32 matrix-core tile leaves lane l with row l % 32 and, for
-  // q = 0..3, columns 8 q + 4 (l / 32) .. + 3: two lanes 32 apart hold the two halves of 8 consecutive outputs;
-  // v_permlane32_swap puts them together (lanes below 32 take chunk q = 0 or 2 of their row, lanes from 32 chunk 1 or 3).
+  // q = 0..3, columns 8 q + 4 (l / 32) .. + 3.  A lane finishes and packs its own values; two lanes 32 apart then hold
+  // the two halves of 8 consecutive outputs and v_permlane32_swap puts them together (lanes below 32 take chunk
+  // q = 0 or 2 of their row, lanes from 32 chunk 1 or 3), one store per 8 outputs.
+  // What the epilogue costs is the time its stores take to drain (every workgroup stores its tile at about the same
+  // time, with the matrix cores idle), and that depends on their order: two stores in a row that together write 64
+  // consecutive bytes of each of their 32 rows (this order: column block, row block, chunk pair) take 322 us on
+  // 8192^3 where the order column block, chunk pair, row block takes 347; eight in a row that fill two whole
+  // 128-byte lines per row are no faster, non-temporal stores are 1.5 times slower, and waiting after every few
+  // stores, or starting the workgroups a few microseconds apart, only costs.
   auto epilogue = [&](const Tile& t) {
     const uint32_t wm0 = t.m0 + wm * (TM2 * 32), wn0 = t.n0 + wn * 128;
+    typename P::Rows rows[TM2];
+#pragma unroll
+    for (int i = 0; i < TM2; ++i) {
+      const uint32_t m = wm0 + 32 * i + l32;
+      rows[i] = p.rows(t.batch, m < p.m ? m : p.m - 1, whole);
+    }
+    const bool narrow = p.narrow(whole);
 #pragma unroll
     for (int j = 0; j < TN2; ++j) {
+      uint32_t first_column[4];  // of this lane's four columns in chunk q of column block j (inside the matrix)
+      typename P::Columns4 columns[4];
 #pragma unroll
-      for (int qp = 0; qp < 2; ++qp) {
-        const uint32_t n = wn0 + 32 * j + 8 * (2 * qp + h);
-        const bool inside = n + 8 <= p.n;
-        const auto columns = p.columns8(t.batch, inside ? n : p.n - 8, whole);
+      for (int q = 0; q < 4; ++q) {
+        const uint32_t n = wn0 + 32 * j + 8 * q + 4 * h;
+        first_column[q] = n + 4 <= p.n ? n : p.n - 4;
+        columns[q] = p.columns4(t.batch, first_column[q], whole);
+      }
 #pragma unroll
-        for (int i = 0; i < TM2; ++i) {
-          const uint32_t m = wm0 + 32 * i + l32;
-          const V16F& v = acc[i][j];
-          float sums[8];
+      for (int i = 0; i < TM2; ++i) {
+        const uint32_t m = wm0 + 32 * i + l32, row = m < p.m ? m : p.m - 1;
+        const V16F& v = acc[i][j];
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const auto swapped = __builtin_amdgcn_permlane32_swap(f32_bits(v[8 * qp + r]), f32_bits(v[8 * qp + 4 + r]), false, false);
-            sums[r] = bits_f32(swapped[0]), sums[4 + r] = bits_f32(swapped[1]);
+        for (int qp = 0; qp < 2; ++qp) {
+          const uint32_t n = wn0 + 32 * j + 8 * (2 * qp + h);
+          const float first[4] = {v[8 * qp], v[8 * qp + 1], v[8 * qp + 2], v[8 * qp + 3]};
+          const float second[4] = {v[8 * qp + 4], v[8 * qp + 5], v[8 * qp + 6], v[8 * qp + 7]};
+          float f0[4], f1[4];
+          p.finish4(t.batch, row, first_column[2 * qp], first, rows[i], columns[2 * qp], whole, f0);
+          p.finish4(t.batch, row, first_column[2 * qp + 1], second, rows[i], columns[2 * qp + 1], whole, f1);
+          uint32_t lo[2], hi[2];
+          p.pack4(f0, whole, lo);
+          p.pack4(f1, whole, hi);
+          const bool inside = m < p.m && n + 8 <= p.n;
+          if (!narrow) {
+            const auto s0 = __builtin_amdgcn_permlane32_swap(lo[0], hi[0], false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(lo[1], hi[1], false, false);
+            if (inside) p.store8(t.batch, m, n, U4{s0[0], s1[0], s0[1], s1[1]});
+          } else {
+            const auto s0 = __builtin_amdgcn_permlane32_swap(lo[0], hi[0], false, false);
+            if (inside) p.store8_narrow(t.batch, m, n, U2{s0[0], s0[1]});
           }
-          if (m < p.m && inside) p.finish8(t.batch, m, n, sums, columns, whole);
         }
       }
     }
@@ -194,16 +234,24 @@ __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_
   __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * PER));  // vmcnt(2 PER): stage 0 has landed
   __syncthreads();
   V8I a_first[TM2], a_second[TM2], b_first[TN2], b_second[TN2];  // of the first / second half of k (kk = 0 / 1)
-  // fragment f of a half step, in the order the matrix-core instructions need them: row block 0, the column blocks, the other row blocks
-  auto read_fragment = [&](int f, V8I (&a)[TM2], V8I (&b)[TN2], int kk, uint32_t stage) {
-    if (f == 0) a[0] = fragment(at_a[kk], 0, stage);
-    else if (f <= TN2) b[f - 1 < TN2 ? f - 1 : 0] = fragment(at_b[kk], f - 1, stage);
-    else a[f - TN2 < TM2 ? f - TN2 : 0] = fragment(at_a[kk], f - TN2, stage);
+  // the fragments of a half step, read between the first TN2 matrix-core instructions of the half step before, in the
+  // order they are needed: with instruction 0 row block 0 and column block 0, with instruction j column block j, with
+  // the last of them the other row blocks (all reads are out within the first half of the instructions, so the wait
+  // for them at the barrier finds them done)
+  auto read_fragments = [&](int n, V8I (&a)[TM2], V8I (&b)[TN2], int kk, uint32_t stage) {
+    if (n >= TN2) return;
+    if (n == 0) a[0] = fragment_a(kk, 0, stage);
+    b[n < TN2 ? n : 0] = fragment_b(kk, n, stage);
+    if (n == TN2 - 1) {
+#pragma unroll
+      for (int i = 1; i < TM2; ++i) a[i] = fragment_a(kk, i, stage);
+    }
   };
 #pragma unroll
-  for (int f = 0; f < FR; ++f) read_fragment(f, a_first, b_first, 0, 0);
+  for (int n = 0; n < TN2; ++n) read_fragments(n, a_first, b_first, 0, 0);
 
   uint32_t tile = 0, s = 0;
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): (as above: nothing scalar pending on the way into the loop either)
   for (uint32_t t = 0; t < stream; ++t) {
     const uint32_t stage = t & 1u;
     // First half of k, with the reads of the second half's fragments between the matrix-core instructions.
@@ -211,7 +259,7 @@ __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_
     for (int n = 0; n < NM; ++n) {
       const int i = n / TN2, j = n % TN2;
       acc[i][j] = multiply(b_first[j], a_first[i], acc[i][j]);
-      if (n < FR) read_fragment(n, a_second, b_second, 1, stage);
+      read_fragments(n, a_second, b_second, 1, stage);
       __builtin_amdgcn_sched_barrier(0);
     }
     // Every fragment of this stage is in registers, and this wave's loads of the next stage have landed.
@@ -227,7 +275,7 @@ __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_
         load_piece(2 * n, stage);
         load_piece(2 * n + 1, stage);
       }
-      if (n < FR) read_fragment(n, a_first, b_first, 0, stage ^ 1u);
+      read_fragments(n, a_first, b_first, 0, stage ^ 1u);
       __builtin_amdgcn_sched_barrier(0);
     }
     if (more) load_advance();
@@ -235,6 +283,7 @@ __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_
       epilogue(tile_at(tile));
       clear();
       s = 0, ++tile;
+      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) and lgkmcnt(0)
     }
   }
   __builtin_amdgcn_s_waitcnt(0x0070);  // nothing of this workgroup may still be on its way into LDS
