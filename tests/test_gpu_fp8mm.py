@@ -225,6 +225,34 @@ def test_scaled_mm_stream_kernel(m, k, n, rowwise, with_bias, fb):
             assert (err[fin] <= (ref_tol(want, mag / 16.0, odt) + HW_WINDOW * mag / 16.0 + step)[fin]).all()
 
 
+def test_scaled_mm_stream_kernel_nan_and_inf():
+    """NaN and infinities through the stream kernel's epilogue, whose bfloat16 conversion looks at its values one by one
+    only where a wave has seen a NaN: NaN operands (both e4m3fn codes), e5m2 infinities of both signs (inf - inf and
+    0 x inf included) and a NaN in the bias.  Every NaN output is 0x7fc0 as c10 writes it, the outputs are bit for bit
+    the tile kernel's, and NaN / infinity sit where the oracle has them."""
+    import _dev
+    m, k, n = 512, 256, 520
+    a = bits(torch.randn(m, k, generator=gen(1095)).to(FLOAT8[0])).copy()
+    bt = bits(torch.randn(n, k, generator=gen(1096)).to(FLOAT8[1])).copy()
+    a[3, 17], a[300, 5] = 0x7F, 0xFF            # e4m3fn NaN of either sign
+    a[7, :] = 0                                  # a zero row: 0 x inf below
+    bt[9, 40], bt[9, 41] = 0x7C, 0xFC            # e5m2 +inf and -inf in one column: inf - inf or +-inf
+    bt[260, 100] = 0x7C                          # +inf alone
+    bt[519, 0] = 0x7E                            # e5m2 NaN
+    bias = torch.randn(n, generator=gen(1097)).numpy()
+    bias[33] = np.nan
+    sa, sb = np.array([0.5], dtype=np.float32), np.array([2.0], dtype=np.float32)
+    got = {v: _dev.scaled_mm(a, oracle.E4M3, bt, oracle.E5M2, sa, sb, False, bias=bias, bias_dtype=oracle.F32, out_dtype=oracle.BF16, variant=v)
+           for v in (11, 8)}
+    assert np.array_equal(got[11], got[8])
+    want = oracle.to_f32(oracle.scaled_mm(a, oracle.E4M3, bt, oracle.E5M2, sa, sb, False, bias, oracle.F32, None, oracle.BF16), oracle.BF16)
+    have = oracle.to_f32(got[11], oracle.BF16)
+    assert np.array_equal(np.isnan(have), np.isnan(want)) and np.isnan(want[3]).all() and np.isnan(want[:, 33]).all() and np.isnan(want[7, 9])
+    assert np.array_equal(np.isinf(have), np.isinf(want)) and np.array_equal(np.sign(have[np.isinf(have)]), np.sign(want[np.isinf(want)]))
+    assert np.isinf(want[:, 260]).sum() > m // 2
+    assert (got[11][np.isnan(have)] == 0x7FC0).all()
+
+
 def test_scaled_mm_zero_sums_keep_their_sign():
     """A negative scale turns a zero sum into -0.0; without a bias it must stay -0.0 in the output (the kernels add the
     bias from registers: an absent bias is -0.0f, whose addition changes nothing), with a bias of +0.0 it becomes +0.0."""
