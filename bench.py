@@ -379,10 +379,10 @@ BASELINE = {
     "c2_m64_k14336_n4096": lambda abi, s, w: wl_q8(abi, 64, 14336, 4096, abi.BF16, s, w),
     "c3_int4_m32": lambda abi, s, w: wl_q4(abi, 32, 4096, 11008, 32, max(s // 4, 5), w),
     "c2_m1_k14336_n4096": lambda abi, s, w: wl_q8(abi, 1, 14336, 4096, abi.BF16, s, w),
-    "c5_fp8_rowwise_70b": lambda abi, s, w: wl_fp8(abi, 4096, 8192, 28672, True, max(s // 10, 5), max(w // 4, 3), seed=1050),
+    "c5_fp8_rowwise_70b": lambda abi, s, w: wl_fp8(abi, 4096, 8192, 28672, True, max(s // 2, 10), max(w, 5), seed=1050),
     "c1_f32_m1_k4096_n4096": lambda abi, s, w: wl_q8(abi, 1, 4096, 4096, abi.F32, s, w, seed=1010),
     "c3_int4_m1": lambda abi, s, w: wl_q4(abi, 1, 4096, 11008, 32, s, w),
-    "c4_fp8_8192": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 10, 5), max(w // 4, 3)),
+    "c4_fp8_8192": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 2, 10), max(w, 5)),
 }
 # Beside the BASELINE configurations (--all, or by name): many rows of the same operators, the steps either side of
 # the path, the planner off the Llama grid, config 4's launch on all-zero operands.
@@ -406,7 +406,7 @@ OTHER = {
     "affine_quantize_256mi": lambda abi, s, w: wl_affine(abi, "quantize", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
     "affine_dequantize_256mi": lambda abi, s, w: wl_affine(abi, "dequantize", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
     "affine_fake_quant_256mi": lambda abi, s, w: wl_affine(abi, "fake_quant", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
-    "c4_fp8_8192_zero_operands": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 10, 5), max(w // 4, 3), zero_operands=True),
+    "c4_fp8_8192_zero_operands": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 2, 10), max(w, 5), zero_operands=True),
 }
 # Ceilings measured in the same run (`ceilings` of the output line; also selectable by name): bare 16-byte loads of
 # each GEMV configuration's weight bytes in its kernel's launch geometry, a persistent-grid read, a device copy of known
