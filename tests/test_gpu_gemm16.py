@@ -72,6 +72,32 @@ def test_gemm16_stream_kernel(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_gemm16_stream_kernel_nan_and_inf(dtype):
+    """NaN and infinities through the stream kernel's epilogue (its bfloat16 conversion looks at its values one by one
+    only where a wave has seen a NaN): a NaN operand of either sign, infinities of both signs in one column (inf - inf)
+    and against a zero row (0 x inf).  Bit for bit the tile kernel's outputs; NaN and infinities where the oracle has
+    them; a bfloat16 NaN is 0x7fc0 as c10 writes it."""
+    import _dev
+    m, k, n = 512, 128, 520
+    a = bits((torch.randn(m, k, generator=gen(16)) * 0.5).to(dtype)).copy()
+    w = bits((torch.randn(n, k, generator=gen(17)) * 0.5).to(dtype)).copy()
+    nan, inf = (0x7FC1, 0x7F80) if dtype == torch.bfloat16 else (0x7E01, 0x7C00)
+    a[3, 17], a[300, 5] = nan, nan | 0x8000
+    a[7, :] = 0
+    w[9, 40], w[9, 41] = inf, inf | 0x8000
+    w[260, 100] = inf
+    got = {v: _dev.gemm16(a, w.T, ODT[dtype], variant=v) for v in (6, 3)}
+    assert np.array_equal(got[6], got[3])
+    want = oracle.to_f32(oracle.gemm16(a, w.T, ODT[dtype]), ODT[dtype])
+    have = oracle.to_f32(got[6], ODT[dtype])
+    assert np.array_equal(np.isnan(have), np.isnan(want)) and np.isnan(want[3]).all() and np.isnan(want[7, 9]) and np.isnan(want[7, 260])
+    assert np.array_equal(np.isinf(have), np.isinf(want)) and np.array_equal(np.sign(have[np.isinf(have)]), np.sign(want[np.isinf(want)]))
+    assert np.isinf(want[:, 260]).sum() > m // 2
+    if dtype == torch.bfloat16:
+        assert (got[6][np.isnan(have)] == 0x7FC0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
 @pytest.mark.parametrize("variant", [0, 3, 4, 5])
 @pytest.mark.parametrize("m,k,n", [(128, 64, 136), (264, 192, 520), (1032, 128, 1024), (8, 64, 8)])
 def test_gemm16_k_major_operands(dtype, variant, m, k, n):
