@@ -92,9 +92,14 @@ __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_
     const Tile t = tile_at(index);
     load_a = p.a + uint64_t(t.batch) * p.a_batch + uint64_t(t.m0) * p.lda - BIAS;
     load_b = p.b + uint64_t(t.batch) * p.b_batch + uint64_t(t.n0) * p.ldb - BIAS;
+    // (The lane's rows and chunks are worked out anew for every tile: as values that do not change in the loop the
+    // compiler computes them once, finds no register to keep them in, and reloads them here from scratch memory,
+    // each reload waiting for every load into LDS in flight: 1.5 us per tile.)
+    uint32_t ln = lane;
+    asm volatile("" : "+v"(ln));
 #pragma unroll
     for (uint32_t i = 0; i < uint32_t(PER); ++i) {
-      const uint32_t r = wave * ROWS + 8 * i + (lane >> 3), c = (lane & 7u) ^ ((r >> 1) & 7u);
+      const uint32_t r = wave * ROWS + 8 * i + (ln >> 3), c = (ln & 7u) ^ ((r >> 1) & 7u);
       const uint32_t ra = t.m0 + r < p.m ? r : p.m - 1 - t.m0, rb = t.n0 + r < p.n ? r : p.n - 1 - t.n0;  // rows past the end repeat the last one
       off_a[i] = ra * p.lda + c * 16 + BIAS - 1024 * (i & 3u);
       off_b[i] = rb * p.ldb + c * 16 + BIAS - 1024 * (i & 3u);
