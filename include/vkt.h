@@ -278,9 +278,13 @@ typedef struct F8Params {
 } F8Params;
 
 /* "probe_read", spec {GEOMETRY} and "probe_mfma_f8", spec {OPERANDS}: calibration kernels for the rooflines (what
- * a launch geometry can stream, what the fp8 matrix cores sustain on given operand bits); they read src [n, k] bytes
- * (probe_read) or run `iters` iterations of 4 matrix-core instructions per wave, 4 waves on every compute unit
- * (probe_mfma_f8), and write nothing (dst must be a valid address).  "probe_delay", spec {}: one wave that waits
+ * a launch geometry can stream, what the fp8 matrix cores sustain on given operand bits).  probe_read reads src and
+ * writes nothing (dst: any valid 4-byte address): GEOMETRY 0, 1, 3 read the n * k bytes at src (k a multiple of 16);
+ * GEOMETRY 2 reads the int4 streaming side-car of an [n, k] weight with blocks of 32, so src holds
+ * vkt_qmm4c_bytes(n, k, 32) bytes and n is a multiple of 16, k of 4096 (anything else is refused).  probe_mfma_f8
+ * runs `iters` iterations of 4 matrix-core instructions per wave, 4 waves on every compute unit, reads no memory
+ * and stores the loop's shader cycles and 100 MHz ticks at dst + 64 and dst + 72: dst holds at least 80 bytes and is
+ * 8-byte aligned.  "probe_delay", spec {}: one wave that waits
  * `iters` microseconds (at most 100000) and exits; a timing loop queues it in front of its launches so that the host
  * has queued them all before the device starts on them.  No counterpart in the reference.  32 bytes. */
 typedef struct ProbeParams {

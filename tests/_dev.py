@@ -308,9 +308,9 @@ def fake_quant(x, dtype, scales, zero_points, qmin, qmax, axis=None, skew=0):
     return out, m
 
 
-def aminmax(x, dtype, ld=None):
+def aminmax(x, dtype, ld=None, static=False):
     """(min, max) float32 per row of a 2-d array (float32, or a uint16 view of float16 / bfloat16 values); ld: row
-    pitch in elements of the device copy (rows further apart than they are long)."""
+    pitch in elements of the device copy (rows further apart than they are long).  static: through vkt_dispatch_static."""
     x = np.ascontiguousarray(x)
     rows, cols = x.shape
     ld = ld or cols
@@ -318,5 +318,5 @@ def aminmax(x, dtype, ld=None):
     padded[:, :cols] = x
     src = abi.Buffer.from_numpy(padded)
     lo, hi = abi.Buffer(4 * rows), abi.Buffer(4 * rows)
-    abi.dispatch("aminmax", [], abi.MinMaxParams(src=src.address, out_min=lo.address, out_max=hi.address, rows=rows, cols=cols, ld=ld, dtype=dtype))
+    abi.dispatch("aminmax", [], abi.MinMaxParams(src=src.address, out_min=lo.address, out_max=hi.address, rows=rows, cols=cols, ld=ld, dtype=dtype), static=static)
     return lo.to_numpy(np.float32, (rows,)), hi.to_numpy(np.float32, (rows,))

@@ -6,6 +6,7 @@
 #include <memory>
 #include <string>
 
+#include "limits.h"
 #include "pool.h"
 
 namespace {
@@ -83,5 +84,8 @@ void vkt_test_pool_stats(void* p, uint64_t* out) {
 }
 
 const char* vkt_test_pool_error(void* p) { return static_cast<TestPool*>(p)->err.c_str(); }
+
+// the stride bound of the stream kernel's 32-bit operand offsets (kernels/limits.h)
+int shim_mma_stream_strides_ok(uint64_t lda, uint64_t ldb) { return vkt::mma_stream_strides_ok(lda, ldb) ? 1 : 0; }
 
 }  // extern "C"

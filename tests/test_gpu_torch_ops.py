@@ -162,6 +162,30 @@ def test_int4_under_inference_mode(tv):
         assert torch.equal(first.cpu(), want) and torch.equal(again.cpu(), want) and torch.equal(one_row.cpu(), want[:1])
 
 
+def test_int4_inference_tensor_rewritten_in_place(tv):
+    """In-place writes under torch.inference_mode() bump no version counter: the op layer's write paths drop the
+    side-cars of the written storage themselves, so the next product sees the new weights (both side-car layouts)."""
+    n, k, bs = 24, 128, 32
+    x = int4_rows(5, k, torch.float32, seed=32)
+    packs = [torch._dyn_quant_pack_4bit_weight(*int4_weights(n, k, bs, seed=s, bias=True), bs, k, n) for s in (41, 42, 43)]
+    wants = [torch._dyn_quant_matmul_4bit(x, p, bs, k, n) for p in packs]
+    with torch.inference_mode(), on_gpu(tv):
+        packed = packs[0].to("vk")
+        assert packed.is_inference()
+        for rows in (5, 1):
+            assert torch.equal(torch._dyn_quant_matmul_4bit(x[:rows].to("vk"), packed, bs, k, n).cpu(), wants[0][:rows])
+        packed.copy_(packs[1])  # host -> device copy into the same storage
+        for rows in (5, 1):
+            assert torch.equal(torch._dyn_quant_matmul_4bit(x[:rows].to("vk"), packed, bs, k, n).cpu(), wants[1][:rows])
+        packed.copy_(packs[2].to("vk"))  # device -> device copy
+        for rows in (5, 1):
+            assert torch.equal(torch._dyn_quant_matmul_4bit(x[:rows].to("vk"), packed, bs, k, n).cpu(), wants[2][:rows])
+        packed.view(-1)[: n * k // 2].zero_()  # a fill through a view: every nibble byte 0, weights -8
+        zeroed = packs[2].clone()
+        zeroed[: n * k // 2] = 0
+        assert torch.equal(torch._dyn_quant_matmul_4bit(x.to("vk"), packed, bs, k, n).cpu(), torch._dyn_quant_matmul_4bit(x, zeroed, bs, k, n))
+
+
 def test_int4_sidecar_follows_writes(tv):
     """A side-car belongs to one version of the packed tensor: writing into the packed weights must show in the
     next product."""

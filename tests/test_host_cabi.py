@@ -176,3 +176,17 @@ def test_pool_zero_and_huge():
     assert z[1] == 256
     with pytest.raises(MemoryError):
         p.alloc((1 << 64) - 1)
+
+
+def test_stream_kernel_stride_bound():
+    """The stream kernel's per-lane operand offsets are 32-bit (row 255 of a tile at 255 * ld bytes, plus chunk
+    offset and bias): strides that would wrap must be refused by the launchers' predicate (kernels/limits.h)."""
+    L = ctypes.CDLL(os.path.join(os.path.dirname(abi.LIB_PATH), "libvkt_hosttest.so"))
+    L.shim_mma_stream_strides_ok.argtypes = [ctypes.c_uint64, ctypes.c_uint64]
+    ok = L.shim_mma_stream_strides_ok
+    assert ok(8192, 8192) and ok(28672, 8192) and ok(1 << 20, 64)
+    limit = ((1 << 32) - 4096) // 255  # the largest stride whose row 255 still fits with the bias
+    assert ok(limit - 1, 16) and ok(16, limit - 1)
+    assert not ok(limit + 1, 16) and not ok(16, limit + 1) and not ok(1 << 25, 1 << 25)
+    for ld in (limit - 1, limit + 1, 1 << 24, 1 << 31):
+        assert bool(ok(ld, 128)) == (255 * ld + 4096 < 1 << 32)

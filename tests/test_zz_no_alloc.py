@@ -2,6 +2,8 @@
 the library instead of pool memory.  Its results are compared with vkt_dispatch's on products that are split over
 workgroups (so that the workspace is really used), on calls in a row of decreasing size (the array keeps the last
 call's contents), and a product whose split needs more than the array holds must be refused."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -49,3 +51,41 @@ def test_static_dispatch_refuses_more_than_the_array_holds():
     _, c64, mag = oracle.qmm8(a, oracle.BF16, b, s, want_f64=True)
     for out in (want, got):
         assert (np.abs(oracle.bf16_to_f32(out) - c64) <= ref_tol(c64, mag, oracle.BF16)).all()
+
+
+def _memory():
+    a, r = abi.u64(), abi.u64()
+    abi.lib().vkt_memory_stats(ctypes.byref(a), ctypes.byref(r))
+    return a.value, r.value
+
+
+def test_static_dispatch_allocates_nothing():
+    """With the pool's kernel memory given back (vkt_empty_cache drops the workspace that vkt_dispatch had taken), a
+    static dispatch of a split product leaves the pool's figures as they were, and its result stands against the oracle
+    without vkt_dispatch having run in between."""
+    abi.device_info()
+    m, k, n = 64, 14336, 4096
+    a, b, s = _case(m, k, n, 300)
+    da, db, ds = abi.Buffer.from_numpy(a), abi.Buffer.from_numpy(b), abi.Buffer.from_numpy(s)
+    dc = abi.Buffer(m * n * 2)
+    p = abi.Q8Params(a=da.address, b=db.address, scales=ds.address, c=dc.address, m=m, n=n, k=k, a_sm=k, a_sk=1)
+    abi.check(abi.lib().vkt_empty_cache())
+    before = _memory()
+    abi.dispatch("qmm8_bf16", [0, 0], p, ((n + 63) // 64, 1), static=True)
+    abi.synchronize()
+    assert _memory() == before
+    got = dc.to_numpy(np.uint16, (m, n))
+    _, c64, mag = oracle.qmm8(a, oracle.BF16, b, s, want_f64=True)
+    assert (np.abs(oracle.bf16_to_f32(got) - c64) <= ref_tol(c64, mag, oracle.BF16)).all()
+
+
+def test_static_dispatch_aminmax():
+    """The other user of the workspace: row ranges whose rows are split over workgroups (partial ranges meet in the
+    workspace).  Two calls in a row, the second smaller; equal to vkt_dispatch's and to numpy's."""
+    abi.device_info()
+    for rows, cols, seed in ((3, 300000, 7), (2, 70000, 8)):
+        x = (torch.randn(rows, cols, generator=gen(seed)) * 3).numpy()
+        want = _dev.aminmax(x, oracle.F32)
+        got = _dev.aminmax(x, oracle.F32, static=True)
+        assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
+        assert np.array_equal(got[0], x.min(axis=1)) and np.array_equal(got[1], x.max(axis=1))

@@ -102,6 +102,8 @@ class F8QuantParams(ctypes.Structure):
 
 
 class ProbeParams(ctypes.Structure):
+    # "probe_read": dst any valid 4-byte address; geometry 2 reads vkt_qmm4c_bytes(n, k, 32) bytes at src (n a multiple
+    # of 16, k of 4096).  "probe_mfma_f8": dst holds at least 80 bytes, 8-byte aligned (clock counts at +64 and +72).
     _fields_ = [("src", u64), ("dst", u64), ("n", u32), ("k", u32), ("iters", u32), ("pad", u32)]
 
 

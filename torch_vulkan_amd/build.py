@@ -84,7 +84,7 @@ def build(force=False, verbose=True):
     # host-only test shim for the allocator policy (no HIP)
     shim = os.path.join(os.path.dirname(HERE), "tests", "pool_shim.cpp")
     if os.path.exists(shim) and (force or _stale(HOSTTEST, [shim] + headers)):
-        subprocess.check_call(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-I", os.path.join(CSRC, "core"), "-o", HOSTTEST, shim])
+        subprocess.check_call(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-I", os.path.join(CSRC, "core"), "-I", os.path.join(CSRC, "kernels"), "-o", HOSTTEST, shim])
     return LIB
 
 

@@ -79,6 +79,9 @@ struct Runtime {
   // widened-weights region, grown on demand.  Guarded by pool_mutex (the Machine fields also by stream_mutex).
   Allocation workspace_alloc{}, widened_alloc{};
   std::atomic<uint64_t> workspace_ready{0}, widened_ready{0};  // bytes of each that dispatches may count on
+  // the smallest widened-weights size the pool has refused since the last vkt_empty_cache: such products run on the
+  // row-block kernels without asking again (every failed attempt may trim the pool and wait for the device)
+  std::atomic<uint64_t> widened_refused{UINT64_MAX};
   uint64_t static_scratch = 0;  // device address of `scratch` on this runtime's device
 
   // Makes sure the workspace exists and the widened-weights region holds `widened` bytes.  Called by vkt_dispatch
@@ -94,10 +97,12 @@ struct Runtime {
       machine.workspace = a.address, machine.workspace_bytes = kWorkspaceBytes;
       workspace_ready.store(kWorkspaceBytes, std::memory_order_release);
     }
-    if (widened > widened_alloc.size && widened <= kMaxWidenedBytes) {
+    if (widened > widened_alloc.size && widened <= kMaxWidenedBytes && widened < widened_refused.load(std::memory_order_relaxed)) {
       Allocation a;
       std::string ignored;  // (without memory for it the row-block kernels run)
-      if (pool->alloc(widened, &a, &ignored)) {
+      if (!pool->alloc(widened, &a, &ignored)) {
+        widened_refused.store(widened, std::memory_order_relaxed);
+      } else {
         std::lock_guard<std::mutex> stream_lock(stream_mutex);
         if (widened_alloc.size) pool->free(widened_alloc);
         widened_alloc = a;
@@ -115,6 +120,7 @@ struct Runtime {
     workspace_alloc = widened_alloc = Allocation{};
     machine.workspace = machine.workspace_bytes = machine.scratch = machine.scratch_bytes = 0;
     workspace_ready.store(0, std::memory_order_release), widened_ready.store(0, std::memory_order_release);
+    widened_refused.store(UINT64_MAX, std::memory_order_relaxed);
   }
 
   ~Runtime() {
@@ -452,11 +458,16 @@ int vkt_dispatch(const char* name, const uint32_t* spec, size_t nspec, const uin
     std::memcpy(&p, push, sizeof(p));
     widened = q8_gemm_scratch_bytes(p, dtype_of_suffix(name + 5), rt->machine);
   }
-  if ((rt->workspace_ready.load(std::memory_order_acquire) == 0 || widened > rt->widened_ready.load(std::memory_order_acquire)) &&
-      !rt->ensure_kernel_memory(widened, &err))
-    return fail(err);
-  std::lock_guard<std::mutex> lock(rt->stream_mutex);
-  return queue_kernel(*rt, rt->machine, name, spec, nspec, push, npush, gx, gy, gz);
+  for (;;) {
+    if ((rt->workspace_ready.load(std::memory_order_acquire) == 0 ||
+         (widened > rt->widened_ready.load(std::memory_order_acquire) && widened < rt->widened_refused.load(std::memory_order_relaxed))) &&
+        !rt->ensure_kernel_memory(widened, &err))
+      return fail(err);
+    std::lock_guard<std::mutex> lock(rt->stream_mutex);
+    // (a vkt_empty_cache between the check above and this lock has taken the workspace away: take it again)
+    if (rt->machine.workspace_bytes == 0) continue;
+    return queue_kernel(*rt, rt->machine, name, spec, nspec, push, npush, gx, gy, gz);
+  }
 }
 
 int vkt_dispatch_static(const char* name, const uint32_t* spec, size_t nspec, const uint8_t* push, size_t npush,

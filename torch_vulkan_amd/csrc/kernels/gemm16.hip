@@ -132,7 +132,8 @@ int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t
     // both operands contiguous along k (x @ w.T): the stream kernel where it serves (8192^3: 0.94-1.00 -> 0.89 ms)
     if (!TRA && !TRB && variant == 3) variant = 6;
   }
-  const bool stream_ok = direct_ok && g.k >= 2 * BK && p.n % 8 == 0 && p.c_sm % 8 == 0 && p.c_sb % 8 == 0 && p.c % 16 == 0;
+  const bool stream_ok = direct_ok && g.k >= 2 * BK && p.n % 8 == 0 && p.c_sm % 8 == 0 && p.c_sb % 8 == 0 && p.c % 16 == 0 &&
+                         mma_stream_strides_ok(g.lda, g.ldb);
   if (variant == 6 && !stream_ok) variant = 3;
   if constexpr (!TRA && !TRB) {
     // 6: the stream kernel (mma_stream.h) where it serves the problem: k a multiple of 64 values and at least 128, n a multiple of 8, C in 16-byte aligned rows
@@ -283,7 +284,7 @@ int launch_q8_gemm_t(const Q8Params& p, const Machine& mc, hipStream_t stream, s
   g.batches = 1, g.a_batch = 0, g.b_batch = 0, g.c = p.c, g.scales = p.scales;
   const bool large = uint64_t((p.m + 255) / 256) * ((p.n + 255) / 256) >= uint64_t(mc.compute_units);
   if (g.k % BK == 0) {
-    if (large && g.k >= 2 * BK && p.n % 8 == 0 && p.c % 16 == 0 && p.scales % 16 == 0)
+    if (large && g.k >= 2 * BK && p.n % 8 == 0 && p.c % 16 == 0 && p.scales % 16 == 0 && mma_stream_strides_ok(g.lda, g.ldb))
       return launch_mma_stream<0, 0, MATH>(g, mc.compute_units, stream, err, "qmm8");
     if (large) return launch_mma_tile<2, 2, 8, 8, 0, 0, true, true, MATH>(g, mc.compute_units, stream, err, "qmm8");
     return launch_mma_tile<2, 2, 4, 4, 0, 0, true, true, MATH>(g, mc.compute_units, stream, err, "qmm8");

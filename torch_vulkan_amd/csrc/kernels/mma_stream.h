@@ -35,6 +35,7 @@
 // k a multiple of 128 bytes and at least 256, n a multiple of 8, 16-byte aligned operand rows.
 #pragma once
 
+#include "limits.h"
 #include "mma_tile.h"
 
 namespace vkt {
@@ -297,7 +298,7 @@ __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_
 // Whether mma_stream serves problem p (the caller has checked the operands' alignment).
 template <class P>
 bool mma_stream_serves(const P& p) {
-  return p.k % BK == 0 && p.k >= 2 * BK && p.n % 8 == 0 && p.n >= 8 && p.m >= 1;
+  return p.k % BK == 0 && p.k >= 2 * BK && p.n % 8 == 0 && p.n >= 8 && p.m >= 1 && mma_stream_strides_ok(p.lda, p.ldb);
 }
 
 template <int FA, int FB, int MATH, class P>

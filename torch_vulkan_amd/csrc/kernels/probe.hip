@@ -142,6 +142,12 @@ int launch_probe_read(const ProbeParams& p, uint32_t geometry, const Machine& mc
     *err = "probe_read: null or unaligned address, or k not a multiple of 16";
     return -1;
   }
+  // geometry 2 walks the int4 streaming side-car of an [n, k] weight in whole tiles of 16 columns and whole rounds of
+  // 4096 values: src holds vkt_qmm4c_bytes(n, k, 32) bytes, of which (n / 16) (k / 4096) 40960 are read
+  if (geometry == 2 && (p.n % 16 != 0 || p.k % 4096 != 0)) {
+    *err = "probe_read: GEOMETRY 2 takes n a multiple of 16 and k a multiple of 4096";
+    return -1;
+  }
   switch (geometry) {
     case 0: hipLaunchKernelGGL((probe_read_gemv<2, 4>), dim3((p.n + 1) / 2), dim3(256), 0, stream, p); break;
     case 1: hipLaunchKernelGGL((probe_read_gemv<2, 2>), dim3((p.n + 3) / 4), dim3(256), 0, stream, p); break;
@@ -174,8 +180,9 @@ int launch_probe_delay(const ProbeParams& p, hipStream_t stream, std::string* er
 }
 
 int launch_probe_mfma(const ProbeParams& p, uint32_t operands, const Machine& mc, hipStream_t stream, std::string* err) {
-  if (!p.dst || p.iters == 0) {
-    *err = "probe_mfma_f8: null address or no iterations";
+  // (the loop's clock counts are stored at dst + 64 and dst + 72: dst holds at least 80 bytes)
+  if (!p.dst || (p.dst & 7) || p.iters == 0) {
+    *err = "probe_mfma_f8: null or unaligned address (dst: 80 bytes, 8-byte aligned), or no iterations";
     return -1;
   }
   const dim3 grid(uint32_t(mc.compute_units));

@@ -104,7 +104,9 @@ uint64_t gpu_address(const at::TensorBase& t) {
 }
 
 uint64_t gpu_address_out(const at::TensorBase& t) {
-  return t.numel() == 0 ? 0 : reinterpret_cast<uint64_t>(t.mutable_data_ptr());  // (materializes copy-on-write storage)
+  if (t.numel() == 0) return 0;
+  note_write(t);
+  return reinterpret_cast<uint64_t>(t.mutable_data_ptr());  // (materializes copy-on-write storage)
 }
 
 namespace {
@@ -266,6 +268,7 @@ const char* float_label(at::ScalarType t) {
 bool copy_strided_on_device(const at::Tensor& dst, uint64_t src_base, const std::vector<int64_t>& src_strides,
                             at::ScalarType src_type) {
   if (dst.is_conj() || dst.is_neg()) return false;
+  note_write(dst);
   const bool same = src_type == dst.scalar_type();
   const char* label = size_label(dst.element_size());
   std::string kernel;
@@ -317,6 +320,7 @@ bool fill_on_device(const at::Tensor& self, const at::Scalar& value) {
   const char* label = size_label(self.element_size());
   if (!label || self.is_conj() || self.is_neg()) return false;
   if (self.numel() == 0) return true;
+  note_write(self);
   at::Tensor v = at::scalar_tensor(value, at::TensorOptions().dtype(self.scalar_type()));
   uint64_t bits[2] = {0, 0};
   std::memcpy(bits, v.const_data_ptr(), size_t(v.element_size()));
@@ -336,6 +340,7 @@ at::Tensor copy_from(const at::Tensor& src, const at::Tensor& dst, bool non_bloc
   TORCH_CHECK(src.sizes() == dst.sizes() || src.numel() == 1 || at::is_expandable_to(src.sizes(), dst.sizes()),
               "copy_: shapes do not broadcast: ", src.sizes(), " -> ", dst.sizes());
   if (dst.numel() == 0) return dst;
+  if (is_vk(dst)) note_write(dst);
   const bool same_layout = src.scalar_type() == dst.scalar_type() && src.sizes() == dst.sizes() &&
                            src.strides() == dst.strides() && plain(src) && plain(dst) && !src.is_conj() &&
                            !src.is_neg();

@@ -14,6 +14,7 @@
 #include <torch/library.h>
 
 #include <algorithm>
+#include <atomic>
 #include <mutex>
 #include <sstream>
 #include <unordered_map>
@@ -146,19 +147,28 @@ struct SideCarKeyHash {
 struct SideCarEntry {
   c10::weak_intrusive_ptr<c10::StorageImpl> owner;
   int64_t version;
+  bool inference;  // built from an inference tensor: no version counter tells it stale, vk::note_write drops it
   at::Tensor compact;
 };
 constexpr size_t kSweepEvery = 64;
 std::mutex g_sidecar_mutex;
 std::unordered_map<SideCarKey, SideCarEntry, SideCarKeyHash> g_sidecars;
 size_t g_sidecar_inserts = 0;
+std::atomic<size_t> g_inference_sidecars{0};  // entries with `inference` set (read without the mutex by note_write)
 
 // The version that tells whether a tensor was written to since its side-car was built.  Inference tensors carry
-// no counter (and cannot be written in place outside inference mode).
+// no counter: in-place writes under torch.inference_mode() are legal and bump nothing, so their entries are dropped
+// by the write paths of the op layer instead (sidecars_note_write).
 int64_t write_version(const at::Tensor& t) { return t.is_inference() ? 0 : static_cast<int64_t>(t._version()); }
 
+std::unordered_map<SideCarKey, SideCarEntry, SideCarKeyHash>::iterator erase_sidecar_locked(
+    std::unordered_map<SideCarKey, SideCarEntry, SideCarKeyHash>::iterator it) {
+  if (it->second.inference) g_inference_sidecars.fetch_sub(1, std::memory_order_relaxed);
+  return g_sidecars.erase(it);
+}
+
 void sweep_sidecars_locked() {
-  for (auto it = g_sidecars.begin(); it != g_sidecars.end();) it = it->second.owner.expired() ? g_sidecars.erase(it) : std::next(it);
+  for (auto it = g_sidecars.begin(); it != g_sidecars.end();) it = it->second.owner.expired() ? erase_sidecar_locked(it) : std::next(it);
 }
 
 at::Tensor sidecar_for(const at::Tensor& packed, int64_t bs, int64_t K, int64_t N, bool with_bias, uint32_t layout) {
@@ -172,18 +182,33 @@ at::Tensor sidecar_for(const at::Tensor& packed, int64_t bs, int64_t K, int64_t 
 
   at::Tensor compact = at::empty({static_cast<int64_t>(bytes)}, packed.options().dtype(at::kByte));
   Q4PackParams p{};
-  p.packed = gpu_address(packed), p.compact = gpu_address_out(compact);
+  // (the new tensor's address directly: gpu_address_out would report a write to the cache, whose mutex is held here)
+  p.packed = gpu_address(packed), p.compact = reinterpret_cast<uint64_t>(compact.mutable_data_ptr());
   p.n = static_cast<uint32_t>(N), p.k = static_cast<uint32_t>(K), p.bs = static_cast<uint32_t>(bs), p.has_bias = with_bias ? 1u : 0u;
   dispatch("qmm4c_pack", {layout}, p, 1);
   if (++g_sidecar_inserts % kSweepEvery == 0) sweep_sidecars_locked();
-  g_sidecars.insert_or_assign(key, SideCarEntry{c10::weak_intrusive_ptr<c10::StorageImpl>(packed.storage().getWeakStorageImpl()), version, compact});
+  if (const auto stale = g_sidecars.find(key); stale != g_sidecars.end()) erase_sidecar_locked(stale);  // (an older version's entry)
+  const bool inference = packed.is_inference();
+  if (inference) g_inference_sidecars.fetch_add(1, std::memory_order_relaxed);
+  g_sidecars.insert_or_assign(key, SideCarEntry{c10::weak_intrusive_ptr<c10::StorageImpl>(packed.storage().getWeakStorageImpl()), version, inference, compact});
   return compact;
+}
+
+// A write into an inference tensor: the side-cars built from its storage go (the next product rebuilds them).
+void sidecars_note_write(const at::TensorBase& t) {
+  if (g_inference_sidecars.load(std::memory_order_relaxed) == 0 || !t.is_inference() || !t.has_storage()) return;
+  const c10::StorageImpl* storage = t.storage().unsafeGetStorageImpl();
+  std::lock_guard<std::mutex> lock(g_sidecar_mutex);
+  for (auto it = g_sidecars.begin(); it != g_sidecars.end();) it = it->first.storage == storage ? erase_sidecar_locked(it) : std::next(it);
 }
 
 // (entries, bytes) of the side-car cache after dropping dead entries; clear = true empties it.
 std::tuple<int64_t, int64_t> sidecar_cache(bool clear) {
   std::lock_guard<std::mutex> lock(g_sidecar_mutex);
-  if (clear) g_sidecars.clear();
+  if (clear) {
+    g_sidecars.clear();
+    g_inference_sidecars.store(0, std::memory_order_relaxed);
+  }
   sweep_sidecars_locked();
   int64_t bytes = 0;
   for (const auto& kv : g_sidecars) bytes += kv.second.compact.numel();
@@ -425,6 +450,9 @@ std::tuple<at::Tensor, at::Tensor> fp8_quant_rowwise(const at::Tensor& x, at::Sc
 }
 
 }  // namespace
+
+void note_write(const at::TensorBase& t) { sidecars_note_write(t); }
+
 }  // namespace vk
 
 TORCH_LIBRARY(vk, m) {

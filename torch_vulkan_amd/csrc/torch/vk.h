@@ -30,6 +30,11 @@ c10::Allocator* allocator();
 uint64_t gpu_address(const at::TensorBase& t);
 uint64_t gpu_address_out(const at::TensorBase& t);
 
+// Tells the op layer that the memory of vk tensor `t` is about to be written: whatever it has derived from the old
+// contents and cannot tell stale by a version counter (inference tensors carry none) is dropped.  Called by
+// gpu_address_out and by the copy and fill paths.
+void note_write(const at::TensorBase& t);
+
 // Records that `op` ran on the CPU instead of the GPU; under TORCH_VK_STRICT raises
 // NotImplementedError instead (reference vk.h: record_fallback).
 void record_fallback(const std::string& op);
