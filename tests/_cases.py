@@ -90,3 +90,45 @@ def float8_case(fa, fb, out_dtype, rowwise, shape=FLOAT8_SHAPE, seeds=FLOAT8_SEE
     bias = draw(("normal", (n,)), seeds["bias"]).bfloat16() if out_dtype == torch.bfloat16 else None
     sr = torch.tensor(2.0) if out_dtype == torch.float8_e4m3fn else None
     return Float8Case(a, b, sa, sb, bias, sr, out_dtype or fa)
+
+
+# ---------------------------------------------------------------- the rows beside the path (tables)
+INF, NAN = float("inf"), float("nan")
+# float8 casts: two normal draws (spreads 3 and 300, 300 values each) and the values at which a conversion saturates,
+# overflows, underflows, or meets NaN, infinities and the signed zero (test_fallback_ops.py:469-485 lists the same)
+CAST_DRAWS = [(("normal", (300,), 3), 0), (("normal", (300,), 300), 1)]
+CAST_EDGES = [0.0, -0.0, INF, -INF, NAN, 448.0, 464.0, 57344.0, 61440.0, 1e-9, -1e-9, 2.0**-9, 2.0**-10, 2.0**-17, 1e30]
+# 16-bit products (m, k, n): whole tiles, ragged edges, k = 1, tall and flat, both tile sizes of the matrix-core kernel
+GEMM16_SHAPES = [(64, 32, 64), (65, 33, 63), (17, 200, 129), (128, 1, 96), (3, 1000, 5), (300, 256, 260), (304, 256, 264)]
+GEMM16_SEEDS = {"a": 1, "b": 2}
+GEMM16_BATCHED = {"a": (("normal", (3, 40, 72)), 3), "b": (("normal", (3, 50, 72)), 4), "bias": (("normal", (50,)), 5)}
+# affine quantisation: 40 values of spread 20 and the ones that meet NaN, infinities, ties and the integer ranges
+AFFINE_DRAW = (("normal", (40,), 20), 0)
+AFFINE_EDGES = [NAN, INF, -INF, 0.05, 0.15, -0.05, 1e30, 3e9]
+AFFINE_QPARAMS = (0.1, 5)
+FAKE_QUANT_ROWS = [[-1.3, 0.0, 0.26, 4.0], [NAN, INF, -0.5, 1e-3]]
+FAKE_QUANT_TENSOR = {"scale": 0.05, "zero_point": 3, "range": (0, 255)}
+FAKE_QUANT_BIG = (("normal", (2, 3, 500), 4), 4)
+# the fused observer: four steps whose inputs widen and drift, the last with a small averaging constant
+OBSERVER_STEPS = [(0.1, 0.0, 0.25), (1.1, -0.5, 0.25), (2.1, -1.0, 0.25), (3.1, -1.5, 0.01)]  # (spread, shift, averaging constant)
+OBSERVER_INPUT = (4, 3, 5)
+
+
+def cast_values():
+    return torch.cat([draw(r, seed) for r, seed in CAST_DRAWS] + [torch.tensor(CAST_EDGES)])
+
+
+def affine_values():
+    return torch.cat([draw(*AFFINE_DRAW), torch.tensor(AFFINE_EDGES)]).view(6, 8)
+
+
+def per_channel_cases():
+    """(input, axis, scales, zero points) of the per-channel fake quantisation: the small matrix with integer and
+    float zero points, a larger tensor along each axis, a 16-bit one, a transposed view."""
+    small, big = torch.tensor(FAKE_QUANT_ROWS), draw(*FAKE_QUANT_BIG)
+    wide_scales = draw(("uniform", (500,), 10), 5) + 0.01
+    return [(small, 0, torch.tensor([0.05, 0.2]), torch.tensor([3, 250], dtype=torch.int32)),
+            (small, 0, torch.tensor([0.05, 0.2]), torch.tensor([3.25, 250.5])),
+            (big, 1, torch.tensor([0.05, 0.2, 0.01]), torch.tensor([3, 250, 128], dtype=torch.int32)),
+            (big.bfloat16(), 2, wide_scales, torch.randint(0, 255, (500,), dtype=torch.int32, generator=torch.Generator().manual_seed(6))),
+            (big.transpose(0, 2), 0, wide_scales, draw(("uniform", (500,)), 7) * 200)]

@@ -3,7 +3,6 @@ to the CPU, against the oracle (and PyTorch's CPU op where it has one), on the r
 (tests/python/test_quant.py:20-21,61-63,101-103, kept as tables in _cases.py), on the frozen fixtures under
 tests/golden/, and on the op layer's own behaviour (side-car cache, inference tensors, empty products, errors).
 The C++ op layer (csrc/torch/quant.cpp) reaches the kernels through the C ABI."""
-import contextlib
 import os
 
 import numpy as np
@@ -11,8 +10,9 @@ import pytest
 import torch
 
 import oracle
-from _cases import (FLOAT8, FLOAT8_OUT, FLOAT8_PAIRS, INT4_SHAPES, INT8_SHAPES, draw, float8_case, int4_rows, int4_weights,
-                    int8_case)
+from _cases import (AFFINE_QPARAMS, FAKE_QUANT_BIG, FAKE_QUANT_ROWS, FAKE_QUANT_TENSOR, FLOAT8, FLOAT8_OUT, FLOAT8_PAIRS, GEMM16_BATCHED,
+                    GEMM16_SEEDS, GEMM16_SHAPES, INF, INT4_SHAPES, INT8_SHAPES, OBSERVER_INPUT, OBSERVER_STEPS, affine_values, cast_values,
+                    draw, float8_case, int4_rows, int4_weights, int8_case, per_channel_cases)
 from _util import ODT, bits, no_fallback as on_gpu, ref_tol, to_device, unbits
 
 pytestmark = pytest.mark.gpu
@@ -366,26 +366,29 @@ def test_fallback_is_counted(tv):
     assert torch.equal(y.cpu(), torch.full((3,), 2.0)) and sum(tv.fallback_counts().values()) > before
 
 
+def same_float_bits(got, want_bits, dtype):
+    """got (host tensor) holds want_bits (a storage array of the oracle) bit for bit; NaNs need only be NaNs."""
+    g, nan = bits(got), np.isnan(oracle.to_f32(want_bits, ODT[dtype]))
+    assert got.dtype == dtype and g.shape == want_bits.shape
+    assert np.array_equal(np.isnan(oracle.to_f32(g, ODT[dtype])), nan) and np.array_equal(g[~nan], want_bits[~nan])
+
+
 @pytest.mark.parametrize("f8", FLOAT8, ids=str)
-@pytest.mark.parametrize("src", [torch.float32, torch.float16, torch.bfloat16], ids=str)
-def test_float8_casts(tv, f8, src):
-    """The reference's float8 cast test for the types _scaled_mm takes
-    (tests/python/test_fallback_ops.py:469-485): every float8 code to the wider type, and values
-    that round, saturate, overflow and are NaN, inf or -0 to float8, bit for bit as the CPU's,
-    converted on the device (cast_fp8 counts its dispatches)."""
+@pytest.mark.parametrize("wide", [torch.float32, torch.float16, torch.bfloat16], ids=str)
+def test_float8_casts(tv, f8, wide):
+    """Tensor.to() between a float8 type and a wider float type, on the device (one cast_fp8 launch each way):
+    the oracle's conversion (pinned against c10's on every code and rounding midpoint) decides, PyTorch's CPU
+    conversion agrees.  Inputs: _cases.cast_values (draws plus the saturating / overflowing / special values) one
+    way, all 256 codes the other."""
+    values = cast_values().to(wide)
     codes = torch.arange(256, dtype=torch.int32).to(torch.uint8).view(f8)
-    x = torch.cat([torch.randn(300, generator=gen(0)) * 3, torch.randn(300, generator=gen(1)) * 300,
-                   torch.tensor([0.0, -0.0, float("inf"), -float("inf"), float("nan"), 448.0, 464.0, 57344.0, 61440.0,
-                                 1e-9, -1e-9, 2.0 ** -9, 2.0 ** -10, 2.0 ** -17, 1e30])]).to(src)
-    dx = x.to("vk")
-    dcodes = codes.to("vk")
-    before = tv.dispatch_count()
-    with on_gpu(tv):
-        got = dx.to(f8)
-        back = dcodes.to(src)
-    assert tv.dispatch_count() - before == 2  # both conversions ran as kernels
-    assert torch.equal(got.cpu().view(torch.uint8), x.to(f8).view(torch.uint8))
-    torch.testing.assert_close(back.cpu(), codes.to(src), equal_nan=True, atol=0, rtol=0)
+    launches = tv.dispatch_count()
+    narrowed, widened = on_vk(tv, lambda v, c: (v.to(f8), c.to(wide)), values, codes)
+    assert tv.dispatch_count() - launches == 2
+    assert np.array_equal(bits(narrowed), oracle.cast(bits(values), ODT[wide], ODT[f8]))
+    assert np.array_equal(bits(narrowed), bits(values.to(f8)))
+    same_float_bits(widened, oracle.cast(bits(codes), ODT[f8], ODT[wide]), wide)
+    same_float_bits(widened, bits(codes.to(wide)), wide)
 
 
 @pytest.mark.parametrize("f8", FLOAT8, ids=str)
@@ -418,54 +421,53 @@ def test_fp8_quant_rowwise_into_scaled_mm(tv, f8, src):
         torch.ops.vk.fp8_quant_rowwise(a.to("vk"), torch.bfloat16)
 
 
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def inside_gemm_band(got, dtype, a, b, cin=None, alpha=1.0, beta=0.0):
+    """got against the oracle's alpha a @ b + beta cin (float32 sums, one rounding): within one unit of the 16-bit
+    type of it plus 2^-20 of the summed magnitudes (the order of the sums is free), the reference's bound for its
+    matrix-core kernel."""
+    want, mag = oracle.gemm16(bits(a), bits(b), ODT[dtype], cin=None if cin is None else bits(cin), alpha=alpha, beta=beta, want_mag=True)
+    want = oracle.to_f32(want, ODT[dtype]).astype(np.float64)
+    assert got.dtype == dtype and tuple(got.shape) == want.shape
+    band = EPS16[dtype] * np.maximum(np.abs(want), 2.0**-14) + 2.0**-20 * mag
+    excess = np.abs(got.double().numpy() - want) - band
+    assert (excess <= 0).all(), excess.max()
+
+
+EPS16 = {torch.float16: 2.0**-10, torch.bfloat16: 2.0**-7}
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
 def test_16bit_matrix_products(tv, dtype):
-    """mm / bmm / addmm of 16-bit tensors on the matrix cores, as the reference tests its
-    cooperative-matrix kernel (tests/python/test_matmul.py:250-284): float32 sums rounded once, one
-    ulp from the CPU's float32 product plus summation-order error relative to the products'
-    magnitudes; every layout, a strided view, batches, alpha / beta with a broadcast bias."""
+    """torch.mm / bmm / addmm / baddbmm / linear of 16-bit tensors on device "vk" run on the matrix-core kernels
+    ("gemmcm_<T>") and stay inside the oracle's band: the shapes of _cases.GEMM16_SHAPES in all four operand
+    layouts and through a row-strided view, then batches with a broadcast bias, an out= that has to be resized,
+    and k = 0."""
+    for m, k, n in GEMM16_SHAPES:
+        a = draw(("normal", (m, k)), GEMM16_SEEDS["a"]).to(dtype)
+        b = draw(("normal", (k, n)), GEMM16_SEEDS["b"]).to(dtype)
+        column_major = lambda t: t.t().contiguous().t()
+        for x, y in ((a, b), (column_major(a), column_major(b)), (a, column_major(b)), (column_major(a), b)):
+            inside_gemm_band(on_vk(tv, torch.mm, x, y), dtype, a, b)
+        inside_gemm_band(on_vk(tv, lambda x, y: x[::2] @ y, a, b), dtype, a[::2], b)
+    a, b, bias = (draw(*GEMM16_BATCHED[name]).to(dtype) for name in ("a", "b", "bias"))
+    bt = b.transpose(1, 2)
+    inside_gemm_band(on_vk(tv, torch.bmm, a, bt), dtype, a, bt)
+    inside_gemm_band(on_vk(tv, lambda c, x, y: torch.addmm(c, x, y, beta=0.5, alpha=2.0), bias, a[0], bt[0]), dtype, a[0], bt[0],
+                     cin=bias, alpha=2.0, beta=0.5)
+    inside_gemm_band(on_vk(tv, lambda c, x, y: torch.baddbmm(c, x, y, beta=0.5, alpha=2.0), bias, a, bt), dtype, a, bt, cin=bias,
+                     alpha=2.0, beta=0.5)
+    inside_gemm_band(on_vk(tv, torch.nn.functional.linear, a, b[0], bias), dtype, a, bt[:1].expand(3, -1, -1), cin=bias, beta=1.0)
 
-    def want(x, y):
-        return (x.float() @ y.float()).to(dtype)
-
-    def close(got, ref, mag):
-        assert got.device.type == "vk" and got.dtype == dtype and got.shape == ref.shape
-        got, ref = got.cpu().float(), ref.float()
-        tol = torch.finfo(dtype).eps * ref.abs().clamp_min(2**-14) + 2**-20 * mag
-        assert ((got - ref).abs() <= tol).all(), (got - ref).abs().max().item()
-
-    for m, k, n in [(64, 32, 64), (65, 33, 63), (17, 200, 129), (128, 1, 96), (3, 1000, 5), (300, 256, 260), (304, 256, 264)]:
-        a, b = torch.randn(m, k, generator=gen(1)).to(dtype), torch.randn(k, n, generator=gen(2)).to(dtype)
-        at, bt = a.t().contiguous().t(), b.t().contiguous().t()  # (column-major)
-        for x, y in [(a, b), (at, bt), (a, bt), (at, b)]:
-            with on_gpu(tv):
-                got = x.to("vk") @ y.to("vk")
-            close(got, want(a, b), a.float().abs() @ b.float().abs())
-        with on_gpu(tv):
-            got = a.to("vk")[::2] @ b.to("vk")
-        close(got, want(a[::2], b), a[::2].float().abs() @ b.float().abs())
-    a, b = torch.randn(3, 40, 72, generator=gen(3)).to(dtype), torch.randn(3, 50, 72, generator=gen(4)).to(dtype)
-    bias = torch.randn(50, generator=gen(5)).to(dtype)
-    with on_gpu(tv):
-        got_t = torch.bmm(a.to("vk"), b.to("vk").transpose(1, 2))
-        got_add = torch.addmm(bias.to("vk"), a[0].to("vk"), b[0].to("vk").t(), beta=0.5, alpha=2.0)
-        got_lin = torch.nn.functional.linear(a.to("vk"), b[0].to("vk"), bias.to("vk"))  # [3,40,72] x [50,72]^T + bias
-        got_badd = torch.baddbmm(bias.to("vk"), a.to("vk"), b.to("vk").transpose(1, 2), beta=0.5, alpha=2.0)
+    def into_empty_out(x, y):
         out = torch.empty(0, dtype=dtype, device="vk")
-        torch.mm(a[1].to("vk"), b[1].to("vk").t(), out=out)
-        empty_k = torch.mm(a[0, :, :0].to("vk"), b[0, :, :0].to("vk").t())
-    mag_t = a.float().abs() @ b.float().abs().transpose(1, 2)
-    close(got_t, want(a, b.transpose(1, 2)), mag_t)
-    close(out, want(a[1], b[1].t()), mag_t[1])
-    close(got_add, (0.5 * bias.float() + 2.0 * (a[0].float() @ b[0].float().t())).to(dtype), 0.5 * bias.float().abs() + 2.0 * mag_t[0])
-    close(got_badd, (0.5 * bias.float() + 2.0 * (a.float() @ b.float().transpose(1, 2))).to(dtype), 0.5 * bias.float().abs() + 2.0 * mag_t)
-    close(got_lin, (a.float() @ b[0].float().t() + bias.float()).to(dtype), a.float().abs() @ b[0].float().abs().t() + bias.float().abs())
-    assert empty_k.shape == (40, 50) and (empty_k.cpu() == 0).all()  # (k = 0: sums of nothing)
+        torch.mm(x, y, out=out)
+        return out
+    inside_gemm_band(on_vk(tv, into_empty_out, a[1], bt[1]), dtype, a[1], bt[1])
+    nothing = on_vk(tv, torch.mm, a[0, :, :0], bt[0, :0])
+    assert nothing.shape == (40, 50) and not nothing.any()
     assert tv.kernel_subgroup_size("gemmcm_bf16") == 64 and tv.kernel_subgroup_size("gemmcm_f16") == 64
-    with pytest.raises(RuntimeError, match="cannot be multiplied"):
-        torch.mm(a[0].to("vk"), b[0].to("vk"))
-    with pytest.raises(RuntimeError, match="same dtype"):
-        torch.mm(a[0].to("vk"), b[0].t().float().to("vk"))
+    raises_each([(RuntimeError, "cannot be multiplied", (a[0], b[0])), (RuntimeError, "same dtype", (a[0], bt[0].float()))],
+                lambda x, y: torch.mm(x.to("vk"), y.to("vk")))
 
 
 def test_strided_copies_and_fills_on_the_device(tv):
@@ -506,82 +508,99 @@ def test_strided_copies_and_fills_on_the_device(tv):
     assert torch.equal(wt.cpu(), wq)
 
 
-@pytest.mark.parametrize("qdtype", [torch.quint8, torch.qint8, torch.qint32])
+QTYPE = {torch.quint8: oracle.QUINT8, torch.qint8: oracle.QINT8, torch.qint32: oracle.QINT32}
+
+
+@pytest.mark.parametrize("qdtype", list(QTYPE), ids=str)
 def test_quantized_per_tensor(tv, qdtype):
-    """Legacy quantised tensors on vk as the reference tests them (tests/python/test_fallback_ops.py:986-1006):
-    quantize_per_tensor, the getters, int_repr, dequantize, flip, clone and copies, bit for bit as the CPU's."""
-    x = torch.cat([torch.randn(40, generator=gen(0)) * 20,
-                   torch.tensor([float("nan"), float("inf"), -float("inf"), 0.05, 0.15, -0.05, 1e30, 3e9])]).view(6, 8)
-    c = torch.quantize_per_tensor(x, 0.1, 5, qdtype)
+    """Per-tensor affine quantised tensors on device "vk" (csrc/torch/quantized.cpp): the integers of
+    quantize_per_tensor are the oracle's (the x86 CPU's arithmetic) on _cases.affine_values, dequantize gives the
+    oracle's floats, and what only moves the integers around (flip, clone, a transposed input, qparams given as
+    tensors, device <-> host) moves them unchanged; the quantiser's parameters read back as set."""
+    x = affine_values()
+    scale, zero_point = AFFINE_QPARAMS
+    ints = oracle.quantize_affine(x.numpy(), scale, zero_point, QTYPE[qdtype])
+    floats = oracle.dequantize_affine(ints, scale, zero_point, QTYPE[qdtype])
     with on_gpu(tv):
-        v = torch.quantize_per_tensor(x.to("vk"), 0.1, 5, qdtype)
-        assert v.is_quantized and v.device.type == "vk" and v.dtype == qdtype
-        assert (v.q_scale(), v.q_zero_point(), v.qscheme()) == (c.q_scale(), c.q_zero_point(), c.qscheme())
-        ints, deq, flipped, cloned = v.int_repr(), v.dequantize(), v.flip((0, 1)), v.clone()
-        t = torch.quantize_per_tensor(x.to("vk").t(), 0.1, 5, qdtype)  # a strided input
-        by_tensor = torch.quantize_per_tensor(x.to("vk"), torch.tensor(0.1).to("vk"), torch.tensor(5).to("vk"), qdtype)
-        e = torch._empty_affine_quantized([5, 5, 5, 5], scale=2, zero_point=3, dtype=qdtype, device="vk")
-    assert torch.equal(ints.cpu(), c.int_repr()) and torch.equal(deq.cpu(), c.dequantize())
-    assert torch.equal(flipped.int_repr().cpu(), c.flip((0, 1)).int_repr()) and torch.equal(cloned.int_repr().cpu(), c.int_repr())
-    assert torch.equal(t.int_repr().cpu(), c.int_repr().t()) and torch.equal(by_tensor.int_repr().cpu(), c.int_repr())
-    assert torch.equal(v.cpu().int_repr(), c.int_repr())
-    back = c.to("vk")
-    assert back.is_quantized and torch.equal(back.int_repr().cpu(), c.int_repr())
-    assert e.flatten(0, -1).shape == (625,) and e.ravel().shape == (625,)
-    with pytest.raises(RuntimeError, match="only works on Float"):
-        torch.quantize_per_tensor(x.half().to("vk"), 0.1, 5, qdtype)
+        q = torch.quantize_per_tensor(x.to("vk"), scale, zero_point, qdtype)
+        assert q.is_quantized and q.device.type == "vk" and q.dtype == qdtype and q.qscheme() == torch.per_tensor_affine
+        assert q.q_scale() == scale and q.q_zero_point() == zero_point
+        moved = {"as quantised": q.int_repr(), "cloned": q.clone().int_repr(), "flipped": q.flip((0, 1)).int_repr(),
+                 "transposed input": torch.quantize_per_tensor(x.to("vk").t(), scale, zero_point, qdtype).int_repr(),
+                 "tensor qparams": torch.quantize_per_tensor(x.to("vk"), torch.tensor(scale).to("vk"), torch.tensor(zero_point).to("vk"),
+                                                             qdtype).int_repr()}
+        back = q.dequantize()
+        blank = torch._empty_affine_quantized([5, 5, 5, 5], scale=2, zero_point=3, dtype=qdtype, device="vk")
+    expect = {"as quantised": ints, "cloned": ints, "flipped": ints[::-1, ::-1], "transposed input": ints.T, "tensor qparams": ints}
+    for name, got in moved.items():
+        assert np.array_equal(got.cpu().numpy(), expect[name]), name
+    assert np.array_equal(back.cpu().numpy(), floats, equal_nan=True)
+    cpu = torch.quantize_per_tensor(x, scale, zero_point, qdtype)
+    assert np.array_equal(cpu.int_repr().numpy(), ints)  # (PyTorch's CPU kernel agrees with the oracle)
+    assert np.array_equal(q.cpu().int_repr().numpy(), ints) and np.array_equal(cpu.to("vk").int_repr().cpu().numpy(), ints)
+    assert blank.flatten(0, -1).shape == (625,) and blank.ravel().shape == (625,)
+    raises_each([(RuntimeError, "only works on Float", (x.half(),))], lambda t: torch.quantize_per_tensor(t.to("vk"), scale, zero_point, qdtype))
+
+
+def same_fake_quant(got, want, dtype):
+    """(output, mask) from the device against the oracle's pair of storage arrays."""
+    same_float_bits(got[0], want[0], dtype)
+    assert np.array_equal(got[1].numpy().astype(np.uint8), want[1])
 
 
 def test_fake_quantize_cachemask_ops(tv):
-    """As the reference's test (tests/python/test_fallback_ops.py:972-984), plus float zero points and 16-bit inputs."""
-    x = torch.tensor([[-1.3, 0.0, 0.26, 4.0], [float("nan"), float("inf"), -0.5, 1e-3]])
-    v = lambda t: t.to("vk")
-    sc, zp = torch.tensor([0.05]), torch.tensor([3], dtype=torch.int32)
-    on = torch.ones(1, dtype=torch.long)
-    f = torch.ops.aten._fake_quantize_per_tensor_affine_cachemask_tensor_qparams
-    with on_gpu(tv):
-        got = f(v(x), v(sc), v(zp), v(on), 0, 255)
-        off = f(v(x), v(sc), v(zp), v(torch.zeros(1, dtype=torch.long)), 0, 255)
-    for a, b in zip(got, f(x, sc, zp, on, 0, 255)):
-        assert torch.equal(a.cpu().nan_to_num(), b.nan_to_num())
-    assert torch.equal(off[0].cpu().nan_to_num(), x.nan_to_num()) and off[1].cpu().all()
-    scs, zps = torch.tensor([0.05, 0.2]), torch.tensor([3, 250], dtype=torch.int32)
-    g = torch.ops.aten.fake_quantize_per_channel_affine_cachemask
-    big = torch.randn(2, 3, 500, generator=gen(4)) * 4
-    for inp, axis, s, z in [(x, 0, scs, zps), (x, 0, scs, torch.tensor([3.25, 250.5])), (big, 1, torch.tensor([0.05, 0.2, 0.01]), torch.tensor([3, 250, 128], dtype=torch.int32)),
-                            (big.bfloat16(), 2, torch.rand(500, generator=gen(5)) * 0.1 + 0.01, torch.randint(0, 255, (500,), dtype=torch.int32, generator=gen(6))),
-                            (big.transpose(0, 2), 0, torch.rand(500, generator=gen(5)) * 0.1 + 0.01, torch.rand(500, generator=gen(7)) * 200)]:
-        with on_gpu(tv):
-            got = g(v(inp), v(s), v(z), axis, 0, 255)
-        for a, b in zip(got, g(inp, s, z, axis, 0, 255)):
-            assert a.shape == b.shape and torch.equal(a.cpu().float().nan_to_num(), b.float().nan_to_num())
-    with on_gpu(tv):
-        got = torch.fake_quantize_per_tensor_affine(v(big), 0.05, 3, 0, 255)
-    assert torch.equal(got.cpu(), torch.fake_quantize_per_tensor_affine(big, 0.05, 3, 0, 255))
-    with pytest.raises(RuntimeError, match="must be between"):
-        g(v(x), v(scs), v(torch.tensor([3, 300], dtype=torch.int32)), 0, 0, 255)
+    """The fake-quantisation operators with their masks on device "vk", one fused kernel each, against the oracle
+    (the CPU's arithmetic, fused multiply-add of the float-zero-point form included): per tensor with qparams in
+    tensors (switched on and off), per channel over _cases.per_channel_cases (integer and float zero points, a
+    16-bit input, a transposed view), and the plain per-tensor operator."""
+    x = torch.tensor(FAKE_QUANT_ROWS)
+    scale, zero_point, (lo, hi) = (FAKE_QUANT_TENSOR[k] for k in ("scale", "zero_point", "range"))
+    per_tensor = torch.ops.aten._fake_quantize_per_tensor_affine_cachemask_tensor_qparams
+    switch = lambda on: torch.full((1,), int(on), dtype=torch.long)
+    want = oracle.fake_quant(x.numpy(), oracle.F32, [scale], np.array([zero_point], np.int32), lo, hi)
+    same_fake_quant(on_vk(tv, per_tensor, x, torch.tensor([scale]), torch.tensor([zero_point], dtype=torch.int32), switch(True), lo, hi),
+                    want, torch.float32)
+    passed, mask = on_vk(tv, per_tensor, x, torch.tensor([scale]), torch.tensor([zero_point], dtype=torch.int32), switch(False), lo, hi)
+    same_float_bits(passed, x.numpy(), torch.float32)  # switched off: the input, every element inside
+    assert mask.all()
+    per_channel = torch.ops.aten.fake_quantize_per_channel_affine_cachemask
+    for inp, axis, scales, zero_points in per_channel_cases():
+        dense = inp.contiguous()
+        want = oracle.fake_quant(bits(dense), ODT[inp.dtype], scales.numpy(), zero_points.numpy(), lo, hi, axis=axis)
+        got = on_vk(tv, per_channel, inp, scales, zero_points, axis, lo, hi)
+        assert got[0].shape == inp.shape
+        same_fake_quant(got, want, inp.dtype)
+    big = draw(*FAKE_QUANT_BIG)
+    plain = on_vk(tv, torch.fake_quantize_per_tensor_affine, big, scale, zero_point, lo, hi)
+    same_float_bits(plain, oracle.fake_quant(big.numpy(), oracle.F32, [scale], np.array([zero_point], np.int32), lo, hi)[0], torch.float32)
+    raises_each([(RuntimeError, "must be between", (torch.tensor([3, 300], dtype=torch.int32),))],
+                lambda zps: per_channel(x.to("vk"), torch.tensor([0.05, 0.2]).to("vk"), zps.to("vk"), 0, lo, hi))
 
 
 @pytest.mark.parametrize("per_row", [False, True])
 @pytest.mark.parametrize("symmetric", [False, True])
 @pytest.mark.parametrize("qrange", [(0, 255), (-128, 127)])
 def test_fused_moving_avg_obs_fake_quant(tv, per_row, symmetric, qrange):
-    """The QAT observer and fake quantisation as the reference tests them (tests/python/test_fallback_ops.py:947-969):
-    bit for bit as the CPU's over several steps (the running min / max start infinite, then move)."""
+    """_fused_moving_avg_obs_fq_helper on device "vk" over _cases.OBSERVER_STEPS: the running range (infinite at
+    first, then a moving average), the scale and zero point chosen from it and the fake-quantised output, each step
+    against the oracle's step and PyTorch's CPU operator, both bit for bit."""
+    channels = OBSERVER_INPUT[0] if per_row else 1
+    fresh = lambda: [torch.full((channels,), INF), torch.full((channels,), -INF), torch.ones(channels), torch.zeros(channels, dtype=torch.int32)]
+    on_device, on_host = [t.to("vk") for t in fresh()], fresh()
+    run_min, run_max = np.full(channels, np.inf, np.float32), np.full(channels, -np.inf, np.float32)
+    helper = torch.ops.aten._fused_moving_avg_obs_fq_helper
+    one = torch.tensor([1])
     g = gen(0)
-    size = 4 if per_row else 1
-    state = {d: [torch.full((size,), float("inf")), torch.full((size,), float("-inf")), torch.ones(size),
-                 torch.zeros(size, dtype=torch.int32)] for d in ("cpu", "vk")}
-    state["vk"] = [t.to("vk") for t in state["vk"]]
-    for step in range(4):
-        x = torch.randn(4, 3, 5, generator=g) * (0.1 + step) - 0.5 * step
-        got = {}
-        for d in ("cpu", "vk"):
-            rmin, rmax, s, z = state[d]
-            with (on_gpu(tv) if d == "vk" else contextlib.nullcontext()):
-                out, mask = torch.ops.aten._fused_moving_avg_obs_fq_helper(
-                    x.to(d), torch.tensor([1]).to(d), torch.tensor([1]).to(d), rmin, rmax, s, z, 0.01 if step == 3 else 0.25,
-                    qrange[0], qrange[1], 0, per_row, symmetric)
-            got[d] = [t.cpu() for t in (out, mask, rmin, rmax, s, z)]
-        for a, b in zip(got["cpu"], got["vk"]):
-            assert torch.equal(a, b)
+    for spread, shift, averaging in OBSERVER_STEPS:
+        x = torch.randn(*OBSERVER_INPUT, generator=g) * spread + shift
+        with on_gpu(tv):
+            out, mask = helper(x.to("vk"), one.to("vk"), one.to("vk"), *on_device, averaging, qrange[0], qrange[1], 0, per_row, symmetric)
+        want_out, want_mask, scales, zero_points = oracle.observe_fake_quant(x.numpy(), oracle.F32, run_min, run_max, averaging, qrange[0],
+                                                                               qrange[1], per_row, symmetric)
+        same_fake_quant((out.cpu(), mask.cpu()), (want_out, want_mask), torch.float32)
+        for got, want in zip(on_device, (run_min, run_max, scales, zero_points)):
+            assert np.array_equal(got.cpu().numpy(), want)
+        host_out, host_mask = helper(x, one, one, *on_host, averaging, qrange[0], qrange[1], 0, per_row, symmetric)
+        assert torch.equal(out.cpu(), host_out) and torch.equal(mask.cpu(), host_mask)
+        for got, want in zip(on_device, on_host):
+            assert torch.equal(got.cpu(), want)
