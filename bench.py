@@ -379,10 +379,10 @@ BASELINE = {
     "c2_m64_k14336_n4096": lambda abi, s, w: wl_q8(abi, 64, 14336, 4096, abi.BF16, s, w),
     "c3_int4_m32": lambda abi, s, w: wl_q4(abi, 32, 4096, 11008, 32, max(s // 4, 5), w),
     "c2_m1_k14336_n4096": lambda abi, s, w: wl_q8(abi, 1, 14336, 4096, abi.BF16, s, w),
-    "c5_fp8_rowwise_70b": lambda abi, s, w: wl_fp8(abi, 4096, 8192, 28672, True, max(s // 2, 10), max(w, 5), seed=1050),
+    "c5_fp8_rowwise_70b": lambda abi, s, w: wl_fp8(abi, 4096, 8192, 28672, True, max(s // 2, 30), max(w, 5), seed=1050),
     "c1_f32_m1_k4096_n4096": lambda abi, s, w: wl_q8(abi, 1, 4096, 4096, abi.F32, s, w, seed=1010),
     "c3_int4_m1": lambda abi, s, w: wl_q4(abi, 1, 4096, 11008, 32, s, w),
-    "c4_fp8_8192": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 2, 10), max(w, 5)),
+    "c4_fp8_8192": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 2, 30), max(w, 5)),
 }
 # Beside the BASELINE configurations (--all, or by name): many rows of the same operators, the steps either side of
 # the path, the planner off the Llama grid, config 4's launch on all-zero operands.
@@ -406,7 +406,7 @@ OTHER = {
     "affine_quantize_256mi": lambda abi, s, w: wl_affine(abi, "quantize", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
     "affine_dequantize_256mi": lambda abi, s, w: wl_affine(abi, "dequantize", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
     "affine_fake_quant_256mi": lambda abi, s, w: wl_affine(abi, "fake_quant", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
-    "c4_fp8_8192_zero_operands": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 2, 10), max(w, 5), zero_operands=True),
+    "c4_fp8_8192_zero_operands": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 2, 30), max(w, 5), zero_operands=True),
 }
 # Ceilings measured in the same run (`ceilings` of the output line; also selectable by name): bare 16-byte loads of
 # each GEMV configuration's weight bytes in its kernel's launch geometry, a persistent-grid read, a device copy of known
@@ -423,6 +423,8 @@ CALIBRATION = {
     "probe_mfma_f8_fresh": lambda abi, s, w: wl_probe_mfma(abi, 2, max(s // 10, 5), max(w // 4, 3)),
     "copy_256mib": lambda abi, s, w: wl_copy(abi, 256 << 20, max(s // 4, 5), w),
 }
+# configurations whose extra entry also carries the op's cost through PyTorch's dispatcher (the headline always does)
+DISPATCHER_TOO = ("c3_int4_m1", "c3_int4_m32", "c4_fp8_8192", "c1_f32_m1_k4096_n4096")
 WORKLOADS = {**BASELINE, **OTHER}
 HEADLINE = "c2_m1_k4096_n14336"
 
@@ -520,29 +522,48 @@ def cpu_baselines(abi, name, r, port=False):
 
 
 def through_dispatcher(abi, name, r, calls=200):
-    """The same op called as torch._weight_int8pack_mm on device "vk" tensors (schema -> op layer -> C ABI -> kernel),
-    one weight tensor over and over: wall time per call with the queue kept full, beside the kernel's own time on
-    the same resident weights, so that the host's share shows."""
+    """The same op called through PyTorch's dispatcher on device "vk" tensors (schema -> op layer -> C ABI -> kernel),
+    one weight tensor over and over: wall time per call with the queue kept full and the host's time to issue a call,
+    beside the kernel's own time on the same resident weights, so that the host's share shows.  int8: torch._weight_int8pack_mm;
+    int4: torch._dyn_quant_matmul_4bit (the side-car of the packed weights is built by the first call and cached);
+    float8: torch._scaled_mm."""
     import torch
     import torch_vulkan_amd.backend as tv
-    if not name.startswith(("c1", "c2", "q8_")) or not r.get("inputs"):
+    if not r.get("inputs"):
         return None
-    x, w, s = (t.to("vk") for t in r["inputs"])
+    if name.startswith(("c1", "c2", "q8_")):
+        x, w, s = (t.to("vk") for t in r["inputs"])
+        op, call = "torch._weight_int8pack_mm", lambda: torch._weight_int8pack_mm(x, w, s)
+    elif name.startswith("c3"):
+        x, packed = (t.to("vk") for t in r["inputs"])
+        (n, bs), k = r["shape"], x.shape[1]
+        op, call = "torch._dyn_quant_matmul_4bit", lambda: torch._dyn_quant_matmul_4bit(x, packed, bs, k, n)
+    elif name.startswith(("c4", "c5")):
+        a, bt, sa, sb = r["inputs"]
+        rowwise = sa.numel() > 1
+        a, b = a.to("vk"), bt.to("vk").t()
+        sa = (sa.reshape(-1, 1) if rowwise else sa.reshape(())).to("vk")
+        sb = (sb.reshape(1, -1) if rowwise else sb.reshape(())).to("vk")
+        op, call = "torch._scaled_mm", lambda: torch._scaled_mm(a, b, sa, sb, out_dtype=torch.bfloat16)
+        calls = min(calls, 50)
+    else:
+        return None
     before = tv.fallback_counts()
-    for _ in range(20):
-        torch._weight_int8pack_mm(x, w, s)
+    for _ in range(min(20, calls)):
+        call()
     abi.synchronize()
     t0 = time.perf_counter()
     for _ in range(calls):
-        torch._weight_int8pack_mm(x, w, s)
+        call()
     t_issue = time.perf_counter()
     abi.synchronize()
     t1 = time.perf_counter()
     if tv.fallback_counts() != before:
-        raise RuntimeError("bench.py: torch._weight_int8pack_mm on device vk fell back to the CPU")
-    return dict(op="torch._weight_int8pack_mm on device vk", calls=calls, us_per_call=round((t1 - t0) * 1e6 / calls, 2),
+        raise RuntimeError(f"bench.py: {op} on device vk fell back to the CPU")
+    resident_ms = r.get("cache_resident_ms") or (r["event_ms"] if r.get("copies") == 1 else None)
+    return dict(op=op + " on device vk", calls=calls, us_per_call=round((t1 - t0) * 1e6 / calls, 2),
                 host_issue_us_per_call=round((t_issue - t0) * 1e6 / calls, 2),
-                kernel_us_cache_resident=round(r["cache_resident_ms"] * 1e3, 2) if r.get("cache_resident_ms") else None)
+                kernel_us_cache_resident=round(resident_ms * 1e3, 2) if resident_ms else None)
 
 
 def load_traffic():
@@ -554,9 +575,25 @@ def load_traffic():
         return {}
 
 
+def load_counters():
+    """Matrix-core busy fraction and the shader clock during the dominant kernel, from rocprofv3 --pmc runs
+    (profiles/counters.json: SQ_VALU_MFMA_BUSY_CYCLES / (4 SIMDs x SQ_BUSY_CU_CYCLES); busy cycles per compute unit
+    / the kernel's duration in the kernel trace), if recorded."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "counters.json")) as f:
+            return json.load(f)
+    except (OSError, ValueError):
+        return {}
+
+
 def compact(key, rr, v, u, rf, cpu):
     """One short entry of `extra`."""
-    e = {"key": key, "value": round(v, 1), "unit": u, "frac": rf["frac"], "kernel_ms": round(rr["event_ms"], 5)}
+    # value and frac from the same clock (HIP events on the runtime's stream); the wall time per step, which includes the
+    # two synchronisations around the timed loop, under its own key
+    e = {"key": key, "value": rf["achieved"], "unit": u, "frac": rf["frac"], "kernel_ms": round(rr["event_ms"], 5),
+         "wall_ms": round(rr["wall_ms"], 5)}
+    if rf.get("counters"):
+        e["counters"] = rf["counters"]
     if "cache_resident" in rf:
         e["resident_ms"] = rf["cache_resident"]["kernel_ms"]
     if rf.get("traffic"):
@@ -583,10 +620,13 @@ def main():
     abi = _abi()
     info = abi.device_info()
     traffic = load_traffic()
+    counters = load_counters()
 
     r = {**WORKLOADS, **CALIBRATION}[args.workload](abi, args.steps, args.warmup)
     value, unit, roof = summarise(r)
     roof["traffic"] = traffic.get(args.workload)
+    if counters.get(args.workload):
+        roof["counters"] = counters[args.workload]
     if r["kind"] == "hbm":
         metric, dtype = "M=1 int8 GEMV GB/s (% of HBM peak)", "f32 accumulate (bf16 activations, int8 weights)"
     else:
@@ -632,8 +672,14 @@ def main():
             rr = fn(abi, args.steps, args.warmup)
             v, u, rf = summarise(rr)
             rf["traffic"] = traffic.get(name)
+            if counters.get(name):
+                rf["counters"] = counters[name]
             cpu = {} if args.no_cpu or name not in BASELINE else cpu_baselines(abi, name, rr)
             e = compact(name, rr, v, u, rf, cpu)
+            if not args.no_cpu and name in DISPATCHER_TOO:  # the full op through the dispatcher, host issue time beside it
+                d = through_dispatcher(abi, name, rr, calls=100)
+                if d:
+                    e["dispatcher"] = {"us_per_call": d["us_per_call"], "host_issue_us": d["host_issue_us_per_call"]}
             if args.verbose:
                 e.update(workload=rr["name"], ms_per_step=round(rr["wall_ms"], 5), roofline=rf, **cpu)
                 if rr["kind"] == "hbm":

@@ -271,24 +271,26 @@ def test_scaled_mm_zero_sums_keep_their_sign():
 
 @pytest.mark.parametrize("fa,fb", [(FLOAT8[0], FLOAT8[0]), (FLOAT8[1], FLOAT8[0]), (FLOAT8[1], FLOAT8[1])])
 def test_scaled_mm_float32_output_large(fa, fb):
-    """float32 output at a size where the path matters (the exact kernel on 256x256 tiles,
-    direct-to-LDS loads): sampled rows / columns inside the reference's bound
-    eps*|want| + 2^-20*sum|a||b|, and within the stated 1e-4 of the float64 closed form."""
+    """float32 output at a size where the path matters (the exact kernel on 256x256 tiles, direct-to-LDS loads):
+    whole rows and whole columns either side of every tile, wave and matrix-core-tile boundary, each inside the
+    reference's bound eps*|want| + 2^-20*sum|a||b| and within the stated 1e-4 of the float64 closed form."""
     import _dev
     m, k, n = 1024, 8192, 1280
     a = torch.randn(m, k, generator=gen(1060)).to(fa)
     bt = torch.randn(n, k, generator=gen(1061)).to(fb)
     sa = torch.empty(m, 1).uniform_(0.5, 2, generator=gen(1062)).numpy()
     sb = torch.empty(1, n).uniform_(0.5, 2, generator=gen(1063)).numpy()
-    got = _dev.scaled_mm(bits(a), ODT[fa], bits(bt), ODT[fb], sa, sb, True, out_dtype=oracle.F32)
-    rows, cols = np.array([0, 31, 32, 255, 256, 700, 1023]), np.array([0, 1, 127, 128, 255, 256, 1279])
-    af = oracle.fp8_table(ODT[fa])[bits(a)[rows]].astype(np.float64)
-    bf = oracle.fp8_table(ODT[fb])[bits(bt)[cols]].astype(np.float64)
-    scale = sa.reshape(-1)[rows][:, None].astype(np.float64) * sb.reshape(-1)[cols][None, :]
-    truth, mag = (af @ bf.T) * scale, (np.abs(af) @ np.abs(bf).T) * scale
-    sub = got[np.ix_(rows, cols)].astype(np.float64)
-    assert (np.abs(sub - truth) <= ref_tol(truth, mag, oracle.F32)).all()
-    assert np.allclose(sub, truth, rtol=1e-4, atol=1e-4)
+    got = _dev.scaled_mm(bits(a), ODT[fa], bits(bt), ODT[fb], sa, sb, True, out_dtype=oracle.F32).astype(np.float64)
+    af = oracle.fp8_table(ODT[fa])[bits(a)].astype(np.float64)
+    bf = oracle.fp8_table(ODT[fb])[bits(bt)].astype(np.float64)
+    rows, cols = np.array([0, 31, 32, 63, 64, 127, 128, 255, 256, 700, 1023]), np.array([0, 1, 31, 32, 127, 128, 255, 256, 1023, 1024, 1279])
+
+    def stripe(sub, x, y, scale):
+        truth, mag = (x @ y.T) * scale, (np.abs(x) @ np.abs(y).T) * scale
+        assert (np.abs(sub - truth) <= ref_tol(truth, mag, oracle.F32)).all()
+        assert np.allclose(sub, truth, rtol=1e-4, atol=1e-4)
+    stripe(got[rows], af[rows], bf, sa.reshape(-1)[rows][:, None].astype(np.float64) * sb.reshape(1, -1))   # whole rows
+    stripe(got[:, cols], af, bf[cols], sa.reshape(-1, 1).astype(np.float64) * sb.reshape(-1)[cols][None, :])  # whole columns
 
 
 def test_scaled_mm_config5_rowwise_70b():
