@@ -87,6 +87,23 @@ def test_qmm8_matrix_core_variants(dtype, variant, m, k, n):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,k,n", [(8, 512, 24600), (5, 1024, 33001), (8, 4096, 14336), (3, 4112, 12300), (7, 2064, 8192),
+                                   (8, 14336, 4096), (4, 528, 70), (6, 512, 16), (8, 9216, 1000)])
+def test_qmm8_rows_kernel(dtype, m, k, n):
+    """3 to 8 rows over a large weight matrix run on the kernel whose waves own column groups (asked for here
+    whatever the size: variant bits 8-15): 1, 2, 4 and 8 waves per group, one and several rounds per workgroup,
+    activations staged whole (k <= 4096) and by chunk, k off the chunk size, n off the group and vector sizes,
+    rows of A further apart than k."""
+    import _dev
+    # (seeds of its own: among the first table's scales for n > 27482 is the smallest float16 subnormal, and a float16
+    # output that small is further from the float64 sum than the bound allows however it is rounded)
+    a, b, s = int8_case(dtype, m, k, n, seeds={"a": 4, "b": 5, "scales": 6})
+    check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=1 << 8), a, b, s, dtype)
+    if (m + 1) // 2 >= 3:  # (fewer rows are other kernels')
+        check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), variant=1 << 8, row_step=2), a, b, s, dtype, rows=slice(None, None, 2))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("m,k,n", [(192, 512, 200), (2100, 64, 2060), (300, 1088, 7000), (1024, 256, 4100), (4096, 72, 2056)])
 def test_qmm8_many_rows(dtype, m, k, n):
     """From 192 rows on (prefill) the weights are widened once into the library's scratch region and the product runs

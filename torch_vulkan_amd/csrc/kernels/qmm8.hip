@@ -716,6 +716,243 @@ bool launch_staged(const Q8Params& p, int mt, int nt, int waves, uint32_t slices
   return false;
 }
 
+// Three to eight rows of 16-bit activations over a large weight matrix (batched decode at small batch, vocabulary-sized
+// projections): the weight stream of the one-row kernels with the arithmetic on the matrix cores.  One workgroup of
+// 8 waves per compute unit stays for the whole launch.  A column group is 16 weight rows; KS waves share its K, each
+// taking every KS-th chunk of 512 bytes of every row: 8 loads of 2 rows x 512 contiguous bytes, into registers, two
+// chunks ahead.  A chunk goes through the wave's own 8 KiB of LDS (16-byte pieces swizzled by the row, so that
+// neither side has a bank conflict) to come back in the matrix core's operand shape (lane (c, g): row c, 16 bytes of
+// k), is widened exactly to the activations' type and multiplied by the activations' fragments.  Those come out of
+// LDS too: all rows of A where they fit (8 rows x K <= 4096 values, staged once per workgroup, asked for before any
+// weights), otherwise the wave's own 8 rows x 512 values, loaded with the weight chunk they meet.  The KS partial
+// tiles of a group meet in LDS, added in wave order.
+// What was measured (8 x 4096 x 14336, timestamps inside the kernel): a compute unit accepts about 64 KiB of loads
+// before the issue of further ones blocks, so the second chunk in flight buys little at the start (the last wave's
+// requests are accepted 4-6 us into the launch) and much in the steady state (1.45 us per chunk and pair of waves,
+// which is the vector units' time: widening 16 weights is 24 instructions of 4-5 cycles, the matrix cores' two
+// instructions of 16 cycles per 64 values of k hide behind them).  The loop over a chunk's eight 64-value steps is
+// rolled (a launch starts with a cold instruction cache).
+constexpr uint32_t kRowsChunk = 512, kRowsRegion = 16 * kRowsChunk, kRowsWaves = 8;
+// a wave's own activations of one chunk (rows longer than 4096): 8 rows x 512 values at the pitch below
+constexpr uint32_t kRowsOwnPitch = 2 * kRowsChunk + 64, kRowsOwn = 8 * kRowsOwnPitch;
+constexpr int kRawBuffer = 0x00020000;  // descriptor word 3: raw (unstructured) buffer, 32-bit data format
+constexpr int kLoadStream = 2;          // the nt bit: read once
+
+// activations in LDS: per row and block of 64 values the eight 16-byte pieces are kept as [first halves of the four
+// k-groups | second halves], so that the 32 distinct pieces one read instruction fetches (8 rows x 4 groups) cover
+// every bank twice; the row pitch is 64 bytes past a multiple of 256
+// (rows run to the end of the last 512-value chunk, zeros past k)
+__host__ __device__ inline uint32_t rows_a_pitch(uint32_t k) { return 2 * ((k + 511) / 512 * 512) + 64; }
+__device__ __forceinline__ uint32_t rows_a_slot(uint32_t piece) { return (piece / 8) * 128 + (piece & 1u) * 64 + ((piece & 7u) >> 1) * 16; }
+
+template <class T, int KS, bool A_LDS>
+__global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t groups) {
+  constexpr uint64_t item = 2;
+  constexpr uint32_t TEAMS = kRowsWaves / KS;
+  extern __shared__ __attribute__((aligned(16))) uint8_t rows_lds[];
+  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t c = lane & 15, g = lane >> 4, team = wave / KS, ks = wave % KS;
+  const uint32_t chunks = (p.k + kRowsChunk - 1) / kRowsChunk, per_wave = (chunks + KS - 1) / KS;
+  const uint32_t a_pitch = A_LDS ? rows_a_pitch(p.k) : kRowsOwnPitch, a_bytes = A_LDS ? 8 * a_pitch : 0;
+  uint8_t* const region = rows_lds + a_bytes + wave * (kRowsRegion + (A_LDS ? 0 : kRowsOwn));
+  uint8_t* const own = region + kRowsRegion;  // (!A_LDS)
+  V4F* const parts = reinterpret_cast<V4F*>(rows_lds + a_bytes + kRowsWaves * (kRowsRegion + (A_LDS ? 0 : kRowsOwn)));  // [2][8 waves][64 lanes]
+  uint16_t* const scales_lds = reinterpret_cast<uint16_t*>(parts + 2 * kRowsWaves * 64);  // [8 waves][16]
+
+  // rounds: in round i team t works on group (i * TEAMS + t) * grid + block (all teams make the same number of
+  // rounds: the barrier below is the workgroup's)
+  const uint32_t span = TEAMS * gridDim.x, rounds = (groups + span - 1) / span;
+  auto group_of = [&](uint32_t round) { return (round * TEAMS + team) * gridDim.x + blockIdx.x; };
+  const uint32_t items = rounds * per_wave;  // (group, chunk) pairs of this wave, some of them past the end
+  // Two chunks are in flight per wave (registers), requested as soon as the registers are free.
+  U4 w[2][8], av[2][A_LDS ? 1 : 8];
+  uint16_t scl[2];
+  // Weights, scales and (long rows) activations are read through buffer descriptors: a load whose offset lies past
+  // the buffer returns zeros and touches no memory, so rows past n, pieces past k and requests past the wave's last
+  // item cost nothing, and every request is the same number of loads on every path (each wait below is then for its
+  // own chunk only: a path without its loads would make every later wait a wait for everything).
+  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(p.b), 0, int(p.n * p.k), kRawBuffer);
+  const __amdgpu_buffer_rsrc_t s_rsrc = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(p.scales), 0, int(p.n * item), kRawBuffer);
+  const __amdgpu_buffer_rsrc_t a_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(p.a), 0, int((uint32_t(p.m - 1) * uint32_t(p.a_sm) + p.k) * item), kRawBuffer);
+  auto request = [&](auto set, uint32_t j) {
+    constexpr int S = decltype(set)::value;
+    // (the fences keep one request's loads together and in program order, which is what the waits count on)
+    __builtin_amdgcn_sched_barrier(0);
+    const uint32_t grp = group_of(j / per_wave), chunk = (j % per_wave) * KS + ks;
+    const uint32_t dead = j < items && grp < groups ? 0u : ~0u;  // (all ones: past every buffer)
+    const uint32_t at = chunk * kRowsChunk + (lane & 31u) * 16;
+    const uint32_t row0 = grp * 16 + (lane >> 5), gone = dead | (at < p.k ? 0u : ~0u);
+#pragma unroll
+    for (int i = 0; i < 8; ++i)  // rows 2 i + lane / 32
+      w[S][i] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, ((row0 + 2 * i) * p.k + at) | gone | (row0 + 2 * i < p.n ? 0u : ~0u), 0, kLoadStream);
+    if constexpr (!A_LDS) {  // row i's piece `lane` of the chunk
+      const uint32_t ka = chunk * kRowsChunk + lane * 8;
+      const uint32_t a_first = (ka * uint32_t(item)) | dead | (ka < p.k ? 0u : ~0u);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        av[S][i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (a_first + i * uint32_t(p.a_sm) * uint32_t(item)) | (uint32_t(i) < p.m ? 0u : ~0u), 0, 0);
+    }
+    // the group's 16 scales come with every chunk and go through LDS with it (loaded in the epilogue they would be
+    // waited for behind two chunks in flight)
+    scl[S] = __builtin_amdgcn_raw_buffer_load_b16(s_rsrc, ((grp * 16 + c) * uint32_t(item)) | dead | (grp * 16 + c < p.n ? 0u : ~0u), 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  if constexpr (A_LDS) {
+    // all rows, once per workgroup: row i's piece `tid` (a row has at most 512 pieces), through the same kind of
+    // descriptor; asked for before any weights: the barrier below waits for the last wave's pieces, and a compute
+    // unit's loads are served in the order they were issued
+    U4 a_regs[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      a_regs[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (tid * 16 + i * uint32_t(p.a_sm) * uint32_t(item)) | (uint32_t(i) < p.m && tid * 8 < p.k ? 0u : ~0u), 0, 0);
+    request(std::integral_constant<int, 0>{}, 0);
+    request(std::integral_constant<int, 1>{}, 1);
+    if (tid * 16 < a_pitch - 64) {
+      uint32_t at = rows_a_slot(tid);
+#pragma unroll
+      for (int i = 0; i < 8; ++i, at += a_pitch) *reinterpret_cast<U4*>(rows_lds + at) = a_regs[i];
+    }
+    __syncthreads();
+  } else {
+    request(std::integral_constant<int, 0>{}, 0);
+    request(std::integral_constant<int, 1>{}, 1);
+  }
+  const uint8_t* const a_frag = (A_LDS ? rows_lds : own) + (c & 7u) * a_pitch + 16 * g;
+
+  V4F acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = acc0;
+  auto work = [&](auto set, uint32_t j) {
+    constexpr int S = decltype(set)::value;
+    const uint32_t round = j / per_wave, chunk = (j % per_wave) * KS + ks, grp = group_of(round);
+    // the chunk's 16 rows into the wave's region: piece q of row r at slot q ^ r
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t r = 2 * i + (lane >> 5);
+      *reinterpret_cast<U4*>(region + r * kRowsChunk + (((lane & 31u) ^ r) * 16)) = w[S][i];
+    }
+    if constexpr (!A_LDS) {
+      const uint32_t at = rows_a_slot(lane);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) *reinterpret_cast<U4*>(own + i * kRowsOwnPitch + at) = av[S][i];
+    }
+    scales_lds[wave * 16 + c] = scl[S];  // (four lanes write each, the same value)
+    request(set, j + 2);
+    if (j < items && chunk < chunks && grp < groups) {
+      const uint32_t k0 = A_LDS ? chunk * kRowsChunk : 0;
+      // a step's operand reads are issued a step ahead (two register sets, used in turn)
+      struct Step {
+        U4 wv, a0, a1;
+      };
+      auto fetch = [&](Step& x, uint32_t s) {
+        // (a wave's LDS operations execute in order: these reads see the writes above)
+        x.wv = *reinterpret_cast<const U4*>(region + c * kRowsChunk + (((4 * s + g) ^ c) * 16));
+        x.a0 = *reinterpret_cast<const U4*>(a_frag + 2 * (k0 + 64 * s));
+        x.a1 = *reinterpret_cast<const U4*>(a_frag + 2 * (k0 + 64 * s) + 64);
+      };
+      auto multiply = [&](const Step& x) {
+        U4 wlo, whi;
+        widen16_to_operands<T>(x.wv, &wlo, &whi);
+        acc0 = mfma16<T>(wlo, x.a0, acc0);
+        acc1 = mfma16<T>(whi, x.a1, acc1);
+      };
+      Step even, odd;
+      fetch(even, 0);
+#pragma clang loop unroll(disable)
+      for (uint32_t s = 0; s < 8; s += 2) {
+        fetch(odd, s + 1);
+        __builtin_amdgcn_sched_barrier(0);  // (the scheduler would move each read down to its first use)
+        multiply(even);
+        fetch(even, s + 2 < 8 ? s + 2 : 7);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(odd);
+      }
+    }
+    if (j < items && (j + 1) % per_wave == 0) {  // the round's last chunk: the team's tiles meet in its first wave, added in wave order
+      V4F sum;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sum[r] = acc0[r] + acc1[r];
+      if constexpr (KS > 1) {
+        V4F* const slot = parts + (round & 1u) * (kRowsWaves * 64);  // (two sets of slots: one barrier per round)
+        slot[wave * 64 + lane] = sum;
+        __syncthreads();
+        if (ks == 0) {
+#pragma unroll
+          for (int q = 1; q < KS; ++q) {
+            const V4F v = slot[(wave + q) * 64 + lane];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sum[r] += v[r];
+          }
+        }
+      }
+      // lane (c, g): row c, columns 16 grp + 4 g .. + 3
+      const uint32_t n = grp * 16 + 4 * g;
+      if (ks == 0 && grp < groups && c < p.m && n < p.n) {
+        const uint64_t to = p.c + (uint64_t(c) * p.n + n) * item;
+        uint32_t h[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const uint16_t bits = scales_lds[wave * 16 + 4 * g + r];
+          const float v = sum[r] * (T::dtype == VKT_BF16 ? bf16_to_f32(bits) : f16_to_f32(bits));
+          h[r] = T::dtype == VKT_BF16 ? f32_to_bf16(v) : f32_to_f16(v);
+        }
+        if ((p.n & 3u) == 0 && (p.c & 7u) == 0) {
+          stg<U2>(to, U2{h[0] | h[1] << 16, h[2] | h[3] << 16});
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (n + r < p.n) stg<uint16_t>(to + r * item, uint16_t(h[r]));
+        }
+      }
+      acc0 = acc1 = V4F{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+  };
+  // (every wave of the workgroup runs the same number of items: the barriers inside are met by all)
+#pragma clang loop unroll(disable)
+  for (uint32_t j = 0; j < items; j += 2) {  // (an odd count's last pass works on nothing: both sets of registers take turns on every path)
+    work(std::integral_constant<int, 0>{}, j);
+    work(std::integral_constant<int, 1>{}, j + 1);
+  }
+}
+
+// The kernel above where it applies: 3 to 8 rows, k a multiple of 16 (checked by the caller), whole 16-byte pieces.
+// False: not this kernel's shape.
+template <class T>
+bool launch_rows_kernel(const Q8Params& p, bool whatever_the_size, const Machine& mc, hipStream_t stream) {
+  if (p.m < 3 || p.m > 8 || p.k < 512 || p.n < 16) return false;
+  // Measured against the slice kernels below (8 rows, microseconds, this kernel first): it streams at 6.2 TB/s once
+  // under way but takes about 7 us to get there and to drain, so it wins on large products only.
+  // K x N 4096 x 14336: 17.2 / 15.3, 14336 x 4096: 18.8 / 15.2, 4096 x 32000: 32.1 / 30.1, 8192 x 28672: 51.2 / 53.9,
+  // 4096 x 65536: 50.9 / 55.4, 4096 x 128256: 94.2 / 100.0, 8192 x 128256: 185.7 / 205.2
+  if (!whatever_the_size && uint64_t(p.n) * p.k < 200000000ull) return false;
+  // (32-bit byte offsets into B and A, each within a buffer descriptor of fewer than 2^31 bytes)
+  if (uint64_t(p.n) * p.k >= (1ull << 31) || p.a_sm < int64_t(p.k) || (uint64_t(p.m - 1) * uint64_t(p.a_sm) + p.k) * 2 >= (1ull << 31)) return false;
+  const uint32_t groups = (p.n + 15) / 16, cus = uint32_t(mc.compute_units);
+  // waves per group: as few as give most of the machine's 8 waves per compute unit a share of a group
+  const int ks = groups >= 6 * cus ? 1 : groups >= 3 * cus ? 2 : groups * 2 >= 3 * cus ? 4 : 8;
+  const bool a_lds = p.k <= 4096;  // (8 rows x 4096 values: 64 KiB, and 8 pieces of 16 bytes per thread to stage them)
+  const uint32_t lds = (a_lds ? 8 * rows_a_pitch(p.k) : kRowsWaves * kRowsOwn) + kRowsWaves * kRowsRegion + 2 * kRowsWaves * 64 * 16 + kRowsWaves * 32;
+  const uint32_t teams = kRowsWaves / uint32_t(ks), units = (groups + teams - 1) / teams;
+  const uint32_t grid = units < cus ? units : cus;
+#define VKT_ROWS_CASE(KS_, AL_)                                                                                              \
+  if (ks == KS_ && a_lds == AL_) {                                                                                           \
+    auto kernel = qmm8_rows<T, KS_, AL_>;                                                                                    \
+    static bool configured = false; /* guarded by the runtime's stream mutex */                                              \
+    if (!configured) {                                                                                                       \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024) != hipSuccess) { \
+        (void)hipGetLastError();                                                                                             \
+        return false;                                                                                                        \
+      }                                                                                                                      \
+      configured = true;                                                                                                     \
+    }                                                                                                                        \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(512), lds, stream, p, groups);                                               \
+    return true;                                                                                                             \
+  }
+  VKT_ROWS_CASE(1, true) VKT_ROWS_CASE(1, false) VKT_ROWS_CASE(2, true) VKT_ROWS_CASE(2, false)
+  VKT_ROWS_CASE(4, true) VKT_ROWS_CASE(4, false) VKT_ROWS_CASE(8, true) VKT_ROWS_CASE(8, false)
+#undef VKT_ROWS_CASE
+  return false;
+}
+
 // 33 to a few hundred rows (batched decode): a tile kernel.  A workgroup of 8 waves owns 64 rows x 128 columns and a
 // slice of K, walked in steps of 128 values.  Both operand tiles of a step are loaded into registers four steps
 // ahead and written to one of two LDS stages a step before they are multiplied: the activations [64 rows][256 bytes]
@@ -1213,6 +1450,10 @@ int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipSt
     // the vector units (measured at K = 4096, N = 14336: 10.5, 16.4, 23.0, 23.4 us for 1 to 4 rows; the matrix
     // cores take 16 us for up to 8).  variant bit 17 forces the GEMV kernels (tests, tuning).
     if (p0.m > 2 && !((variant >> 17) & 1)) {
+      // 3 to 8 rows over 200 MB of weights or more: the wave-per-column-group kernel (variant bit 23 keeps the kernels below)
+      // (bits 8-15 with bits 0-7 clear ask for it whatever the size: tests, tuning)
+      const bool asked = !(variant & 0xff) && ((variant >> 8) & 0xff);
+      if ((asked || !(variant & 0xffff)) && !((variant >> 18) & 3) && !((variant >> 23) & 1) && launch_rows_kernel<T>(p0, asked, mc, stream)) return 0;
       for (uint32_t r0 = 0; r0 < p0.m; r0 += 64) {
         Q8Params p = p0;
         p.m = p0.m - r0 < 64 ? p0.m - r0 : 64;
