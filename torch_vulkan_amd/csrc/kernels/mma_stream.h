@@ -96,8 +96,9 @@ __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_
     // (The lane's rows and chunks are worked out anew for every tile: as values that do not change in the loop the
     // compiler computes them once, finds no register to keep them in, and reloads them here from scratch memory,
     // each reload waiting for every load into LDS in flight: 1.5 us per tile.)
-    uint32_t ln = lane;
-    asm volatile("" : "+v"(ln));
+    // (the lane number likewise: counted anew, two instructions, rather than kept or reloaded)
+    uint32_t ln;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
 #pragma unroll
     for (uint32_t i = 0; i < uint32_t(PER); ++i) {
       const uint32_t r = wave * ROWS + 8 * i + (ln >> 3), c = (ln & 7u) ^ ((r >> 1) & 7u);
@@ -171,15 +172,14 @@ __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_
   const auto whole = p.whole();
 
   // The epilogue, straight from the accumulators.  A 32 x 32 matrix-core tile leaves lane l with row l % 32 and, for
-  // q = 0..3, columns 8 q + 4 (l / 32) .. + 3.  A lane finishes and packs its own values; two lanes 32 apart then hold
-  // the two halves of 8 consecutive outputs and v_permlane32_swap puts them together (lanes below 32 take chunk
-  // q = 0 or 2 of their row, lanes from 32 chunk 1 or 3), one store per 8 outputs.
+  // q = 0..3, columns 8 q + 4 (l / 32) .. + 3.  A lane finishes and packs its own values; three exchanges between lanes
+  // (32, 16 and 8 apart: two swap instructions and a row rotation) then bring the 128 bytes that two column blocks
+  // side by side hold of a row into 8 neighbouring lanes, so that a store instruction writes 8 whole 128-byte lines.
   // What the epilogue costs is the time its stores take to drain (every workgroup stores its tile at about the same
-  // time, with the matrix cores idle), and that depends on their order: two stores in a row that together write 64
-  // consecutive bytes of each of their 32 rows (this order: column block, row block, chunk pair) take 322 us on
-  // 8192^3 where the order column block, chunk pair, row block takes 347; eight in a row that fill two whole
-  // 128-byte lines per row are no faster, non-temporal stores are 1.5 times slower, and waiting after every few
-  // stores, or starting the workgroups a few microseconds apart, only costs.
+  // time, with the matrix cores idle).  Stores that write 32 or 64 bytes of each of their rows take as long, in any
+  // order tried, but put 1.5 times the output's bytes on the way to memory (counted: 201 MiB for the 128 MiB of
+  // 8192 x 8192 bfloat16 outputs); with whole lines the count is the output's size.  Non-temporal stores are 1.5 times
+  // slower, and waiting after every few stores, or starting the workgroups a few microseconds apart, only costs.
   auto epilogue = [&](const Tile& t) {
     const uint32_t wm0 = t.m0 + wm * (TM2 * 32), wn0 = t.n0 + wn * 128;
     typename P::Rows rows[TM2];
@@ -189,39 +189,86 @@ __global__ __launch_bounds__(512) void mma_stream(P p, uint32_t tiles_m, uint32_
       rows[i] = p.rows(t.batch, m < p.m ? m : p.m - 1, whole);
     }
     const bool narrow = p.narrow(whole);
+    // One 32 x 32 tile, finished, packed and exchanged twice: [0] the 8 outputs (16-bit: 4 words, 8-bit: 2) at
+    // row lane % 16, [1] at row 16 + lane % 16, both of chunk {0, 2, 1, 3}[lane / 16] of the tile's four chunks of 8
+    // columns.  (First exchange, lanes 32 apart: the two halves of a chunk meet.  Second, lanes 16 apart: the lanes of
+    // rows 16 .. 31 give their first chunk for the second chunk of the lanes 16 below.)
+    struct Packed {
+      uint32_t w[2][4];
+    };
+    auto packed_tile = [&](int i, int j, const uint32_t (&first_column)[4], const typename P::Columns4 (&columns)[4]) {
+      const uint32_t m = wm0 + 32 * i + l32, row = m < p.m ? m : p.m - 1;
+      const V16F& v = acc[i][j];
+      Packed out;
 #pragma unroll
-    for (int j = 0; j < TN2; ++j) {
-      uint32_t first_column[4];  // of this lane's four columns in chunk q of column block j (inside the matrix)
-      typename P::Columns4 columns[4];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const uint32_t n = wn0 + 32 * j + 8 * q + 4 * h;
-        first_column[q] = n + 4 <= p.n ? n : p.n - 4;
-        columns[q] = p.columns4(t.batch, first_column[q], whole);
+      for (int qp = 0; qp < 2; ++qp) {
+        const float first[4] = {v[8 * qp], v[8 * qp + 1], v[8 * qp + 2], v[8 * qp + 3]};
+        const float second[4] = {v[8 * qp + 4], v[8 * qp + 5], v[8 * qp + 6], v[8 * qp + 7]};
+        float f0[4], f1[4];
+        p.finish4(t.batch, row, first_column[2 * qp], first, rows[i], columns[2 * qp], whole, f0);
+        p.finish4(t.batch, row, first_column[2 * qp + 1], second, rows[i], columns[2 * qp + 1], whole, f1);
+        uint32_t lo[2] = {0, 0}, hi[2] = {0, 0};
+        p.pack4(f0, whole, lo);
+        p.pack4(f1, whole, hi);
+        const auto s0 = __builtin_amdgcn_permlane32_swap(lo[0], hi[0], false, false);
+        const auto s1 = __builtin_amdgcn_permlane32_swap(lo[1], hi[1], false, false);
+        out.w[qp][0] = s0[0], out.w[qp][1] = narrow ? s0[1] : s1[0], out.w[qp][2] = s0[1], out.w[qp][3] = s1[1];
       }
 #pragma unroll
-      for (int i = 0; i < TM2; ++i) {
-        const uint32_t m = wm0 + 32 * i + l32, row = m < p.m ? m : p.m - 1;
-        const V16F& v = acc[i][j];
+      for (int e = 0; e < 4; ++e) {
+        const auto x = __builtin_amdgcn_permlane16_swap(out.w[0][e], out.w[1][e], false, false);
+        out.w[0][e] = x[0], out.w[1][e] = x[1];
+      }
+      return out;
+    };
+    // Two column blocks side by side are 128 bytes of a row of 16-bit outputs.  A third exchange, between lanes 8 apart
+    // (lanes 8 .. 15 of every 16 give their left block's words for the right block's of the lanes 8 below), leaves a
+    // store instruction with whole 128-byte lines: rows lane % 8 (+ 8, 16, 24 for the four stores), left or right block
+    // by lane / 8 % 2, chunk by lane / 16.  (Stores of 32 or 64 bytes per row wrote 1.5 times the output's bytes to
+    // memory, whatever their order: counted.)
+    const bool upper8 = (lane & 8u) != 0;
+    auto exchange8 = [&](uint32_t& left, uint32_t& right) {
+      const uint32_t give = upper8 ? left : right;
+      const uint32_t got = uint32_t(__builtin_amdgcn_update_dpp(0, int(give), 0x128 /* row_ror:8 */, 0xf, 0xf, false));
+      left = upper8 ? got : left;
+      right = upper8 ? right : got;
+    };
 #pragma unroll
-        for (int qp = 0; qp < 2; ++qp) {
-          const uint32_t n = wn0 + 32 * j + 8 * (2 * qp + h);
-          const float first[4] = {v[8 * qp], v[8 * qp + 1], v[8 * qp + 2], v[8 * qp + 3]};
-          const float second[4] = {v[8 * qp + 4], v[8 * qp + 5], v[8 * qp + 6], v[8 * qp + 7]};
-          float f0[4], f1[4];
-          p.finish4(t.batch, row, first_column[2 * qp], first, rows[i], columns[2 * qp], whole, f0);
-          p.finish4(t.batch, row, first_column[2 * qp + 1], second, rows[i], columns[2 * qp + 1], whole, f1);
-          uint32_t lo[2], hi[2];
-          p.pack4(f0, whole, lo);
-          p.pack4(f1, whole, hi);
-          const bool inside = m < p.m && n + 8 <= p.n;
-          if (!narrow) {
-            const auto s0 = __builtin_amdgcn_permlane32_swap(lo[0], hi[0], false, false);
-            const auto s1 = __builtin_amdgcn_permlane32_swap(lo[1], hi[1], false, false);
-            if (inside) p.store8(t.batch, m, n, U4{s0[0], s1[0], s0[1], s1[1]});
-          } else {
-            const auto s0 = __builtin_amdgcn_permlane32_swap(lo[0], hi[0], false, false);
-            if (inside) p.store8_narrow(t.batch, m, n, U2{s0[0], s0[1]});
+    for (int jp = 0; jp < TN2 / 2; ++jp) {
+      Packed left[TM2];
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj) {
+        const int j = 2 * jp + jj;
+        uint32_t first_column[4];  // of this lane's four columns in chunk q of column block j (inside the matrix)
+        typename P::Columns4 columns[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t n = wn0 + 32 * j + 8 * q + 4 * h;
+          first_column[q] = n + 4 <= p.n ? n : p.n - 4;
+          columns[q] = p.columns4(t.batch, first_column[q], whole);
+        }
+#pragma unroll
+        for (int i = 0; i < TM2; ++i) {
+          if (jj == 0) {
+            left[i] = packed_tile(i, j, first_column, columns);
+            continue;
+          }
+          Packed right = packed_tile(i, j, first_column, columns);
+#pragma unroll
+          for (int half = 0; half < 2; ++half)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) exchange8(left[i].w[half][e], right.w[half][e]);
+          const uint32_t n = wn0 + 32 * (2 * jp + ((lane >> 3) & 1u)) + 8 * (2 * ((lane >> 4) & 1u) + h);
+#pragma unroll
+          for (int part = 0; part < 4; ++part) {  // rows lane % 8 + 8 part: left[half = 0], right[0], left[1], right[1]
+            const uint32_t mm = wm0 + 32 * i + 8 * part + (lane & 7u);
+            const uint32_t(&w)[4] = (part & 1) ? right.w[part >> 1] : left[i].w[part >> 1];
+            const bool inside = mm < p.m && n + 8 <= p.n;
+            if (!narrow) {
+              if (inside) p.store8(t.batch, mm, n, U4{w[0], w[1], w[2], w[3]});
+            } else {
+              if (inside) p.store8_narrow(t.batch, mm, n, U2{w[0], w[1]});
+            }
           }
         }
       }
