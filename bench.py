@@ -396,6 +396,7 @@ OTHER = {
     "q8_m1_k8192_n8192": lambda abi, s, w: wl_q8(abi, 1, 8192, 8192, abi.BF16, s, w, seed=1120),
     "q8_m8_k5120_n13824": lambda abi, s, w: wl_q8(abi, 8, 5120, 13824, abi.BF16, s, w, seed=1110),
     "q8_m64_k8192_n8192": lambda abi, s, w: wl_q8(abi, 64, 8192, 8192, abi.BF16, s, w, seed=1120),
+    "q8_m8_k4096_n128256": lambda abi, s, w: wl_q8(abi, 8, 4096, 128256, abi.BF16, max(s // 4, 10), w, seed=1130),  # (a vocabulary-sized projection)
     "f8_cast_bf16_e4m3_256mi": lambda abi, s, w: wl_cast(abi, 1 << 28, max(s // 10, 5), max(w // 4, 3)),
     "f8_quant_rowwise_bf16_16384x16384": lambda abi, s, w: wl_quant(abi, 16384, 16384, max(s // 10, 5), max(w // 4, 3)),
     "mm_bf16_8192": lambda abi, s, w: wl_gemm16(abi, 8192, 8192, 8192, max(s // 10, 5), max(w // 4, 3)),
@@ -438,7 +439,7 @@ def summarise(r):
         value, unit, peak = r["work"] / r["wall_ms"] / 1e9, "TFLOP/s", r.get("peak", FP8_PEAK_TFLOPS)
         achieved = r["work"] / r["event_ms"] / 1e9
     roof = dict(bound=r["kind"], achieved=round(achieved, 1), peak=peak, unit=unit, frac=round(achieved / peak, 4),
-                traffic=None)
+                traffic=None, algorithmic=r["work"])  # algorithmic: bytes (or operations) per step that `achieved` prices
     if r.get("event_ms_median"):  # the same figure from the median fifth of the timed loop
         roof["achieved_median_of_5"] = round(achieved * r["event_ms"] / r["event_ms_median"], 1)
     if r.get("cache_resident_ms"):  # one weight copy over and over: L2 / Infinity Cache, not HBM (reported, not priced)
