@@ -1354,7 +1354,13 @@ int launch_mfma(const Q8Params& p, uint32_t variant, const Machine& mc, hipStrea
   bool staged = (variant >> 18) & 1;
   if (!(variant & 0xffff) && !((variant >> 19) & 1) && p.m <= 8 && p.k >= 2048 && p.n >= 64) {
     staged = true;
-    nt = (p.k >= 16384 || (p.n >= 12288 && p.k <= 4096)) ? 2 : 1, waves = 8, slices = 1;  // (measured on the Llama shapes)
+    // 32 columns per workgroup where 16 would make two or more workgroups per compute unit and the 32 columns' share of
+    // the weights stays within 192 KiB; otherwise 16.  Measured at 8 rows, microseconds with 16 / 32 columns (K x N):
+    // 5120 x 13824: 21.0 / 17.7, 6144 x 16384: 25.3 / 21.5, 4096 x 14336: 20.0 / 15.1, 4096 x 28672: 34.8 / 27.6,
+    // 3072 x 9216: 11.8 / 11.3, 2048 x 8192: 7.1 / 6.7, 4096 x 4096: 8.3 / 8.6, 8192 x 8192: 18.7 / 20.5,
+    // 14336 x 4096: 15.2 / 19.8, 16384 x 4096: 19.7 / 22.1, 8192 x 28672: 52.9 / 56.2; 4 rows order the same way.
+    const uint32_t groups16 = (p.n + 15) / 16;
+    nt = (groups16 >= 2u * uint32_t(mc.compute_units) && 32ull * p.k <= 192 * 1024) ? 2 : 1, waves = 8, slices = 1;
   } else if (!(variant & 0xffff) && !((variant >> 19) & 1) && p.m <= 32 && p.k >= 2048 && p.k <= 8192 && p.n >= 8192) {
     // 9 to 32 rows against many short weight rows: 64 columns per workgroup (K = 4096, N = 14336: 17.3 and 21.7 us
     // at 16 and 32 rows against 18.6 and 23.3; with long rows and few columns the unstaged kernel stays ahead)
