@@ -119,7 +119,9 @@ uint64_t vkt_qmm4c_q_bytes(uint32_t m, uint32_t k);
  * kernel, 17 the vector-unit kernels, 18 / 19 the matrix-core kernel with / without staging through LDS, 20 no
  * widened-weights product for many rows, 21 / 22 the 64 x 128 tile kernel forced / off; one row: bit 23 keeps the
  * kernel with a workgroup per pair of columns, bits 8-11 / 12-15 (bits 0-7 clear) ask for the persistent streaming
- * kernel with that many workgroups per compute unit / rows per iteration. */
+ * kernel with that many workgroups per compute unit / rows per iteration; 3 to 8 rows: bit 23 keeps the slice
+ * kernels where the planner would take the kernel whose waves own column groups (large products), bits 8-15 (bits
+ * 0-7 clear) ask for that kernel whatever the size. */
 typedef struct Q8Params {
   uint64_t a, b, scales, c; /* A [m,k] (row stride a_sm, a_sk must be 1), B int8 [n,k], scales [n], C [m,n] */
   uint32_t m, n, k;
