@@ -800,20 +800,28 @@ __global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t groups) {
   };
   if constexpr (A_LDS) {
     // all rows, once per workgroup: row i's piece `tid` (a row has at most 512 pieces), through the same kind of
-    // descriptor; asked for before any weights: the barrier below waits for the last wave's pieces, and a compute
-    // unit's loads are served in the order they were issued
+    // descriptor; asked for before any weights.  The two barriers before the one that publishes A are barriers of
+    // ISSUE, not of data: a compute unit accepts ~64 KiB of loads and lets the oldest wave's instructions go first, so
+    // without them the first waves' second chunks are accepted before the last wave's first one, that wave cannot
+    // reach the code that writes its pieces of A to LDS, and everyone waits for it (compute started 5.7 us into the
+    // launch; with them 3.8-4.6)
     U4 a_regs[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       a_regs[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (tid * 16 + i * uint32_t(p.a_sm) * uint32_t(item)) | (uint32_t(i) < p.m && tid * 8 < p.k ? 0u : ~0u), 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
     request(std::integral_constant<int, 0>{}, 0);
-    request(std::integral_constant<int, 1>{}, 1);
+    __builtin_amdgcn_s_barrier();  // (every wave's first chunk before any wave's second)
+    __builtin_amdgcn_sched_barrier(0);
     if (tid * 16 < a_pitch - 64) {
       uint32_t at = rows_a_slot(tid);
 #pragma unroll
       for (int i = 0; i < 8; ++i, at += a_pitch) *reinterpret_cast<U4*>(rows_lds + at) = a_regs[i];
     }
     __syncthreads();
+    request(std::integral_constant<int, 1>{}, 1);
   } else {
     request(std::integral_constant<int, 0>{}, 0);
     request(std::integral_constant<int, 1>{}, 1);
