@@ -727,11 +727,13 @@ bool launch_staged(const Q8Params& p, int mt, int nt, int waves, uint32_t slices
 // weights), otherwise the wave's own 8 rows x 512 values, loaded with the weight chunk they meet.  The KS partial
 // tiles of a group meet in LDS, added in wave order.
 // What was measured (8 x 4096 x 14336, timestamps inside the kernel): a compute unit accepts about 64 KiB of loads
-// before the issue of further ones blocks, so the second chunk in flight buys little at the start (the last wave's
-// requests are accepted 4-6 us into the launch) and much in the steady state (1.45 us per chunk and pair of waves,
-// which is the vector units' time: widening 16 weights is 24 instructions of 4-5 cycles, the matrix cores' two
-// instructions of 16 cycles per 64 values of k hide behind them).  The loop over a chunk's eight 64-value steps is
-// rolled (a launch starts with a cold instruction cache).
+// before the issue of further ones blocks, and its older waves issue first.  So the second chunk in flight buys
+// little at the start and much in the steady state (the stream runs at 6.2 TB/s; a chunk costs a pair of waves
+// 1.45 us, which is the vector units' time: widening 16 weights is 24 instructions of 4-5 cycles, the matrix cores'
+// two instructions of 16 cycles per 64 values of k hide behind them), and the younger wave of every SIMD gets its
+// chunks later than the older one throughout: a unit's last two microseconds stream for half of its waves.  (A
+// barrier of issue per chunk, which keeps the waves level, costs more than that: 17.6 against 16.6 us.)  The loop
+// over a chunk's eight 64-value steps is rolled (a launch starts with a cold instruction cache).
 constexpr uint32_t kRowsChunk = 512, kRowsRegion = 16 * kRowsChunk, kRowsWaves = 8;
 // a wave's own activations of one chunk (rows longer than 4096): 8 rows x 512 values at the pitch below
 constexpr uint32_t kRowsOwnPitch = 2 * kRowsChunk + 64, kRowsOwn = 8 * kRowsOwnPitch;
