@@ -718,7 +718,8 @@ bool launch_staged(const Q8Params& p, int mt, int nt, int waves, uint32_t slices
 
 // Three to eight rows of 16-bit activations over a large weight matrix (batched decode at small batch, vocabulary-sized
 // projections): the weight stream of the one-row kernels with the arithmetic on the matrix cores.  One workgroup of
-// 8 waves per compute unit stays for the whole launch.  A column group is 16 weight rows; KS waves share its K, each
+// 8 waves per compute unit stays for the whole launch and owns a run of consecutive columns, the same count for every
+// workgroup.  A column group is 16 weight rows; KS waves share its K, each
 // taking every KS-th chunk of 512 bytes of every row: 8 loads of 2 rows x 512 contiguous bytes, into registers, two
 // chunks ahead.  A chunk goes through the wave's own 8 KiB of LDS (16-byte pieces swizzled by the row, so that
 // neither side has a bank conflict) to come back in the matrix core's operand shape (lane (c, g): row c, 16 bytes of
@@ -748,7 +749,7 @@ __host__ __device__ inline uint32_t rows_a_pitch(uint32_t k) { return 2 * ((k + 
 __device__ __forceinline__ uint32_t rows_a_slot(uint32_t piece) { return (piece / 8) * 128 + (piece & 1u) * 64 + ((piece & 7u) >> 1) * 16; }
 
 template <class T, int KS, bool A_LDS>
-__global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t groups) {
+__global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t cols_per_wg) {
   constexpr uint64_t item = 2;
   constexpr uint32_t TEAMS = kRowsWaves / KS;
   extern __shared__ __attribute__((aligned(16))) uint8_t rows_lds[];
@@ -761,10 +762,14 @@ __global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t groups) {
   V4F* const parts = reinterpret_cast<V4F*>(rows_lds + a_bytes + kRowsWaves * (kRowsRegion + (A_LDS ? 0 : kRowsOwn)));  // [2][8 waves][64 lanes]
   uint16_t* const scales_lds = reinterpret_cast<uint16_t*>(parts + 2 * kRowsWaves * 64);  // [8 waves][16]
 
-  // rounds: in round i team t works on group (i * TEAMS + t) * grid + block (all teams make the same number of
-  // rounds: the barrier below is the workgroup's)
-  const uint32_t span = TEAMS * gridDim.x, rounds = (groups + span - 1) / span;
-  auto group_of = [&](uint32_t round) { return (round * TEAMS + team) * gridDim.x + blockIdx.x; };
+  // A workgroup owns cols_per_wg consecutive columns (a multiple of 8; the same count for every workgroup, so that
+  // every compute unit streams the same bytes: with whole groups of 16 dealt out, 896 groups leave 32 of 256 units
+  // idle or give 192 of them twice the work of the rest), as groups of 16 of which the last may be partial.  In round
+  // i team t works on the workgroup's group i * TEAMS + t (all teams make the same number of rounds: the barrier
+  // below is the workgroup's).
+  const uint32_t col_begin = blockIdx.x * cols_per_wg, col_end = min(col_begin + cols_per_wg, p.n);
+  const uint32_t rounds = ((cols_per_wg + 15) / 16 + TEAMS - 1) / TEAMS;
+  auto first_col = [&](uint32_t round) { return col_begin + (round * TEAMS + team) * 16; };  // (at or past col_end: no group)
   const uint32_t items = rounds * per_wave;  // (group, chunk) pairs of this wave, some of them past the end
   // Two chunks are in flight per wave (registers), requested as soon as the registers are free.
   U4 w[2][8], av[2][A_LDS ? 1 : 8];
@@ -781,13 +786,13 @@ __global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t groups) {
     constexpr int S = decltype(set)::value;
     // (the fences keep one request's loads together and in program order, which is what the waits count on)
     __builtin_amdgcn_sched_barrier(0);
-    const uint32_t grp = group_of(j / per_wave), chunk = (j % per_wave) * KS + ks;
-    const uint32_t dead = j < items && grp < groups ? 0u : ~0u;  // (all ones: past every buffer)
+    const uint32_t n0 = first_col(j / per_wave), chunk = (j % per_wave) * KS + ks;
+    const uint32_t dead = j < items && n0 < col_end ? 0u : ~0u;  // (all ones: past every buffer)
     const uint32_t at = chunk * kRowsChunk + (lane & 31u) * 16;
-    const uint32_t row0 = grp * 16 + (lane >> 5), gone = dead | (at < p.k ? 0u : ~0u);
+    const uint32_t row0 = n0 + (lane >> 5), gone = dead | (at < p.k ? 0u : ~0u);
 #pragma unroll
     for (int i = 0; i < 8; ++i)  // rows 2 i + lane / 32
-      w[S][i] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, ((row0 + 2 * i) * p.k + at) | gone | (row0 + 2 * i < p.n ? 0u : ~0u), 0, kLoadStream);
+      w[S][i] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, ((row0 + 2 * i) * p.k + at) | gone | (row0 + 2 * i < col_end ? 0u : ~0u), 0, kLoadStream);
     if constexpr (!A_LDS) {  // row i's piece `lane` of the chunk
       const uint32_t ka = chunk * kRowsChunk + lane * 8;
       const uint32_t a_first = (ka * uint32_t(item)) | dead | (ka < p.k ? 0u : ~0u);
@@ -797,7 +802,7 @@ __global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t groups) {
     }
     // the group's 16 scales come with every chunk and go through LDS with it (loaded in the epilogue they would be
     // waited for behind two chunks in flight)
-    scl[S] = __builtin_amdgcn_raw_buffer_load_b16(s_rsrc, ((grp * 16 + c) * uint32_t(item)) | dead | (grp * 16 + c < p.n ? 0u : ~0u), 0, 0);
+    scl[S] = __builtin_amdgcn_raw_buffer_load_b16(s_rsrc, ((n0 + c) * uint32_t(item)) | dead | (n0 + c < col_end ? 0u : ~0u), 0, 0);
     __builtin_amdgcn_sched_barrier(0);
   };
   if constexpr (A_LDS) {
@@ -833,7 +838,7 @@ __global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t groups) {
   V4F acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = acc0;
   auto work = [&](auto set, uint32_t j) {
     constexpr int S = decltype(set)::value;
-    const uint32_t round = j / per_wave, chunk = (j % per_wave) * KS + ks, grp = group_of(round);
+    const uint32_t round = j / per_wave, chunk = (j % per_wave) * KS + ks, n0 = first_col(round);
     // the chunk's 16 rows into the wave's region: piece q of row r at slot q ^ r
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -847,7 +852,7 @@ __global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t groups) {
     }
     scales_lds[wave * 16 + c] = scl[S];  // (four lanes write each, the same value)
     request(set, j + 2);
-    if (j < items && chunk < chunks && grp < groups) {
+    if (j < items && chunk < chunks && n0 < col_end) {
       const uint32_t k0 = A_LDS ? chunk * kRowsChunk : 0;
       // a step's operand reads are issued a step ahead (two register sets, used in turn)
       struct Step {
@@ -894,9 +899,9 @@ __global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t groups) {
           }
         }
       }
-      // lane (c, g): row c, columns 16 grp + 4 g .. + 3
-      const uint32_t n = grp * 16 + 4 * g;
-      if (ks == 0 && grp < groups && c < p.m && n < p.n) {
+      // lane (c, g): row c, columns n0 + 4 g .. + 3 (a partial group ends at col_end, a multiple of 8 or n)
+      const uint32_t n = n0 + 4 * g;
+      if (ks == 0 && c < p.m && n < col_end) {
         const uint64_t to = p.c + (uint64_t(c) * p.n + n) * item;
         uint32_t h[4];
 #pragma unroll
@@ -910,7 +915,7 @@ __global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t groups) {
         } else {
 #pragma unroll
           for (int r = 0; r < 4; ++r)
-            if (n + r < p.n) stg<uint16_t>(to + r * item, uint16_t(h[r]));
+            if (n + r < col_end) stg<uint16_t>(to + r * item, uint16_t(h[r]));
         }
       }
       acc0 = acc1 = V4F{0.0f, 0.0f, 0.0f, 0.0f};
@@ -929,20 +934,34 @@ __global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t groups) {
 template <class T>
 bool launch_rows_kernel(const Q8Params& p, bool whatever_the_size, const Machine& mc, hipStream_t stream) {
   if (p.m < 3 || p.m > 8 || p.k < 512 || p.n < 16) return false;
-  // Measured against the slice kernels below (8 rows, microseconds, this kernel first): it streams at 6.2 TB/s once
-  // under way but takes about 7 us to get there and to drain, so it wins on large products only.
-  // K x N 4096 x 14336: 17.2 / 15.3, 14336 x 4096: 18.8 / 15.2, 4096 x 32000: 32.1 / 30.1, 8192 x 28672: 51.2 / 53.9,
-  // 4096 x 65536: 50.9 / 55.4, 4096 x 128256: 94.2 / 100.0, 8192 x 128256: 185.7 / 205.2
-  if (!whatever_the_size && uint64_t(p.n) * p.k < 200000000ull) return false;
+  // Measured against the slice kernels below (8 rows, microseconds, this kernel first).  It streams faster than they
+  // do once under way (5.9 TB/s over a whole launch at 4096 x 128256) but takes ~6.5 us to get there and to drain, and
+  // its waves own whole groups: it pays where a workgroup has 8 groups or more and the activations stay in LDS,
+  //   K x N 1024 x 131072: 28.0 / 31.5, 2048 x 32768: 15.9 / 17.2, 2048 x 65536: 26.5 / 29.7 (5 rows), 3072 x 32768: 21.2 /
+  //   22.0, 4096 x 32000: 29.3 / 29.9, 4096 x 49152: 43.0 / 43.1, 4096 x 65536: 50.9 / 55.3, 4096 x 128256: 89.4 / 100.1
+  //   (and not 4096 x 14336: 16.4 / 15.3, 4096 x 20480: 22.7 / 22.1, 4096 x 24576: 25.8 / 24.9),
+  // and with longer rows (a wave then asks for its own activations with every chunk, as many bytes again, from L2)
+  // only where the slice kernels run their 16-column form and the product is large,
+  //   8192 x 16384: 30.8 / 32.6, 8192 x 28672: 50.4 / 54.1, 16384 x 16384: 54.2 / 61.0, 12288 x 32768: 83.0 / 84.7,
+  //   8192 x 128256: 185.7 / 205.2 (and not 14336 x 4096: 18.6 / 15.1, 5120 x 51200: 63.3 / 50.8, 6144 x 65536: 76.9 / 69.2,
+  //   7168 x 28672: 46.2 / 46.1).
+  {
+    const uint32_t cus0 = uint32_t(mc.compute_units), units = (p.n + 15) / 16 < cus0 ? (p.n + 15) / 16 : cus0;
+    const bool pays = p.k <= 4096 ? (p.n + units - 1) / units >= 121 : p.k >= 8192 && uint64_t(p.n) * p.k >= (128ull << 20);
+    if (!whatever_the_size && !pays) return false;
+  }
   // (32-bit byte offsets into B and A, each within a buffer descriptor of fewer than 2^31 bytes)
   if (uint64_t(p.n) * p.k >= (1ull << 31) || p.a_sm < int64_t(p.k) || (uint64_t(p.m - 1) * uint64_t(p.a_sm) + p.k) * 2 >= (1ull << 31)) return false;
-  const uint32_t groups = (p.n + 15) / 16, cus = uint32_t(mc.compute_units);
-  // waves per group: as few as give most of the machine's 8 waves per compute unit a share of a group
-  const int ks = groups >= 6 * cus ? 1 : groups >= 3 * cus ? 2 : groups * 2 >= 3 * cus ? 4 : 8;
+  const uint32_t cus = uint32_t(mc.compute_units), groups = (p.n + 15) / 16;
+  // columns per workgroup: the same for every compute unit, a multiple of 8; waves per group: as few as give most of
+  // the workgroup's 8 waves a share of a group
+  uint32_t grid = groups < cus ? groups : cus;
+  const uint32_t cols_per_wg = ((p.n + grid - 1) / grid + 7) / 8 * 8;
+  grid = (p.n + cols_per_wg - 1) / cols_per_wg;
+  const uint32_t local = (cols_per_wg + 15) / 16;
+  const int ks = local >= 5 ? 1 : local >= 3 ? 2 : local == 2 ? 4 : 8;
   const bool a_lds = p.k <= 4096;  // (8 rows x 4096 values: 64 KiB, and 8 pieces of 16 bytes per thread to stage them)
   const uint32_t lds = (a_lds ? 8 * rows_a_pitch(p.k) : kRowsWaves * kRowsOwn) + kRowsWaves * kRowsRegion + 2 * kRowsWaves * 64 * 16 + kRowsWaves * 32;
-  const uint32_t teams = kRowsWaves / uint32_t(ks), units = (groups + teams - 1) / teams;
-  const uint32_t grid = units < cus ? units : cus;
 #define VKT_ROWS_CASE(KS_, AL_)                                                                                              \
   if (ks == KS_ && a_lds == AL_) {                                                                                           \
     auto kernel = qmm8_rows<T, KS_, AL_>;                                                                                    \
@@ -954,7 +973,7 @@ bool launch_rows_kernel(const Q8Params& p, bool whatever_the_size, const Machine
       }                                                                                                                      \
       configured = true;                                                                                                     \
     }                                                                                                                        \
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(512), lds, stream, p, groups);                                               \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(512), lds, stream, p, cols_per_wg);                                               \
     return true;                                                                                                             \
   }
   VKT_ROWS_CASE(1, true) VKT_ROWS_CASE(1, false) VKT_ROWS_CASE(2, true) VKT_ROWS_CASE(2, false)
@@ -1466,7 +1485,7 @@ int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipSt
     // the vector units (measured at K = 4096, N = 14336: 10.5, 16.4, 23.0, 23.4 us for 1 to 4 rows; the matrix
     // cores take 16 us for up to 8).  variant bit 17 forces the GEMV kernels (tests, tuning).
     if (p0.m > 2 && !((variant >> 17) & 1)) {
-      // 3 to 8 rows over 200 MB of weights or more: the wave-per-column-group kernel (variant bit 23 keeps the kernels below)
+      // 3 to 8 rows over large weights: the wave-per-column-group kernel where it pays (variant bit 23 keeps the kernels below)
       // (bits 8-15 with bits 0-7 clear ask for it whatever the size: tests, tuning)
       const bool asked = !(variant & 0xff) && ((variant >> 8) & 0xff);
       if ((asked || !(variant & 0xffff)) && !((variant >> 18) & 3) && !((variant >> 23) & 1) && launch_rows_kernel<T>(p0, asked, mc, stream)) return 0;
