@@ -411,7 +411,8 @@ __device__ __forceinline__ V4F mfma16(const U4& w, const U4& a, const V4F& acc) 
 // The epilogue of the matrix-core kernels: lane (c = lane % 16, g = lane / 16) holds, per
 // tile (mt, t), the sums of row 16 mt + c for columns n0 + 16 t + 4 g .. + 3.
 template <class T, int MT, int NT>
-__device__ __forceinline__ void store_tiles(const Q8Params& p, uint32_t n0, const V4F (&acc)[MT][NT], int lane) {
+__device__ __forceinline__ void store_tiles(const Q8Params& p, uint32_t n0, const V4F (&acc)[MT][NT], int lane, uint32_t n_end = ~0u) {
+  n_end = n_end < p.n ? n_end : p.n;  // (columns from n_end on are another workgroup's; a multiple of 4, or n)
   constexpr uint64_t item = 2;
   const int c = lane & 15, g = lane >> 4;
   const bool vec_ok = (p.n & 3u) == 0 && (p.c & 7u) == 0;
@@ -424,7 +425,7 @@ __device__ __forceinline__ void store_tiles(const Q8Params& p, uint32_t n0, cons
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const uint32_t m = 16 * mt + c;
-      if (m >= p.m || n >= p.n) continue;
+      if (m >= p.m || n >= n_end) continue;
       const uint64_t at = p.c + (uint64_t(m) * p.n + n) * item;
       uint32_t h[4];
 #pragma unroll
@@ -432,12 +433,12 @@ __device__ __forceinline__ void store_tiles(const Q8Params& p, uint32_t n0, cons
         const float v = acc[mt][t][r] * scale[r];
         h[r] = T::dtype == VKT_BF16 ? f32_to_bf16(v) : f32_to_f16(v);
       }
-      if (vec_ok && n + 3 < p.n) {
+      if (vec_ok && n + 3 < n_end) {
         stg<U2>(at, U2{h[0] | h[1] << 16, h[2] | h[3] << 16});
       } else {
 #pragma unroll
         for (int r = 0; r < 4; ++r)
-          if (n + r < p.n) stg<uint16_t>(at + r * item, uint16_t(h[r]));
+          if (n + r < n_end) stg<uint16_t>(at + r * item, uint16_t(h[r]));
       }
     }
   }
@@ -557,7 +558,7 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma(Q8Params p, uint32_t chu
 // values of k: all loads of a chunk are issued, awaited (vmcnt(0)) and consumed; the waves of a
 // workgroup drift apart and keep the memory pipeline full between them.
 template <class T, int MT, int NT, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void qmm8_mfma_staged(Q8Params p, uint32_t chunks_per_slice, uint64_t workspace) {
+__global__ __launch_bounds__(WAVES * 64) void qmm8_mfma_staged(Q8Params p, uint32_t chunks_per_slice, uint64_t workspace, uint32_t cols_per_wg) {
   constexpr uint64_t item = 2;
   constexpr uint32_t TILE = 16 * 256, REGION = NT * TILE;  // bytes of LDS per tile of 16 rows, per wave
   extern __shared__ __attribute__((aligned(16))) uint8_t staged[];
@@ -566,7 +567,8 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma_staged(Q8Params p, uint3
   const uint32_t total = (p.k + 255) / 256;
   const uint32_t q_begin = blockIdx.y * chunks_per_slice;
   const uint32_t q_end = q_begin + chunks_per_slice < total ? q_begin + chunks_per_slice : total;
-  const uint32_t n0 = blockIdx.x * 16 * NT;
+  // the workgroup's columns: cols_per_wg of them (at most 16 NT, a multiple of 4; 16 NT when K is sliced over workgroups)
+  const uint32_t n0 = blockIdx.x * cols_per_wg, n_end = n0 + cols_per_wg < p.n ? n0 + cols_per_wg : p.n;
   // loads: instruction i of tile t fetches rows 4 i .. 4 i + 3; this lane row 4 i + (lane / 16), slot lane % 16
   uint64_t wsrc[NT][4];
   uint32_t wk[4];  // byte offset within the chunk of the 16 bytes this lane fetches
@@ -576,7 +578,7 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma_staged(Q8Params p, uint3
     wk[i] = ((uint32_t(c) ^ row) & 15u) * 16;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      const uint32_t n = n0 + 16 * t + row < p.n ? n0 + 16 * t + row : p.n - 1;
+      const uint32_t n = n0 + 16 * t + row < n_end ? n0 + 16 * t + row : n_end - 1;  // (rows past the end: the last one again, from the caches)
       wsrc[t][i] = p.b + uint64_t(n) * p.k;
     }
   }
@@ -654,7 +656,7 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma_staged(Q8Params p, uint3
     for (int i = 0; i < MT * NT; ++i) out[i * 64 + lane] = acc[i / NT][i % NT];
     return;
   }
-  store_tiles<T, MT, NT>(p, n0, acc, lane);
+  store_tiles<T, MT, NT>(p, n0, acc, lane, n_end);
 }
 
 // Adds up the slices of one column group (one wave per group), in slice order.
@@ -697,9 +699,18 @@ bool launch_staged_one(const Q8Params& p, uint32_t slices, const Machine& mc, hi
     }
     configured = true;
   }
-  const dim3 grid((p.n + 16 * NT - 1) / (16 * NT), slices);
+  // One slice: the columns are dealt out evenly over a whole number of workgroups per compute unit (N = 14336 in 32s is
+  // 448 workgroups, two for 192 of 256 units and one for the rest, and the launch lasts as long as the two take; in 28s
+  // it is 512, two for each: the same bytes everywhere).  Several slices: whole tiles, which the second launch expects.
+  uint32_t cols = 16 * NT;
+  if (slices == 1) {
+    const uint32_t cus = uint32_t(mc.compute_units), wgs = (p.n + cols - 1) / cols, even = (wgs + cus - 1) / cus * cus;
+    const uint32_t fewer = ((p.n + even - 1) / even + 3) / 4 * 4;
+    if (fewer >= 8 && fewer < cols) cols = fewer;
+  }
+  const dim3 grid((p.n + cols - 1) / cols, slices);
   const uint32_t chunks = (p.k + 255) / 256, per_slice = (chunks + slices - 1) / slices;
-  hipLaunchKernelGGL(kernel, grid, dim3(WAVES * 64), lds, stream, p, per_slice, mc.workspace);
+  hipLaunchKernelGGL(kernel, grid, dim3(WAVES * 64), lds, stream, p, per_slice, mc.workspace, cols);
   if (slices > 1) hipLaunchKernelGGL((qmm8_mfma_finish<T, MT, NT>), dim3(grid.x), dim3(64), 0, stream, p, slices, mc.workspace);
   return true;
 }
@@ -936,18 +947,17 @@ bool launch_rows_kernel(const Q8Params& p, bool whatever_the_size, const Machine
   if (p.m < 3 || p.m > 8 || p.k < 512 || p.n < 16) return false;
   // Measured against the slice kernels below (8 rows, microseconds, this kernel first).  It streams faster than they
   // do once under way (5.9 TB/s over a whole launch at 4096 x 128256) but takes ~6.5 us to get there and to drain, and
-  // its waves own whole groups: it pays where a workgroup has 8 groups or more and the activations stay in LDS,
-  //   K x N 1024 x 131072: 28.0 / 31.5, 2048 x 32768: 15.9 / 17.2, 2048 x 65536: 26.5 / 29.7 (5 rows), 3072 x 32768: 21.2 /
-  //   22.0, 4096 x 32000: 29.3 / 29.9, 4096 x 49152: 43.0 / 43.1, 4096 x 65536: 50.9 / 55.3, 4096 x 128256: 89.4 / 100.1
-  //   (and not 4096 x 14336: 16.4 / 15.3, 4096 x 20480: 22.7 / 22.1, 4096 x 24576: 25.8 / 24.9),
+  // its waves own whole groups.  It pays where a workgroup has 8 groups or more and the activations stay in LDS,
+  //   K x N 1024 x 131072: 28.0 / 31.2, 2048 x 32768: 15.9 / 17.2, 2048 x 65536: 26.4 / 31.8, 3072 x 32768: 21.4 / 22.0,
+  //   4096 x 32000: 29.3 / 29.7, 4096 x 49152: 42.8 / 43.1, 4096 x 65536: 50.5 / 55.1, 4096 x 128256: 89.7 / 99.5
+  //   (and not 4096 x 14336: 16.4 / 14.3, 4096 x 20480: 22.7 / 22.1, 4096 x 24576: 25.8 / 24.9),
   // and with longer rows (a wave then asks for its own activations with every chunk, as many bytes again, from L2)
-  // only where the slice kernels run their 16-column form and the product is large,
-  //   8192 x 16384: 30.8 / 32.6, 8192 x 28672: 50.4 / 54.1, 16384 x 16384: 54.2 / 61.0, 12288 x 32768: 83.0 / 84.7,
-  //   8192 x 128256: 185.7 / 205.2 (and not 14336 x 4096: 18.6 / 15.1, 5120 x 51200: 63.3 / 50.8, 6144 x 65536: 76.9 / 69.2,
-  //   7168 x 28672: 46.2 / 46.1).
+  // from 16 groups per workgroup on,
+  //   8192 x 128256: 179.5 / 208.7 (and not 14336 x 4096: 18.6 / 15.1, 8192 x 28672: 51.2 / 44.3, 12288 x 32768: 82.8 / 73.6,
+  //   5120 x 51200: 63.3 / 50.8, 6144 x 65536: 76.9 / 69.2; about level: 16384 x 16384: 53.3 / 54.9, 8192 x 16384: 30.9 / 33.3).
   {
     const uint32_t cus0 = uint32_t(mc.compute_units), units = (p.n + 15) / 16 < cus0 ? (p.n + 15) / 16 : cus0;
-    const bool pays = p.k <= 4096 ? (p.n + units - 1) / units >= 121 : p.k >= 8192 && uint64_t(p.n) * p.k >= (128ull << 20);
+    const bool pays = (p.n + units - 1) / units >= (p.k <= 4096 ? 121u : 241u);
     if (!whatever_the_size && !pays) return false;
   }
   // (32-bit byte offsets into B and A, each within a buffer descriptor of fewer than 2^31 bytes)
@@ -1383,13 +1393,15 @@ int launch_mfma(const Q8Params& p, uint32_t variant, const Machine& mc, hipStrea
   bool staged = (variant >> 18) & 1;
   if (!(variant & 0xffff) && !((variant >> 19) & 1) && p.m <= 8 && p.k >= 2048 && p.n >= 64) {
     staged = true;
-    // 32 columns per workgroup where 16 would make two or more workgroups per compute unit and the 32 columns' share of
-    // the weights stays within 192 KiB; otherwise 16.  Measured at 8 rows, microseconds with 16 / 32 columns (K x N):
-    // 5120 x 13824: 21.0 / 17.7, 6144 x 16384: 25.3 / 21.5, 4096 x 14336: 20.0 / 15.1, 4096 x 28672: 34.8 / 27.6,
-    // 3072 x 9216: 11.8 / 11.3, 2048 x 8192: 7.1 / 6.7, 4096 x 4096: 8.3 / 8.6, 8192 x 8192: 18.7 / 20.5,
-    // 14336 x 4096: 15.2 / 19.8, 16384 x 4096: 19.7 / 22.1, 8192 x 28672: 52.9 / 56.2; 4 rows order the same way.
+    // 32 columns per workgroup where 16 would make two or more workgroups per compute unit, otherwise 16 (the launch
+    // below then deals the columns out evenly, 28 or 20 per workgroup where 32 do not divide them over the machine).
+    // Measured at 8 rows, microseconds with 16 / 32 columns (K x N): 5120 x 13824: 21.0 / 17.5, 6144 x 16384: 24.8 / 21.5,
+    // 4096 x 14336: 19.6 / 14.3, 4096 x 28672: 34.6 / 25.0, 3072 x 9216: 12.0 / 10.3, 2048 x 8192: 7.1 / 6.7, 4096 x 8192:
+    // 11.7 / 10.6, 8192 x 9216: 22.1 / 20.8, 14336 x 8192: 28.1 / 23.8, 8192 x 28672: 53.0 / 43.0, 14336 x 14336: 48.6 / 39.2,
+    // 16384 x 16384: 59.8 / 54.0, 12288 x 32768: 83.4 / 72.6; and 4096 x 4096: 8.2 / 8.6, 14336 x 4096: 15.4 / 17.4,
+    // 16384 x 4096: 19.5 / 21.4.  (One shape goes against the rule: 8192 x 8192 18.4 / 20.4.)  4 rows order the same way.
     const uint32_t groups16 = (p.n + 15) / 16;
-    nt = (groups16 >= 2u * uint32_t(mc.compute_units) && 32ull * p.k <= 192 * 1024) ? 2 : 1, waves = 8, slices = 1;
+    nt = groups16 >= 2u * uint32_t(mc.compute_units) ? 2 : 1, waves = 8, slices = 1;
   } else if (!(variant & 0xffff) && !((variant >> 19) & 1) && p.m <= 32 && p.k >= 2048 && p.k <= 8192 && p.n >= 8192) {
     // 9 to 32 rows against many short weight rows: 64 columns per workgroup (K = 4096, N = 14336: 17.3 and 21.7 us
     // at 16 and 32 rows against 18.6 and 23.3; with long rows and few columns the unstaged kernel stays ahead)
