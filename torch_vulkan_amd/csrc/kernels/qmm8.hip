@@ -1343,11 +1343,22 @@ int launch_tile_kernel(const Q8Params& p, uint32_t want_slices, const Machine& m
   }
   const uint32_t gx = (p.n + 127) / 128, gy = (p.m + 63) / 64, steps = p.k / kTileStepK;
   uint32_t slices = want_slices;
-  if (slices == 0) {  // about one workgroup per compute unit (measured: more slices cost more than they fill), 2 steps per slice at least
-    slices = (uint32_t(mc.compute_units) + gx * gy / 2) / (gx * gy);
-    const uint32_t most = steps / 4 ? steps / 4 : 1;
-    slices = slices > most ? most : slices;
-    slices = slices < 1 ? 1 : slices;
+  if (slices == 0) {
+    // The count of slices with the shortest estimated launch, 4 steps per slice at least.  The estimate, in
+    // microseconds, from what was measured at 64 rows: every round of workgroups over the machine takes 3 (until its
+    // first operands are in LDS) + 0.72 per step (three times that with float32 activations, whose planes are
+    // multiplied one after the other); more than one slice costs the second launch, 4.5, and its partial tiles written
+    // and read back at 5 TB/s.  (Rounding tiles x slices to the nearest count of compute units, the rule before, gave
+    // N = 11008 three slices: 258 workgroups on 256 units, two rounds of 11 steps, 31.2-32.6 us; two slices, one round
+    // of 16 steps: 22.6-22.9.)
+    const uint32_t cus = uint32_t(mc.compute_units), most = steps / 4 ? steps / 4 : 1;
+    const float step_us = T::dtype == VKT_F32 ? 2.2f : 0.72f, partial_us = float(p.m) * float(p.n) * 8.0f / 5e6f;
+    float best = 1e30f;
+    for (uint32_t s = 1; s <= most && s <= 64; ++s) {
+      const uint32_t rounds = (gx * gy * s + cus - 1) / cus;
+      const float cost = float(rounds) * (3.0f + step_us * float((steps + s - 1) / s)) + (s > 1 ? 4.5f + partial_us * float(s) : 0.0f);
+      if (cost < best) best = cost, slices = s;
+    }
   }
   if (slices > 1 && workspace_refused(mc, uint64_t(slices) * p.m * p.n * 4, err)) return -1;
   while (slices > 1 && uint64_t(slices) * p.m * p.n * 4 > mc.workspace_bytes) --slices;
