@@ -87,6 +87,21 @@ def test_qmm8_matrix_core_variants(dtype, variant, m, k, n):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,k,n", [(8, 2048, 8195), (5, 2048, 9216), (8, 2048, 13824), (3, 2048, 8200), (20, 2048, 8196),
+                                   (32, 2048, 14336), (8, 2048, 2049), (8, 2304, 2100), (8, 2048, 14336)])
+def test_qmm8_columns_dealt_out_evenly(dtype, m, k, n):
+    """3 to 32 rows on the kernel that stages weights through LDS, planned by the library: the launch deals the columns
+    out over a whole number of workgroups per compute unit, so a workgroup owns 12, 20, 28, 36 or 56 columns and not
+    whole tiles of 16; n off the vector width (scalar stores), a last workgroup with fewer columns, rows of A further
+    apart than k."""
+    import _dev
+    a, b, s = int8_case(dtype, m, k, n, seeds={"a": 4, "b": 5, "scales": 6})
+    check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s)), a, b, s, dtype)
+    if (m + 1) // 2 >= 3:
+        check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), row_step=2), a, b, s, dtype, rows=slice(None, None, 2))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("m,k,n", [(8, 512, 24600), (5, 1024, 33001), (8, 4096, 14336), (3, 4112, 12300), (7, 2064, 8192),
                                    (8, 14336, 4096), (4, 528, 70), (6, 512, 16), (8, 9216, 1000)])
 def test_qmm8_rows_kernel(dtype, m, k, n):
