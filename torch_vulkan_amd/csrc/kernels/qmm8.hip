@@ -609,8 +609,13 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma_staged(Q8Params p, uint3
         wr[t][i] = ldg_stream<U4>(wsrc[t][i] + (k0 + wk[i] < p.k ? k0 + wk[i] : 0u));
       }
   };
-  if (q_begin + wave < q_end) request(q_begin + wave);
-  for (uint32_t q = q_begin + wave; q < q_end; q += WAVES) {
+  // Workgroups start at different chunks of their slice and wrap around: with rows a power of two apart, all
+  // workgroups reading the same offsets of their rows at the same time keep to a few memory channels.
+  const uint32_t count = q_end - q_begin, rot = (blockIdx.x * 5u) % count;
+  auto chunk_at = [&](uint32_t i) { return q_begin + (i + rot) % count; };  // the i-th chunk this workgroup works on
+  if (uint32_t(wave) < count) request(chunk_at(wave));
+  for (uint32_t i = wave; i < count; i += WAVES) {
+    const uint32_t q = chunk_at(i);
     const uint32_t k0 = q * 256;
     U4 a0[MT][4], a1[MT][4];
 #pragma unroll
@@ -628,7 +633,7 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma_staged(Q8Params p, uint3
     for (int t = 0; t < NT; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) *reinterpret_cast<U4*>(mine + (t * 16 + 4 * i) * 256 + lane * 16) = wr[t][i];
-    if (q + WAVES < q_end) request(q + WAVES);
+    if (i + WAVES < count) request(chunk_at(i + WAVES));
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -1410,7 +1415,8 @@ int launch_mfma(const Q8Params& p, uint32_t variant, const Machine& mc, hipStrea
     // 4096 x 14336: 19.6 / 14.3, 4096 x 28672: 34.6 / 25.0, 3072 x 9216: 12.0 / 10.3, 2048 x 8192: 7.1 / 6.7, 4096 x 8192:
     // 11.7 / 10.6, 8192 x 9216: 22.1 / 20.8, 14336 x 8192: 28.1 / 23.8, 8192 x 28672: 53.0 / 43.0, 14336 x 14336: 48.6 / 39.2,
     // 16384 x 16384: 59.8 / 54.0, 12288 x 32768: 83.4 / 72.6; and 4096 x 4096: 8.2 / 8.6, 14336 x 4096: 15.4 / 17.4,
-    // 16384 x 4096: 19.5 / 21.4.  (One shape goes against the rule: 8192 x 8192 18.4 / 20.4.)  4 rows order the same way.
+    // 16384 x 4096: 19.5 / 21.4.  4 rows order the same way.  (8192 x 8192 read 18.4 / 20.4 until the workgroups' chunk
+    // orders were rotated against each other: 17.9 / 15.6 since.)
     const uint32_t groups16 = (p.n + 15) / 16;
     nt = groups16 >= 2u * uint32_t(mc.compute_units) ? 2 : 1, waves = 8, slices = 1;
   } else if (!(variant & 0xffff) && !((variant >> 19) & 1) && p.m <= 32 && p.k >= 2048 && p.k <= 8192 && p.n >= 8192) {
