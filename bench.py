@@ -397,6 +397,7 @@ OTHER = {
     "q8_m8_k5120_n13824": lambda abi, s, w: wl_q8(abi, 8, 5120, 13824, abi.BF16, s, w, seed=1110),
     "q8_m64_k8192_n8192": lambda abi, s, w: wl_q8(abi, 64, 8192, 8192, abi.BF16, s, w, seed=1120),
     "q8_m8_k4096_n128256": lambda abi, s, w: wl_q8(abi, 8, 4096, 128256, abi.BF16, max(s // 4, 10), w, seed=1130),  # (a vocabulary-sized projection)
+    "q8_m8_k2048_n128256": lambda abi, s, w: wl_q8(abi, 8, 2048, 128256, abi.BF16, max(s // 4, 10), w, seed=1140),  # (the same of a smaller model)
     "f8_cast_bf16_e4m3_256mi": lambda abi, s, w: wl_cast(abi, 1 << 28, max(s // 10, 5), max(w // 4, 3)),
     "f8_quant_rowwise_bf16_16384x16384": lambda abi, s, w: wl_quant(abi, 16384, 16384, max(s // 10, 5), max(w // 4, 3)),
     "mm_bf16_8192": lambda abi, s, w: wl_gemm16(abi, 8192, 8192, 8192, max(s // 10, 5), max(w // 4, 3)),

@@ -102,13 +102,13 @@ def test_qmm8_columns_dealt_out_evenly(dtype, m, k, n):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("m,k,n", [(8, 512, 24600), (5, 1024, 33001), (8, 4096, 14336), (3, 4112, 12300), (7, 2064, 8192),
-                                   (8, 14336, 4096), (4, 528, 70), (6, 512, 16), (8, 9216, 1000)])
+@pytest.mark.parametrize("m,k,n", [(8, 512, 24600), (5, 1024, 33001), (8, 4096, 14336), (3, 3088, 12300), (7, 2064, 8192),
+                                   (8, 4080, 4096), (4, 528, 70), (6, 512, 16), (8, 3600, 1000), (8, 2048, 34000)])
 def test_qmm8_rows_kernel(dtype, m, k, n):
-    """3 to 8 rows over a large weight matrix run on the kernel whose waves own column groups (asked for here
-    whatever the size: variant bits 8-15): 1, 2, 4 and 8 waves per group, one and several rounds per workgroup,
-    activations staged whole (k <= 4096) and by chunk, k off the chunk size, n off the group and vector sizes,
-    rows of A further apart than k."""
+    """3 to 8 short rows against many columns run on the kernel whose waves own column groups (asked for here
+    whatever the size: variant bits 8-15; the last shape is one the planner sends there itself): 1, 2, 4 and 8 waves
+    per group, one and several rounds per workgroup, a partial last group, k off the chunk size, n off the group and
+    vector sizes, rows of A further apart than k."""
     import _dev
     # (seeds of its own: among the first table's scales for n > 27482 is the smallest float16 subnormal, and a float16
     # output that small is further from the float64 sum than the bound allows however it is rounded)

@@ -732,17 +732,19 @@ bool launch_staged(const Q8Params& p, int mt, int nt, int waves, uint32_t slices
   return false;
 }
 
-// Three to eight rows of 16-bit activations over a large weight matrix (batched decode at small batch, vocabulary-sized
-// projections): the weight stream of the one-row kernels with the arithmetic on the matrix cores.  One workgroup of
-// 8 waves per compute unit stays for the whole launch and owns a run of consecutive columns, the same count for every
-// workgroup.  A column group is 16 weight rows; KS waves share its K, each
-// taking every KS-th chunk of 512 bytes of every row: 8 loads of 2 rows x 512 contiguous bytes, into registers, two
-// chunks ahead.  A chunk goes through the wave's own 8 KiB of LDS (16-byte pieces swizzled by the row, so that
-// neither side has a bank conflict) to come back in the matrix core's operand shape (lane (c, g): row c, 16 bytes of
-// k), is widened exactly to the activations' type and multiplied by the activations' fragments.  Those come out of
-// LDS too: all rows of A where they fit (8 rows x K <= 4096 values, staged once per workgroup, asked for before any
-// weights), otherwise the wave's own 8 rows x 512 values, loaded with the weight chunk they meet.  The KS partial
-// tiles of a group meet in LDS, added in wave order.
+// Three to eight rows of 16-bit activations, rows of up to 4096 values, many columns (batched decode at small batch
+// against a vocabulary-sized projection of a small model: K = 2048 or 3072, N = 128256): the weight stream of the
+// one-row kernels with the arithmetic on the matrix cores.  One workgroup of 8 waves per compute unit stays for the
+// whole launch and owns a run of consecutive columns, the same count for every workgroup.  A column group is 16
+// weight rows; KS waves share its K, each taking every KS-th chunk of 512 bytes of every row: 8 loads of 2 rows x 512
+// contiguous bytes, into registers, two chunks ahead.  A chunk goes through the wave's own 8 KiB of LDS (16-byte
+// pieces swizzled by the row, so that neither side has a bank conflict) to come back in the matrix core's operand
+// shape (lane (c, g): row c, 16 bytes of k), is widened exactly to the activations' type and multiplied by the
+// activations' fragments.  Those come out of LDS too: all rows of A (8 rows x K <= 4096 values), staged once per
+// workgroup and asked for before any weights.  The KS partial tiles of a group meet in LDS, added in wave order.
+// (The slice kernels above give a workgroup's waves K / 256 chunks to share: with short rows that is one chunk per
+// wave and nothing to overlap.  With longer rows they win: K = 4096, N = 128256: 89.9 us against 88.4 here, K = 8192:
+// 172 against 180 with the activations loaded per chunk, a form this kernel had and lost.)
 // What was measured (8 x 4096 x 14336, timestamps inside the kernel): a compute unit accepts about 64 KiB of loads
 // before the issue of further ones blocks, and its older waves issue first.  So the second chunk in flight buys
 // little at the start and much in the steady state (the stream runs at 6.2 TB/s; a chunk costs a pair of waves
@@ -752,8 +754,6 @@ bool launch_staged(const Q8Params& p, int mt, int nt, int waves, uint32_t slices
 // barrier of issue per chunk, which keeps the waves level, costs more than that: 17.6 against 16.6 us.)  The loop
 // over a chunk's eight 64-value steps is rolled (a launch starts with a cold instruction cache).
 constexpr uint32_t kRowsChunk = 512, kRowsRegion = 16 * kRowsChunk, kRowsWaves = 8;
-// a wave's own activations of one chunk (rows longer than 4096): 8 rows x 512 values at the pitch below
-constexpr uint32_t kRowsOwnPitch = 2 * kRowsChunk + 64, kRowsOwn = 8 * kRowsOwnPitch;
 constexpr int kRawBuffer = 0x00020000;  // descriptor word 3: raw (unstructured) buffer, 32-bit data format
 constexpr int kLoadStream = 2;          // the nt bit: read once
 
@@ -764,7 +764,7 @@ constexpr int kLoadStream = 2;          // the nt bit: read once
 __host__ __device__ inline uint32_t rows_a_pitch(uint32_t k) { return 2 * ((k + 511) / 512 * 512) + 64; }
 __device__ __forceinline__ uint32_t rows_a_slot(uint32_t piece) { return (piece / 8) * 128 + (piece & 1u) * 64 + ((piece & 7u) >> 1) * 16; }
 
-template <class T, int KS, bool A_LDS>
+template <class T, int KS>
 __global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t cols_per_wg) {
   constexpr uint64_t item = 2;
   constexpr uint32_t TEAMS = kRowsWaves / KS;
@@ -772,10 +772,9 @@ __global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t cols_per_w
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t c = lane & 15, g = lane >> 4, team = wave / KS, ks = wave % KS;
   const uint32_t chunks = (p.k + kRowsChunk - 1) / kRowsChunk, per_wave = (chunks + KS - 1) / KS;
-  const uint32_t a_pitch = A_LDS ? rows_a_pitch(p.k) : kRowsOwnPitch, a_bytes = A_LDS ? 8 * a_pitch : 0;
-  uint8_t* const region = rows_lds + a_bytes + wave * (kRowsRegion + (A_LDS ? 0 : kRowsOwn));
-  uint8_t* const own = region + kRowsRegion;  // (!A_LDS)
-  V4F* const parts = reinterpret_cast<V4F*>(rows_lds + a_bytes + kRowsWaves * (kRowsRegion + (A_LDS ? 0 : kRowsOwn)));  // [2][8 waves][64 lanes]
+  const uint32_t a_pitch = rows_a_pitch(p.k), a_bytes = 8 * a_pitch;
+  uint8_t* const region = rows_lds + a_bytes + wave * kRowsRegion;
+  V4F* const parts = reinterpret_cast<V4F*>(rows_lds + a_bytes + kRowsWaves * kRowsRegion);  // [2][8 waves][64 lanes]
   uint16_t* const scales_lds = reinterpret_cast<uint16_t*>(parts + 2 * kRowsWaves * 64);  // [8 waves][16]
 
   // A workgroup owns cols_per_wg consecutive columns (a multiple of 8; the same count for every workgroup, so that
@@ -786,11 +785,14 @@ __global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t cols_per_w
   const uint32_t col_begin = blockIdx.x * cols_per_wg, col_end = min(col_begin + cols_per_wg, p.n);
   const uint32_t rounds = ((cols_per_wg + 15) / 16 + TEAMS - 1) / TEAMS;
   auto first_col = [&](uint32_t round) { return col_begin + (round * TEAMS + team) * 16; };  // (at or past col_end: no group)
+  // (workgroups walk K from different starting chunks and wrap around: with rows a power of two apart, all of them
+  // reading the same offsets of their rows at the same time keep to a few memory channels)
+  const uint32_t rot = (blockIdx.x * 3u) % chunks;
   const uint32_t items = rounds * per_wave;  // (group, chunk) pairs of this wave, some of them past the end
   // Two chunks are in flight per wave (registers), requested as soon as the registers are free.
-  U4 w[2][8], av[2][A_LDS ? 1 : 8];
+  U4 w[2][8];
   uint16_t scl[2];
-  // Weights, scales and (long rows) activations are read through buffer descriptors: a load whose offset lies past
+  // Weights, scales and activations are read through buffer descriptors: a load whose offset lies past
   // the buffer returns zeros and touches no memory, so rows past n, pieces past k and requests past the wave's last
   // item cost nothing, and every request is the same number of loads on every path (each wait below is then for its
   // own chunk only: a path without its loads would make every later wait a wait for everything).
@@ -802,26 +804,19 @@ __global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t cols_per_w
     constexpr int S = decltype(set)::value;
     // (the fences keep one request's loads together and in program order, which is what the waits count on)
     __builtin_amdgcn_sched_barrier(0);
-    const uint32_t n0 = first_col(j / per_wave), chunk = (j % per_wave) * KS + ks;
-    const uint32_t dead = j < items && n0 < col_end ? 0u : ~0u;  // (all ones: past every buffer)
+    const uint32_t n0 = first_col(j / per_wave), turn = (j % per_wave) * KS + ks, chunk = (turn + rot) % chunks;
+    const uint32_t dead = j < items && n0 < col_end && turn < chunks ? 0u : ~0u;  // (all ones: past every buffer)
     const uint32_t at = chunk * kRowsChunk + (lane & 31u) * 16;
     const uint32_t row0 = n0 + (lane >> 5), gone = dead | (at < p.k ? 0u : ~0u);
 #pragma unroll
     for (int i = 0; i < 8; ++i)  // rows 2 i + lane / 32
       w[S][i] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, ((row0 + 2 * i) * p.k + at) | gone | (row0 + 2 * i < col_end ? 0u : ~0u), 0, kLoadStream);
-    if constexpr (!A_LDS) {  // row i's piece `lane` of the chunk
-      const uint32_t ka = chunk * kRowsChunk + lane * 8;
-      const uint32_t a_first = (ka * uint32_t(item)) | dead | (ka < p.k ? 0u : ~0u);
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        av[S][i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (a_first + i * uint32_t(p.a_sm) * uint32_t(item)) | (uint32_t(i) < p.m ? 0u : ~0u), 0, 0);
-    }
     // the group's 16 scales come with every chunk and go through LDS with it (loaded in the epilogue they would be
     // waited for behind two chunks in flight)
     scl[S] = __builtin_amdgcn_raw_buffer_load_b16(s_rsrc, ((n0 + c) * uint32_t(item)) | dead | (n0 + c < col_end ? 0u : ~0u), 0, 0);
     __builtin_amdgcn_sched_barrier(0);
   };
-  if constexpr (A_LDS) {
+  {
     // all rows, once per workgroup: row i's piece `tid` (a row has at most 512 pieces), through the same kind of
     // descriptor; asked for before any weights.  The two barriers before the one that publishes A are barriers of
     // ISSUE, not of data: a compute unit accepts ~64 KiB of loads and lets the oldest wave's instructions go first, so
@@ -845,31 +840,23 @@ __global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t cols_per_w
     }
     __syncthreads();
     request(std::integral_constant<int, 1>{}, 1);
-  } else {
-    request(std::integral_constant<int, 0>{}, 0);
-    request(std::integral_constant<int, 1>{}, 1);
   }
-  const uint8_t* const a_frag = (A_LDS ? rows_lds : own) + (c & 7u) * a_pitch + 16 * g;
+  const uint8_t* const a_frag = rows_lds + (c & 7u) * a_pitch + 16 * g;
 
   V4F acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = acc0;
   auto work = [&](auto set, uint32_t j) {
     constexpr int S = decltype(set)::value;
-    const uint32_t round = j / per_wave, chunk = (j % per_wave) * KS + ks, n0 = first_col(round);
+    const uint32_t round = j / per_wave, turn = (j % per_wave) * KS + ks, chunk = (turn + rot) % chunks, n0 = first_col(round);
     // the chunk's 16 rows into the wave's region: piece q of row r at slot q ^ r
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const uint32_t r = 2 * i + (lane >> 5);
       *reinterpret_cast<U4*>(region + r * kRowsChunk + (((lane & 31u) ^ r) * 16)) = w[S][i];
     }
-    if constexpr (!A_LDS) {
-      const uint32_t at = rows_a_slot(lane);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) *reinterpret_cast<U4*>(own + i * kRowsOwnPitch + at) = av[S][i];
-    }
     scales_lds[wave * 16 + c] = scl[S];  // (four lanes write each, the same value)
     request(set, j + 2);
-    if (j < items && chunk < chunks && n0 < col_end) {
-      const uint32_t k0 = A_LDS ? chunk * kRowsChunk : 0;
+    if (j < items && turn < chunks && n0 < col_end) {
+      const uint32_t k0 = chunk * kRowsChunk;
       // a step's operand reads are issued a step ahead (two register sets, used in turn)
       struct Step {
         U4 wv, a0, a1;
@@ -945,24 +932,21 @@ __global__ __launch_bounds__(512) void qmm8_rows(Q8Params p, uint32_t cols_per_w
   }
 }
 
-// The kernel above where it applies: 3 to 8 rows, k a multiple of 16 (checked by the caller), whole 16-byte pieces.
+// The kernel above where it applies: 3 to 8 rows of at most 4096 values, k a multiple of 16 (checked by the caller).
 // False: not this kernel's shape.
 template <class T>
 bool launch_rows_kernel(const Q8Params& p, bool whatever_the_size, const Machine& mc, hipStream_t stream) {
-  if (p.m < 3 || p.m > 8 || p.k < 512 || p.n < 16) return false;
-  // Measured against the slice kernels below (8 rows, microseconds, this kernel first).  It streams faster than they
-  // do once under way (5.9 TB/s over a whole launch at 4096 x 128256) but takes ~6.5 us to get there and to drain, and
-  // its waves own whole groups.  It pays where a workgroup has 8 groups or more and the activations stay in LDS,
-  //   K x N 1024 x 131072: 28.0 / 31.2, 2048 x 32768: 15.9 / 17.2, 2048 x 65536: 26.4 / 31.8, 3072 x 32768: 21.4 / 22.0,
-  //   4096 x 32000: 29.3 / 29.7, 4096 x 49152: 42.8 / 43.1, 4096 x 65536: 50.5 / 55.1, 4096 x 128256: 89.7 / 99.5
-  //   (and not 4096 x 14336: 16.4 / 14.3, 4096 x 20480: 22.7 / 22.1, 4096 x 24576: 25.8 / 24.9),
-  // and with longer rows (a wave then asks for its own activations with every chunk, as many bytes again, from L2)
-  // from 16 groups per workgroup on,
-  //   8192 x 128256: 179.5 / 208.7 (and not 14336 x 4096: 18.6 / 15.1, 8192 x 28672: 51.2 / 44.3, 12288 x 32768: 82.8 / 73.6,
-  //   5120 x 51200: 63.3 / 50.8, 6144 x 65536: 76.9 / 69.2; about level: 16384 x 16384: 53.3 / 54.9, 8192 x 16384: 30.9 / 33.3).
+  // (rows of A as a whole in LDS: 8 x 4096 values at most; 16-byte pieces)
+  if (p.m < 3 || p.m > 8 || p.k < 512 || p.k > 4096 || p.n < 16) return false;
+  // Measured against the slice kernels below (8 rows, microseconds, this kernel first).  It pays with rows shorter
+  // than 4096 values, of which a slice kernel's waves get one chunk each, where a workgroup has 8 groups or more:
+  //   K x N 1024 x 131072: 28.4 / 31.3, 2048 x 32768: 16.2 / 17.3, 2048 x 50304: 24.5 / 26.9, 2048 x 65536: 26.5 / 31.8,
+  //   2048 x 128256: 47.6 / 58.3, 3072 x 32768: 21.0 / 22.2, 3072 x 65536: 37.2 / 40.6;
+  // not with K = 4096 (4096 x 14336: 15.3 / 14.2, 4096 x 32000: 25.7 / 26.1, 4096 x 49152: 38.6 / 37.2, 4096 x 65536: 48.4 /
+  // 48.4, 4096 x 128256: 88.4 / 89.9, at 4 rows 86.8 / 86.2) and not with few columns per compute unit.
   {
     const uint32_t cus0 = uint32_t(mc.compute_units), units = (p.n + 15) / 16 < cus0 ? (p.n + 15) / 16 : cus0;
-    const bool pays = (p.n + units - 1) / units >= (p.k <= 4096 ? 121u : 241u);
+    const bool pays = p.k < 4096 && (p.n + units - 1) / units >= 121;
     if (!whatever_the_size && !pays) return false;
   }
   // (32-bit byte offsets into B and A, each within a buffer descriptor of fewer than 2^31 bytes)
@@ -975,11 +959,10 @@ bool launch_rows_kernel(const Q8Params& p, bool whatever_the_size, const Machine
   grid = (p.n + cols_per_wg - 1) / cols_per_wg;
   const uint32_t local = (cols_per_wg + 15) / 16;
   const int ks = local >= 5 ? 1 : local >= 3 ? 2 : local == 2 ? 4 : 8;
-  const bool a_lds = p.k <= 4096;  // (8 rows x 4096 values: 64 KiB, and 8 pieces of 16 bytes per thread to stage them)
-  const uint32_t lds = (a_lds ? 8 * rows_a_pitch(p.k) : kRowsWaves * kRowsOwn) + kRowsWaves * kRowsRegion + 2 * kRowsWaves * 64 * 16 + kRowsWaves * 32;
-#define VKT_ROWS_CASE(KS_, AL_)                                                                                              \
-  if (ks == KS_ && a_lds == AL_) {                                                                                           \
-    auto kernel = qmm8_rows<T, KS_, AL_>;                                                                                    \
+  const uint32_t lds = 8 * rows_a_pitch(p.k) + kRowsWaves * kRowsRegion + 2 * kRowsWaves * 64 * 16 + kRowsWaves * 32;
+#define VKT_ROWS_CASE(KS_)                                                                                                   \
+  if (ks == KS_) {                                                                                                           \
+    auto kernel = qmm8_rows<T, KS_>;                                                                                         \
     static bool configured = false; /* guarded by the runtime's stream mutex */                                              \
     if (!configured) {                                                                                                       \
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024) != hipSuccess) { \
@@ -988,11 +971,10 @@ bool launch_rows_kernel(const Q8Params& p, bool whatever_the_size, const Machine
       }                                                                                                                      \
       configured = true;                                                                                                     \
     }                                                                                                                        \
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(512), lds, stream, p, cols_per_wg);                                               \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(512), lds, stream, p, cols_per_wg);                                          \
     return true;                                                                                                             \
   }
-  VKT_ROWS_CASE(1, true) VKT_ROWS_CASE(1, false) VKT_ROWS_CASE(2, true) VKT_ROWS_CASE(2, false)
-  VKT_ROWS_CASE(4, true) VKT_ROWS_CASE(4, false) VKT_ROWS_CASE(8, true) VKT_ROWS_CASE(8, false)
+  VKT_ROWS_CASE(1) VKT_ROWS_CASE(2) VKT_ROWS_CASE(4) VKT_ROWS_CASE(8)
 #undef VKT_ROWS_CASE
   return false;
 }
@@ -1514,7 +1496,7 @@ int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipSt
     // the vector units (measured at K = 4096, N = 14336: 10.5, 16.4, 23.0, 23.4 us for 1 to 4 rows; the matrix
     // cores take 16 us for up to 8).  variant bit 17 forces the GEMV kernels (tests, tuning).
     if (p0.m > 2 && !((variant >> 17) & 1)) {
-      // 3 to 8 rows over large weights: the wave-per-column-group kernel where it pays (variant bit 23 keeps the kernels below)
+      // 3 to 8 short rows against many columns: the wave-per-column-group kernel where it pays (variant bit 23 keeps the kernels below)
       // (bits 8-15 with bits 0-7 clear ask for it whatever the size: tests, tuning)
       const bool asked = !(variant & 0xff) && ((variant >> 8) & 0xff);
       if ((asked || !(variant & 0xffff)) && !((variant >> 18) & 3) && !((variant >> 23) & 1) && launch_rows_kernel<T>(p0, asked, mc, stream)) return 0;
