@@ -1379,11 +1379,16 @@ int launch_mfma(const Q8Params& p, uint32_t variant, const Machine& mc, hipStrea
   } else {
     const uint32_t groups = (p.n + 16 * nt - 1) / (16 * nt), chunks = (p.k + 63) / 64;
     while (waves > 4 && chunks < uint32_t(waves)) waves /= 2;
-    const uint32_t want = (uint32_t(mc.compute_units) + groups / 2) / groups;  // about one workgroup per compute unit
-    const uint32_t most = chunks / (2u * waves) ? chunks / (2u * waves) : 1;   // >= 2 chunks per wave
-    slices = want < most ? want : most;
-    if (slices < 1) slices = 1;
-    if (slices > 16) slices = 16;
+    // The count of slices that leaves the busiest compute unit the least work: (workgroups on it) x (a slice's share
+    // of K), plus a little per slice for its partial tile; at least 2 chunks per wave.  (Rounding groups x slices to
+    // the nearest count of compute units, the rule before, gave N = 6400 three slices, 300 workgroups on 256 units;
+    // five make 500, two for nearly every unit: 38.9 -> 29.5 us at 16 rows, K = 14336.)
+    const uint32_t cus = uint32_t(mc.compute_units), most = chunks / (2u * waves) ? chunks / (2u * waves) : 1;
+    float best = 1e30f;
+    for (uint32_t s = 1; s <= most && s <= 16; ++s) {
+      const float cost = float((groups * s + cus - 1) / cus) / float(s) + 0.005f * float(s);
+      if (cost < best) best = cost, slices = s;
+    }
   }
   // Up to 8 rows the kernel that stages the weights through LDS wins (measured at K = 4096 / N = 14336 and the
   // reverse: 15.8 against 17.1 us, 15.1-16.4 against 17.3-18.4); from 16 rows on the activations' own traffic
