@@ -163,7 +163,7 @@ def wl_q8(abi, m, k, n, dtype, steps, warmup, seed=1020, prefill=False, variant=
                 **timed(abi, fns, steps, warmup))
 
 
-def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030, prefill=False):
+def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030, prefill=False, phase=2):
     """_dyn_quant_matmul_4bit on the compact side-car: up to 4 rows the streaming layout with
     row quantisation fused into the launch, above that the matrix-core layout (two launches)."""
     import torch
@@ -195,7 +195,7 @@ def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030, prefill=False):
     for c in copies:
         p = abi.Q4CParams(inp=dx.address, q=dq.address, rows=dr.address, compact=c.address, out=out.address, m=m, n=n,
                           k=k, bs=bs, has_bias=1)
-        fns.append(Launch(abi, "qmm4c_f32", [2, 1, layout], p))  # row quantisation + product
+        fns.append(Launch(abi, "qmm4c_f32", [phase, 1, layout], p))  # row quantisation + product
     work = n * k // 2 + 4 * n * (k // bs) + 4 * n + 4 * m * k + 4 * m * n
     if prefill:  # many rows: the matrix cores' int8 rate is the published bound
         return dict(kind="mfma", peak=INT8_PEAK_TOPS, metric="int4-weight prefill TOP/s (% of int8 MFMA peak)", work=2 * m * n * k,

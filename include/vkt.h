@@ -165,7 +165,8 @@ typedef struct Q4PackParams {
  * be quantised from registers (k a multiple of 8, at most 16384), otherwise as PHASE 0
  * then 1.  Results are bit-identical to qmm4.  With LAYOUT 1, bits 4-7 of PHASE override the choice
  * between the two product kernels, which give the same bits (tests, tuning): 16 keeps the kernel whose four waves
- * split K, 32 forces the one whose waves each walk all of K (| 64, 128, 192: 1, 2, 4 tiles of 16 x 16 per wave). */
+ * split K, 32 forces the one whose waves each walk all of K (| 64, 128, 192: 1, 2, 4 tiles of 16 x 16 per wave).
+ * With LAYOUT 0, PHASE 2 with 1, 2 or 3 in bits 8-9 fixes the column tiles per workgroup (same bits). */
 typedef struct Q4CParams {
   uint64_t inp, q, rows, compact, out;
   uint32_t m, n, k, bs, has_bias, pad;

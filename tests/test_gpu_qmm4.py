@@ -91,6 +91,23 @@ def test_q4_config3(m):
     assert np.array_equal(got_b.view(np.uint32), cpu_b.view(np.uint32))
 
 
+@pytest.mark.parametrize("m,k,n,bs,bias", [(2, 4096, 4128, 32, True), (3, 2048, 8200, 64, False), (2, 1024, 40, 128, True),
+                                           (3, 4096, 16, 4096, False), (2, 512, 12300, 256, True)])
+def test_q4_several_tiles_per_workgroup(m, k, n, bs, bias):
+    """Two and three rows on the streaming kernel with two and three column tiles per workgroup (the launcher's choice
+    when a compute unit has that many tiles; forced here through the phase word's bits 8-9), tile counts that leave
+    the last workgroup short of tiles."""
+    import _dev
+    w, sc, bvec = int4_weights(n, k, bs, bias=bias)
+    x = int4_rows(m, k, torch.float32)
+    packed = torch._dyn_quant_pack_4bit_weight(w, sc, bvec, bs, k, n).numpy()
+    want = oracle.q4_matmul(bits(x), oracle.F32, packed, bs, k, n)
+    cw = _dev.CompactWeights(packed, bs, k, n)
+    for teams in (0, 1, 2, 3):
+        got = _dev.q4_compact(bits(x), oracle.F32, cw, flags=teams << 8)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), teams
+
+
 def test_q4_golden_fixtures():
     import _dev
     g = np.load(os.path.join(GOLDEN, "q4.npz"))

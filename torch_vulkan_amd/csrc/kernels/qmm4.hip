@@ -98,14 +98,17 @@ __device__ __forceinline__ void row_range(uint64_t row, uint32_t k, float* mn_ou
   *mx_out = fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3]));
 }
 
-// Workgroup-wide min / max of per-thread values (256 threads).
+// Workgroup-wide min / max of per-thread values (NW waves).
+template <int NW = 4>
 __device__ __forceinline__ void block_range(float* mn, float* mx) {
-  __shared__ float bmin[4], bmax[4];
+  __shared__ float bmin[NW], bmax[NW];
   const float a = wave_min(*mn), b = wave_max(*mx);
   if ((threadIdx.x & 63) == 0) bmin[threadIdx.x >> 6] = a, bmax[threadIdx.x >> 6] = b;
   __syncthreads();
-  *mn = fminf(fminf(bmin[0], bmin[1]), fminf(bmin[2], bmin[3]));
-  *mx = fmaxf(fmaxf(bmax[0], bmax[1]), fmaxf(bmax[2], bmax[3]));
+  float lo = bmin[0], hi = bmax[0];
+#pragma unroll
+  for (int w = 1; w < NW; ++w) lo = fminf(lo, bmin[w]), hi = fmaxf(hi, bmax[w]);
+  *mn = lo, *mx = hi;
 }
 
 // 8 consecutive elements at a 16-byte aligned address (float32: 32-byte aligned pairs).
@@ -290,8 +293,10 @@ __device__ __forceinline__ void nibble_planes(const int (&q)[8], uint32_t* hi, u
 __host__ __device__ inline uint32_t q_row_bytes(uint32_t kpad) { return kpad + kpad / 256 * 16; }
 constexpr uint32_t kTermPitch = 132;  // floats per (row, column) of a round's block terms: 128 + 4, so that the 16
                                       // columns' 16-byte reads fall on different banks
-__host__ __device__ inline uint32_t q_lds_bytes(uint32_t rows, uint32_t kpad) {
-  return rows * q_row_bytes(kpad) + rows * kTileCols * 4 + 64 + rows * kTileCols * kTermPitch * 4;
+// (per team of 4 waves: the carried sums [rows][16], 64 bytes, and a round's block terms)
+__host__ __device__ inline uint32_t q_team_bytes(uint32_t rows) { return rows * kTileCols * 4 + 64 + rows * kTileCols * kTermPitch * 4; }
+__host__ __device__ inline uint32_t q_lds_bytes(uint32_t rows, uint32_t kpad, uint32_t teams = 1) {
+  return rows * q_row_bytes(kpad) + teams * q_team_bytes(rows);
 }
 __device__ __forceinline__ uint32_t q_group_offset(uint32_t g) {  // byte offset of 8 values' hi word
   const uint32_t unit = g >> 2, d = g & 3;
@@ -333,19 +338,24 @@ __global__ __launch_bounds__(256) void qmm4c_rowquant(Q4CParams p, uint32_t grou
 // folded in: no second launch, no scratch round trip); otherwise it stages the planes that
 // phase 0 left in global memory.  The inner loop reads activations from LDS and weights
 // straight from HBM.
-template <class T, int MR, int UPB, int XG>
-__global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L, uint32_t m0, uint32_t groupwise) {
+template <class T, int MR, int UPB, int XG, int TEAMS>
+__global__ __launch_bounds__(256 * TEAMS) void qmm4c_stream(Q4CParams p, CompactLayout L, uint32_t m0, uint32_t groupwise) {
   constexpr bool FUSED = XG != 0;  // XG: groups of 8 activations a thread quantises (k <= 2048 * XG)
   constexpr uint64_t item = sizeof(typename T::storage);
   constexpr int BPL = UPB ? kUnitsPerLane / UPB : 1;  // blocks per lane per round
   constexpr int UN = UPB ? UPB : kUnitsPerLane;       // units of a block within a lane
   extern __shared__ __attribute__((aligned(16))) uint8_t q_lds[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr int XGT = (XG + TEAMS - 1) / TEAMS;  // groups of 8 activations per thread of the whole workgroup
+  // A team of 4 waves per column tile; the teams of a workgroup share the quantised activation rows (read and
+  // quantised once per workgroup).  tid, wave: within the team; wtid: within the workgroup.
+  const int wtid = threadIdx.x, team = wtid >> 8, tid = wtid & 255, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, grp = lane >> 4, part = wave * 4 + grp;
-  const uint32_t tile = blockIdx.x, n = tile * kTileCols + col;
+  // (a team past the last tile works on the last tile again and stores nothing: it keeps to the barriers)
+  const bool live = blockIdx.x * TEAMS + team < L.tiles;
+  const uint32_t tile = live ? blockIdx.x * TEAMS + team : L.tiles - 1, n = tile * kTileCols + col;
   const uint32_t nblocks = UPB ? p.k / p.bs : 1;
   const uint32_t qs = q_row_bytes(L.kpad);
-  float* const carry = reinterpret_cast<float*>(q_lds + MR * qs);      // [MR][16]
+  float* const carry = reinterpret_cast<float*>(q_lds + MR * qs + team * q_team_bytes(MR));  // [MR][16]
   int* const itotal = reinterpret_cast<int*>(carry);                    // (channelwise: integer totals)
   float* const terms = carry + MR * kTileCols + 16;                     // [MR][16][kTermPitch]: a round's block terms
 
@@ -392,27 +402,27 @@ __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L
       // No branch goes around a load (groups past the row read its first group again): the compiler then knows how
       // many younger loads there are and waits for the row alone, not for the weights requested after it.
       const uint32_t groups = p.k / 8;
-      float x[XG ? XG : 1][8];
+      float x[XGT ? XGT : 1][8];
       float mn = 3.40282347e38f, mx = -3.40282347e38f;
 #pragma unroll
-      for (int i = 0; i < XG; ++i) {
-        const uint32_t g = tid + 256 * i;
+      for (int i = 0; i < XGT; ++i) {
+        const uint32_t g = wtid + 256 * TEAMS * i;
         load8_f32<T>(row + uint64_t(g < groups ? g : 0) * 8 * item, x[i]);
       }
       if (r == 0) request_round(0);
 #pragma unroll
-      for (int i = 0; i < XG; ++i) {
-        const bool inside = uint32_t(tid + 256 * i) < groups;
+      for (int i = 0; i < XGT; ++i) {
+        const bool inside = uint32_t(wtid + 256 * TEAMS * i) < groups;
 #pragma unroll
         for (int e = 0; e < 8; ++e) mn = fminf(mn, inside ? x[i][e] : mn), mx = fmaxf(mx, inside ? x[i][e] : mx);
       }
-      block_range(&mn, &mx);
+      block_range<4 * TEAMS>(&mn, &mx);
       const RowQuant rq = row_quant(mn, mx, groupwise != 0);
       nzp8[r] = 8 - rq.izp;
       recip[r] = rq.recip;
 #pragma unroll
-      for (int i = 0; i < XG; ++i) {
-        const uint32_t g = tid + 256 * i;
+      for (int i = 0; i < XGT; ++i) {
+        const uint32_t g = wtid + 256 * TEAMS * i;
         if (g < L.kpad / 8) {
           uint32_t hi = 0, lo = 0x88888888u;  // beyond k: value 0 = planes (0, 0 - 8)
           if (g < groups) {
@@ -431,7 +441,7 @@ __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L
       nzp8[r] = 8 + ldg<int32_t>(p.rows + 8ull * m + 4);
       recip[r] = bits_f32(ldg<uint32_t>(p.rows + 8ull * m));
       const uint64_t src = p.q + uint64_t(m) * L.kpad;
-      for (uint32_t c = tid; c < L.kpad / 16; c += 256)
+      for (uint32_t c = wtid; c < L.kpad / 16; c += 256 * TEAMS)
         *reinterpret_cast<U4*>(q_lds + r * qs + c * 16 + c / 16 * 16) = ldg<U4>(src + c * 16ull);
     }
   }
@@ -560,13 +570,13 @@ __global__ __launch_bounds__(256) void qmm4c_stream(Q4CParams p, CompactLayout L
     }
   }
   if constexpr (UPB != 0) {
-    if (wave == 0 && grp < MR && n < p.n && m0 + grp < p.m) {
+    if (live && wave == 0 && grp < MR && n < p.n && m0 + grp < p.m) {
       float rc = recip[0];
 #pragma unroll
       for (int r = 1; r < MR; ++r) rc = grp == r ? recip[r] : rc;
       finish_store<T>(p.out + (uint64_t(m0 + grp) * p.n + n) * item, acc[0], rc, p.has_bias != 0, bias);
     }
-  } else if (part == 15 && n < p.n) {
+  } else if (live && part == 15 && n < p.n) {
 #pragma unroll
     for (int r = 0; r < MR; ++r)
       if (m0 + r < p.m) finish_store<T>(p.out + (uint64_t(m0 + r) * p.n + n) * item, acc[r], recip[r], p.has_bias != 0, bias);
@@ -1139,11 +1149,11 @@ bool check_q4_shape(uint32_t m, uint32_t n, uint32_t k, uint32_t bs, std::string
   return true;
 }
 
-template <class T, int MR, int UPB, int XG>
+template <class T, int MR, int UPB, int XG, int TEAMS>
 int launch_stream_one(const Q4CParams& p, const CompactLayout& L, uint32_t m0, uint32_t groupwise, hipStream_t stream,
                       std::string* err) {
-  auto kernel = qmm4c_stream<T, MR, UPB, XG>;
-  const uint32_t lds = q_lds_bytes(MR, L.kpad);
+  auto kernel = qmm4c_stream<T, MR, UPB, XG, TEAMS>;
+  const uint32_t lds = q_lds_bytes(MR, L.kpad, TEAMS);
   static uint32_t reserved = 48 * 1024;  // guarded by the runtime's stream mutex
   if (lds > reserved) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds) !=
@@ -1154,28 +1164,52 @@ int launch_stream_one(const Q4CParams& p, const CompactLayout& L, uint32_t m0, u
     }
     reserved = lds;
   }
-  hipLaunchKernelGGL(kernel, dim3(L.tiles), dim3(256), lds, stream, p, L, m0, groupwise);
+  hipLaunchKernelGGL(kernel, dim3((L.tiles + TEAMS - 1) / TEAMS), dim3(256 * TEAMS), lds, stream, p, L, m0, groupwise);
   return 0;
 }
 
-template <class T, int MR, int XG>
+template <class T, int MR, int XG, int TEAMS>
 int launch_stream_upb(const Q4CParams& p, const CompactLayout& L, uint32_t m0, uint32_t groupwise, hipStream_t stream,
                       std::string* err) {
   switch (L.upb) {
-    case 0: return launch_stream_one<T, MR, 0, XG>(p, L, m0, groupwise, stream, err);
-    case 1: return launch_stream_one<T, MR, 1, XG>(p, L, m0, groupwise, stream, err);
-    case 2: return launch_stream_one<T, MR, 2, XG>(p, L, m0, groupwise, stream, err);
-    case 4: return launch_stream_one<T, MR, 4, XG>(p, L, m0, groupwise, stream, err);
-    case 8: return launch_stream_one<T, MR, 8, XG>(p, L, m0, groupwise, stream, err);
+    case 0: return launch_stream_one<T, MR, 0, XG, TEAMS>(p, L, m0, groupwise, stream, err);
+    case 1: return launch_stream_one<T, MR, 1, XG, TEAMS>(p, L, m0, groupwise, stream, err);
+    case 2: return launch_stream_one<T, MR, 2, XG, TEAMS>(p, L, m0, groupwise, stream, err);
+    case 4: return launch_stream_one<T, MR, 4, XG, TEAMS>(p, L, m0, groupwise, stream, err);
+    case 8: return launch_stream_one<T, MR, 8, XG, TEAMS>(p, L, m0, groupwise, stream, err);
   }
   *err = "qmm4c: bad layout";
   return -1;
 }
 
+// Column tiles per workgroup.  Every workgroup reads (and, fused, quantises) the activation rows for itself.  With
+// two rows and more, and up to three tiles per compute unit, one workgroup per unit with that many tiles is ~10 %
+// faster than as many workgroups (K = 4096, 2 rows, 256 units: 8192 columns 8.8 against 9.8 us, 11008 columns 11.0
+// against 12.3).  With one row it is level to slower (the launch is a chain of waits, not of bytes, and three
+// workgroups a unit that start at different times overlap their waits better than twelve waves in step), and so it
+// is with more workgroups than units (16384 columns as 512 workgroups of two tiles: 16.1 against 14.5 us).
+inline int stream_teams(const CompactLayout& L, uint32_t rows, int cus) {
+  const uint32_t per_unit = (L.tiles + cus - 1) / cus;
+  return rows >= 2 && per_unit <= 3 && q_lds_bytes(rows, L.kpad, per_unit) <= 144 * 1024 ? int(per_unit) : 1;
+}
+
+template <class T, int MR, int XG>
+int launch_stream_teams(const Q4CParams& p, const CompactLayout& L, uint32_t m0, uint32_t groupwise, int teams,
+                        hipStream_t stream, std::string* err) {
+  // (several tiles per workgroup only in the fused form for rows of up to 4096 values, the one decode runs on, and
+  // only with two rows and more)
+  if constexpr (XG == 2 && MR >= 2) {
+    if (teams == 3) return launch_stream_upb<T, MR, XG, 3>(p, L, m0, groupwise, stream, err);
+    if (teams == 2) return launch_stream_upb<T, MR, XG, 2>(p, L, m0, groupwise, stream, err);
+  }
+  return launch_stream_upb<T, MR, XG, 1>(p, L, m0, groupwise, stream, err);
+}
+
 // Rows in groups of at most 4 (fewer when the activations of 4 rows would not fit in LDS).
+// forced_teams: 0 = by the rule above.
 template <class T, int XG>
-int launch_stream_rows(const Q4CParams& p, const CompactLayout& L, uint32_t groupwise, hipStream_t stream,
-                       std::string* err) {
+int launch_stream_rows(const Q4CParams& p, const CompactLayout& L, uint32_t groupwise, uint32_t forced_teams, int cus,
+                       hipStream_t stream, std::string* err) {
   uint32_t per = 4;
   while (per > 1 && q_lds_bytes(per, L.kpad) > 144 * 1024) per /= 2;
   if (q_lds_bytes(per, L.kpad) > 144 * 1024) {
@@ -1184,11 +1218,13 @@ int launch_stream_rows(const Q4CParams& p, const CompactLayout& L, uint32_t grou
   }
   for (uint32_t m0 = 0; m0 < p.m; m0 += per) {
     const uint32_t rows = p.m - m0 < per ? p.m - m0 : per;
+    int teams = XG == 2 ? stream_teams(L, rows, cus) : 1;
+    if (forced_teams != 0 && q_lds_bytes(rows, L.kpad, forced_teams) <= 144 * 1024) teams = int(forced_teams);
     int rc;
-    if (rows >= 4) rc = launch_stream_upb<T, 4, XG>(p, L, m0, groupwise, stream, err);
-    else if (rows == 3) rc = launch_stream_upb<T, 3, XG>(p, L, m0, groupwise, stream, err);
-    else if (rows == 2) rc = launch_stream_upb<T, 2, XG>(p, L, m0, groupwise, stream, err);
-    else rc = launch_stream_upb<T, 1, XG>(p, L, m0, groupwise, stream, err);
+    if (rows >= 4) rc = launch_stream_teams<T, 4, XG>(p, L, m0, groupwise, teams, stream, err);
+    else if (rows == 3) rc = launch_stream_teams<T, 3, XG>(p, L, m0, groupwise, teams, stream, err);
+    else if (rows == 2) rc = launch_stream_teams<T, 2, XG>(p, L, m0, groupwise, teams, stream, err);
+    else rc = launch_stream_teams<T, 1, XG>(p, L, m0, groupwise, teams, stream, err);
     if (rc != 0) return rc;
   }
   return 0;
@@ -1375,6 +1411,9 @@ int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwi
     *err = "qmm4c: GROUPWISE must be 1 exactly when bs != k";
     return -1;
   }
+  // (phase 2 with 1, 2 or 3 in bits 8-9: that many column tiles per workgroup instead of the launcher's choice; tests, tuning)
+  uint32_t forced_teams = 0;
+  if ((phase & 255u) == 2 && (phase >> 8) <= 3) forced_teams = phase >> 8, phase = 2;
   if (!p.inp || !p.out || (phase != 2 && (!p.q || !p.rows || (p.q & 15)))) {
     *err = "qmm4c: null or unaligned tensor address";
     return -1;
@@ -1393,8 +1432,8 @@ int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwi
       *err = "qmm4c: null or unaligned side-car address";
       return -1;
     }
-    const int rc = dtype == VKT_F32 ? launch_stream_rows<f32_t, 0>(p, L, groupwise, stream, err)
-                                    : launch_stream_rows<bf16_t, 0>(p, L, groupwise, stream, err);
+    const int rc = dtype == VKT_F32 ? launch_stream_rows<f32_t, 0>(p, L, groupwise, 0, mc.compute_units, stream, err)
+                                    : launch_stream_rows<bf16_t, 0>(p, L, groupwise, 0, mc.compute_units, stream, err);
     if (rc != 0) return rc;
   } else if (phase == 2) {
     // both phases in one launch per group of rows when the rows can be quantised from
@@ -1412,10 +1451,10 @@ int launch_qmm4c(const Q4CParams& p, int dtype, uint32_t phase, uint32_t groupwi
     }
     // (a thread quantises 2 groups of 8 activations where that covers the row, else up to kFusedGroups)
     const bool few = p.k <= 4096;
-    const int rc = dtype == VKT_F32 ? (few ? launch_stream_rows<f32_t, 2>(p, L, groupwise, stream, err)
-                                           : launch_stream_rows<f32_t, kFusedGroups>(p, L, groupwise, stream, err))
-                                    : (few ? launch_stream_rows<bf16_t, 2>(p, L, groupwise, stream, err)
-                                           : launch_stream_rows<bf16_t, kFusedGroups>(p, L, groupwise, stream, err));
+    const int rc = dtype == VKT_F32 ? (few ? launch_stream_rows<f32_t, 2>(p, L, groupwise, forced_teams, mc.compute_units, stream, err)
+                                           : launch_stream_rows<f32_t, kFusedGroups>(p, L, groupwise, 0, mc.compute_units, stream, err))
+                                    : (few ? launch_stream_rows<bf16_t, 2>(p, L, groupwise, forced_teams, mc.compute_units, stream, err)
+                                           : launch_stream_rows<bf16_t, kFusedGroups>(p, L, groupwise, 0, mc.compute_units, stream, err));
     if (rc != 0) return rc;
   } else {
     *err = "qmm4c: PHASE must be 0, 1 or 2";
