@@ -691,6 +691,14 @@ void launch_mfma_waves(const Q8Params& p, int waves, uint32_t slices, const Mach
   if (slices > 1) hipLaunchKernelGGL((qmm8_mfma_finish<T, MT, NT>), dim3(grid.x), dim3(64), 0, stream, p, slices, mc.workspace);
 }
 
+// Columns per workgroup of the staged kernel with one slice: at most 16 nt, fewer where that deals the columns out
+// over a whole number of workgroups per compute unit (a multiple of 4, at least 8).
+inline uint32_t staged_cols(uint32_t n, int nt, uint32_t cus) {
+  const uint32_t cols = 16 * nt, wgs = (n + cols - 1) / cols, even = (wgs + cus - 1) / cus * cus;
+  const uint32_t fewer = ((n + even - 1) / even + 3) / 4 * 4;
+  return fewer >= 8 && fewer < cols ? fewer : cols;
+}
+
 template <class T, int MT, int NT, int WAVES>
 bool launch_staged_one(const Q8Params& p, uint32_t slices, const Machine& mc, hipStream_t stream) {
   auto kernel = qmm8_mfma_staged<T, MT, NT, WAVES>;
@@ -707,12 +715,7 @@ bool launch_staged_one(const Q8Params& p, uint32_t slices, const Machine& mc, hi
   // One slice: the columns are dealt out evenly over a whole number of workgroups per compute unit (N = 14336 in 32s is
   // 448 workgroups, two for 192 of 256 units and one for the rest, and the launch lasts as long as the two take; in 28s
   // it is 512, two for each: the same bytes everywhere).  Several slices: whole tiles, which the second launch expects.
-  uint32_t cols = 16 * NT;
-  if (slices == 1) {
-    const uint32_t cus = uint32_t(mc.compute_units), wgs = (p.n + cols - 1) / cols, even = (wgs + cus - 1) / cus * cus;
-    const uint32_t fewer = ((p.n + even - 1) / even + 3) / 4 * 4;
-    if (fewer >= 8 && fewer < cols) cols = fewer;
-  }
+  const uint32_t cols = slices == 1 ? staged_cols(p.n, NT, uint32_t(mc.compute_units)) : 16 * NT;
   const dim3 grid((p.n + cols - 1) / cols, slices);
   const uint32_t chunks = (p.k + 255) / 256, per_slice = (chunks + slices - 1) / slices;
   hipLaunchKernelGGL(kernel, grid, dim3(WAVES * 64), lds, stream, p, per_slice, mc.workspace, cols);
@@ -1313,6 +1316,28 @@ bool workspace_refused(const Machine& mc, uint64_t need, std::string* err) {
   return true;
 }
 
+// The tile kernel's count of K-slices with the shortest estimated launch (4 steps per slice at least), and that
+// estimate in microseconds, from what was measured at 64 rows: every round of workgroups over the machine takes 3
+// (until its first operands are in LDS) + 0.72 per step (three times that with float32 activations, whose planes are
+// multiplied one after the other); more than one slice costs the second launch, 4.5, and its partial tiles written
+// and read back at 5 TB/s.  (Rounding tiles x slices to the nearest count of compute units, the rule before, gave
+// N = 11008 three slices: 258 workgroups on 256 units, two rounds of 11 steps, 31.2-32.6 us; two slices, one round
+// of 16 steps: 22.6-22.9.)
+template <class T>
+float tile_estimate_us(const Q8Params& p, const Machine& mc, uint32_t* slices) {
+  const uint32_t gx = (p.n + 127) / 128, gy = (p.m + 63) / 64, steps = p.k / kTileStepK;
+  const uint32_t cus = uint32_t(mc.compute_units), most = steps / 4 ? steps / 4 : 1;
+  const float step_us = T::dtype == VKT_F32 ? 2.2f : 0.72f, partial_us = float(p.m) * float(p.n) * 8.0f / 5e6f;
+  float best = 1e30f;
+  *slices = 1;
+  for (uint32_t s = 1; s <= most && s <= 64; ++s) {
+    const uint32_t rounds = (gx * gy * s + cus - 1) / cus;
+    const float cost = float(rounds) * (3.0f + step_us * float((steps + s - 1) / s)) + (s > 1 ? 4.5f + partial_us * float(s) : 0.0f);
+    if (cost < best) best = cost, *slices = s;
+  }
+  return best;
+}
+
 // Launches the tile kernel if it takes the product (k a multiple of its step, 16-byte aligned activation rows):
 // 1 launched, 0 not this kernel's shape, -1 refused (*err set).
 template <class T>
@@ -1330,23 +1355,7 @@ int launch_tile_kernel(const Q8Params& p, uint32_t want_slices, const Machine& m
   }
   const uint32_t gx = (p.n + 127) / 128, gy = (p.m + 63) / 64, steps = p.k / kTileStepK;
   uint32_t slices = want_slices;
-  if (slices == 0) {
-    // The count of slices with the shortest estimated launch, 4 steps per slice at least.  The estimate, in
-    // microseconds, from what was measured at 64 rows: every round of workgroups over the machine takes 3 (until its
-    // first operands are in LDS) + 0.72 per step (three times that with float32 activations, whose planes are
-    // multiplied one after the other); more than one slice costs the second launch, 4.5, and its partial tiles written
-    // and read back at 5 TB/s.  (Rounding tiles x slices to the nearest count of compute units, the rule before, gave
-    // N = 11008 three slices: 258 workgroups on 256 units, two rounds of 11 steps, 31.2-32.6 us; two slices, one round
-    // of 16 steps: 22.6-22.9.)
-    const uint32_t cus = uint32_t(mc.compute_units), most = steps / 4 ? steps / 4 : 1;
-    const float step_us = T::dtype == VKT_F32 ? 2.2f : 0.72f, partial_us = float(p.m) * float(p.n) * 8.0f / 5e6f;
-    float best = 1e30f;
-    for (uint32_t s = 1; s <= most && s <= 64; ++s) {
-      const uint32_t rounds = (gx * gy * s + cus - 1) / cus;
-      const float cost = float(rounds) * (3.0f + step_us * float((steps + s - 1) / s)) + (s > 1 ? 4.5f + partial_us * float(s) : 0.0f);
-      if (cost < best) best = cost, slices = s;
-    }
-  }
+  if (slices == 0) tile_estimate_us<T>(p, mc, &slices);
   if (slices > 1 && workspace_refused(mc, uint64_t(slices) * p.m * p.n * 4, err)) return -1;
   while (slices > 1 && uint64_t(slices) * p.m * p.n * 4 > mc.workspace_bytes) --slices;
   uint32_t per_slice = (steps + slices - 1) / slices;
@@ -1367,11 +1376,17 @@ int launch_tile_kernel(const Q8Params& p, uint32_t want_slices, const Machine& m
 // columns per workgroup that traffic is several times the weight stream once M reaches 64),
 // and K is cut into slices across workgroups until the grid covers the machine about
 // twice.  variant = NT | WAVES << 8 | SLICES << 24 overrides the plan (tuning, tests).
-template <class T>
-int launch_mfma(const Q8Params& p, uint32_t variant, const Machine& mc, hipStream_t stream, std::string* err) {
-  const int mt = p.m <= 16 ? 1 : p.m <= 32 ? 2 : 4;
+struct MfmaPlan {
+  bool staged;
+  int nt, waves;
+  uint32_t slices;
+  float estimate_us;  // of the launch, for 9 to 32 rows (0: none made)
+};
+
+inline MfmaPlan plan_mfma(const Q8Params& p, uint32_t variant, const Machine& mc) {
   int nt = p.n >= 64 ? 4 : 1, waves = p.m > 32 ? 4 : 8;  // (measured: K = 4096 and 14336, N = 14336 and 4096)
   uint32_t slices = 1;
+  float estimate = 0.0f;
   if (variant & 0xffff) {
     nt = variant & 0xff;
     waves = (variant >> 8) & 0xff;
@@ -1406,12 +1421,39 @@ int launch_mfma(const Q8Params& p, uint32_t variant, const Machine& mc, hipStrea
     // orders were rotated against each other: 17.9 / 15.6 since.)
     const uint32_t groups16 = (p.n + 15) / 16;
     nt = groups16 >= 2u * uint32_t(mc.compute_units) ? 2 : 1, waves = 8, slices = 1;
-  } else if (!(variant & 0xffff) && !((variant >> 19) & 1) && p.m <= 32 && p.k >= 2048 && p.k <= 8192 && p.n >= 8192) {
-    // 9 to 32 rows against many short weight rows: 64 columns per workgroup (K = 4096, N = 14336: 17.3 and 21.7 us
-    // at 16 and 32 rows against 18.6 and 23.3; with long rows and few columns the unstaged kernel stays ahead)
-    staged = true;
-    nt = 4, waves = 4, slices = 1;
+  } else if (!(variant & 0xffff) && !((variant >> 19) & 1) && p.m <= 32 && p.k >= 2048 && p.n >= 64) {
+    // 9 to 32 rows.  Every workgroup reads all rows of the activations next to its own weights, and what a launch
+    // lasts is what its busiest compute unit takes in: (workgroups on it) x (columns + 2 rows) x K bytes, at ~30 KB/us
+    // with the weights staged, ~23 with the plain kernel (whose K-slices cost a second launch, ~4.5 us).  16, 32 or 64
+    // columns per workgroup, whichever leaves the busiest unit least (64 as one workgroup per unit runs a quarter
+    // slower than its bytes say).  Measured, us at 9 / 16 / 32 rows with this choice against the rule before it (64
+    // columns for K <= 8192 and N >= 8192, else the plain kernel): K = N = 8192: 16.2 / 18.9 / 25.3 against 23.0 /
+    // 23.9 / 29.2; K = N = 4096: 7.5 / 8.6 / 12.2 against 9.3 / 9.7 / 12.2; K = 4096, N = 14336: 14.3 / 16.8 / 21.1
+    // against 16.3 / 16.9 / 21.1; K = 14336, N = 4096: 16.2 / 18.9 / 24.1 against 18.0 / 18.9 / 24.1.
+    const uint32_t cus = uint32_t(mc.compute_units);
+    const auto busiest = [&](uint32_t workgroups, uint32_t cols, uint32_t k_share) {
+      return float((workgroups + cus - 1) / cus) * float(cols + 2 * p.m) * float(k_share);
+    };
+    const uint32_t plain_groups = (p.n + 16 * nt - 1) / (16 * nt);
+    float best = busiest(plain_groups * slices, 16 * nt, (p.k + slices - 1) / slices) / 23e3f + (slices > 1 ? 4.5f : 0.0f);
+    for (int t = 1; t <= 4; t *= 2) {
+      const uint32_t cols = staged_cols(p.n, t, cus), workgroups = (p.n + cols - 1) / cols;
+      const float cost = busiest(workgroups, cols, p.k) / 30e3f * (t == 4 && workgroups <= cus ? 1.25f : 1.0f);
+      if (cost < best) best = cost, staged = true, nt = t;
+    }
+    if (staged) waves = nt < 4 && p.k >= 16 * 256 ? 8 : 4, slices = 1;
+    estimate = best;
   }
+  return MfmaPlan{staged, nt, waves, slices, estimate};
+}
+
+template <class T>
+int launch_mfma(const Q8Params& p, uint32_t variant, const Machine& mc, hipStream_t stream, std::string* err) {
+  const int mt = p.m <= 16 ? 1 : p.m <= 32 ? 2 : 4;
+  const MfmaPlan plan = plan_mfma(p, variant, mc);
+  const bool staged = plan.staged;
+  const int nt = plan.nt, waves = plan.waves;
+  uint32_t slices = plan.slices;
   if (staged) {  // chunks of 256 values of k
     const uint64_t sgroups = (p.n + 16 * nt - 1) / (16 * nt);
     const uint32_t schunks = (p.k + 255) / 256;
@@ -1491,8 +1533,18 @@ int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipSt
     // (variant bit 20 keeps the row-block kernels, for tests and tuning)
     const uint64_t need = q8_gemm_scratch_bytes(p0, T::dtype, mc);
     if (need != 0 && need <= mc.scratch_bytes && !((variant >> 20) & 1) && !(variant & 0xffff)) return launch_q8_gemm(p0, T::dtype, mc, stream, err);
-    // more than 32 rows (batched decode): the tile kernel (variant bit 21 forces it with bits 24+ slices, bit 22 keeps it off)
-    if (((p0.m > 32 && !(variant & 0xffff)) || ((variant >> 21) & 1)) && !((variant >> 22) & 1) && !((variant >> 17) & 1) && !((variant >> 18) & 1) &&
+    // more than 32 rows (batched decode): the tile kernel (variant bit 21 forces it with bits 24+ slices, bit 22 keeps it off).
+    // 17 to 32 rows: where its estimated launch is the shorter one by 5 % or more (it multiplies 64 rows whatever the
+    // count, but reads the activations once per 128 columns; measured at 24 rows, tile kernel / the others: K = 28672,
+    // N = 4096: 31.1 / 38.5 us, 14336 x 4096: 21.1 / 23.2, 8192 x 8192: 22.1 / 23.2, 2048 x 32000: 19.2 / 20.9; 4096 x 14336:
+    // 20.6 / 19.5, 4096 x 4096: 12.8 / 10.9 stay).
+    bool tile = p0.m > 32;
+    if (variant == 0 && p0.m > 16 && p0.m <= 32 && p0.k % kTileStepK == 0) {
+      uint32_t unused;
+      const MfmaPlan other = plan_mfma(p0, 0, mc);
+      tile = other.estimate_us > 0.0f && tile_estimate_us<T>(p0, mc, &unused) < 0.95f * other.estimate_us;
+    }
+    if (((tile && !(variant & 0xffff)) || ((variant >> 21) & 1)) && !((variant >> 22) & 1) && !((variant >> 17) & 1) && !((variant >> 18) & 1) &&
         !((variant >> 19) & 1) && !((variant >> 20) & 1)) {
       const int rc = launch_tile_kernel<T>(p0, variant >> 24, mc, stream, err);
       if (rc != 0) return rc < 0 ? -1 : 0;
