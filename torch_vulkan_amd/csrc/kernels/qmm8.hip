@@ -1568,10 +1568,21 @@ int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipSt
     }
   }
   if constexpr (T::dtype == VKT_F32) {
-    // More than 16 rows of float32 activations: the tile kernel on the activations' three bfloat16 parts, one pass
-    // over the weights per 64 rows (the one-row kernels below read them once per 16).  variant bit 21 forces it
-    // (bits 24+ slices), bit 22 keeps it off.
-    if (((p0.m > 16 && !(variant & 0xffff)) || ((variant >> 21) & 1)) && !((variant >> 22) & 1) && !((variant >> 17) & 1)) {
+    // More than 16 rows of float32 activations: the tile kernel on the activations' three bfloat16 parts, one pass over
+    // the weights per 64 rows.  3 to 16 rows: where its estimated launch is well below that of the one-row kernels
+    // below, which multiply every weight once per row on the vector units (kernels of 4, 8 and 16 rows: ~2.5 us + rows
+    // x weights / 3.8 MB/us) and read the weights once per 16 rows.  Measured, us at 3 / 4 / 8 / 16 rows, one-row
+    // kernels against the tile kernel: K = N = 4096: 16.8 / 18.2 / 34.5 / 64.5 against 17.4-18.7; K = 4096, N = 14336:
+    // 50.4 / 54.4 / 102 / 111 against 47; K = N = 8192: 63 / 69 / 124 / 126 against 49-50; K = N = 2048: 5.6 / 5.9 / 10.7 /
+    // 18.8 against 15.2-15.4 (so only 16 rows move); K = N = 1024: 3.7 / 3.7 / 4.6 / 7.0 against 14.6-14.9 (none do).
+    // variant bit 21 forces the tile kernel (bits 24+ slices), bit 22 keeps it off.
+    bool tile = p0.m > 16;
+    if (variant == 0 && p0.m >= 3 && p0.m <= 16 && p0.k % kTileStepK == 0) {
+      uint32_t unused;
+      const float rows = p0.m <= 4 ? 4.0f : p0.m <= 8 ? 8.0f : 16.0f, one_row_us = 2.5f + rows * float(p0.n) * float(p0.k) / 3.8e6f;
+      tile = tile_estimate_us<T>(p0, mc, &unused) < 0.8f * one_row_us;
+    }
+    if (((tile && !(variant & 0xffff)) || ((variant >> 21) & 1)) && !((variant >> 22) & 1) && !((variant >> 17) & 1)) {
       const int rc = launch_tile_kernel<T>(p0, variant >> 24, mc, stream, err);
       if (rc != 0) return rc < 0 ? -1 : 0;
     }
