@@ -183,6 +183,44 @@ def test_qmm8_float32_rows_special_values():
     assert (np.abs(got - want)[fin] <= (2.0 ** -23 * np.abs(want) + 2.0 ** -20 * mag)[fin]).all()
 
 
+@pytest.mark.parametrize("variant", [0, 1 << 18, 1 << 19])
+@pytest.mark.parametrize("m,k,n", [(2, 1024, 64), (3, 2064, 200), (5, 4096, 1000), (8, 1040, 77), (13, 3072, 4100), (16, 4096, 4128), (9, 8192, 520)])
+def test_qmm8_float32_few_rows_on_matrix_cores(variant, m, k, n):
+    """2 to 16 rows of float32 activations: split into three bfloat16 planes by a launch of its own and multiplied by
+    the staged matrix-core kernel (forced with bit 18, planned, and switched off with bit 19); rows of k not a multiple
+    of 256, every column count per workgroup, strided rows as well."""
+    import _dev
+    a, b, s = int8_case(torch.float32, m, k, n)
+    check_q8(_dev.qmm8(bits(a), ODT[torch.float32], b.numpy(), bits(s), variant=variant), a, b, s, torch.float32)
+    check_q8(_dev.qmm8(bits(a), ODT[torch.float32], b.numpy(), bits(s), variant=variant, row_step=2), a, b, s, torch.float32,
+             rows=slice(None, None, 2))
+
+
+def test_qmm8_float32_few_rows_special_values():
+    """The same special values through the three-plane split of the few-row path: infinities and NaNs come out where
+    float64 arithmetic has them, the rest within the bound."""
+    import _dev
+    m, k, n = 8, 1024, 64
+    a, b, s = int8_case(torch.float32, m, k, n)
+    a = a.clone()
+    a[1, 5] = float("inf")
+    a[2, 7] = float("-inf")
+    a[3, 9] = float("nan")
+    a[4, 11] = torch.tensor(0x7f800001, dtype=torch.int32).view(torch.float32)
+    a[5, :] = 0.0
+    a[6, 3] = 1e-41
+    a[7, 2] = 3.0e38
+    b = b.clone()
+    b[:, 2] = 1  # (keeps row 7 finite)
+    got = unbits(_dev.qmm8(bits(a), ODT[torch.float32], b.numpy(), bits(s), variant=1 << 18), torch.float32).numpy().astype(np.float64)
+    want = (a.double() @ b.double().t() * s.double()).numpy()
+    nan, inf = np.isnan(want), np.isinf(want)
+    assert np.array_equal(np.isnan(got), nan) and np.array_equal(got[inf], want[inf])
+    fin = ~(nan | inf)
+    mag = (a.double().abs() @ b.double().abs().t() * s.double().abs()).numpy()
+    assert (np.abs(got - want)[fin] <= (2.0 ** -23 * np.abs(want) + 2.0 ** -20 * mag)[fin]).all()
+
+
 def test_qmm8_config1_vs_torch_cpu():
     """BASELINE config 1: fp32, M=1, K=N=4096, within rtol/atol 1e-4 of PyTorch's CPU op."""
     import _dev

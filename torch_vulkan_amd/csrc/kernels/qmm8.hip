@@ -413,9 +413,10 @@ __device__ __forceinline__ V4F mfma16(const U4& w, const U4& a, const V4F& acc) 
 template <class T, int MT, int NT>
 __device__ __forceinline__ void store_tiles(const Q8Params& p, uint32_t n0, const V4F (&acc)[MT][NT], int lane, uint32_t n_end = ~0u) {
   n_end = n_end < p.n ? n_end : p.n;  // (columns from n_end on are another workgroup's; a multiple of 4, or n)
-  constexpr uint64_t item = 2;
+  constexpr uint64_t item = sizeof(typename T::storage);  // (scales and outputs have the activations' type)
+  constexpr bool F32 = T::dtype == VKT_F32;
   const int c = lane & 15, g = lane >> 4;
-  const bool vec_ok = (p.n & 3u) == 0 && (p.c & 7u) == 0;
+  const bool vec_ok = (p.n & 3u) == 0 && (p.c & (4 * item - 1)) == 0;
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     const uint32_t n = n0 + 16 * t + 4 * g;
@@ -427,18 +428,28 @@ __device__ __forceinline__ void store_tiles(const Q8Params& p, uint32_t n0, cons
       const uint32_t m = 16 * mt + c;
       if (m >= p.m || n >= n_end) continue;
       const uint64_t at = p.c + (uint64_t(m) * p.n + n) * item;
-      uint32_t h[4];
+      float v[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float v = acc[mt][t][r] * scale[r];
-        h[r] = T::dtype == VKT_BF16 ? f32_to_bf16(v) : f32_to_f16(v);
-      }
-      if (vec_ok && n + 3 < n_end) {
-        stg<U2>(at, U2{h[0] | h[1] << 16, h[2] | h[3] << 16});
+      for (int r = 0; r < 4; ++r) v[r] = acc[mt][t][r] * scale[r];
+      if constexpr (F32) {
+        if (vec_ok && n + 3 < n_end) {
+          stg<F4>(at, F4{v[0], v[1], v[2], v[3]});
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (n + r < n_end) stg<float>(at + r * item, v[r]);
+        }
       } else {
+        uint32_t h[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (n + r < n_end) stg<uint16_t>(at + r * item, uint16_t(h[r]));
+        for (int r = 0; r < 4; ++r) h[r] = T::dtype == VKT_BF16 ? f32_to_bf16(v[r]) : f32_to_f16(v[r]);
+        if (vec_ok && n + 3 < n_end) {
+          stg<U2>(at, U2{h[0] | h[1] << 16, h[2] | h[3] << 16});
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (n + r < n_end) stg<uint16_t>(at + r * item, uint16_t(h[r]));
+        }
       }
     }
   }
@@ -557,9 +568,13 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma(Q8Params p, uint32_t chu
 // lane simply fetches the chunk that belongs in its slot.  A wave works on chunks of 256
 // values of k: all loads of a chunk are issued, awaited (vmcnt(0)) and consumed; the waves of a
 // workgroup drift apart and keep the memory pipeline full between them.
-template <class T, int MT, int NT, int WAVES>
+// PLANES = 3 (float32 outputs): the activations are three bfloat16 planes [3][m][k] whose sum the float32 activations
+// are, exactly (qmm8_split_rows wrote them); every weight fragment multiplies the three planes' fragments one after
+// the other into the same sums, which is the product of the float32 values added up in float32.
+template <class T, int MT, int NT, int WAVES, int PLANES>
 __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma_staged(Q8Params p, uint32_t chunks_per_slice, uint64_t workspace, uint32_t cols_per_wg) {
-  constexpr uint64_t item = 2;
+  constexpr uint64_t item = 2;  // (of the activations as this kernel reads them)
+  const uint64_t plane_bytes = PLANES > 1 ? uint64_t(p.m) * p.k * item : 0;  // (planes: rows k values apart)
   constexpr uint32_t TILE = 16 * 256, REGION = NT * TILE;  // bytes of LDS per tile of 16 rows, per wave
   extern __shared__ __attribute__((aligned(16))) uint8_t staged[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
@@ -617,18 +632,20 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma_staged(Q8Params p, uint3
   for (uint32_t i = wave; i < count; i += WAVES) {
     const uint32_t q = chunk_at(i);
     const uint32_t k0 = q * 256;
-    U4 a0[MT][4], a1[MT][4];
+    U4 a0[PLANES][MT][4], a1[PLANES][MT][4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const bool inside = k0 + 64 * j + 16 * g < p.k;  // (k is a multiple of 16)
+    for (int pl = 0; pl < PLANES; ++pl)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        // (rows past m are zeros, not loads: with 8 rows that is half of the activation traffic)
-        const bool real = inside && uint32_t(16 * mt + c) < p.m;
-        a0[mt][j] = real ? ldg<U4>(arow[mt] + (k0 + 64 * j) * item) : zero;
-        a1[mt][j] = real ? ldg<U4>(arow[mt] + (k0 + 64 * j) * item + 16) : zero;
+      for (int j = 0; j < 4; ++j) {
+        const bool inside = k0 + 64 * j + 16 * g < p.k;  // (k is a multiple of 16)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          // (rows past m are zeros, not loads: with 8 rows that is half of the activation traffic)
+          const bool real = inside && uint32_t(16 * mt + c) < p.m;
+          a0[pl][mt][j] = real ? ldg<U4>(arow[mt] + pl * plane_bytes + (k0 + 64 * j) * item) : zero;
+          a1[pl][mt][j] = real ? ldg<U4>(arow[mt] + pl * plane_bytes + (k0 + 64 * j) * item + 16) : zero;
+        }
       }
-    }
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
@@ -643,10 +660,12 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma_staged(Q8Params p, uint3
         U4 wlo, whi;
         widen16_to_operands<T>(wv, &wlo, &whi);
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          acc[mt][t] = mfma16<T>(wlo, a0[mt][j], acc[mt][t]);
-          acc[mt][t] = mfma16<T>(whi, a1[mt][j], acc[mt][t]);
-        }
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int pl = 0; pl < PLANES; ++pl) {
+            acc[mt][t] = mfma16<T>(wlo, a0[pl][mt][j], acc[mt][t]);
+            acc[mt][t] = mfma16<T>(whi, a1[pl][mt][j], acc[mt][t]);
+          }
       }
     }
   }
@@ -699,9 +718,9 @@ inline uint32_t staged_cols(uint32_t n, int nt, uint32_t cus) {
   return fewer >= 8 && fewer < cols ? fewer : cols;
 }
 
-template <class T, int MT, int NT, int WAVES>
+template <class T, int MT, int NT, int WAVES, int PLANES = 1>
 bool launch_staged_one(const Q8Params& p, uint32_t slices, const Machine& mc, hipStream_t stream) {
-  auto kernel = qmm8_mfma_staged<T, MT, NT, WAVES>;
+  auto kernel = qmm8_mfma_staged<T, MT, NT, WAVES, PLANES>;
   constexpr uint32_t stage_bytes = WAVES * NT * 16 * 256, part_bytes = kPartSlots<MT, NT, WAVES> * MT * NT * 1024;
   constexpr uint32_t lds = stage_bytes > part_bytes ? stage_bytes : part_bytes;
   static bool configured = false;  // guarded by the runtime's stream mutex
@@ -1017,6 +1036,62 @@ __device__ __forceinline__ void split_f32x8(const U4& x0, const U4& x1, U4* hi, 
     return U4{v[0] >> 16 | v[1], v[2] >> 16 | v[3], v[4] >> 16 | v[5], v[6] >> 16 | v[7]};
   };
   *hi = pack(h), *mid = pack(m), *lo = pack(l);
+}
+
+bool workspace_refused(const Machine& mc, uint64_t need, std::string* err);
+
+// float32 activation rows [m][k] (rows a_sm values apart) as three bfloat16 planes [3][m][k]: a thread per 8 values.
+__global__ __launch_bounds__(256) void qmm8_split_rows(Q8Params p, uint64_t planes) {
+  const uint32_t per_row = p.k / 8, id = blockIdx.x * 256 + threadIdx.x;  // (k is a multiple of 16)
+  if (id >= p.m * per_row) return;
+  const uint32_t m = id / per_row, piece = id % per_row;
+  const uint64_t src = p.a + uint64_t(int64_t(m) * p.a_sm * 4) + piece * 32ull;
+  const U4 x0 = ldg<U4>(src), x1 = ldg<U4>(src + 16);
+  U4 part[3];
+  split_f32x8(x0, x1, &part[0], &part[1], &part[2]);
+  const uint64_t plane = uint64_t(p.m) * p.k * 2;
+#pragma unroll
+  for (int q = 0; q < 3; ++q) stg<U4>(planes + q * plane + (uint64_t(m) * p.k + piece * 8ull) * 2, part[q]);
+}
+
+// 2 to 16 rows of float32 activations on the matrix cores: the rows are split into their three bfloat16 planes by a
+// launch of its own (into the workspace), and the staged kernel multiplies every weight fragment by the planes'
+// fragments.  Columns per workgroup as for 16-bit activations, with three times their activation bytes.  Returns the
+// estimated microseconds of both launches in *estimate_us when stream is null (nothing is launched then); false
+// where the path does not apply.
+inline bool launch_split_staged(const Q8Params& p0, const Machine& mc, hipStream_t stream, bool launch, float* estimate_us, std::string* err, int* rc) {
+  *rc = 0;
+  if (p0.m < 2 || p0.m > 16 || p0.k < 1024 || p0.n < 64 || uint64_t(p0.m) * p0.k >= (1ull << 28)) return false;
+  const uint64_t need = 3ull * p0.m * p0.k * 2;
+  const uint32_t cus = uint32_t(mc.compute_units);
+  int nt = 1;
+  float best = 1e30f;
+  for (int t = 1; t <= 4; t *= 2) {
+    const uint32_t cols = staged_cols(p0.n, t, cus), workgroups = (p0.n + cols - 1) / cols;
+    const float cost = float((workgroups + cus - 1) / cus) * float(cols + 6 * p0.m) * float(p0.k) / 30e3f * (t == 4 && workgroups <= cus ? 1.25f : 1.0f);
+    if (cost < best) best = cost, nt = t;
+  }
+  *estimate_us = best + 6.5f;  // (what two launches in a row cost before their bytes: K = N = 1024 takes 6.3-8.1 us)
+  if (!launch) return need <= mc.workspace_bytes || mc.workspace_fixed;
+  if (workspace_refused(mc, need, err)) {
+    *rc = -1;
+    return true;
+  }
+  if (need > mc.workspace_bytes) return false;
+  const uint32_t threads = p0.m * (p0.k / 8);
+  hipLaunchKernelGGL(qmm8_split_rows, dim3((threads + 255) / 256), dim3(256), 0, stream, p0, mc.workspace);
+  Q8Params p = p0;
+  p.a = mc.workspace, p.a_sm = p0.k;
+  const int waves = nt < 4 && p0.k >= 16 * 256 ? 8 : 4;
+  bool ok = false;
+  if (nt == 1) ok = waves == 8 ? launch_staged_one<f32_t, 1, 1, 8, 3>(p, 1, mc, stream) : launch_staged_one<f32_t, 1, 1, 4, 3>(p, 1, mc, stream);
+  else if (nt == 2) ok = waves == 8 ? launch_staged_one<f32_t, 1, 2, 8, 3>(p, 1, mc, stream) : launch_staged_one<f32_t, 1, 2, 4, 3>(p, 1, mc, stream);
+  else ok = launch_staged_one<f32_t, 1, 4, 4, 3>(p, 1, mc, stream);
+  if (!ok) {
+    *err = "qmm8: cannot reserve LDS for the staged kernel";
+    *rc = -1;
+  }
+  return true;
 }
 
 template <class T>
@@ -1576,11 +1651,21 @@ int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipSt
     // 50.4 / 54.4 / 102 / 111 against 47; K = N = 8192: 63 / 69 / 124 / 126 against 49-50; K = N = 2048: 5.6 / 5.9 / 10.7 /
     // 18.8 against 15.2-15.4 (so only 16 rows move); K = N = 1024: 3.7 / 3.7 / 4.6 / 7.0 against 14.6-14.9 (none do).
     // variant bit 21 forces the tile kernel (bits 24+ slices), bit 22 keeps it off.
+    // 2 to 16 rows: split into bfloat16 planes by a launch of its own and multiplied by the staged matrix-core kernel,
+    // where the estimate of the two launches is the shortest of the three (variant bit 18 asks for that path, bit 19
+    // keeps it off).
     bool tile = p0.m > 16;
-    if (variant == 0 && p0.m >= 3 && p0.m <= 16 && p0.k % kTileStepK == 0) {
+    if ((variant == 0 || variant == (1u << 18) || variant == (1u << 19)) && p0.m >= 2 && p0.m <= 16) {
       uint32_t unused;
-      const float rows = p0.m <= 4 ? 4.0f : p0.m <= 8 ? 8.0f : 16.0f, one_row_us = 2.5f + rows * float(p0.n) * float(p0.k) / 3.8e6f;
-      tile = tile_estimate_us<T>(p0, mc, &unused) < 0.8f * one_row_us;
+      const float rows = p0.m <= 2 ? 2.0f : p0.m <= 4 ? 4.0f : p0.m <= 8 ? 8.0f : 16.0f, one_row_us = 2.5f + rows * float(p0.n) * float(p0.k) / 3.8e6f;
+      const float tile_us = p0.m >= 3 && p0.k % kTileStepK == 0 ? tile_estimate_us<T>(p0, mc, &unused) : 1e30f;
+      float split_us = 1e30f;
+      int rc = 0;
+      const bool can_split = !((variant >> 19) & 1) && launch_split_staged(p0, mc, stream, false, &split_us, err, &rc);
+      if (can_split && (((variant >> 18) & 1) || (split_us < 0.9f * one_row_us && split_us < tile_us))) {
+        if (launch_split_staged(p0, mc, stream, true, &split_us, err, &rc)) return rc;
+      }
+      tile = variant != (1u << 18) && tile_us < 0.8f * one_row_us;
     }
     if (((tile && !(variant & 0xffff)) || ((variant >> 21) & 1)) && !((variant >> 22) & 1) && !((variant >> 17) & 1)) {
       const int rc = launch_tile_kernel<T>(p0, variant >> 24, mc, stream, err);
