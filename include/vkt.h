@@ -121,7 +121,8 @@ uint64_t vkt_qmm4c_q_bytes(uint32_t m, uint32_t k);
  * kernel with a workgroup per pair of columns, bits 8-11 / 12-15 (bits 0-7 clear) ask for the persistent streaming
  * kernel with that many workgroups per compute unit / rows per iteration; 3 to 8 rows: bit 23 keeps the slice
  * kernels where the planner would take the kernel whose waves own column groups (large products), bits 8-15 (bits
- * 0-7 clear) ask for that kernel whatever the size. */
+ * 0-7 clear) ask for that kernel whatever the size; float32 activations, 2 to 16 rows: exactly bit 18 / bit 19 asks for /
+ * keeps off the path that splits the rows into bfloat16 planes for the staged matrix-core kernel. */
 typedef struct Q8Params {
   uint64_t a, b, scales, c; /* A [m,k] (row stride a_sm, a_sk must be 1), B int8 [n,k], scales [n], C [m,n] */
   uint32_t m, n, k;
