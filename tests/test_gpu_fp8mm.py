@@ -28,7 +28,7 @@ HW_WINDOW = 2.0**-13
 def on_matrix_cores(odt, variant, k):
     if variant in (6, 7, 255) or k % 16:
         return False
-    return variant in (1, 2, 3, 4, 5, 8, 11) or odt in (oracle.BF16, oracle.E4M3, oracle.E5M2)
+    return variant in (1, 2, 3, 4, 5, 8, 11, 12) or odt in (oracle.BF16, oracle.E4M3, oracle.E5M2)
 
 
 def run_case(m, k, n, fa, fb, out_dtype, rowwise, bias_dtype=None, scale_result=None, variant=0, seed=1, scale=1.0):
@@ -86,6 +86,21 @@ def test_scaled_mm_tile_edges(m, k, n, variant, rowwise):
     unaligned kernel), every tile variant and the one-thread-per-output kernel (255)."""
     run_case(m, k, n, FLOAT8[0], FLOAT8[0], torch.bfloat16, rowwise, torch.float32, variant=variant, seed=20)
     run_case(m, k, n, FLOAT8[1], FLOAT8[0], torch.float32, rowwise, variant=variant, seed=30)
+
+
+@pytest.mark.parametrize("fa,fb", [(FLOAT8[0], FLOAT8[0]), (FLOAT8[1], FLOAT8[0]), (FLOAT8[0], FLOAT8[1]), (FLOAT8[1], FLOAT8[1])])
+@pytest.mark.parametrize("m,k,n,out_dtype,rowwise", [
+    (1, 1024, 64, torch.bfloat16, False), (7, 2064, 200, torch.bfloat16, True), (16, 4096, 1000, torch.float8_e4m3fn, True),
+    (17, 1040, 77, torch.bfloat16, True), (32, 3072, 4100, torch.bfloat16, False), (33, 1024, 130, torch.float8_e5m2, False),
+    (64, 4096, 4128, torch.bfloat16, True), (50, 8192, 520, torch.bfloat16, True)])
+def test_scaled_mm_few_rows(fa, fb, m, k, n, out_dtype, rowwise):
+    """Up to 64 rows with bfloat16 or float8 outputs run on the kernel whose workgroups own runs of columns and whose
+    waves split K (planned, which is what these shapes get, and asked for as variant 12): every row-tile count, rows of
+    k not a multiple of 256, column counts that leave short workgroups and ragged vectors, bias and output scale."""
+    bias_dtype = torch.bfloat16 if out_dtype == torch.bfloat16 else None
+    sr = 2.0 if out_dtype != torch.bfloat16 else None
+    for variant in (0, 12):
+        run_case(m, k, n, fa, fb, out_dtype, rowwise, bias_dtype, sr, variant=variant, seed=m + n)
 
 
 def test_scaled_mm_fp8_output_saturation_and_nan():

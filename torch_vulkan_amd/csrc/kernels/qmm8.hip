@@ -28,6 +28,7 @@
 #include <type_traits>
 
 #include "kernels.h"
+#include "wave_tiles.h"
 
 namespace vkt {
 namespace {
@@ -371,7 +372,6 @@ __global__ __launch_bounds__(256) void qmm8_generic(Q8Params p) {
   }
 }
 
-using V4F = float __attribute__((ext_vector_type(4)));
 using V8BF = __bf16 __attribute__((ext_vector_type(8)));
 using V8H = _Float16 __attribute__((ext_vector_type(8)));
 
@@ -450,44 +450,6 @@ __device__ __forceinline__ void store_tiles(const Q8Params& p, uint32_t n0, cons
           for (int r = 0; r < 4; ++r)
             if (n + r < n_end) stg<uint16_t>(at + r * item, uint16_t(h[r]));
         }
-      }
-    }
-  }
-}
-
-// The partial tiles of a workgroup's waves added up in wave 0.  Where LDS holds half the waves' tiles, a
-// tree: in each round the upper half of the remaining waves hands its tiles to the lower half (two
-// barriers per round, log2(WAVES) rounds, a fixed order); otherwise wave by wave.
-template <int MT, int NT, int WAVES>
-constexpr int kPartSlots = (WAVES / 2) * MT * NT <= 32 ? WAVES / 2 : 1;
-
-template <int MT, int NT, int WAVES>
-__device__ __forceinline__ void add_wave_tiles(V4F (&acc)[MT][NT], V4F* part, int wave, int lane) {
-  if constexpr (kPartSlots<MT, NT, WAVES> > 1) {
-#pragma unroll
-    for (int half = WAVES / 2; half >= 1; half /= 2) {
-      if (wave >= half && wave < 2 * half) {
-#pragma unroll
-        for (int i = 0; i < MT * NT; ++i) part[((wave - half) * MT * NT + i) * 64 + lane] = acc[i / NT][i % NT];
-      }
-      __syncthreads();
-      if (wave < half) {
-#pragma unroll
-        for (int i = 0; i < MT * NT; ++i) acc[i / NT][i % NT] += part[(wave * MT * NT + i) * 64 + lane];
-      }
-      if (half > 1) __syncthreads();
-    }
-  } else {
-    for (int w = 1; w < WAVES; ++w) {
-      __syncthreads();
-      if (wave == w) {
-#pragma unroll
-        for (int i = 0; i < MT * NT; ++i) part[i * 64 + lane] = acc[i / NT][i % NT];
-      }
-      __syncthreads();
-      if (wave == 0) {
-#pragma unroll
-        for (int i = 0; i < MT * NT; ++i) acc[i / NT][i % NT] += part[i * 64 + lane];
       }
     }
   }
@@ -708,14 +670,6 @@ void launch_mfma_waves(const Q8Params& p, int waves, uint32_t slices, const Mach
     default: hipLaunchKernelGGL((qmm8_mfma<T, MT, NT, 16>), grid, dim3(1024), 0, stream, p, per_slice, mc.workspace); break;
   }
   if (slices > 1) hipLaunchKernelGGL((qmm8_mfma_finish<T, MT, NT>), dim3(grid.x), dim3(64), 0, stream, p, slices, mc.workspace);
-}
-
-// Columns per workgroup of the staged kernel with one slice: at most 16 nt, fewer where that deals the columns out
-// over a whole number of workgroups per compute unit (a multiple of 4, at least 8).
-inline uint32_t staged_cols(uint32_t n, int nt, uint32_t cus) {
-  const uint32_t cols = 16 * nt, wgs = (n + cols - 1) / cols, even = (wgs + cus - 1) / cus * cus;
-  const uint32_t fewer = ((n + even - 1) / even + 3) / 4 * 4;
-  return fewer >= 8 && fewer < cols ? fewer : cols;
 }
 
 template <class T, int MT, int NT, int WAVES, int PLANES = 1>
