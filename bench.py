@@ -206,7 +206,7 @@ def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030, prefill=False, phase=2):
                 shape=(n, bs), reference_layout_bytes=int(packed.numel()) * 4 + 4 * m * k + 4 * m * n, **timed(abi, fns, steps, warmup))
 
 
-def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False):
+def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False, variant=0):
     """_scaled_mm e4m3fn x e4m3fn -> bf16; A row-major, B column-major.  zero_operands: the same
     launch on all-zero matrices: the matrix cores' sustained rate depends on how many operand
     bits toggle (the part is power limited), and this is the data-independent end of that range."""
@@ -226,7 +226,7 @@ def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False)
     out = abi.Buffer(m * n * 2)
     p = abi.F8Params(a=da.address, b=db.address, scale_a=dsa.address, scale_b=dsb.address, out=out.address, m=m, n=n,
                      k=k, lda=k, ldb=k, ldo=n, fmt_a=abi.E4M3, fmt_b=abi.E4M3, out_dtype=abi.BF16, rowwise=int(rowwise))
-    fns = [Launch(abi, "fp8mm", [0], p)]
+    fns = [Launch(abi, "fp8mm", [variant], p)]
     tm = time_steps(abi, fns, steps, warmup)
     return dict(kind="mfma", work=2 * m * n * k, wall_ms=tm[0], event_ms=tm[1], event_ms_median=tm.median, bytes=m * k + n * k + 2 * m * n,
                 inputs=(a, bt, sa, sb), copies=1,

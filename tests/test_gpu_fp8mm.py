@@ -92,14 +92,16 @@ def test_scaled_mm_tile_edges(m, k, n, variant, rowwise):
 @pytest.mark.parametrize("m,k,n,out_dtype,rowwise", [
     (1, 1024, 64, torch.bfloat16, False), (7, 2064, 200, torch.bfloat16, True), (16, 4096, 1000, torch.float8_e4m3fn, True),
     (17, 1040, 77, torch.bfloat16, True), (32, 3072, 4100, torch.bfloat16, False), (33, 1024, 130, torch.float8_e5m2, False),
-    (64, 4096, 4128, torch.bfloat16, True), (50, 8192, 520, torch.bfloat16, True)])
+    (64, 4096, 4128, torch.bfloat16, True), (50, 8192, 520, torch.bfloat16, True),
+    # float32 and float16 outputs: the same kernel on operands widened exactly to bfloat16 (no window in the bound)
+    (5, 2064, 300, torch.float32, True), (40, 1024, 64, torch.float16, False), (16, 4096, 4100, torch.float32, False)])
 def test_scaled_mm_few_rows(fa, fb, m, k, n, out_dtype, rowwise):
     """Up to 64 rows with bfloat16 or float8 outputs run on the kernel whose workgroups own runs of columns and whose
     waves split K (planned, which is what these shapes get, and asked for as variant 12): every row-tile count, rows of
     k not a multiple of 256, column counts that leave short workgroups and ragged vectors, bias and output scale."""
     bias_dtype = torch.bfloat16 if out_dtype == torch.bfloat16 else None
-    sr = 2.0 if out_dtype != torch.bfloat16 else None
-    for variant in (0, 12):
+    sr = 2.0 if out_dtype in (torch.float8_e4m3fn, torch.float8_e5m2) else None
+    for variant in (0, 12) if sr or bias_dtype else (0,):
         run_case(m, k, n, fa, fb, out_dtype, rowwise, bias_dtype, sr, variant=variant, seed=m + n)
 
 

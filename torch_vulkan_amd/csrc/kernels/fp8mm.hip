@@ -226,7 +226,16 @@ __device__ __forceinline__ V4F mfma_f8x32(long w, long a, const V4F& acc) {
   else return __builtin_amdgcn_mfma_f32_16x16x32_bf8_bf8(w, a, acc, 0, 0, 0);
 }
 
-template <int MT, int NT, int WAVES, int FA, int FB>
+// WIDE (float32 and float16 outputs): both operands are widened exactly to bfloat16 in registers (two values per
+// conversion instruction) and multiplied by V_MFMA_F32_16X16X32_BF16, which adds at float32 precision.
+template <int F>
+__device__ __forceinline__ V8BF widen8(uint32_t lo, uint32_t hi) {
+  const V2BF p0 = widen_pair<F, false>(int(lo)), p1 = widen_pair<F, true>(int(lo));
+  const V2BF p2 = widen_pair<F, false>(int(hi)), p3 = widen_pair<F, true>(int(hi));
+  return V8BF{p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
+}
+
+template <int MT, int NT, int WAVES, int FA, int FB, bool WIDE>
 __global__ __launch_bounds__(WAVES * 64) void fp8mm_skinny(F8Problem p, uint32_t cols_per_wg) {
   constexpr uint32_t TILE = 16 * 256, REGION = NT * TILE;  // bytes of LDS per tile of 16 weight rows, per wave
   extern __shared__ __attribute__((aligned(16))) uint8_t staged[];
@@ -294,16 +303,30 @@ __global__ __launch_bounds__(WAVES * 64) void fp8mm_skinny(F8Problem p, uint32_t
     if (i + WAVES < count) request(chunk_at(i + WAVES));
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
+      V8BF wide_a[WIDE ? MT : 1][2];
+      if constexpr (WIDE) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) wide_a[mt][0] = widen8<FA>(a[mt][j][0], a[mt][j][1]), wide_a[mt][1] = widen8<FA>(a[mt][j][2], a[mt][j][3]);
+      }
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         // (a wave's LDS operations execute in order: these reads see the writes above)
         const U4 wv = *reinterpret_cast<const U4*>(mine + (t * 16 + c) * 256 + (((4 * j + g) ^ c) & 15) * 16);
-        const long w0 = long(uint64_t(wv[0]) | uint64_t(wv[1]) << 32), w1 = long(uint64_t(wv[2]) | uint64_t(wv[3]) << 32);
+        if constexpr (WIDE) {
+          const V8BF w0 = widen8<FB>(wv[0], wv[1]), w1 = widen8<FB>(wv[2], wv[3]);
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          const long a0 = long(uint64_t(a[mt][j][0]) | uint64_t(a[mt][j][1]) << 32), a1 = long(uint64_t(a[mt][j][2]) | uint64_t(a[mt][j][3]) << 32);
-          acc[mt][t] = mfma_f8x32<FA, FB>(w0, a0, acc[mt][t]);
-          acc[mt][t] = mfma_f8x32<FA, FB>(w1, a1, acc[mt][t]);
+          for (int mt = 0; mt < MT; ++mt) {
+            acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, wide_a[mt][0], acc[mt][t], 0, 0, 0);
+            acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, wide_a[mt][1], acc[mt][t], 0, 0, 0);
+          }
+        } else {
+          const long w0 = long(uint64_t(wv[0]) | uint64_t(wv[1]) << 32), w1 = long(uint64_t(wv[2]) | uint64_t(wv[3]) << 32);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            const long a0 = long(uint64_t(a[mt][j][0]) | uint64_t(a[mt][j][1]) << 32), a1 = long(uint64_t(a[mt][j][2]) | uint64_t(a[mt][j][3]) << 32);
+            acc[mt][t] = mfma_f8x32<FA, FB>(w0, a0, acc[mt][t]);
+            acc[mt][t] = mfma_f8x32<FA, FB>(w1, a1, acc[mt][t]);
+          }
         }
       }
     }
@@ -329,9 +352,9 @@ __global__ __launch_bounds__(WAVES * 64) void fp8mm_skinny(F8Problem p, uint32_t
   }
 }
 
-template <int MT, int NT, int WAVES, int FA, int FB>
+template <int MT, int NT, int WAVES, int FA, int FB, bool WIDE>
 int launch_skinny_one(const F8Problem& p, uint32_t cols, hipStream_t stream, std::string* err) {
-  auto kernel = fp8mm_skinny<MT, NT, WAVES, FA, FB>;
+  auto kernel = fp8mm_skinny<MT, NT, WAVES, FA, FB, WIDE>;
   constexpr uint32_t stage_bytes = WAVES * NT * 16 * 256, part_bytes = kPartSlots<MT, NT, WAVES> * MT * NT * 1024;
   constexpr uint32_t lds = stage_bytes > part_bytes ? stage_bytes : part_bytes;
   static bool configured = false;  // guarded by the runtime's stream mutex
@@ -347,14 +370,15 @@ int launch_skinny_one(const F8Problem& p, uint32_t cols, hipStream_t stream, std
   return 0;
 }
 
-// The few-row kernel where it serves: up to 64 rows, rows of k of 1024 bytes and more, bfloat16 or float8 outputs (the
-// precision the fp8 matrix cores are used for).  16, 32 or 64 columns per workgroup, whichever leaves the busiest
+// The few-row kernel where it serves: up to 64 rows, rows of k of 1024 bytes and more; bfloat16 and float8 outputs on
+// the fp8 matrix-core instruction, float32 and float16 outputs on exactly widened operands (the precision rule of the
+// tile kernels).  16, 32 or 64 columns per workgroup, whichever leaves the busiest
 // compute unit the fewest bytes to take in, (workgroups on it) x (columns + rows) x K: every workgroup reads all rows
 // of A beside its weights.  -2: not this kernel's problem.
 template <int FA, int FB>
-int launch_skinny(const F8Params& p0, int compute_units, hipStream_t stream, std::string* err) {
-  const bool narrow_out = p0.out_dtype == VKT_BF16 || p0.out_dtype == VKT_E4M3 || p0.out_dtype == VKT_E5M2;
-  if (p0.m > 64 || p0.k < 1024 || p0.n < 64 || !narrow_out) return -2;
+int launch_skinny(const F8Params& p0, int compute_units, uint32_t forced_nt, hipStream_t stream, std::string* err) {
+  const bool wide = p0.out_dtype == VKT_F32 || p0.out_dtype == VKT_F16;
+  if (p0.m > 64 || p0.k < 1024 || p0.n < 64) return -2;
   F8Problem p;
   static_cast<F8Params&>(p) = p0;
   const uint32_t cus = uint32_t(compute_units);
@@ -366,11 +390,14 @@ int launch_skinny(const F8Params& p0, int compute_units, hipStream_t stream, std
     if (cost < best) best = cost, nt = t;
   }
   const int mt = p.m <= 16 ? 1 : p.m <= 32 ? 2 : 4;
+  if (forced_nt) nt = int(forced_nt);
   if (mt == 1 && nt == 4) nt = 2;  // (the shapes that are built)
   if (mt == 4 && nt == 1) nt = 2;
   const uint32_t cols = staged_cols(p.n, nt, cus);
-#define VKT_SKINNY_CASE(MT_, NT_, W_) \
-  if (mt == MT_ && nt == NT_) return launch_skinny_one<MT_, NT_, W_, FA, FB>(p, cols, stream, err);
+#define VKT_SKINNY_CASE(MT_, NT_, W_)                                                                         \
+  if (mt == MT_ && nt == NT_)                                                                                \
+    return wide ? launch_skinny_one<MT_, NT_, W_, FA, FB, true>(p, cols, stream, err) \
+                : launch_skinny_one<MT_, NT_, W_, FA, FB, false>(p, cols, stream, err);
   VKT_SKINNY_CASE(1, 1, 8) VKT_SKINNY_CASE(1, 2, 8) VKT_SKINNY_CASE(2, 1, 8) VKT_SKINNY_CASE(2, 2, 8) VKT_SKINNY_CASE(2, 4, 4)
   VKT_SKINNY_CASE(4, 2, 8) VKT_SKINNY_CASE(4, 4, 4)
 #undef VKT_SKINNY_CASE
@@ -407,8 +434,8 @@ int launch_formats(const F8Params& p, uint32_t variant, int compute_units, hipSt
   // 6 / 7: the exact path (float8 widened to bfloat16 in registers, 32x32x16 bfloat16 MFMA) on
   // 256x256 / 128x128 tiles: what float32 and float16 outputs get.
   const bool big = uint64_t(p.m) * p.n >= (1ull << 20);
-  if (variant == 0 || variant == 12) {  // 12: the few-row kernel where it serves (what up to 64 rows get), else as planned
-    const int rc = launch_skinny<FA, FB>(p, compute_units, stream, err);
+  if (variant == 0 || (variant & 0xff) == 12) {  // 12: the few-row kernel where it serves (what up to 64 rows get), else as planned; bits 8-11: 16s of columns per workgroup
+    const int rc = launch_skinny<FA, FB>(p, compute_units, (variant >> 8) & 15u, stream, err);
     if (rc != -2) return rc;
     variant = 0;
   }
