@@ -206,10 +206,12 @@ def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030, prefill=False, phase=2):
                 shape=(n, bs), reference_layout_bytes=int(packed.numel()) * 4 + 4 * m * k + 4 * m * n, **timed(abi, fns, steps, warmup))
 
 
-def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False, variant=0):
+def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False, variant=0, decode=False):
     """_scaled_mm e4m3fn x e4m3fn -> bf16; A row-major, B column-major.  zero_operands: the same
     launch on all-zero matrices: the matrix cores' sustained rate depends on how many operand
-    bits toggle (the part is power limited), and this is the data-independent end of that range."""
+    bits toggle (the part is power limited), and this is the data-independent end of that range.
+    decode: few rows; the product is the weight stream, priced against HBM, over copies of the weights taken in
+    turn (one copy would stay in the last-level cache)."""
     import torch
     g = torch.Generator().manual_seed(seed)
     a = torch.randn(m, k, generator=g).clamp(-448, 448).to(torch.float8_e4m3fn)
@@ -226,6 +228,20 @@ def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False,
     out = abi.Buffer(m * n * 2)
     p = abi.F8Params(a=da.address, b=db.address, scale_a=dsa.address, scale_b=dsb.address, out=out.address, m=m, n=n,
                      k=k, lda=k, ldb=k, ldo=n, fmt_a=abi.E4M3, fmt_b=abi.E4M3, out_dtype=abi.BF16, rowwise=int(rowwise))
+    if decode:
+        copies = [db]
+        for _ in range(rotation(n * k) - 1):
+            b = abi.Buffer(n * k)
+            abi.check(abi.lib().vkt_copy_on_device(b.address, db.address, n * k))
+            copies.append(b)
+        fns = []
+        for c in copies:
+            q = abi.F8Params(a=da.address, b=c.address, scale_a=dsa.address, scale_b=dsb.address, out=out.address, m=m, n=n,
+                             k=k, lda=k, ldb=k, ldo=n, fmt_a=abi.E4M3, fmt_b=abi.E4M3, out_dtype=abi.BF16, rowwise=int(rowwise))
+            fns.append(Launch(abi, "fp8mm", [variant], q))
+        return dict(kind="hbm", work=n * k + m * k + 2 * m * n + 4 * (m + n if rowwise else 2), flops=2 * m * n * k, inputs=None,
+                    name=f"_scaled_mm e4m3fn {'rowwise' if rowwise else 'per-tensor'} M={m} K={k} N={n} -> bf16 (decode)",
+                    **timed(abi, fns, steps, warmup))
     fns = [Launch(abi, "fp8mm", [variant], p)]
     tm = time_steps(abi, fns, steps, warmup)
     return dict(kind="mfma", work=2 * m * n * k, wall_ms=tm[0], event_ms=tm[1], event_ms_median=tm.median, bytes=m * k + n * k + 2 * m * n,
@@ -408,6 +424,9 @@ OTHER = {
     "affine_quantize_256mi": lambda abi, s, w: wl_affine(abi, "quantize", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
     "affine_dequantize_256mi": lambda abi, s, w: wl_affine(abi, "dequantize", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
     "affine_fake_quant_256mi": lambda abi, s, w: wl_affine(abi, "fake_quant", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
+    "f8_decode_m1_k8192_n8192": lambda abi, s, w: wl_fp8(abi, 1, 8192, 8192, True, s, w, decode=True),  # (_scaled_mm at decode: few rows)
+    "f8_decode_m16_k8192_n28672": lambda abi, s, w: wl_fp8(abi, 16, 8192, 28672, True, s, w, decode=True),
+    "f8_decode_m64_k8192_n8192": lambda abi, s, w: wl_fp8(abi, 64, 8192, 8192, True, s, w, decode=True),
     "c4_fp8_8192_zero_operands": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 2, 30), max(w, 5), zero_operands=True),
 }
 # Ceilings measured in the same run (`ceilings` of the output line; also selectable by name): bare 16-byte loads of
