@@ -55,6 +55,24 @@ def test_gemm16_tile_variants(dtype, variant, m, k, n):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("variant", [0, 7, 7 | 1 << 8, 7 | 2 << 8, 7 | 4 << 8])
+@pytest.mark.parametrize("m,k,n", [(1, 512, 64), (7, 1032, 200), (16, 2048, 1000), (17, 520, 77), (33, 1536, 4100), (64, 2048, 4128), (50, 4096, 520)])
+def test_gemm16_few_rows(dtype, variant, m, k, n):
+    """Up to 64 rows in the Linear layout (x @ w.T at decode) run on the kernel whose workgroups own runs of columns
+    and whose waves split K: planned (what these shapes get) and asked for with 16, 32 and 64 columns per workgroup;
+    every row-tile count, k not a multiple of 128, short last workgroups and ragged vectors; alpha, beta and a bias;
+    a strided view of the rows."""
+    import _dev
+    a = bits((torch.randn(2 * m, k, generator=gen(23)) * 0.5).to(dtype))
+    w = bits((torch.randn(n, k, generator=gen(24)) * 0.5).to(dtype))  # B = w.T: rows of k
+    want, mag = oracle.gemm16(a[::2], w.T, ODT[dtype], want_mag=True)
+    close(_dev.gemm16(a[::2], w.T, ODT[dtype], variant=variant), want, mag, dtype)
+    bias = bits(torch.randn(n, generator=gen(25)).to(dtype))
+    want2, mag2 = oracle.gemm16(a[:m], w.T, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, want_mag=True)
+    close(_dev.gemm16(a[:m], w.T, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, variant=variant), want2, mag2, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
 def test_gemm16_stream_kernel(dtype):
     """The stream kernel (variant 6; what large products in the Linear layout get): more tiles than workgroups, so
     streams that run through two tiles; batches; a broadcast bias; rows and columns past the last whole tile.  Every

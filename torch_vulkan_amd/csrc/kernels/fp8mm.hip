@@ -33,7 +33,7 @@
 #include "kernels.h"
 #include "mma_stream.h"
 #include "mma_tile.h"
-#include "wave_tiles.h"
+#include "mma_skinny.h"
 
 namespace vkt {
 namespace {
@@ -205,203 +205,14 @@ __global__ __launch_bounds__(256) void fp8mm_generic(F8Params p) {
   store_out(p, uint64_t(m) * p.ldo + n, finish(p, acc, sa, sb, n, output_inv(p)));
 }
 
-// Up to 64 rows of A (decode at small batch): the product is the weight stream, N x K bytes read once, and the tile
-// kernels above, which give a workgroup 128 rows x 128 columns, cover a quarter of the machine at N = 8192.  Here a
-// workgroup owns a run of at most 16 NT columns (weight rows) and all rows of A, and its waves take the chunks of 256
-// values of k in turn (rotated against the other workgroups', so that rows a power of two apart are not all read at
-// the same offsets at the same time).  A wave's load instruction fetches 4 weight rows x 256 contiguous bytes, into
-// registers a chunk ahead, and from there into the wave's own LDS region, 16-byte pieces swizzled by the row, to come
-// back in the matrix core's operand shape: lane (c, g) holds 16 bytes of weight row c, two operands of
-// V_MFMA_F32_16X16X32_{FP8,BF8}_{FP8,BF8} (weights first, so a lane ends with 4 consecutive columns of one row), against
-// the same 16 values of k of activation row c, loaded from global memory (the rows of A come from L2).  The waves'
-// partial tiles meet in wave 0, which applies scales, bias and the cast.  (This instruction runs at half the rate of
-// the 128-deep one the tile kernels use: at 64 rows the matrix cores' share is ~4 us of a launch the weights hold to
-// 12 and more.)
-template <int FA, int FB>
-__device__ __forceinline__ V4F mfma_f8x32(long w, long a, const V4F& acc) {
-  // first operand: weights (format FB), second: activations (format FA); 0 = e4m3fn, 1 = e5m2
-  if constexpr (FB == 0 && FA == 0) return __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w, a, acc, 0, 0, 0);
-  else if constexpr (FB == 0 && FA == 1) return __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(w, a, acc, 0, 0, 0);
-  else if constexpr (FB == 1 && FA == 0) return __builtin_amdgcn_mfma_f32_16x16x32_bf8_fp8(w, a, acc, 0, 0, 0);
-  else return __builtin_amdgcn_mfma_f32_16x16x32_bf8_bf8(w, a, acc, 0, 0, 0);
-}
-
-// WIDE (float32 and float16 outputs): both operands are widened exactly to bfloat16 in registers (two values per
-// conversion instruction) and multiplied by V_MFMA_F32_16X16X32_BF16, which adds at float32 precision.
-template <int F>
-__device__ __forceinline__ V8BF widen8(uint32_t lo, uint32_t hi) {
-  const V2BF p0 = widen_pair<F, false>(int(lo)), p1 = widen_pair<F, true>(int(lo));
-  const V2BF p2 = widen_pair<F, false>(int(hi)), p3 = widen_pair<F, true>(int(hi));
-  return V8BF{p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
-}
-
-template <int MT, int NT, int WAVES, int FA, int FB, bool WIDE>
-__global__ __launch_bounds__(WAVES * 64) void fp8mm_skinny(F8Problem p, uint32_t cols_per_wg) {
-  constexpr uint32_t TILE = 16 * 256, REGION = NT * TILE;  // bytes of LDS per tile of 16 weight rows, per wave
-  extern __shared__ __attribute__((aligned(16))) uint8_t staged[];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
-  uint8_t* const mine = staged + uint32_t(wave) * REGION;
-  const uint32_t count = (p.k + 255) / 256;
-  const uint32_t n0 = blockIdx.x * cols_per_wg, n_end = n0 + cols_per_wg < p.n ? n0 + cols_per_wg : p.n;
-  // loads: instruction i of tile t fetches rows 4 i .. 4 i + 3; this lane row 4 i + (lane / 16), slot lane % 16
-  uint64_t wsrc[NT][4];
-  uint32_t wk[4];  // byte offset within the chunk of the 16 bytes this lane fetches
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const uint32_t row = 4 * i + g;
-    wk[i] = ((uint32_t(c) ^ row) & 15u) * 16;
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      const uint32_t n = n0 + 16 * t + row < n_end ? n0 + 16 * t + row : n_end - 1;  // (rows past the end: the last one again, from the caches)
-      wsrc[t][i] = p.b + uint64_t(n) * p.ldb;
-    }
-  }
-  uint64_t arow[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const uint32_t m = uint32_t(16 * mt + c) < p.m ? 16 * mt + c : p.m - 1;
-    arow[mt] = p.a + uint64_t(m) * p.lda + 16 * g;
-  }
-  V4F acc[MT][NT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-    for (int t = 0; t < NT; ++t) acc[mt][t] = V4F{0.0f, 0.0f, 0.0f, 0.0f};
-
-  const U4 zero = {0, 0, 0, 0};
-  U4 wr[NT][4];
-  auto request = [&](uint32_t q) {
-    const uint32_t k0 = q * 256;
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        // (bytes past k are fetched from the row's start instead: their activations are zeros below, and a NaN among
-        // them is one of the row's own values)
-        wr[t][i] = ldg_stream<U4>(wsrc[t][i] + (k0 + wk[i] < p.k ? k0 + wk[i] : 0u));
-      }
-  };
-  const uint32_t rot = (blockIdx.x * 5u) % count;
-  auto chunk_at = [&](uint32_t i) { return (i + rot) % count; };  // the i-th chunk this workgroup works on
-  if (uint32_t(wave) < count) request(chunk_at(wave));
-  for (uint32_t i = wave; i < count; i += WAVES) {
-    const uint32_t k0 = chunk_at(i) * 256;
-    U4 a[MT][4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const bool inside = k0 + 64 * j + 16 * g < p.k;  // (k is a multiple of 16)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const bool real = inside && uint32_t(16 * mt + c) < p.m;  // (rows past m are zeros, not loads)
-        a[mt][j] = real ? ldg<U4>(arow[mt] + k0 + 64 * j) : zero;
-      }
-    }
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-      for (int i2 = 0; i2 < 4; ++i2) *reinterpret_cast<U4*>(mine + (t * 16 + 4 * i2) * 256 + lane * 16) = wr[t][i2];
-    if (i + WAVES < count) request(chunk_at(i + WAVES));
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      V8BF wide_a[WIDE ? MT : 1][2];
-      if constexpr (WIDE) {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) wide_a[mt][0] = widen8<FA>(a[mt][j][0], a[mt][j][1]), wide_a[mt][1] = widen8<FA>(a[mt][j][2], a[mt][j][3]);
-      }
-#pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        // (a wave's LDS operations execute in order: these reads see the writes above)
-        const U4 wv = *reinterpret_cast<const U4*>(mine + (t * 16 + c) * 256 + (((4 * j + g) ^ c) & 15) * 16);
-        if constexpr (WIDE) {
-          const V8BF w0 = widen8<FB>(wv[0], wv[1]), w1 = widen8<FB>(wv[2], wv[3]);
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, wide_a[mt][0], acc[mt][t], 0, 0, 0);
-            acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, wide_a[mt][1], acc[mt][t], 0, 0, 0);
-          }
-        } else {
-          const long w0 = long(uint64_t(wv[0]) | uint64_t(wv[1]) << 32), w1 = long(uint64_t(wv[2]) | uint64_t(wv[3]) << 32);
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            const long a0 = long(uint64_t(a[mt][j][0]) | uint64_t(a[mt][j][1]) << 32), a1 = long(uint64_t(a[mt][j][2]) | uint64_t(a[mt][j][3]) << 32);
-            acc[mt][t] = mfma_f8x32<FA, FB>(w0, a0, acc[mt][t]);
-            acc[mt][t] = mfma_f8x32<FA, FB>(w1, a1, acc[mt][t]);
-          }
-        }
-      }
-    }
-  }
-
-  // the waves' partial tiles meet in wave 0 (through the staging memory, once every wave is done with it)
-  __syncthreads();
-  add_wave_tiles<MT, NT, WAVES>(acc, reinterpret_cast<V4F*>(staged), wave, lane);
-  if (wave != 0) return;
-  // lane (c, g) holds, per tile (mt, t), row 16 mt + c, columns n0 + 16 t + 4 g .. + 3
-  const F8Problem::Whole whole = p.whole();
-#pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const uint32_t col = n0 + 16 * t + 4 * g;
-    if (col >= n_end) continue;
-    const F8Problem::Columns cs = p.columns(0, col, whole);
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const uint32_t row = 16 * mt + c;
-      if (row >= p.m) continue;
-      p.for_output_type(col + 3 < p.n, whole, [&](auto dt) { p.template store<decltype(dt)::value>(0, row, col, acc[mt][t], cs, whole); });
-    }
-  }
-}
-
-template <int MT, int NT, int WAVES, int FA, int FB, bool WIDE>
-int launch_skinny_one(const F8Problem& p, uint32_t cols, hipStream_t stream, std::string* err) {
-  auto kernel = fp8mm_skinny<MT, NT, WAVES, FA, FB, WIDE>;
-  constexpr uint32_t stage_bytes = WAVES * NT * 16 * 256, part_bytes = kPartSlots<MT, NT, WAVES> * MT * NT * 1024;
-  constexpr uint32_t lds = stage_bytes > part_bytes ? stage_bytes : part_bytes;
-  static bool configured = false;  // guarded by the runtime's stream mutex
-  if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
-      (void)hipGetLastError();
-      *err = "fp8mm: cannot reserve " + std::to_string(lds) + " bytes of LDS";
-      return -1;
-    }
-    configured = true;
-  }
-  hipLaunchKernelGGL(kernel, dim3((p.n + cols - 1) / cols), dim3(WAVES * 64), lds, stream, p, cols);
-  return 0;
-}
-
-// The few-row kernel where it serves: up to 64 rows, rows of k of 1024 bytes and more; bfloat16 and float8 outputs on
-// the fp8 matrix-core instruction, float32 and float16 outputs on exactly widened operands (the precision rule of the
-// tile kernels).  16, 32 or 64 columns per workgroup, whichever leaves the busiest
-// compute unit the fewest bytes to take in, (workgroups on it) x (columns + rows) x K: every workgroup reads all rows
-// of A beside its weights.  -2: not this kernel's problem.
+// The few-row kernel (mma_skinny.h) where it serves; bfloat16 and float8 outputs on the fp8 matrix-core instruction,
+// float32 and float16 outputs on exactly widened operands (the precision rule of the tile kernels).  -2: not served.
 template <int FA, int FB>
 int launch_skinny(const F8Params& p0, int compute_units, uint32_t forced_nt, hipStream_t stream, std::string* err) {
-  const bool wide = p0.out_dtype == VKT_F32 || p0.out_dtype == VKT_F16;
-  if (p0.m > 64 || p0.k < 1024 || p0.n < 64) return -2;
   F8Problem p;
   static_cast<F8Params&>(p) = p0;
-  const uint32_t cus = uint32_t(compute_units);
-  int nt = 1;
-  float best = 1e30f;
-  for (int t = 1; t <= 4; t *= 2) {
-    const uint32_t cols = staged_cols(p.n, t, cus), workgroups = (p.n + cols - 1) / cols;
-    const float cost = float((workgroups + cus - 1) / cus) * float(cols + p.m) * float(p.k) * (t == 4 && workgroups <= cus ? 1.25f : 1.0f);
-    if (cost < best) best = cost, nt = t;
-  }
-  const int mt = p.m <= 16 ? 1 : p.m <= 32 ? 2 : 4;
-  if (forced_nt) nt = int(forced_nt);
-  if (mt == 1 && nt == 4) nt = 2;  // (the shapes that are built)
-  if (mt == 4 && nt == 1) nt = 2;
-  const uint32_t cols = staged_cols(p.n, nt, cus);
-#define VKT_SKINNY_CASE(MT_, NT_, W_)                                                                         \
-  if (mt == MT_ && nt == NT_)                                                                                \
-    return wide ? launch_skinny_one<MT_, NT_, W_, FA, FB, true>(p, cols, stream, err) \
-                : launch_skinny_one<MT_, NT_, W_, FA, FB, false>(p, cols, stream, err);
-  VKT_SKINNY_CASE(1, 1, 8) VKT_SKINNY_CASE(1, 2, 8) VKT_SKINNY_CASE(2, 1, 8) VKT_SKINNY_CASE(2, 2, 8) VKT_SKINNY_CASE(2, 4, 4)
-  VKT_SKINNY_CASE(4, 2, 8) VKT_SKINNY_CASE(4, 4, 4)
-#undef VKT_SKINNY_CASE
-  return -2;
+  if (p0.out_dtype == VKT_F32 || p0.out_dtype == VKT_F16) return launch_mma_skinny<FA, FB, kMathFp8Wide>(p, compute_units, forced_nt, stream, err, "fp8mm");
+  return launch_mma_skinny<FA, FB, kMathFp8>(p, compute_units, forced_nt, stream, err, "fp8mm");
 }
 
 template <int WAVES_M, int WAVES_N, int TM, int TN, int FA, int FB, bool MF32 = false, bool DIRECT = false, bool WIDE = false>

@@ -15,6 +15,7 @@
 #include "kernels.h"
 #include "mma_stream.h"
 #include "mma_tile.h"
+#include "mma_skinny.h"
 
 namespace vkt {
 namespace {
@@ -119,6 +120,16 @@ int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t
   g.c = p.c, g.cin = use_cin ? p.cin : 0;
   g.alpha = bits_f32_host(uint32_t(p.alpha)), g.beta = bits_f32_host(uint32_t(p.beta));
   g.c_sm = p.c_sm, g.c_sb = p.c_sb, g.cin_sm = p.cin_sm, g.cin_sn = p.cin_sn, g.cin_sb = p.cin_sb;
+  // Up to 64 rows against weights in rows of k (x @ w.T at decode): the few-row kernel (mma_skinny.h), whose
+  // workgroups own runs of columns and whose waves split K: the product is the weight stream, and 128 x 128 tiles put
+  // 64 workgroups on the machine at N = 8192 (variant 7 asks for it; bits 8-11: 16s of columns per workgroup).
+  if constexpr (!TRA && !TRB) {
+    if ((variant == 0 || (variant & 0xff) == 7) && batch == 1) {
+      const int rc = launch_mma_skinny<0, 0, MATH>(g, mc.compute_units, (variant >> 8) & 15u, stream, err, "gemmcm");
+      if (rc != -2) return rc;
+    }
+  }
+  if ((variant & 0xff) == 7) variant = 0;
   const bool direct_ok = g.k % BK == 0;
   // variant 0: planned; 1: 128x128 tiles; 2: 256x128; 3: 256x256 with direct loads; 4: 128x128 with direct loads;
   // 5: 256x256 with direct loads over 8 waves; 6: the stream kernel (mma_stream.h; else 3)
