@@ -250,7 +250,7 @@ def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False,
                      + (" (all-zero operands)" if zero_operands else ""))
 
 
-def wl_gemm16(abi, m, k, n, steps, warmup, seed=1090, layout="nt"):
+def wl_gemm16(abi, m, k, n, steps, warmup, seed=1090, layout="nt", decode=False):
     """bfloat16 mm, x [m,k] @ w -> [m,n]: the unquantised product next to the path.  layout "nt": w stored
     [n,k] (x @ w.T, the Linear layout); "nn": w stored [k,n] (x @ w); "tn": x stored [k,m] as well (x.t() @ w)."""
     import torch
@@ -264,6 +264,19 @@ def wl_gemm16(abi, m, k, n, steps, warmup, seed=1090, layout="nt"):
         p.b_sk, p.b_sn = n, 1
     if layout == "tn":
         p.a_sm, p.a_sk = 1, m
+    if decode:  # few rows: the product is the weight stream, over copies of the weights taken in turn, priced against HBM
+        copies = [dw]
+        for _ in range(rotation(2 * n * k) - 1):
+            b = abi.Buffer(2 * n * k)
+            abi.check(abi.lib().vkt_copy_on_device(b.address, dw.address, 2 * n * k))
+            copies.append(b)
+        fns = []
+        for c in copies:
+            q = abi.GemmParams.from_buffer_copy(p)
+            q.b = c.address
+            fns.append(Launch(abi, "gemmcm_bf16", [0], q))
+        return dict(kind="hbm", work=2 * (n * k + m * k + m * n), flops=2 * m * n * k, inputs=None,
+                    name=f"mm bf16 M={m} K={k} N={n} ({layout}, decode)", **timed(abi, fns, steps, warmup))
     tm = time_steps(abi, [Launch(abi, "gemmcm_bf16", [0], p)], steps, warmup)
     return dict(kind="mfma", peak=BF16_PEAK_TFLOPS, metric="bf16 mm TFLOP/s (% of MFMA peak)", work=2 * m * n * k, wall_ms=tm[0], event_ms=tm[1], event_ms_median=tm.median,
                 bytes=2 * (m * k + n * k + m * n), inputs=None, copies=1, name=f"mm bf16 M={m} K={k} N={n} ({layout}: " + {"nt": "x @ w.T, the Linear layout", "nn": "x @ w", "tn": "x.T @ w"}[layout] + ")")
@@ -400,6 +413,15 @@ BASELINE = {
     "c3_int4_m1": lambda abi, s, w: wl_q4(abi, 1, 4096, 11008, 32, s, w),
     "c4_fp8_8192": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 2, 30), max(w, 5)),
 }
+# The same operators at decode off the BASELINE grid (in `extra` of the default run, after the BASELINE configurations):
+# few rows of _scaled_mm, float32 rows and 16 rows of _weight_int8pack_mm, and the unquantised Linear beside them.
+DECODE = {
+    "f8_decode_m1_k8192_n8192": lambda abi, s, w: wl_fp8(abi, 1, 8192, 8192, True, s, w, decode=True),
+    "f8_decode_m16_k8192_n28672": lambda abi, s, w: wl_fp8(abi, 16, 8192, 28672, True, s, w, decode=True),
+    "q8_f32_m8_k4096_n14336": lambda abi, s, w: wl_q8(abi, 8, 4096, 14336, abi.F32, s, w, seed=1150),
+    "q8_m16_k8192_n8192": lambda abi, s, w: wl_q8(abi, 16, 8192, 8192, abi.BF16, s, w, seed=1160),
+    "mm_bf16_decode_m8_k8192_n8192": lambda abi, s, w: wl_gemm16(abi, 8, 8192, 8192, s, w, decode=True),
+}
 # Beside the BASELINE configurations (--all, or by name): many rows of the same operators, the steps either side of
 # the path, the planner off the Llama grid, config 4's launch on all-zero operands.
 OTHER = {
@@ -424,8 +446,6 @@ OTHER = {
     "affine_quantize_256mi": lambda abi, s, w: wl_affine(abi, "quantize", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
     "affine_dequantize_256mi": lambda abi, s, w: wl_affine(abi, "dequantize", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
     "affine_fake_quant_256mi": lambda abi, s, w: wl_affine(abi, "fake_quant", 1 << 28, max(s // 10, 5), max(w // 4, 3)),
-    "f8_decode_m1_k8192_n8192": lambda abi, s, w: wl_fp8(abi, 1, 8192, 8192, True, s, w, decode=True),  # (_scaled_mm at decode: few rows)
-    "f8_decode_m16_k8192_n28672": lambda abi, s, w: wl_fp8(abi, 16, 8192, 28672, True, s, w, decode=True),
     "f8_decode_m64_k8192_n8192": lambda abi, s, w: wl_fp8(abi, 64, 8192, 8192, True, s, w, decode=True),
     "c4_fp8_8192_zero_operands": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 2, 30), max(w, 5), zero_operands=True),
 }
@@ -446,7 +466,7 @@ CALIBRATION = {
 }
 # configurations whose extra entry also carries the op's cost through PyTorch's dispatcher (the headline always does)
 DISPATCHER_TOO = ("c3_int4_m1", "c3_int4_m32", "c4_fp8_8192", "c1_f32_m1_k4096_n4096")
-WORKLOADS = {**BASELINE, **OTHER}
+WORKLOADS = {**BASELINE, **DECODE, **OTHER}
 HEADLINE = "c2_m1_k4096_n14336"
 
 
@@ -687,7 +707,7 @@ def main():
             del rr
         line["ceilings"] = ceilings
         extra = []
-        for name, fn in ({**OTHER, **BASELINE} if args.all else BASELINE).items():
+        for name, fn in ({**OTHER, **BASELINE, **DECODE} if args.all else {**BASELINE, **DECODE}).items():
             if name == args.workload:
                 continue
             rr = fn(abi, args.steps, args.warmup)
