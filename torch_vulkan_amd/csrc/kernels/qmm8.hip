@@ -1581,7 +1581,11 @@ int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipSt
     // From 3 rows on the matrix cores win: the GEMV kernels convert every weight and multiply it once per row on
     // the vector units (measured at K = 4096, N = 14336: 10.5, 16.4, 23.0, 23.4 us for 1 to 4 rows; the matrix
     // cores take 16 us for up to 8).  variant bit 17 forces the GEMV kernels (tests, tuning).
-    if (p0.m > 2 && !((variant >> 17) & 1)) {
+    // (two rows against 32 column groups and more per compute unit pair go there too: 3-6 % ahead of the vector units,
+    //  K = 4096, N = 14336: 13.5 against 13.9 us, N = 128256: 86 against 92; with fewer columns 9 % behind.  Bit 18: the
+    //  staged matrix-core kernel for one and two rows whatever the shape.)
+    const bool two_rows = p0.m == 2 && variant == 0 && p0.k >= 2048 && (p0.n + 15) / 16 >= 2u * uint32_t(mc.compute_units);
+    if ((p0.m > 2 || two_rows || ((variant >> 18) & 1)) && !((variant >> 17) & 1)) {
       // 3 to 8 short rows against many columns: the wave-per-column-group kernel where it pays (variant bit 23 keeps the kernels below)
       // (bits 8-15 with bits 0-7 clear ask for it whatever the size: tests, tuning)
       const bool asked = !(variant & 0xff) && ((variant >> 8) & 0xff);
