@@ -25,6 +25,10 @@ def _q8_shapes():
             out.append((m, k, n))
     # enough 128 x 128 tiles for the widened-weights product, and one short of it
     out += [(256, 512, 128 * 128), (256, 512, 128 * 127), (192, 256, 128 * 170)]
+    # two rows on both sides of 32 column groups per pair of compute units; 9 to 32 rows where 16, 32 and 64 columns per
+    # workgroup are the plan, and 17 to 32 where the tile kernel is; float32 rows on the three-plane path and off it
+    out += [(2, 2048, 8192), (2, 2048, 8176), (9, 2048, 4096), (12, 2048, 8200), (16, 2304, 14336), (24, 4096, 2048), (24, 7168, 1024),
+            (32, 2048, 6400), (3, 1024, 2048), (4, 4096, 1024), (8, 2048, 4100), (16, 1024, 8192)]
     return out
 
 
