@@ -94,7 +94,9 @@ def test_scaled_mm_tile_edges(m, k, n, variant, rowwise):
     (17, 1040, 77, torch.bfloat16, True), (32, 3072, 4100, torch.bfloat16, False), (33, 1024, 130, torch.float8_e5m2, False),
     (64, 4096, 4128, torch.bfloat16, True), (50, 8192, 520, torch.bfloat16, True),
     # float32 and float16 outputs: the same kernel on operands widened exactly to bfloat16 (no window in the bound)
-    (5, 2064, 300, torch.float32, True), (40, 1024, 64, torch.float16, False), (16, 4096, 4100, torch.float32, False)])
+    (5, 2064, 300, torch.float32, True), (40, 1024, 64, torch.float16, False), (16, 4096, 4100, torch.float32, False),
+    # few columns against long rows: 8 columns and 16 waves per workgroup
+    (4, 8192, 264, torch.bfloat16, True), (9, 16384, 100, torch.float32, False)])
 def test_scaled_mm_few_rows(fa, fb, m, k, n, out_dtype, rowwise):
     """Up to 64 rows with bfloat16 or float8 outputs run on the kernel whose workgroups own runs of columns and whose
     waves split K (planned, which is what these shapes get, and asked for as variant 12): every row-tile count, rows of

@@ -56,7 +56,8 @@ def test_gemm16_tile_variants(dtype, variant, m, k, n):
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
 @pytest.mark.parametrize("variant", [0, 7, 7 | 1 << 8, 7 | 2 << 8, 7 | 4 << 8])
-@pytest.mark.parametrize("m,k,n", [(1, 512, 64), (7, 1032, 200), (16, 2048, 1000), (17, 520, 77), (33, 1536, 4100), (64, 2048, 4128), (50, 4096, 520)])
+@pytest.mark.parametrize("m,k,n", [(1, 512, 64), (7, 1032, 200), (16, 2048, 1000), (17, 520, 77), (33, 1536, 4100), (64, 2048, 4128), (50, 4096, 520),
+                                   (3, 4096, 264), (12, 8192, 100)])  # (few columns against long rows: 8 columns and 16 waves per workgroup)
 def test_gemm16_few_rows(dtype, variant, m, k, n):
     """Up to 64 rows in the Linear layout (x @ w.T at decode) run on the kernel whose workgroups own runs of columns
     and whose waves split K: planned (what these shapes get) and asked for with 16, 32 and 64 columns per workgroup;

@@ -209,6 +209,10 @@ int launch_mma_skinny(const Problem& p, int compute_units, uint32_t forced_nt, h
   if (mt == 1 && nt == 4) nt = 2;  // (the shapes that are built)
   if (mt == 4 && nt == 1) nt = 2;
   const uint32_t cols = staged_cols(p.n, nt, cus);
+  // few columns against long rows: 16 waves per workgroup where half of the compute units or more would have none (a
+  // workgroup's waves take the chunks of k in turn: twice the waves, half the turns)
+  if (mt == 1 && nt == 1 && (p.n + cols - 1) / cols * 2 <= cus && p.k >= 32 * 256)
+    return launch_skinny_one<1, 1, 16, FA, FB, MATH>(p, cols, stream, err, name);
 #define VKT_SKINNY_CASE(MT_, NT_, W_) \
   if (mt == MT_ && nt == NT_) return launch_skinny_one<MT_, NT_, W_, FA, FB, MATH>(p, cols, stream, err, name);
   VKT_SKINNY_CASE(1, 1, 8) VKT_SKINNY_CASE(1, 2, 8) VKT_SKINNY_CASE(2, 1, 8) VKT_SKINNY_CASE(2, 2, 8) VKT_SKINNY_CASE(2, 4, 4)

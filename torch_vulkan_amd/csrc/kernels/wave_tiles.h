@@ -49,8 +49,10 @@ __device__ __forceinline__ void add_wave_tiles(V4F (&acc)[MT][NT], V4F* part, in
 // out over a whole number of workgroups per compute unit (a multiple of 4, at least 8).
 inline uint32_t staged_cols(uint32_t n, int nt, uint32_t cus) {
   const uint32_t cols = 16 * nt, wgs = (n + cols - 1) / cols, even = (wgs + cus - 1) / cus * cus;
-  const uint32_t fewer = ((n + even - 1) / even + 3) / 4 * 4;
-  return fewer >= 8 && fewer < cols ? fewer : cols;
+  // (not below 8: half of a matrix-core tile's columns are then zeros, and fewer columns than compute units x 8
+  // leave some units without a workgroup, which costs less than workgroups of 16 on a quarter of them)
+  const uint32_t share = ((n + even - 1) / even + 3) / 4 * 4, fewer = share < 8 ? 8 : share;
+  return fewer < cols ? fewer : cols;
 }
 
 }  // namespace vkt
