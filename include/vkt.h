@@ -272,7 +272,8 @@ typedef struct MinMaxParams {
  * (quant.cpp:279-300 fused into one kernel).  A: fp8 [m,k] row-major (lda bytes);
  * B: fp8, column-major, i.e. [n,k] rows ldb bytes apart.  104 bytes.  An optional entry overrides the launcher's
  * choice of kernel (tests, tuning; 0 or absent: planned): 1-9 tile shapes, 11 the stream kernel, 12 the few-row kernel
- * (up to 64 rows; bits 8-11: 16s of columns per workgroup), 255 one thread per output. */
+ * (up to 64 rows; bits 8-11: 16s of columns per workgroup), 13 the vector-unit kernel (up to 4 rows), 255 one thread per
+ * output. */
 typedef struct F8Params {
   uint64_t a, b, scale_a, scale_b, bias, scale_result, out; /* bias / scale_result may be 0 */
   uint32_t m, n, k;

@@ -28,6 +28,8 @@ HW_WINDOW = 2.0**-13
 def on_matrix_cores(odt, variant, k):
     if variant in (6, 7, 255) or k % 16:
         return False
+    if variant == 13:  # the vector-unit kernel for up to four rows: float32 sums whatever the output type
+        return False
     return variant in (1, 2, 3, 4, 5, 8, 11, 12) or odt in (oracle.BF16, oracle.E4M3, oracle.E5M2)
 
 
@@ -105,6 +107,21 @@ def test_scaled_mm_few_rows(fa, fb, m, k, n, out_dtype, rowwise):
     sr = 2.0 if out_dtype in (torch.float8_e4m3fn, torch.float8_e5m2) else None
     for variant in (0, 12) if sr or bias_dtype else (0,):
         run_case(m, k, n, fa, fb, out_dtype, rowwise, bias_dtype, sr, variant=variant, seed=m + n)
+
+
+@pytest.mark.parametrize("fa,fb", [(FLOAT8[0], FLOAT8[0]), (FLOAT8[1], FLOAT8[0]), (FLOAT8[0], FLOAT8[1]), (FLOAT8[1], FLOAT8[1])])
+@pytest.mark.parametrize("m,k,n,out_dtype,rowwise", [
+    (1, 1024, 64, torch.bfloat16, False), (1, 4096, 1001, torch.bfloat16, True), (2, 2064, 200, torch.float8_e4m3fn, True),
+    (2, 8192, 77, torch.float32, True), (1, 16384, 30, torch.float16, False), (3, 1040, 130, torch.bfloat16, True),
+    (4, 4096, 520, torch.float8_e5m2, False), (4, 1024, 9, torch.float32, True)])
+def test_scaled_mm_one_to_four_rows_on_vector_units(fa, fb, m, k, n, out_dtype, rowwise):
+    """One and two rows (and three and four against few columns) run on the vector-unit kernel: both operands widened
+    exactly to bfloat16, two-element dot products into float32 sums.  Asked for as variant 13 and as planned; every
+    split of K over a workgroup's waves, column counts that leave the last workgroup short, every output type."""
+    bias_dtype = torch.bfloat16 if out_dtype == torch.bfloat16 else None
+    sr = 2.0 if out_dtype in (torch.float8_e4m3fn, torch.float8_e5m2) else None
+    for variant in (13, 0):
+        run_case(m, k, n, fa, fb, out_dtype, rowwise, bias_dtype, sr, variant=variant, seed=3 * m + n)
 
 
 def test_scaled_mm_fp8_output_saturation_and_nan():

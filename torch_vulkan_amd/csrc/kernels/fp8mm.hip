@@ -205,6 +205,116 @@ __global__ __launch_bounds__(256) void fp8mm_generic(F8Params p) {
   store_out(p, uint64_t(m) * p.ldo + n, finish(p, acc, sa, sb, n, output_inv(p)));
 }
 
+// One and two rows of A on the vector units (the shape of the int8 op's one-row kernel): a wave streams COLS weight
+// rows with 16-byte non-temporal loads, KSPLIT waves of the workgroup share a row's k; both operands are widened
+// exactly to bfloat16 (two values per conversion instruction) and multiplied by two-element dot products into float32
+// sums (products of two float8 values are exact in float32), so every output type is served at float32 precision.
+// Many small workgroups have the whole weight stream in flight at once, and a workgroup may own as few as 2 columns:
+// few columns against long rows keep the machine busy where the matrix-core kernel's 8 to 16 columns per workgroup do
+// not (K = 8192, N = 1024: 4.5 against 6.8 us).
+template <int F>
+__device__ __forceinline__ void widen16_pairs(const U4& v, uint32_t (&out)[8]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    out[2 * i] = __builtin_bit_cast(uint32_t, widen_pair<F, false>(int(v[i])));
+    out[2 * i + 1] = __builtin_bit_cast(uint32_t, widen_pair<F, true>(int(v[i])));
+  }
+}
+
+template <int ROWS, int COLS, int KSPLIT, int FA, int FB>
+__global__ __launch_bounds__(256) void fp8mm_gemv(F8Params p) {
+  constexpr int WAVES = 4, GROUPS = WAVES / KSPLIT;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int grp = wave / KSPLIT, ks = wave % KSPLIT;
+  const uint32_t n0 = (blockIdx.x * GROUPS + grp) * COLS;
+  float acc[ROWS][COLS];
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) acc[r][c] = 0.0f;
+  // (clamped: the tail group re-reads the last row, masked at the store)
+  uint64_t brow[COLS], arow[ROWS];
+#pragma unroll
+  for (int c = 0; c < COLS; ++c) brow[c] = p.b + uint64_t(n0 + c < p.n ? n0 + c : p.n - 1) * p.ldb;
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) arow[r] = p.a + uint64_t(uint32_t(r) < p.m ? uint32_t(r) : p.m - 1) * p.lda;
+
+  for (uint32_t k = (ks * 64 + lane) * 16; k < p.k; k += 1024 * KSPLIT) {  // (k is a multiple of 16)
+    U4 wv[COLS], av[ROWS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) wv[c] = ldg_stream<U4>(brow[c] + k);
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) av[r] = ldg<U4>(arow[r] + k);
+    uint32_t w[COLS][8], a[ROWS][8];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) widen16_pairs<FB>(wv[c], w[c]);
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) widen16_pairs<FA>(av[r], a[r]);
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+      for (int c = 0; c < COLS; ++c)
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          acc[r][c] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(V2BF, a[r][i]), __builtin_bit_cast(V2BF, w[c][i]), acc[r][c], false);
+  }
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) acc[r][c] = wave_sum(acc[r][c]);
+
+  __shared__ float part[WAVES][ROWS * COLS];
+  if constexpr (KSPLIT > 1) {
+    if (lane == 0) {
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) part[wave][r * COLS + c] = acc[r][c];
+    }
+    __syncthreads();
+    if (ks != 0) return;
+  }
+  // lane (r, c) of the group's first wave finishes output (r, n0 + c)
+  if (lane < ROWS * COLS) {
+    const int r = lane / COLS, c = lane % COLS;
+    float sum = 0.0f;
+#pragma unroll
+    for (int rr = 0; rr < ROWS; ++rr)
+#pragma unroll
+      for (int cc = 0; cc < COLS; ++cc)
+        if (rr == r && cc == c) sum = acc[rr][cc];  // (no dynamic register indexing)
+    if constexpr (KSPLIT > 1) {
+      sum = part[wave][lane];
+#pragma unroll
+      for (int s = 1; s < KSPLIT; ++s) sum += part[wave + s][lane];
+    }
+    const uint32_t n = n0 + c;
+    if (uint32_t(r) < p.m && n < p.n) {
+      const float sa = ldg<float>(p.scale_a + (p.rowwise ? 4ull * r : 0)), sb = ldg<float>(p.scale_b + (p.rowwise ? 4ull * n : 0));
+      store_out(p, uint64_t(r) * p.ldo + n, finish(p, sum, sa, sb, n, output_inv(p)));
+    }
+  }
+}
+
+// -2: not this kernel's problem (more than four rows, short rows).
+// One and two rows always; three and four where the matrix-core kernel would have fewer workgroups than half the
+// machine's compute units (us at 3 rows, this kernel / that one: K = 8192, N = 1024: 4.8 / 7.0; K = 16384, N = 512:
+// 8.3 / 9.4; but K = 4096, N = 14336: 16.9 / 12.4); forced: whatever the column count.
+template <int FA, int FB>
+int launch_gemv(const F8Params& p, int compute_units, bool forced, hipStream_t stream) {
+  if (p.m > 4 || p.k < 1024) return -2;
+  if (p.m > 2 && !forced && p.n > 8u * uint32_t(compute_units)) return -2;
+  const int rows = p.m <= 1 ? 1 : p.m <= 2 ? 2 : 4;
+  const int ksplit = p.k >= 4096 ? (p.k <= 8192 ? 4 : 2) : (p.k >= 2048 ? 2 : 1);  // (the int8 op's rule: a wave keeps one full 1 KiB load per column)
+  const dim3 grid((p.n + 2 * (4 / ksplit) - 1) / (2 * (4 / ksplit)));
+#define VKT_F8_GEMV_CASE(R_, KS_) \
+  if (rows == R_ && ksplit == KS_) { hipLaunchKernelGGL((fp8mm_gemv<R_, 2, KS_, FA, FB>), grid, dim3(256), 0, stream, p); return 0; }
+  VKT_F8_GEMV_CASE(1, 1) VKT_F8_GEMV_CASE(1, 2) VKT_F8_GEMV_CASE(1, 4) VKT_F8_GEMV_CASE(2, 1) VKT_F8_GEMV_CASE(2, 2) VKT_F8_GEMV_CASE(2, 4)
+  VKT_F8_GEMV_CASE(4, 1) VKT_F8_GEMV_CASE(4, 2) VKT_F8_GEMV_CASE(4, 4)
+#undef VKT_F8_GEMV_CASE
+  return -2;
+}
+
 // The few-row kernel (mma_skinny.h) where it serves; bfloat16 and float8 outputs on the fp8 matrix-core instruction,
 // float32 and float16 outputs on exactly widened operands (the precision rule of the tile kernels).  -2: not served.
 template <int FA, int FB>
@@ -245,6 +355,11 @@ int launch_formats(const F8Params& p, uint32_t variant, int compute_units, hipSt
   // 6 / 7: the exact path (float8 widened to bfloat16 in registers, 32x32x16 bfloat16 MFMA) on
   // 256x256 / 128x128 tiles: what float32 and float16 outputs get.
   const bool big = uint64_t(p.m) * p.n >= (1ull << 20);
+  if (variant == 0 || variant == 13) {  // 13: the vector-unit kernel for one and two rows where it serves (what they get), else as planned
+    const int rc = launch_gemv<FA, FB>(p, compute_units, variant == 13, stream);
+    if (rc != -2) return rc;
+    variant = 0;
+  }
   if (variant == 0 || (variant & 0xff) == 12) {  // 12: the few-row kernel where it serves (what up to 64 rows get), else as planned; bits 8-11: 16s of columns per workgroup
     const int rc = launch_skinny<FA, FB>(p, compute_units, (variant >> 8) & 15u, stream, err);
     if (rc != -2) return rc;
