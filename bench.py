@@ -250,7 +250,7 @@ def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False,
                      + (" (all-zero operands)" if zero_operands else ""))
 
 
-def wl_gemm16(abi, m, k, n, steps, warmup, seed=1090, layout="nt", decode=False):
+def wl_gemm16(abi, m, k, n, steps, warmup, seed=1090, layout="nt", decode=False, variant=0):
     """bfloat16 mm, x [m,k] @ w -> [m,n]: the unquantised product next to the path.  layout "nt": w stored
     [n,k] (x @ w.T, the Linear layout); "nn": w stored [k,n] (x @ w); "tn": x stored [k,m] as well (x.t() @ w)."""
     import torch
@@ -274,7 +274,7 @@ def wl_gemm16(abi, m, k, n, steps, warmup, seed=1090, layout="nt", decode=False)
         for c in copies:
             q = abi.GemmParams.from_buffer_copy(p)
             q.b = c.address
-            fns.append(Launch(abi, "gemmcm_bf16", [0], q))
+            fns.append(Launch(abi, "gemmcm_bf16", [0, 0, 0, variant], q))
         return dict(kind="hbm", work=2 * (n * k + m * k + m * n), flops=2 * m * n * k, inputs=None,
                     name=f"mm bf16 M={m} K={k} N={n} ({layout}, decode)", **timed(abi, fns, steps, warmup))
     tm = time_steps(abi, [Launch(abi, "gemmcm_bf16", [0], p)], steps, warmup)

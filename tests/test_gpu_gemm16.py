@@ -74,6 +74,23 @@ def test_gemm16_few_rows(dtype, variant, m, k, n):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("variant", [0, 8])
+@pytest.mark.parametrize("m,k,n", [(1, 512, 64), (1, 2048, 1001), (2, 1032, 200), (2, 4096, 77), (1, 8192, 30), (3, 520, 130), (4, 2048, 520), (4, 512, 9)])
+def test_gemm16_one_to_four_rows_on_vector_units(dtype, variant, m, k, n):
+    """One and two rows in the Linear layout (three and four against few columns) run on the vector-unit kernel:
+    two-element dot products into float32 sums; planned and asked for (variant 8); every split of K over a workgroup's
+    waves, short last workgroups; alpha, beta and a bias; a strided view of the rows."""
+    import _dev
+    a = bits((torch.randn(2 * m, k, generator=gen(33)) * 0.5).to(dtype))
+    w = bits((torch.randn(n, k, generator=gen(34)) * 0.5).to(dtype))  # B = w.T: rows of k
+    want, mag = oracle.gemm16(a[::2], w.T, ODT[dtype], want_mag=True)
+    close(_dev.gemm16(a[::2], w.T, ODT[dtype], variant=variant), want, mag, dtype)
+    bias = bits(torch.randn(n, generator=gen(35)).to(dtype))
+    want2, mag2 = oracle.gemm16(a[:m], w.T, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, want_mag=True)
+    close(_dev.gemm16(a[:m], w.T, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, variant=variant), want2, mag2, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
 def test_gemm16_stream_kernel(dtype):
     """The stream kernel (variant 6; what large products in the Linear layout get): more tiles than workgroups, so
     streams that run through two tiles; batches; a broadcast bias; rows and columns past the last whole tile.  Every

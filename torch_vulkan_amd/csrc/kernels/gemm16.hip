@@ -109,6 +109,106 @@ __global__ __launch_bounds__(256) void gemm16_generic(GemmParams p, uint32_t use
   store_f32<T>(p.c + uint64_t((int64_t(batch) * p.c_sb + int64_t(m) * p.c_sm + int64_t(n) * p.c_sn) * 2), v);
 }
 
+// One and two rows of A in the Linear layout on the vector units (three and four against few columns): a wave streams
+// 2 weight rows with 16-byte non-temporal loads, 1, 2 or 4 waves of the workgroup share a row's k, two-element dot
+// products into float32 sums (products of two 16-bit values are exact in float32), wave sums by DPP, the K-parts
+// through LDS.  Many small workgroups have the whole weight stream in flight at once; the matrix-core kernel needs 8
+// to 16 columns per workgroup and leaves most of the machine idle against few columns.  g.k, g.lda, g.ldb in bytes.
+template <class T, int ROWS, int COLS, int KSPLIT>
+__global__ __launch_bounds__(256) void gemm16_gemv(GemmProblem<T> g) {
+  constexpr int WAVES = 4, GROUPS = WAVES / KSPLIT;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int grp = wave / KSPLIT, ks = wave % KSPLIT;
+  const uint32_t n0 = (blockIdx.x * GROUPS + grp) * COLS;
+  float acc[ROWS][COLS];
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) acc[r][c] = 0.0f;
+  // (clamped: the tail group re-reads the last row, masked at the store)
+  uint64_t brow[COLS], arow[ROWS];
+#pragma unroll
+  for (int c = 0; c < COLS; ++c) brow[c] = g.b + uint64_t(n0 + c < g.n ? n0 + c : g.n - 1) * g.ldb;
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) arow[r] = g.a + uint64_t(uint32_t(r) < g.m ? uint32_t(r) : g.m - 1) * g.lda;
+  for (uint32_t k = (ks * 64 + lane) * 16; k < g.k; k += 1024 * KSPLIT) {  // (k is a multiple of 16 bytes)
+    U4 wv[COLS], av[ROWS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) wv[c] = ldg_stream<U4>(brow[c] + k);
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) av[r] = ldg<U4>(arow[r] + k);
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+      for (int c = 0; c < COLS; ++c)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t x = av[r][i], y = wv[c][i];  // (values: a bit cast of a vector's element expression reads element 0)
+          if constexpr (T::dtype == VKT_BF16) {
+            acc[r][c] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(V2BF, x), __builtin_bit_cast(V2BF, y), acc[r][c], false);
+          } else {
+            typedef _Float16 V2H __attribute__((ext_vector_type(2)));
+            acc[r][c] = __builtin_amdgcn_fdot2(__builtin_bit_cast(V2H, x), __builtin_bit_cast(V2H, y), acc[r][c], false);
+          }
+        }
+  }
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) acc[r][c] = wave_sum(acc[r][c]);
+  __shared__ float part[WAVES][ROWS * COLS];
+  if constexpr (KSPLIT > 1) {
+    if (lane == 0) {
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) part[wave][r * COLS + c] = acc[r][c];
+    }
+    __syncthreads();
+    if (ks != 0) return;
+  }
+  // lane (r, c) of the group's first wave finishes output (r, n0 + c)
+  if (lane < ROWS * COLS) {
+    const int r = lane / COLS, c = lane % COLS;
+    float sum = 0.0f;
+#pragma unroll
+    for (int rr = 0; rr < ROWS; ++rr)
+#pragma unroll
+      for (int cc = 0; cc < COLS; ++cc)
+        if (rr == r && cc == c) sum = acc[rr][cc];  // (no dynamic register indexing)
+    if constexpr (KSPLIT > 1) {
+      sum = part[wave][lane];
+#pragma unroll
+      for (int s = 1; s < KSPLIT; ++s) sum += part[wave + s][lane];
+    }
+    const uint32_t n = n0 + c;
+    if (uint32_t(r) < g.m && n < g.n) {
+      float v = g.alpha * sum;
+      if (g.cin != 0) v += g.beta * load_f32<T>(g.cin + uint64_t((int64_t(r) * g.cin_sm + int64_t(n) * g.cin_sn) * 2));  // (beta == 0 never reads Cin: then cin is 0)
+      store_f32<T>(g.c + uint64_t((int64_t(r) * g.c_sm + int64_t(n)) * 2), v);
+    }
+  }
+}
+
+// One and two rows always; three and four where the matrix-core kernel would have fewer workgroups than half the
+// machine's compute units; forced: up to four rows whatever the column count.  -2: not this kernel's problem.
+template <class T>
+int launch_gemv16(const GemmProblem<T>& g, int compute_units, bool forced, hipStream_t stream) {
+  if (g.m > 4 || g.k < 1024) return -2;
+  if (g.m > 2 && !forced && g.n > 8u * uint32_t(compute_units)) return -2;
+  // (two long rows against many columns: 25.3 against 23.6 us at K = N = 8192; level at K = 4096, N = 14336; ahead elsewhere)
+  if (g.m == 2 && !forced && g.k >= 2 * 8192 && g.n >= 8192) return -2;
+  const int rows = g.m <= 1 ? 1 : g.m <= 2 ? 2 : 4;
+  const int ksplit = g.k >= 4096 ? (g.k <= 8192 ? 4 : 2) : (g.k >= 2048 ? 2 : 1);  // (a wave keeps one full 1 KiB load per column)
+  const dim3 grid((g.n + 2 * (4 / ksplit) - 1) / (2 * (4 / ksplit)));
+#define VKT_G16_GEMV_CASE(R_, KS_) \
+  if (rows == R_ && ksplit == KS_) { hipLaunchKernelGGL((gemm16_gemv<T, R_, 2, KS_>), grid, dim3(256), 0, stream, g); return 0; }
+  VKT_G16_GEMV_CASE(1, 1) VKT_G16_GEMV_CASE(1, 2) VKT_G16_GEMV_CASE(1, 4) VKT_G16_GEMV_CASE(2, 1) VKT_G16_GEMV_CASE(2, 2) VKT_G16_GEMV_CASE(2, 4)
+  VKT_G16_GEMV_CASE(4, 1) VKT_G16_GEMV_CASE(4, 2) VKT_G16_GEMV_CASE(4, 4)
+#undef VKT_G16_GEMV_CASE
+  return -2;
+}
+
 template <class T, bool TRA, bool TRB>
 int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t variant, const Machine& mc, hipStream_t stream,
                  std::string* err) {
@@ -124,6 +224,11 @@ int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t
   // workgroups own runs of columns and whose waves split K: the product is the weight stream, and 128 x 128 tiles put
   // 64 workgroups on the machine at N = 8192 (variant 7 asks for it; bits 8-11: 16s of columns per workgroup).
   if constexpr (!TRA && !TRB) {
+    if ((variant == 0 || variant == 8) && batch == 1) {  // 8: the vector-unit kernel for up to four rows
+      const int rc = launch_gemv16<T>(g, mc.compute_units, variant == 8, stream);
+      if (rc != -2) return rc;
+    }
+    if (variant == 8) variant = 0;
     if ((variant == 0 || (variant & 0xff) == 7) && batch == 1) {
       const int rc = launch_mma_skinny<0, 0, MATH>(g, mc.compute_units, (variant >> 8) & 15u, stream, err, "gemmcm");
       if (rc != -2) return rc;
