@@ -542,8 +542,8 @@ void orc_observe(float* run_min, float* run_max, const float* cur_min, const flo
   }
 }
 
-/* The float8 producer in front of _scaled_mm (no counterpart in the reference; SURVEY lists it
- * as the step a float8 pipeline needs on the device).  Per row, or with one given scale:
+/* The float8 producer in front of _scaled_mm (no counterpart in the reference: the step a float8
+ * pipeline needs on the device before the product).  Per row, or with one given scale:
  *   a = max(max_k |x|, 1e-12) (NaN elements do not count); scale = a / fmax;
  *   q = cast(clamp(x * (fmax / a), -fmax, fmax)); every step one float32 operation.
  * rowwise 0: scales[0] is an input and a = scales[0] * fmax. */
