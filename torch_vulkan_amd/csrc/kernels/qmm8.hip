@@ -1585,7 +1585,13 @@ int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipSt
     //  K = 4096, N = 14336: 13.5 against 13.9 us, N = 128256: 86 against 92; with fewer columns 9 % behind.  Bit 18: the
     //  staged matrix-core kernel for one and two rows whatever the shape.)
     const bool two_rows = p0.m == 2 && variant == 0 && p0.k >= 2048 && (p0.n + 15) / 16 >= 2u * uint32_t(mc.compute_units);
-    if ((p0.m > 2 || two_rows || ((variant >> 18) & 1)) && !((variant >> 17) & 1)) {
+    // (few columns: the matrix-core kernels give a workgroup 8 columns at least, the vector-unit kernels 1 or 2, and
+    //  there the many small workgroups win although they multiply every weight once per row: K = 8192, N = 1024 at 3 / 4 /
+    //  8 rows 5.8 / 5.9 / 8.6 us against 8.6 / 8.8 / 9.3; K = 4096, N = 2048 at 3 / 4: 5.4 against 6.3 / 6.4; N = 4096: 8.0
+    //  against 7.0, the other way round)
+    const uint32_t few = 8u * uint32_t(mc.compute_units);
+    const bool few_columns = variant == 0 && ((p0.m <= 4 && p0.n <= few) || (p0.m <= 8 && 2 * p0.n <= few && p0.k <= 8192));  // (K = 16384, N = 512 at 8 rows: 17.7 against 14.4)
+    if ((p0.m > 2 || two_rows || ((variant >> 18) & 1)) && !few_columns && !((variant >> 17) & 1)) {
       // 3 to 8 short rows against many columns: the wave-per-column-group kernel where it pays (variant bit 23 keeps the kernels below)
       // (bits 8-15 with bits 0-7 clear ask for it whatever the size: tests, tuning)
       const bool asked = !(variant & 0xff) && ((variant >> 8) & 0xff);
