@@ -1058,6 +1058,10 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
   constexpr uint32_t PLANE = 64 * 256, A_BYTES = PLANES * PLANE, B_BYTES = 128 * 128, STAGE = A_BYTES + B_BYTES;
   constexpr uint32_t ITEM = F32 ? 4 : 2, OUT_ITEM = ITEM;
   constexpr int PER_STEP = 2 * A_LOADS + 2;  // loads per lane and step
+  // steps in flight from memory (even: a step's parity names its register sets).  float32 activations: two, whose
+  // steps take three times as long and whose loads are half as many again (four would not fit the registers: 80
+  // bytes per lane went to scratch memory)
+  constexpr int AHEAD = F32 ? 2 : int(kTileAhead);
   static_assert(2 * STAGE <= kTileLds, "two stages");
   extern __shared__ __attribute__((aligned(16))) uint8_t tile_lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
@@ -1087,7 +1091,7 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
     b_src[i] = p.b + uint64_t(n) * p.k + ((slot ^ ((row >> 1) & 7u)) * 16);
     b_dst[i] = A_BYTES + (wave * 2 + i) * 1024 + lane * 16;
   }
-  U4 ra[kTileAhead][2][A_LOADS], rb[kTileAhead][2];
+  U4 ra[AHEAD][2][A_LOADS], rb[AHEAD][2];
   auto request = [&](auto set, uint32_t step) {
     constexpr int R = decltype(set)::value;
     const uint32_t st = step < s_end ? step : s_end - 1;  // (past the end the last step again, never published: the count of loads in flight stays the same)
@@ -1164,19 +1168,19 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
       for (int mt = 0; mt < 4; ++mt) acc[mt][t + 1] = mfma16<T>(w1, fa[S][mt], acc[mt][t + 1]);
     }
   };
-  // J = (step - s_begin) % kTileAhead.  The weights' register set is the step's parity; the activations' set changes
+  // J = (step - s_begin) % AHEAD.  The weights' register set is the step's parity; the activations' set changes
   // with every plane: sub-step (step, plane) uses set (PLANES * J + plane) % 2.
   auto iteration = [&](auto index, auto guarded, uint32_t step) {
-    constexpr int J = decltype(index)::value, NEXT = (J + 1) % kTileAhead;
+    constexpr int J = decltype(index)::value, NEXT = (J + 1) % AHEAD;
     constexpr bool GUARDED = decltype(guarded)::value;  // the last steps of the slice: step + 1 may be past the end
     // the registers of step + 1 have landed; they go to the stage that step - 1 was read from, and the register set
-    // takes the loads of step + 1 + kTileAhead.  16-bit activations: every wave's reads of that stage had returned
+    // takes the loads of step + 1 + AHEAD.  16-bit activations: every wave's reads of that stage had returned
     // before it passed the last barrier.  float32: a wave reads planes 1 and 2 of a step during the step itself, so
     // a barrier of its own comes first.
     if constexpr (F32) __syncthreads();
-    __builtin_amdgcn_s_waitcnt(vmcnt_only(3 * PER_STEP));
+    __builtin_amdgcn_s_waitcnt(vmcnt_only((AHEAD - 1) * PER_STEP));
     if (!GUARDED || step + 1 < s_end) publish(std::integral_constant<int, NEXT>{}, step + 1);
-    request(std::integral_constant<int, NEXT>{}, step + 1 + kTileAhead);
+    request(std::integral_constant<int, NEXT>{}, step + 1 + AHEAD);
     __syncthreads();
 #pragma unroll
     for (int plane = 0; plane < PLANES; ++plane) {
@@ -1197,11 +1201,13 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
   };
   request(std::integral_constant<int, 0>{}, s_begin);
   request(std::integral_constant<int, 1>{}, s_begin + 1);
-  request(std::integral_constant<int, 2>{}, s_begin + 2);
-  request(std::integral_constant<int, 3>{}, s_begin + 3);
-  __builtin_amdgcn_s_waitcnt(vmcnt_only(3 * PER_STEP));  // the first of four steps has landed
+  if constexpr (AHEAD == 4) {
+    request(std::integral_constant<int, 2>{}, s_begin + 2);
+    request(std::integral_constant<int, 3>{}, s_begin + 3);
+  }
+  __builtin_amdgcn_s_waitcnt(vmcnt_only((AHEAD - 1) * PER_STEP));  // the first of the steps in flight has landed
   publish(std::integral_constant<int, 0>{}, s_begin);
-  request(std::integral_constant<int, 0>{}, s_begin + kTileAhead);
+  request(std::integral_constant<int, 0>{}, s_begin + AHEAD);
   __syncthreads();
   read_activations(std::integral_constant<int, 0>{}, s_begin, 0);
   read_weights(std::integral_constant<int, 0>{}, s_begin);
@@ -1209,16 +1215,20 @@ __global__ __launch_bounds__(512) void qmm8_tile(Q8Params p, uint32_t steps_per_
   uint32_t step = s_begin;
   constexpr std::false_type plain{};
   constexpr std::true_type guarded{};
-  for (; step + kTileAhead < s_end; step += kTileAhead) {
+  for (; step + AHEAD < s_end; step += AHEAD) {
     iteration(std::integral_constant<int, 0>{}, plain, step);
     iteration(std::integral_constant<int, 1>{}, plain, step + 1);
-    iteration(std::integral_constant<int, 2>{}, plain, step + 2);
-    iteration(std::integral_constant<int, 3>{}, plain, step + 3);
+    if constexpr (AHEAD == 4) {
+      iteration(std::integral_constant<int, 2>{}, plain, step + 2);
+      iteration(std::integral_constant<int, 3>{}, plain, step + 3);
+    }
   }
   iteration(std::integral_constant<int, 0>{}, guarded, step);
   if (step + 1 < s_end) iteration(std::integral_constant<int, 1>{}, guarded, step + 1);
-  if (step + 2 < s_end) iteration(std::integral_constant<int, 2>{}, guarded, step + 2);
-  if (step + 3 < s_end) iteration(std::integral_constant<int, 3>{}, guarded, step + 3);
+  if constexpr (AHEAD == 4) {
+    if (step + 2 < s_end) iteration(std::integral_constant<int, 2>{}, guarded, step + 2);
+    if (step + 3 < s_end) iteration(std::integral_constant<int, 3>{}, guarded, step + 3);
+  }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // (the re-reads of the last step, requested past the end)
 
   // The four k-parts of a column half meet through LDS (8 waves x 16 tiles x 1 KiB = 128 KiB): wave
