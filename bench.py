@@ -206,7 +206,7 @@ def wl_q4(abi, m, k, n, bs, steps, warmup, seed=1030, prefill=False, phase=2):
                 shape=(n, bs), reference_layout_bytes=int(packed.numel()) * 4 + 4 * m * k + 4 * m * n, **timed(abi, fns, steps, warmup))
 
 
-def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False, variant=0, decode=False):
+def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False, variant=0, decode=False, f32_out=False):
     """_scaled_mm e4m3fn x e4m3fn -> bf16; A row-major, B column-major.  zero_operands: the same
     launch on all-zero matrices: the matrix cores' sustained rate depends on how many operand
     bits toggle (the part is power limited), and this is the data-independent end of that range.
@@ -225,9 +225,9 @@ def wl_fp8(abi, m, k, n, rowwise, steps, warmup, seed=1040, zero_operands=False,
         sa, sb = torch.tensor([0.5]), torch.tensor([0.5])
     da, db = abi.Buffer.from_numpy(a.view(torch.uint8).numpy()), abi.Buffer.from_numpy(bt.view(torch.uint8).numpy())
     dsa, dsb = abi.Buffer.from_numpy(sa.numpy()), abi.Buffer.from_numpy(sb.numpy())
-    out = abi.Buffer(m * n * 2)
+    out = abi.Buffer(m * n * (4 if f32_out else 2))
     p = abi.F8Params(a=da.address, b=db.address, scale_a=dsa.address, scale_b=dsb.address, out=out.address, m=m, n=n,
-                     k=k, lda=k, ldb=k, ldo=n, fmt_a=abi.E4M3, fmt_b=abi.E4M3, out_dtype=abi.BF16, rowwise=int(rowwise))
+                     k=k, lda=k, ldb=k, ldo=n, fmt_a=abi.E4M3, fmt_b=abi.E4M3, out_dtype=abi.F32 if f32_out else abi.BF16, rowwise=int(rowwise))
     if decode:
         copies = [db]
         for _ in range(rotation(n * k) - 1):

@@ -365,7 +365,13 @@ int launch_formats(const F8Params& p, uint32_t variant, int compute_units, hipSt
     if (rc != -2) return rc;
     variant = 0;
   }
-  if (variant == 0) variant = (p.out_dtype == VKT_F32 || p.out_dtype == VKT_F16) ? (big ? 6 : 7) : (big ? 11 : 1);
+  // (256 x 256 tiles where they give the machine enough workgroups, else 128 x 128: the exact path from one tile per
+  //  compute unit on (2048 x 4096 x 4096: 94 us on 128 x 128 tiles against 116; 1024 x 8192 x 8192: 164 against 200),
+  //  the float8 path from one per four units on (512 x 8192 x 8192: 64 against 82 us; at 1024 rows the stream kernel
+  //  is ahead, 91 against 99))
+  const uint64_t tiles256 = uint64_t((p.m + 255) / 256) * ((p.n + 255) / 256), cus = uint64_t(compute_units);
+  if (variant == 0)
+    variant = (p.out_dtype == VKT_F32 || p.out_dtype == VKT_F16) ? (big && tiles256 >= cus ? 6 : 7) : (big && 4 * tiles256 > cus ? 11 : 1);
   switch (variant) {
     case 6:
       if (p.k % BK == 0) return launch_tile<2, 2, 8, 8, FA, FB, true, true, true>(p, compute_units, stream, err);

@@ -1168,15 +1168,21 @@ int launch_stream_one(const Q4CParams& p, const CompactLayout& L, uint32_t m0, u
   return 0;
 }
 
+// Several tiles per workgroup only where the kernel keeps to its registers with 512 or 768 threads (blocks of 32 and
+// 64 values up to three rows, blocks of 128 at two rows, or three rows and two tiles): the other forms spill 100 to
+// 760 bytes per lane and run with one tile per workgroup.
+template <int MR, int UPB, int TEAMS>
+constexpr int kTeamsThatFit = TEAMS == 1 || (MR <= 3 && (UPB == 1 || UPB == 2)) || (UPB == 4 && (MR == 2 || (MR == 3 && TEAMS == 2))) ? TEAMS : 1;
+
 template <class T, int MR, int XG, int TEAMS>
 int launch_stream_upb(const Q4CParams& p, const CompactLayout& L, uint32_t m0, uint32_t groupwise, hipStream_t stream,
                       std::string* err) {
   switch (L.upb) {
-    case 0: return launch_stream_one<T, MR, 0, XG, TEAMS>(p, L, m0, groupwise, stream, err);
-    case 1: return launch_stream_one<T, MR, 1, XG, TEAMS>(p, L, m0, groupwise, stream, err);
-    case 2: return launch_stream_one<T, MR, 2, XG, TEAMS>(p, L, m0, groupwise, stream, err);
-    case 4: return launch_stream_one<T, MR, 4, XG, TEAMS>(p, L, m0, groupwise, stream, err);
-    case 8: return launch_stream_one<T, MR, 8, XG, TEAMS>(p, L, m0, groupwise, stream, err);
+    case 0: return launch_stream_one<T, MR, 0, XG, kTeamsThatFit<MR, 0, TEAMS>>(p, L, m0, groupwise, stream, err);
+    case 1: return launch_stream_one<T, MR, 1, XG, kTeamsThatFit<MR, 1, TEAMS>>(p, L, m0, groupwise, stream, err);
+    case 2: return launch_stream_one<T, MR, 2, XG, kTeamsThatFit<MR, 2, TEAMS>>(p, L, m0, groupwise, stream, err);
+    case 4: return launch_stream_one<T, MR, 4, XG, kTeamsThatFit<MR, 4, TEAMS>>(p, L, m0, groupwise, stream, err);
+    case 8: return launch_stream_one<T, MR, 8, XG, kTeamsThatFit<MR, 8, TEAMS>>(p, L, m0, groupwise, stream, err);
   }
   *err = "qmm4c: bad layout";
   return -1;
