@@ -277,7 +277,7 @@ def wl_gemm16(abi, m, k, n, steps, warmup, seed=1090, layout="nt", decode=False,
             fns.append(Launch(abi, "gemmcm_bf16", [0, 0, 0, variant], q))
         return dict(kind="hbm", work=2 * (n * k + m * k + m * n), flops=2 * m * n * k, inputs=None,
                     name=f"mm bf16 M={m} K={k} N={n} ({layout}, decode)", **timed(abi, fns, steps, warmup))
-    tm = time_steps(abi, [Launch(abi, "gemmcm_bf16", [0], p)], steps, warmup)
+    tm = time_steps(abi, [Launch(abi, "gemmcm_bf16", [0, 0, 0, variant], p)], steps, warmup)
     return dict(kind="mfma", peak=BF16_PEAK_TFLOPS, metric="bf16 mm TFLOP/s (% of MFMA peak)", work=2 * m * n * k, wall_ms=tm[0], event_ms=tm[1], event_ms_median=tm.median,
                 bytes=2 * (m * k + n * k + m * n), inputs=None, copies=1, name=f"mm bf16 M={m} K={k} N={n} ({layout}: " + {"nt": "x @ w.T, the Linear layout", "nn": "x @ w", "tn": "x.T @ w"}[layout] + ")")
 

@@ -241,7 +241,9 @@ int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t
   // (direct loads: k a multiple of 64; k-major operands run on the direct forms only)
   if (variant == 0) {
     // 256 x 256 tiles where they give every compute unit one, else 128 x 128
-    const bool large = uint64_t((p.m + 255) / 256) * ((p.n + 255) / 256) * batch >= uint64_t(mc.compute_units);
+    // (from three quarters of a tile per unit on: 1024 x 4096 x 14336 is 224 tiles on 256 units, 121 us on the stream
+    //  kernel against 163 on 128 x 128 tiles; at 128 tiles the small tiles are level or ahead)
+    const bool large = uint64_t((p.m + 255) / 256) * ((p.n + 255) / 256) * batch * 4 >= uint64_t(mc.compute_units) * 3;
     // (both operands k-major: 8 waves, whose transposing LDS reads cover each other: 8192^3 0.94 -> 1.11-1.13 PFLOP/s;
     //  with k-contiguous operands the 8-wave form reads 1.5x the LDS bytes and is 3-5 % slower)
     variant = large ? (direct_ok ? (TRA && TRB ? 5 : 3) : 2) : (TRA || TRB ? 4 : 1);
