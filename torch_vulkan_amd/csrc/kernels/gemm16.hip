@@ -400,7 +400,7 @@ int launch_q8_gemm_t(const Q8Params& p, const Machine& mc, hipStream_t stream, s
   Q8GemmProblem<T> g;
   g.a = p.a, g.b = mc.scratch, g.m = p.m, g.n = p.n, g.k = p.k * 2, g.lda = uint32_t(p.a_sm) * 2, g.ldb = p.k * 2;
   g.batches = 1, g.a_batch = 0, g.b_batch = 0, g.c = p.c, g.scales = p.scales;
-  const bool large = uint64_t((p.m + 255) / 256) * ((p.n + 255) / 256) >= uint64_t(mc.compute_units);
+  const bool large = uint64_t((p.m + 255) / 256) * ((p.n + 255) / 256) * 4 >= uint64_t(mc.compute_units) * 3;  // (as for the 16-bit product)
   if (g.k % BK == 0) {
     if (large && g.k >= 2 * BK && p.n % 8 == 0 && p.c % 16 == 0 && p.scales % 16 == 0 && mma_stream_strides_ok(g.lda, g.ldb))
       return launch_mma_stream<0, 0, MATH>(g, mc.compute_units, stream, err, "qmm8");
