@@ -241,9 +241,9 @@ int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t
   // (direct loads: k a multiple of 64; k-major operands run on the direct forms only)
   if (variant == 0) {
     // 256 x 256 tiles where they give every compute unit one, else 128 x 128
-    // (from three quarters of a tile per unit on: 1024 x 4096 x 14336 is 224 tiles on 256 units, 121 us on the stream
-    //  kernel against 163 on 128 x 128 tiles; at 128 tiles the small tiles are level or ahead)
-    const bool large = uint64_t((p.m + 255) / 256) * ((p.n + 255) / 256) * batch * 4 >= uint64_t(mc.compute_units) * 3;
+    // (from five eighths of a tile per unit on: 1024 x 4096 x 14336 is 224 tiles on 256 units, 121 us on the stream
+    //  kernel against 163 on 128 x 128 tiles; 168 tiles: 142 against 152; at 128 tiles the small tiles are level or ahead)
+    const bool large = uint64_t((p.m + 255) / 256) * ((p.n + 255) / 256) * batch * 8 >= uint64_t(mc.compute_units) * 5;
     // (both operands k-major: 8 waves, whose transposing LDS reads cover each other: 8192^3 0.94 -> 1.11-1.13 PFLOP/s;
     //  with k-contiguous operands the 8-wave form reads 1.5x the LDS bytes and is 3-5 % slower)
     variant = large ? (direct_ok ? (TRA && TRB ? 5 : 3) : 2) : (TRA || TRB ? 4 : 1);
@@ -400,7 +400,7 @@ int launch_q8_gemm_t(const Q8Params& p, const Machine& mc, hipStream_t stream, s
   Q8GemmProblem<T> g;
   g.a = p.a, g.b = mc.scratch, g.m = p.m, g.n = p.n, g.k = p.k * 2, g.lda = uint32_t(p.a_sm) * 2, g.ldb = p.k * 2;
   g.batches = 1, g.a_batch = 0, g.b_batch = 0, g.c = p.c, g.scales = p.scales;
-  const bool large = uint64_t((p.m + 255) / 256) * ((p.n + 255) / 256) * 4 >= uint64_t(mc.compute_units) * 3;  // (as for the 16-bit product)
+  const bool large = uint64_t((p.m + 255) / 256) * ((p.n + 255) / 256) * 8 >= uint64_t(mc.compute_units) * 5;  // (as for the 16-bit product)
   if (g.k % BK == 0) {
     if (large && g.k >= 2 * BK && p.n % 8 == 0 && p.c % 16 == 0 && p.scales % 16 == 0 && mma_stream_strides_ok(g.lda, g.ldb))
       return launch_mma_stream<0, 0, MATH>(g, mc.compute_units, stream, err, "qmm8");
