@@ -91,6 +91,24 @@ def test_gemm16_one_to_four_rows_on_vector_units(dtype, variant, m, k, n):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_gemm16_few_rows_infinite_weights(dtype):
+    """Rows of k that end inside a chunk of the few-row kernel, weight rows that start with an infinity: the outputs
+    are the infinities float arithmetic gives (what stands in for the values past k must not meet them as 0 x inf)."""
+    import _dev
+    m, k, n = 5, 520, 80
+    a = (torch.randn(m, k, generator=gen(43)) * 0.5).to(dtype)
+    w = (torch.randn(n, k, generator=gen(44)) * 0.5).to(dtype)
+    a[:, 0] = 1.0
+    w[:, 0] = float("inf")
+    w[3, 0] = float("-inf")
+    for variant in (7, 7 | 1 << 8, 0):
+        got = oracle.to_f32(_dev.gemm16(bits(a), bits(w).T, ODT[dtype], variant=variant), ODT[dtype])
+        want = np.full((m, n), np.inf, np.float32)
+        want[:, 3] = -np.inf
+        assert np.array_equal(got, want), variant
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
 def test_gemm16_stream_kernel(dtype):
     """The stream kernel (variant 6; what large products in the Linear layout get): more tiles than workgroups, so
     streams that run through two tiles; batches; a broadcast bias; rows and columns past the last whole tile.  Every

@@ -114,9 +114,11 @@ __global__ __launch_bounds__(WAVES * 64) void mma_skinny(Problem p, uint32_t col
     for (int t = 0; t < NT; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        // (bytes past k are fetched from the row's start instead: their activations are zeros below, and a NaN among
-        // them is one of the row's own values)
-        wr[t][i] = ldg_stream<U4>(wsrc[t][i] + (k0 + wk[i] < p.k ? k0 + wk[i] : 0u));
+        // (no branch around a load: bytes past k are fetched from the row's start and replaced by zeros, so that an
+        // infinity there does not meet the zeros that stand for the activations past k)
+        const bool inside = k0 + wk[i] < p.k;
+        const U4 v = ldg_stream<U4>(wsrc[t][i] + (inside ? k0 + wk[i] : 0u));
+        wr[t][i] = inside ? v : zero;
       }
   };
   const uint32_t rot = (blockIdx.x * 5u) % count;
