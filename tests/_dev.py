@@ -98,8 +98,9 @@ def q4_compact(x, odt, cw, fused=True, flags=0):
 
 
 def scaled_mm(a, fmt_a, bt, fmt_b, sa, sb, rowwise, bias=None, bias_dtype=oracle.F32, scale_result=None,
-              out_dtype=oracle.BF16, variant=0):
-    """_scaled_mm ("fp8mm").  a: uint8 codes [M,K]; bt: uint8 codes [N,K] (mat2 column-major)."""
+              out_dtype=oracle.BF16, variant=0, static=False):
+    """_scaled_mm ("fp8mm").  a: uint8 codes [M,K]; bt: uint8 codes [N,K] (mat2 column-major).  static: through
+    vkt_dispatch_static."""
     a = np.ascontiguousarray(a, dtype=np.uint8)
     bt = np.ascontiguousarray(bt, dtype=np.uint8)
     (m, k), n = a.shape, bt.shape[0]
@@ -116,7 +117,7 @@ def scaled_mm(a, fmt_a, bt, fmt_b, sa, sb, rowwise, bias=None, bias_dtype=oracle
                      n=n, k=k, lda=k, ldb=k, ldo=n, fmt_a=fmt_a, fmt_b=fmt_b, out_dtype=out_dtype,
                      bias_dtype=bias_dtype, rowwise=int(bool(rowwise)))
     if m and n:
-        abi.dispatch("fp8mm", [variant], p)
+        abi.dispatch("fp8mm", [variant], p, static=static)
     return do.to_numpy(_NP[out_dtype], (m, n))
 
 
@@ -171,9 +172,9 @@ def _device_view(arr):
     return buf, buf.address - lo, [st // arr.itemsize for st in arr.strides]
 
 
-def gemm16(a, b, dtype, cin=None, alpha=1.0, beta=0.0, variant=0):
+def gemm16(a, b, dtype, cin=None, alpha=1.0, beta=0.0, variant=0, static=False):
     """alpha * a @ b (+ beta * cin) through "gemmcm_<T>": a [B,]M,K and b [B,]K,N as uint16 views with
-    any strides; cin broadcastable to the result (zero strides)."""
+    any strides; cin broadcastable to the result (zero strides).  static: through vkt_dispatch_static."""
     a3 = np.asarray(a) if np.asarray(a).ndim == 3 else np.asarray(a)[None]
     b3 = np.asarray(b) if np.asarray(b).ndim == 3 else np.asarray(b)[None]
     B, M, K = a3.shape
@@ -190,7 +191,7 @@ def gemm16(a, b, dtype, cin=None, alpha=1.0, beta=0.0, variant=0):
         bc, pc, sc = _device_view(c3)
         p.cin, p.cin_sb, p.cin_sm, p.cin_sn = pc, sc[0], sc[1], sc[2]
     if B and M and N:
-        abi.dispatch("gemmcm_" + abi.SUFFIX[dtype], [int(use_cin), 0, 0, variant], p, (1, 1, B))
+        abi.dispatch("gemmcm_" + abi.SUFFIX[dtype], [int(use_cin), 0, 0, variant], p, (1, 1, B), static=static)
     res = out.to_numpy(np.uint16, (B, M, N))
     return res if np.asarray(a).ndim == 3 else res[0]
 

@@ -26,6 +26,7 @@ HW_WINDOW = 2.0**-13
 
 
 def on_matrix_cores(odt, variant, k):
+    variant &= 0xff  # (the bits above: columns per workgroup and slices of the few-row kernel)
     if variant in (6, 7, 255) or k % 16:
         return False
     if variant == 13:  # the vector-unit kernel for up to four rows: float32 sums whatever the output type
@@ -107,6 +108,23 @@ def test_scaled_mm_few_rows(fa, fb, m, k, n, out_dtype, rowwise):
     sr = 2.0 if out_dtype in (torch.float8_e4m3fn, torch.float8_e5m2) else None
     for variant in (0, 12) if sr or bias_dtype else (0,):
         run_case(m, k, n, fa, fb, out_dtype, rowwise, bias_dtype, sr, variant=variant, seed=m + n)
+
+
+@pytest.mark.parametrize("fa,fb", [(FLOAT8[0], FLOAT8[0]), (FLOAT8[1], FLOAT8[1])])
+@pytest.mark.parametrize("m,k,n,out_dtype,rowwise,nt,slices", [
+    (5, 4096, 80, torch.bfloat16, True, 1, 2), (16, 2064, 64, torch.float8_e4m3fn, False, 2, 2), (33, 8192, 200, torch.bfloat16, True, 2, 4),
+    (20, 4112, 1000, torch.float32, True, 1, 3), (64, 16400, 520, torch.bfloat16, False, 4, 8), (50, 28672, 100, torch.float16, True, 2, 16),
+    (64, 4096, 72, torch.bfloat16, True, 2, 31),
+    # planned: few columns against long rows (slices of K over workgroups)
+    (8, 16384, 1024, torch.bfloat16, True, 0, 0), (32, 8192, 1024, torch.float32, False, 0, 0), (32, 28672, 1024, torch.bfloat16, True, 0, 0),
+    (64, 8192, 2000, torch.float8_e5m2, True, 0, 0)])
+def test_scaled_mm_few_rows_k_slices(fa, fb, m, k, n, out_dtype, rowwise, nt, slices):
+    """The few-row kernel with K cut into slices over workgroups (their tiles through the workspace, added up by a
+    second launch, which runs the epilogue): asked for (slices that do not divide the chunks of k, a short last slice,
+    more slices asked for than half the chunks) and planned (what N = 1024 and 2048 get); every output type."""
+    bias_dtype = torch.bfloat16 if out_dtype == torch.bfloat16 else None
+    sr = 2.0 if out_dtype in (torch.float8_e4m3fn, torch.float8_e5m2) else None
+    run_case(m, k, n, fa, fb, out_dtype, rowwise, bias_dtype, sr, variant=12 | nt << 8 | slices << 12 if nt else 0, seed=m + n)
 
 
 @pytest.mark.parametrize("fa,fb", [(FLOAT8[0], FLOAT8[0]), (FLOAT8[1], FLOAT8[0]), (FLOAT8[0], FLOAT8[1]), (FLOAT8[1], FLOAT8[1])])

@@ -91,6 +91,27 @@ def test_gemm16_one_to_four_rows_on_vector_units(dtype, variant, m, k, n):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("m,k,n,nt,slices", [(5, 2048, 80, 1, 2), (16, 1032, 64, 2, 2), (33, 4096, 200, 2, 4), (20, 2056, 1000, 1, 3), (64, 8200, 520, 4, 8),
+                                              (50, 28672, 100, 2, 16), (64, 2048, 72, 2, 31),
+                                              # planned: few columns against long rows (slices of K over workgroups)
+                                              (8, 8192, 1024, 0, 0), (32, 4096, 1024, 0, 0), (32, 16384, 2048, 0, 0), (64, 8192, 1000, 0, 0)])
+def test_gemm16_few_rows_k_slices(dtype, m, k, n, nt, slices):
+    """The few-row kernel with K cut into slices over workgroups (their tiles through the workspace, added up by a
+    second launch): asked for (columns per workgroup and slice count in the variant word: slices that do not divide the
+    chunks of k, a last slice that is short, more slices asked for than half the chunks) and planned (few columns:
+    what N = 1024 and 2048 get); alpha, beta and a bias through the second launch's epilogue."""
+    import _dev
+    variant = 7 | nt << 8 | slices << 12 if nt else 0
+    a = bits((torch.randn(m, k, generator=gen(53)) * 0.5).to(dtype))
+    w = bits((torch.randn(n, k, generator=gen(54)) * 0.5).to(dtype))
+    want, mag = oracle.gemm16(a, w.T, ODT[dtype], want_mag=True)
+    close(_dev.gemm16(a, w.T, ODT[dtype], variant=variant), want, mag, dtype)
+    bias = bits(torch.randn(n, generator=gen(55)).to(dtype))
+    want2, mag2 = oracle.gemm16(a, w.T, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, want_mag=True)
+    close(_dev.gemm16(a, w.T, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, variant=variant), want2, mag2, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
 def test_gemm16_few_rows_infinite_weights(dtype):
     """Rows of k that end inside a chunk of the few-row kernel, weight rows that start with an infinity: the outputs
     are the infinities float arithmetic gives (what stands in for the values past k must not meet them as 0 x inf)."""

@@ -37,6 +37,31 @@ def test_static_dispatch_matches_dispatch():
             assert (np.abs(oracle.bf16_to_f32(got) - c64) <= ref_tol(c64, mag, oracle.BF16)).all()
 
 
+def test_static_dispatch_few_row_products_in_slices():
+    """The few-row kernel of the float8 and 16-bit products cuts K into slices over workgroups where columns are few,
+    their tiles in the workspace: the same outputs from the fixed array, on calls in a row of decreasing size."""
+    abi.device_info()
+    for i, (m, k, n) in enumerate([(64, 8192, 2048), (32, 8192, 1024), (8, 4096, 1024)]):
+        a = bits((torch.randn(m, k, generator=gen(300 + i)) * 0.5).bfloat16())
+        w = bits((torch.randn(n, k, generator=gen(310 + i)) * 0.5).bfloat16())
+        want = _dev.gemm16(a, w.T, oracle.BF16, variant=7 | 2 << 8 | 4 << 12)
+        assert np.array_equal(_dev.gemm16(a, w.T, oracle.BF16, variant=7 | 2 << 8 | 4 << 12, static=True), want), (m, k, n)
+        assert np.array_equal(_dev.gemm16(a, w.T, oracle.BF16, static=True), _dev.gemm16(a, w.T, oracle.BF16)), (m, k, n)
+        a8 = bits((torch.randn(m, k, generator=gen(320 + i))).to(torch.float8_e4m3fn))
+        w8 = bits((torch.randn(n, k, generator=gen(330 + i))).to(torch.float8_e4m3fn))
+        sa, sb = np.full(m, 0.5, np.float32), np.full(n, 1.5, np.float32)
+        for variant in (12 | 1 << 8 | 8 << 12, 0):
+            want = _dev.scaled_mm(a8, oracle.E4M3, w8, oracle.E4M3, sa, sb, True, variant=variant)
+            assert np.array_equal(_dev.scaled_mm(a8, oracle.E4M3, w8, oracle.E4M3, sa, sb, True, variant=variant, static=True), want), (m, k, n)
+    # more partial sums than the array holds: refused, not re-planned
+    m, k, n = 64, 8192, 16384
+    a = bits((torch.randn(m, k, generator=gen(340)) * 0.5).bfloat16())
+    w = bits((torch.randn(n, k, generator=gen(341)) * 0.5).bfloat16())
+    assert (n // 32) * 31 * 4 * 2 * 1024 > abi.STATIC_SCRATCH_BYTES
+    with pytest.raises(abi.VktError, match="fixed workspace holds"):
+        _dev.gemm16(a, w.T, oracle.BF16, variant=7 | 2 << 8 | 31 << 12, static=True)
+
+
 def test_static_dispatch_refuses_more_than_the_array_holds():
     abi.device_info()
     a, b, s = _case(64, 4096, 4096, 200)

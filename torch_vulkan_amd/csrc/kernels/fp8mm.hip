@@ -318,11 +318,11 @@ int launch_gemv(const F8Params& p, int compute_units, bool forced, hipStream_t s
 // The few-row kernel (mma_skinny.h) where it serves; bfloat16 and float8 outputs on the fp8 matrix-core instruction,
 // float32 and float16 outputs on exactly widened operands (the precision rule of the tile kernels).  -2: not served.
 template <int FA, int FB>
-int launch_skinny(const F8Params& p0, int compute_units, uint32_t forced_nt, hipStream_t stream, std::string* err) {
+int launch_skinny(const F8Params& p0, const Machine& mc, uint32_t forced_nt, uint32_t forced_slices, hipStream_t stream, std::string* err) {
   F8Problem p;
   static_cast<F8Params&>(p) = p0;
-  if (p0.out_dtype == VKT_F32 || p0.out_dtype == VKT_F16) return launch_mma_skinny<FA, FB, kMathFp8Wide>(p, compute_units, forced_nt, stream, err, "fp8mm");
-  return launch_mma_skinny<FA, FB, kMathFp8>(p, compute_units, forced_nt, stream, err, "fp8mm");
+  if (p0.out_dtype == VKT_F32 || p0.out_dtype == VKT_F16) return launch_mma_skinny<FA, FB, kMathFp8Wide>(p, mc, forced_nt, forced_slices, stream, err, "fp8mm");
+  return launch_mma_skinny<FA, FB, kMathFp8>(p, mc, forced_nt, forced_slices, stream, err, "fp8mm");
 }
 
 template <int WAVES_M, int WAVES_N, int TM, int TN, int FA, int FB, bool MF32 = false, bool DIRECT = false, bool WIDE = false>
@@ -344,7 +344,8 @@ int launch_stream(const F8Params& p, int compute_units, hipStream_t stream, std:
 }
 
 template <int FA, int FB>
-int launch_formats(const F8Params& p, uint32_t variant, int compute_units, hipStream_t stream, std::string* err) {
+int launch_formats(const F8Params& p, uint32_t variant, const Machine& mc, hipStream_t stream, std::string* err) {
+  const int compute_units = mc.compute_units;
   // variant 0: planned.  Explicit variants run the MFMA kernel whatever the output dtype
   // (tests, tuning): 1: 128x128 tiles (4 waves of 64x64, 16x16x128 MFMA); 2: 256x256 (4 waves of
   // 128x128, 16x16x128); 3: 256x128; 4: 256x256 with the 32x32x64 MFMA (measured ~10 % faster
@@ -360,8 +361,8 @@ int launch_formats(const F8Params& p, uint32_t variant, int compute_units, hipSt
     if (rc != -2) return rc;
     variant = 0;
   }
-  if (variant == 0 || (variant & 0xff) == 12) {  // 12: the few-row kernel where it serves (what up to 64 rows get), else as planned; bits 8-11: 16s of columns per workgroup
-    const int rc = launch_skinny<FA, FB>(p, compute_units, (variant >> 8) & 15u, stream, err);
+  if (variant == 0 || (variant & 0xff) == 12) {  // 12: the few-row kernel where it serves (what up to 64 rows get), else as planned; bits 8-11: 16s of columns per workgroup, bits 12-16: slices of K
+    const int rc = launch_skinny<FA, FB>(p, mc, (variant >> 8) & 15u, (variant >> 12) & 31u, stream, err);
     if (rc != -2) return rc;
     variant = 0;
   }
@@ -435,13 +436,13 @@ int launch_fp8mm(const F8Params& p, uint32_t variant, const Machine& mc, hipStre
     hipLaunchKernelGGL(fp8mm_generic, dim3((p.n + 63) / 64, (p.m + 3) / 4), dim3(256), 0, stream, p);
     rc = 0;
   } else if (p.fmt_a == VKT_E4M3 && p.fmt_b == VKT_E4M3) {
-    rc = launch_formats<0, 0>(p, variant, mc.compute_units, stream, err);
+    rc = launch_formats<0, 0>(p, variant, mc, stream, err);
   } else if (p.fmt_a == VKT_E5M2 && p.fmt_b == VKT_E4M3) {
-    rc = launch_formats<1, 0>(p, variant, mc.compute_units, stream, err);
+    rc = launch_formats<1, 0>(p, variant, mc, stream, err);
   } else if (p.fmt_a == VKT_E4M3 && p.fmt_b == VKT_E5M2) {
-    rc = launch_formats<0, 1>(p, variant, mc.compute_units, stream, err);
+    rc = launch_formats<0, 1>(p, variant, mc, stream, err);
   } else {
-    rc = launch_formats<1, 1>(p, variant, mc.compute_units, stream, err);
+    rc = launch_formats<1, 1>(p, variant, mc, stream, err);
   }
   if (rc == 0 && hipGetLastError() != hipSuccess) {
     *err = "fp8mm: kernel launch failed";

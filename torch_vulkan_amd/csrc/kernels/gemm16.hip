@@ -35,10 +35,13 @@ struct GemmProblem {
   float alpha, beta;
   int32_t c_sm, c_sb, cin_sm, cin_sn, cin_sb;  // elements (c_sn is 1 here)
   struct Whole {
-    bool vec_ok;
+    uint32_t vec_ok;
   };
   struct Columns {};
-  __device__ __forceinline__ Whole whole() const { return Whole{(c_sm & 3) == 0 && (c_sb & 3) == 0 && (c & 7u) == 0}; }
+  // (a word, not a bool: the one-byte struct stayed in memory, 8 bytes of scratch per lane in the kernels that use it; in
+  // the few-row kernel's second launch it went through LDS, indexed by a workgroup size read from the dispatch packet
+  // in host memory: 12 us in a 3 us kernel)
+  __device__ __forceinline__ Whole whole() const { return Whole{((uint32_t(c_sm) & 3u) | (uint32_t(c_sb) & 3u) | (uint32_t(c) & 7u)) == 0 ? 1u : 0u}; }
   __device__ __forceinline__ Columns columns(uint32_t, uint32_t, const Whole&) const { return Columns{}; }
   template <int DT>
   __device__ __forceinline__ void store(uint32_t batch, uint32_t row, uint32_t col, const V4F& t, const Columns&,
@@ -230,7 +233,7 @@ int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t
     }
     if (variant == 8) variant = 0;
     if ((variant == 0 || (variant & 0xff) == 7) && batch == 1) {
-      const int rc = launch_mma_skinny<0, 0, MATH>(g, mc.compute_units, (variant >> 8) & 15u, stream, err, "gemmcm");
+      const int rc = launch_mma_skinny<0, 0, MATH>(g, mc, (variant >> 8) & 15u, (variant >> 12) & 31u, stream, err, "gemmcm");
       if (rc != -2) return rc;
     }
   }
@@ -308,12 +311,12 @@ struct Q8GemmProblem {
   uint64_t a_batch, b_batch;
   uint64_t c, scales;
   struct Whole {
-    bool vec_ok;
+    uint32_t vec_ok;  // (a word, as in GemmProblem)
   };
   struct Columns {
     float s[4];
   };
-  __device__ __forceinline__ Whole whole() const { return Whole{(n & 3u) == 0 && (c & 7u) == 0}; }
+  __device__ __forceinline__ Whole whole() const { return Whole{((n & 3u) | (uint32_t(c) & 7u)) == 0 ? 1u : 0u}; }
   __device__ __forceinline__ Columns columns(uint32_t, uint32_t col, const Whole&) const {
     Columns cs;
 #pragma unroll

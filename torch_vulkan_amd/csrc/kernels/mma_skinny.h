@@ -17,6 +17,7 @@
 #include <string>
 #include <type_traits>
 
+#include "kernels.h"
 #include "mma_tile.h"
 #include "wave_tiles.h"
 
@@ -72,14 +73,36 @@ __device__ __forceinline__ void skinny_step(const U4& wv, const U4 (&a)[MT][4], 
   }
 }
 
-// p.k, p.lda, p.ldb in bytes; k a multiple of 16, rows and bases 16-byte aligned; p.m <= 16 MT.
+// The epilogue of one workgroup's tiles: lane (c, g) holds, per tile (mt, t), row 16 mt + c, columns n0 + 16 t + 4 g .. + 3.
+template <int MT, int NT, class Problem>
+__device__ __forceinline__ void skinny_store(const Problem& p, uint32_t n0, uint32_t n_end, const V4F (&acc)[MT][NT], int lane) {
+  const int c = lane & 15, g = lane >> 4;
+  const auto whole = p.whole();
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const uint32_t col = n0 + 16 * t + 4 * g;
+    if (col >= n_end) continue;
+    const auto cs = p.columns(0, col, whole);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const uint32_t row = 16 * mt + c;
+      if (row >= p.m) continue;
+      p.for_output_type(col + 3 < p.n, whole, [&](auto dt) { p.template store<decltype(dt)::value>(0, row, col, acc[mt][t], cs, whole); });
+    }
+  }
+}
+
+// p.k, p.lda, p.ldb in bytes; k a multiple of 16, rows and bases 16-byte aligned; p.m <= 16 MT.  gridDim.y slices of K
+// (chunks_per_slice chunks of 256 bytes each), one per workgroup of the column group: with more than one, wave 0
+// leaves the workgroup's tiles in the workspace and mma_skinny_finish adds the slices up in slice order.
 template <int MT, int NT, int WAVES, int FA, int FB, int MATH, class Problem>
-__global__ __launch_bounds__(WAVES * 64) void mma_skinny(Problem p, uint32_t cols_per_wg) {
+__global__ __launch_bounds__(WAVES * 64) void mma_skinny(Problem p, uint32_t cols_per_wg, uint32_t chunks_per_slice, uint64_t workspace) {
   constexpr uint32_t TILE = 16 * 256, REGION = NT * TILE;  // bytes of LDS per tile of 16 weight rows, per wave
   extern __shared__ __attribute__((aligned(16))) uint8_t staged[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
   uint8_t* const mine = staged + uint32_t(wave) * REGION;
-  const uint32_t count = (p.k + 255) / 256;
+  const uint32_t total = (p.k + 255) / 256, q_begin = blockIdx.y * chunks_per_slice;
+  const uint32_t count = (q_begin + chunks_per_slice < total ? q_begin + chunks_per_slice : total) - q_begin;  // (no slice is empty)
   const uint32_t n0 = blockIdx.x * cols_per_wg, n_end = n0 + cols_per_wg < p.n ? n0 + cols_per_wg : p.n;
   // loads: instruction i of tile t fetches rows 4 i .. 4 i + 3; this lane row 4 i + (lane / 16), slot lane % 16
   uint64_t wsrc[NT][4];
@@ -122,7 +145,7 @@ __global__ __launch_bounds__(WAVES * 64) void mma_skinny(Problem p, uint32_t col
       }
   };
   const uint32_t rot = (blockIdx.x * 5u) % count;
-  auto chunk_at = [&](uint32_t i) { return (i + rot) % count; };  // the i-th chunk this workgroup works on
+  auto chunk_at = [&](uint32_t i) { return q_begin + (i + rot) % count; };  // the i-th chunk this workgroup works on
   if (uint32_t(wave) < count) request(chunk_at(wave));
   for (uint32_t i = wave; i < count; i += WAVES) {
     const uint32_t k0 = chunk_at(i) * 256;
@@ -156,24 +179,33 @@ __global__ __launch_bounds__(WAVES * 64) void mma_skinny(Problem p, uint32_t col
   __syncthreads();
   add_wave_tiles<MT, NT, WAVES>(acc, reinterpret_cast<V4F*>(staged), wave, lane);
   if (wave != 0) return;
-  // lane (c, g) holds, per tile (mt, t), row 16 mt + c, columns n0 + 16 t + 4 g .. + 3
-  const auto whole = p.whole();
+  if (gridDim.y > 1) {
+    V4F* const out = reinterpret_cast<V4F*>(workspace) + (uint64_t(blockIdx.x) * gridDim.y + blockIdx.y) * (MT * NT * 64);
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const uint32_t col = n0 + 16 * t + 4 * g;
-    if (col >= n_end) continue;
-    const auto cs = p.columns(0, col, whole);
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const uint32_t row = 16 * mt + c;
-      if (row >= p.m) continue;
-      p.for_output_type(col + 3 < p.n, whole, [&](auto dt) { p.template store<decltype(dt)::value>(0, row, col, acc[mt][t], cs, whole); });
-    }
+    for (int i = 0; i < MT * NT; ++i) out[i * 64 + lane] = acc[i / NT][i % NT];
+    return;
   }
+  skinny_store<MT, NT>(p, n0, n_end, acc, lane);
+}
+
+// Adds up the slices of one column group (one wave per group), in slice order, and runs the epilogue.
+template <int MT, int NT, class Problem>
+__global__ __launch_bounds__(64) void mma_skinny_finish(Problem p, uint32_t cols_per_wg, uint32_t slices, uint64_t workspace) {
+  const int lane = threadIdx.x;
+  const V4F* const tiles = reinterpret_cast<const V4F*>(workspace) + uint64_t(blockIdx.x) * slices * (MT * NT * 64);
+  V4F acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT * NT; ++i) acc[i / NT][i % NT] = tiles[i * 64 + lane];
+  for (uint32_t sl = 1; sl < slices; ++sl) {
+#pragma unroll
+    for (int i = 0; i < MT * NT; ++i) acc[i / NT][i % NT] += tiles[uint64_t(sl) * (MT * NT * 64) + i * 64 + lane];
+  }
+  const uint32_t n0 = blockIdx.x * cols_per_wg;
+  skinny_store<MT, NT>(p, n0, n0 + cols_per_wg < p.n ? n0 + cols_per_wg : p.n, acc, lane);
 }
 
 template <int MT, int NT, int WAVES, int FA, int FB, int MATH, class Problem>
-int launch_skinny_one(const Problem& p, uint32_t cols, hipStream_t stream, std::string* err, const char* name) {
+int launch_skinny_one(const Problem& p, uint32_t cols, uint32_t slices, uint64_t workspace, hipStream_t stream, std::string* err, const char* name) {
   auto kernel = mma_skinny<MT, NT, WAVES, FA, FB, MATH, Problem>;
   constexpr uint32_t stage_bytes = WAVES * NT * 16 * 256, part_bytes = kPartSlots<MT, NT, WAVES> * MT * NT * 1024;
   constexpr uint32_t lds = stage_bytes > part_bytes ? stage_bytes : part_bytes;
@@ -186,37 +218,70 @@ int launch_skinny_one(const Problem& p, uint32_t cols, hipStream_t stream, std::
     }
     configured = true;
   }
-  hipLaunchKernelGGL(kernel, dim3((p.n + cols - 1) / cols), dim3(WAVES * 64), lds, stream, p, cols);
+  const uint32_t chunks = (p.k + 255) / 256, per_slice = (chunks + slices - 1) / slices, groups = (p.n + cols - 1) / cols;
+  slices = (chunks + per_slice - 1) / per_slice;  // (no empty slice)
+  hipLaunchKernelGGL(kernel, dim3(groups, slices), dim3(WAVES * 64), lds, stream, p, cols, per_slice, workspace);
+  if (slices > 1) hipLaunchKernelGGL((mma_skinny_finish<MT, NT, Problem>), dim3(groups), dim3(64), 0, stream, p, cols, slices, workspace);
   return 0;
 }
 
 // Launches the few-row kernel where it serves: up to 64 rows, rows of k of 1024 bytes and more, 64 columns and more.
-// 16, 32 or 64 columns per workgroup, whichever leaves the busiest compute unit the fewest bytes to take in,
-// (workgroups on it) x (columns + rows) x K: every workgroup reads all rows of A beside its weights (64 columns as one
-// workgroup per unit run a quarter slower than their bytes say).  forced_nt: that many 16s of columns instead (tests,
-// tuning).  -2: not this kernel's problem.
+// Enough columns to give every compute unit a workgroup: 16, 32 or 64 columns per workgroup, whichever leaves the
+// busiest compute unit the fewest bytes to take in, (workgroups on it) x (columns + rows) x K: every workgroup reads all
+// rows of A beside its weights (64 columns as one workgroup per unit run a quarter slower than their bytes say).
+// Fewer columns (N = 1024 or 2048: the key / value projections of a model with grouped heads): K is cut into slices
+// over workgroups, a power of two of them that brings the workgroups up to about one per unit while a slice keeps 8
+// chunks, and a second launch adds the slices' tiles up in slice order; measured on ten shapes x three row counts
+// x every (columns, slices), us before / with slices, fp8: 64 rows, K = 28672, N = 1024: 74.9 / 22.4; K = 8192, N =
+// 1024: 25.5 / 14.8; K = 8192, N = 4096: 27.2 / 21.3; 8 rows, K = 16384, N = 512: 11.4 / 7.8; K = 8192, N = 8192:
+// 14.8 as it was (no slices).  forced_nt: that many 16s of columns instead; forced_slices likewise (tests, tuning).
+// -2: not this kernel's problem; -1: the workspace is fixed and too small for the plan (*err says so).
 template <int FA, int FB, int MATH, class Problem>
-int launch_mma_skinny(const Problem& p, int compute_units, uint32_t forced_nt, hipStream_t stream, std::string* err, const char* name) {
+int launch_mma_skinny(const Problem& p, const Machine& mc, uint32_t forced_nt, uint32_t forced_slices, hipStream_t stream, std::string* err,
+                      const char* name) {
   if (p.m > 64 || p.k < 1024 || p.n < 64) return -2;
-  const uint32_t cus = uint32_t(compute_units);
-  int nt = 1;
-  float best = 1e30f;
-  for (int t = 1; t <= 4; t *= 2) {
-    const uint32_t cols = staged_cols(p.n, t, cus), workgroups = (p.n + cols - 1) / cols;
-    const float cost = float((workgroups + cus - 1) / cus) * float(cols + p.m) * float(p.k) * (t == 4 && workgroups <= cus ? 1.25f : 1.0f);
-    if (cost < best) best = cost, nt = t;
-  }
+  const uint32_t cus = uint32_t(mc.compute_units), chunks = (p.k + 255) / 256;
   const int mt = p.m <= 16 ? 1 : p.m <= 32 ? 2 : 4;
-  if (forced_nt) nt = int(forced_nt);
-  if (mt == 1 && nt == 4) nt = 2;  // (the shapes that are built)
-  if (mt == 4 && nt == 1) nt = 2;
-  const uint32_t cols = staged_cols(p.n, nt, cus);
-  // few columns against long rows: 16 waves per workgroup where half of the compute units or more would have none (a
-  // workgroup's waves take the chunks of k in turn: twice the waves, half the turns)
-  if (mt == 1 && nt == 1 && (p.n + cols - 1) / cols * 2 <= cus && p.k >= 32 * 256)
-    return launch_skinny_one<1, 1, 16, FA, FB, MATH>(p, cols, stream, err, name);
+  auto built = [&](int t) { return !((mt == 1 && t == 4) || (mt == 4 && t == 1)); };  // (the shapes that are built)
+  int nt = 2;
+  uint32_t slices = 1;
+  {
+    // (17 to 32 rows: 32 columns per workgroup from 24 MiB of weights on, 16 below: 8192 x 2048 bf16, 14.6 against 16.5 us;
+    //  4096 x 1024, 9.4 against 8.5)
+    const int sliced_nt = p.m <= 16 ? 1 : p.m <= 32 ? (uint64_t(p.k) * p.n >= (24u << 20) ? 2 : 1) : 2;
+    const uint32_t groups = (p.n + 16 * sliced_nt - 1) / (16 * sliced_nt);
+    while (groups * slices * 2 <= cus && chunks / (slices * 2) >= 8) slices *= 2;
+    if (slices > 1 && p.m <= 16 && chunks / slices >= 16) slices *= 2;  // (few rows: two workgroups per unit)
+    if (slices > 1) nt = sliced_nt;
+  }
+  if (slices == 1) {
+    float best = 1e30f;
+    for (int t = 1; t <= 4; t *= 2) {
+      if (!built(t)) continue;
+      const uint32_t cols = staged_cols(p.n, t, cus), workgroups = (p.n + cols - 1) / cols;
+      const float cost = float((workgroups + cus - 1) / cus) * float(cols + p.m) * float(p.k) * (t == 4 && workgroups <= cus ? 1.25f : 1.0f);
+      if (cost < best) best = cost, nt = t;
+    }
+  }
+  if (forced_nt && built(int(forced_nt))) nt = int(forced_nt), slices = 1;
+  if (forced_slices) slices = forced_slices;
+  while (slices > 1 && slices * 2 > chunks) --slices;
+  const uint32_t cols = slices == 1 ? staged_cols(p.n, nt, cus) : 16u * nt;
+  const uint64_t need = slices > 1 ? uint64_t((p.n + cols - 1) / cols) * slices * mt * nt * 1024 : 0;
+  if (need > mc.workspace_bytes) {
+    if (mc.workspace_fixed) {
+      *err = std::string(name) + ": this product's partial sums need " + std::to_string(need) + " bytes of workspace, the fixed workspace holds " +
+             std::to_string(mc.workspace_bytes);
+      return -1;
+    }
+    return -2;
+  }
+  // few columns against long rows without slices: 16 waves per workgroup where half of the compute units or more would
+  // have none (a workgroup's waves take the chunks of k in turn: twice the waves, half the turns)
+  if (mt == 1 && nt == 1 && slices == 1 && (p.n + cols - 1) / cols * 2 <= cus && p.k >= 32 * 256)
+    return launch_skinny_one<1, 1, 16, FA, FB, MATH>(p, cols, 1, 0, stream, err, name);
 #define VKT_SKINNY_CASE(MT_, NT_, W_) \
-  if (mt == MT_ && nt == NT_) return launch_skinny_one<MT_, NT_, W_, FA, FB, MATH>(p, cols, stream, err, name);
+  if (mt == MT_ && nt == NT_) return launch_skinny_one<MT_, NT_, W_, FA, FB, MATH>(p, cols, slices, mc.workspace, stream, err, name);
   VKT_SKINNY_CASE(1, 1, 8) VKT_SKINNY_CASE(1, 2, 8) VKT_SKINNY_CASE(2, 1, 8) VKT_SKINNY_CASE(2, 2, 8) VKT_SKINNY_CASE(2, 4, 4)
   VKT_SKINNY_CASE(4, 2, 8) VKT_SKINNY_CASE(4, 4, 4)
 #undef VKT_SKINNY_CASE
