@@ -178,8 +178,8 @@ typedef struct Q4CParams {
  * accumulation, one rounding (the reference's block, linalg.cpp:25-34, and kernel,
  * shaders/gemmcm.slang).  Strides in elements; alpha and beta hold float32 bits in their low
  * words.  112 bytes.  VARIANT (tests, tuning; 0: planned): 1-5 tile shapes, 6 the stream kernel, 7 the few-row kernel
- * (x @ w.T with up to 64 rows; bits 8-11: 16s of columns per workgroup), 8 the vector-unit kernel (x @ w.T, up to 4 rows),
- * 255 one thread per output. */
+ * (x @ w.T with up to 64 rows; bits 8-11: 16s of columns per workgroup, bits 12-16: slices of K over workgroups), 8 the
+ * vector-unit kernel (x @ w.T, up to 4 rows), 255 one thread per output. */
 typedef struct GemmParams {
   uint64_t a, b, c, cin;
   uint64_t alpha, beta;
@@ -273,8 +273,8 @@ typedef struct MinMaxParams {
  * (quant.cpp:279-300 fused into one kernel).  A: fp8 [m,k] row-major (lda bytes);
  * B: fp8, column-major, i.e. [n,k] rows ldb bytes apart.  104 bytes.  An optional entry overrides the launcher's
  * choice of kernel (tests, tuning; 0 or absent: planned): 1-9 tile shapes, 11 the stream kernel, 12 the few-row kernel
- * (up to 64 rows; bits 8-11: 16s of columns per workgroup), 13 the vector-unit kernel (up to 4 rows), 255 one thread per
- * output. */
+ * (up to 64 rows; bits 8-11: 16s of columns per workgroup, bits 12-16: slices of K over workgroups), 13 the vector-unit
+ * kernel (up to 4 rows), 255 one thread per output. */
 typedef struct F8Params {
   uint64_t a, b, scale_a, scale_b, bias, scale_result, out; /* bias / scale_result may be 0 */
   uint32_t m, n, k;
