@@ -241,12 +241,18 @@ int launch_skinny_one(const Problem& p, uint32_t cols, uint32_t slices, uint64_t
 // Enough columns to give every compute unit a workgroup: 16, 32 or 64 columns per workgroup, whichever leaves the
 // busiest compute unit the fewest bytes to take in, (workgroups on it) x (columns + rows) x K: every workgroup reads all
 // rows of A beside its weights (64 columns as one workgroup per unit run a quarter slower than their bytes say).
-// Fewer columns (N = 1024 or 2048: the key / value projections of a model with grouped heads): K is cut into slices
-// over workgroups, a power of two of them that brings the workgroups up to about one per unit while a slice keeps 8
-// chunks, and a second launch adds the slices' tiles up in slice order; measured on ten shapes x three row counts
-// x every (columns, slices), us before / with slices, fp8: 64 rows, K = 28672, N = 1024: 74.9 / 22.4; K = 8192, N =
-// 1024: 25.5 / 14.8; K = 8192, N = 4096: 27.2 / 21.3; 8 rows, K = 16384, N = 512: 11.4 / 7.8; K = 8192, N = 8192:
-// 14.8 as it was (no slices).  forced_nt: that many 16s of columns instead; forced_slices likewise (tests, tuning).
+// K in slices over workgroups (a second launch adds the slices' tiles up in slice order) where that brings more of
+// the machine to bear.  The rules are read off every (columns, slices) of 14 shapes x 5 row counts x both element
+// sizes (what they pick is 0.7 % behind the best form on average, 11 % at worst):
+//  - 32 columns per workgroup and a power of two of slices that brings the workgroups up to one per compute unit
+//    while a slice keeps two chunks (rows of k of 4096 bytes and more; 2048 from 33 rows on); up to 16 rows: twice the
+//    slices where they stay 14 chunks long (two workgroups per unit: 8 x 14336 x 4096 bf16, 28.5 -> 23.5 us), and no
+//    slices where 16 columns per workgroup fill the machine anyway;
+//  - 49 to 64 rows against 4096 columns and more, 17 to 32 against 8192 and more (rows of k of 8192 bytes and more):
+//    64 columns per workgroup, which halves the activations the workgroups re-read, and slices up to one workgroup
+//    per unit (two at 32 rows): 64 x 8192 x 8192, 30.6 -> 27.3 us fp8, 50.0 -> 42.2 bf16.
+// us before / with slices, fp8: 64 rows, K = 28672, N = 1024: 74.9 / 18.8; K = 8192, N = 1024: 25.5 / 11.2; 8 rows,
+// K = 16384, N = 512: 11.4 / 7.8.  forced_nt: that many 16s of columns instead; forced_slices likewise (tests, tuning).
 // -2: not this kernel's problem; -1: the workspace is fixed and too small for the plan (*err says so).
 template <int FA, int FB, int MATH, class Problem>
 int launch_mma_skinny(const Problem& p, const Machine& mc, uint32_t forced_nt, uint32_t forced_slices, hipStream_t stream, std::string* err,
@@ -257,14 +263,22 @@ int launch_mma_skinny(const Problem& p, const Machine& mc, uint32_t forced_nt, u
   auto built = [&](int t) { return !((mt == 1 && t == 4) || (mt == 4 && t == 1)); };  // (the shapes that are built)
   int nt = 2;
   uint32_t slices = 1;
-  {
-    // (17 to 32 rows: 32 columns per workgroup from 24 MiB of weights on, 16 below: 8192 x 2048 bf16, 14.6 against 16.5 us;
-    //  4096 x 1024, 9.4 against 8.5)
-    const int sliced_nt = p.m <= 16 ? 1 : p.m <= 32 ? (uint64_t(p.k) * p.n >= (24u << 20) ? 2 : 1) : 2;
-    const uint32_t groups = (p.n + 16 * sliced_nt - 1) / (16 * sliced_nt);
-    while (groups * slices * 2 <= cus && chunks / (slices * 2) >= 8) slices *= 2;
-    if (slices > 1 && p.m <= 16 && chunks / slices >= 16) slices *= 2;  // (few rows: two workgroups per unit)
-    if (slices > 1) nt = sliced_nt;
+  auto fill = [&](uint32_t groups, uint32_t limit) {  // slices that bring `groups` up to `limit` workgroups
+    uint32_t sl = 1;
+    while (groups * sl * 2 <= limit && chunks / (sl * 2) >= 2) sl *= 2;
+    return sl;
+  };
+  if (mt == 4 && p.m > 48 && p.n >= 4096 && p.k >= 8192) {
+    nt = 4, slices = fill((p.n + 63) / 64, cus);
+  } else if (mt == 2 && p.n >= 8192 && p.k >= 8192) {
+    nt = 4, slices = fill((p.n + 63) / 64, 2 * cus);
+  } else if (p.k >= (mt == 4 ? 2048u : 4096u)) {
+    const uint32_t groups = (p.n + 31) / 32;
+    slices = fill(groups, cus);
+    if (p.m <= 16 && slices > 1) {
+      if (groups * slices <= cus && chunks / (slices * 2) >= 14) slices *= 2;
+      else if ((p.n + 15) / 16 >= cus) slices = 1;
+    }
   }
   if (slices == 1) {
     float best = 1e30f;
