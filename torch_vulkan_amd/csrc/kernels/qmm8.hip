@@ -409,9 +409,9 @@ __device__ __forceinline__ V4F mfma16(const U4& w, const U4& a, const V4F& acc) 
 // k0 + 16 g (two MFMA operands) and the matching 16 activations of rows 16 mt + c; the
 // MFMA's first operand is the weights, so the lane ends with C[16 mt + c][n0 + 16 t + 4 g + r].
 // The epilogue of the matrix-core kernels: lane (c = lane % 16, g = lane / 16) holds, per
-// tile (mt, t), the sums of row 16 mt + c for columns n0 + 16 t + 4 g .. + 3.
+// tile (mt, t), the sums of row m0 + 16 mt + c for columns n0 + 16 t + 4 g .. + 3.
 template <class T, int MT, int NT>
-__device__ __forceinline__ void store_tiles(const Q8Params& p, uint32_t n0, const V4F (&acc)[MT][NT], int lane, uint32_t n_end = ~0u) {
+__device__ __forceinline__ void store_tiles(const Q8Params& p, uint32_t n0, const V4F (&acc)[MT][NT], int lane, uint32_t n_end = ~0u, uint32_t m0 = 0) {
   n_end = n_end < p.n ? n_end : p.n;  // (columns from n_end on are another workgroup's; a multiple of 4, or n)
   constexpr uint64_t item = sizeof(typename T::storage);  // (scales and outputs have the activations' type)
   constexpr bool F32 = T::dtype == VKT_F32;
@@ -425,7 +425,7 @@ __device__ __forceinline__ void store_tiles(const Q8Params& p, uint32_t n0, cons
     for (int r = 0; r < 4; ++r) scale[r] = load_f32<T>(p.scales + (n + r < p.n ? n + r : p.n - 1) * item);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      const uint32_t m = 16 * mt + c;
+      const uint32_t m = m0 + 16 * mt + c;
       if (m >= p.m || n >= n_end) continue;
       const uint64_t at = p.c + (uint64_t(m) * p.n + n) * item;
       float v[4];
@@ -645,19 +645,26 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma_staged(Q8Params p, uint3
   store_tiles<T, MT, NT>(p, n0, acc, lane, n_end);
 }
 
-// Adds up the slices of one column group (one wave per group), in slice order.
+// Adds up the slices of one column group, in slice order, and runs the epilogue: a workgroup per group, its waves (one
+// per 16 x 16 tile, 16 at most) take the tiles in turn, four slices' loads in flight.
+template <int MT, int NT>
+constexpr int kFinishWaves = MT * NT < 16 ? MT * NT : 16;
 template <class T, int MT, int NT>
-__global__ __launch_bounds__(64) void qmm8_mfma_finish(Q8Params p, uint32_t slices, uint64_t workspace) {
-  const int lane = threadIdx.x;
-  const V4F* const tiles = reinterpret_cast<const V4F*>(workspace) + uint64_t(blockIdx.x) * slices * (MT * NT * 64);
-  V4F acc[MT][NT];
-#pragma unroll
-  for (int i = 0; i < MT * NT; ++i) acc[i / NT][i % NT] = tiles[i * 64 + lane];
-  for (uint32_t sl = 1; sl < slices; ++sl) {
-#pragma unroll
-    for (int i = 0; i < MT * NT; ++i) acc[i / NT][i % NT] += tiles[uint64_t(sl) * (MT * NT * 64) + i * 64 + lane];
+__global__ __launch_bounds__((64 * kFinishWaves<MT, NT>)) void qmm8_mfma_finish(Q8Params p, uint32_t slices, uint64_t workspace) {
+  constexpr uint32_t GROUP = MT * NT * 64;  // V4F per slice of a group
+  const int lane = threadIdx.x & 63;
+  for (int tile = threadIdx.x >> 6; tile < MT * NT; tile += kFinishWaves<MT, NT>) {
+    const V4F* const mine = reinterpret_cast<const V4F*>(workspace) + uint64_t(blockIdx.x) * slices * GROUP + tile * 64 + lane;
+    V4F acc[1][1];
+    acc[0][0] = mine[0];
+    uint32_t sl = 1;
+    for (; sl + 4 <= slices; sl += 4) {
+      const V4F a = mine[uint64_t(sl) * GROUP], b = mine[uint64_t(sl + 1) * GROUP], c = mine[uint64_t(sl + 2) * GROUP], d = mine[uint64_t(sl + 3) * GROUP];
+      acc[0][0] += a, acc[0][0] += b, acc[0][0] += c, acc[0][0] += d;
+    }
+    for (; sl < slices; ++sl) acc[0][0] += mine[uint64_t(sl) * GROUP];
+    store_tiles<T, 1, 1>(p, blockIdx.x * 16 * NT + 16 * (tile % NT), acc, lane, ~0u, 16 * (tile / NT));
   }
-  store_tiles<T, MT, NT>(p, blockIdx.x * 16 * NT, acc, lane);
 }
 
 template <class T, int MT, int NT>
@@ -669,7 +676,7 @@ void launch_mfma_waves(const Q8Params& p, int waves, uint32_t slices, const Mach
     case 8: hipLaunchKernelGGL((qmm8_mfma<T, MT, NT, 8>), grid, dim3(512), 0, stream, p, per_slice, mc.workspace); break;
     default: hipLaunchKernelGGL((qmm8_mfma<T, MT, NT, 16>), grid, dim3(1024), 0, stream, p, per_slice, mc.workspace); break;
   }
-  if (slices > 1) hipLaunchKernelGGL((qmm8_mfma_finish<T, MT, NT>), dim3(grid.x), dim3(64), 0, stream, p, slices, mc.workspace);
+  if (slices > 1) hipLaunchKernelGGL((qmm8_mfma_finish<T, MT, NT>), dim3(grid.x), dim3(64 * kFinishWaves<MT, NT>), 0, stream, p, slices, mc.workspace);
 }
 
 template <class T, int MT, int NT, int WAVES, int PLANES = 1>
@@ -692,7 +699,7 @@ bool launch_staged_one(const Q8Params& p, uint32_t slices, const Machine& mc, hi
   const dim3 grid((p.n + cols - 1) / cols, slices);
   const uint32_t chunks = (p.k + 255) / 256, per_slice = (chunks + slices - 1) / slices;
   hipLaunchKernelGGL(kernel, grid, dim3(WAVES * 64), lds, stream, p, per_slice, mc.workspace, cols);
-  if (slices > 1) hipLaunchKernelGGL((qmm8_mfma_finish<T, MT, NT>), dim3(grid.x), dim3(64), 0, stream, p, slices, mc.workspace);
+  if (slices > 1) hipLaunchKernelGGL((qmm8_mfma_finish<T, MT, NT>), dim3(grid.x), dim3(64 * kFinishWaves<MT, NT>), 0, stream, p, slices, mc.workspace);
   return true;
 }
 
