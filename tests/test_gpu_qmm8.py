@@ -102,6 +102,19 @@ def test_qmm8_columns_dealt_out_evenly(dtype, m, k, n):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,k,n", [(8, 8192, 1024), (7, 28672, 64), (16, 4096, 1000), (5, 16384, 516), (20, 4112, 264), (32, 16384, 520), (32, 8192, 2048)])
+def test_qmm8_few_columns_k_slices(dtype, m, k, n):
+    """Few columns against long rows, planned by the library: the staged kernel with K in slices over workgroups, the
+    slices' tiles added up in slice order by a second launch (a wave per tile); slices that do not divide the chunks
+    of k, column counts that leave a short last workgroup and ragged vectors, rows of A further apart than k."""
+    import _dev
+    a, b, s = int8_case(dtype, m, k, n, seeds={"a": 14, "b": 15, "scales": 16})
+    check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s)), a, b, s, dtype)
+    if (m + 1) // 2 >= 5:
+        check_q8(_dev.qmm8(bits(a), ODT[dtype], b.numpy(), bits(s), row_step=2), a, b, s, dtype, rows=slice(None, None, 2))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("m,k,n", [(8, 512, 24600), (5, 1024, 33001), (8, 4096, 14336), (3, 3088, 12300), (7, 2064, 8192),
                                    (8, 4080, 4096), (4, 528, 70), (6, 512, 16), (8, 3600, 1000), (8, 2048, 34000)])
 def test_qmm8_rows_kernel(dtype, m, k, n):

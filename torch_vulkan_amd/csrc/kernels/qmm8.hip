@@ -1451,6 +1451,22 @@ inline MfmaPlan plan_mfma(const Q8Params& p, uint32_t variant, const Machine& mc
       if (cost < best) best = cost, slices = s;
     }
   }
+  // Few columns against long rows (N = 1024 or 2048, the key / value projections of a model with grouped heads; rows
+  // of 4096 values and more): the staged kernel with 32 columns per workgroup and K in slices over workgroups, a power
+  // of two that brings them up to one per compute unit while a slice keeps two chunks of 256 values (up to 16 rows:
+  // twice that where slices stay 14 chunks long), their tiles added up by a second launch.  Read off every (columns,
+  // slices) of 14 shapes x 3 row counts; us before / after at 8 rows: K = 28672, N = 1024: 23.5 / 11.5; K = 16384, N =
+  // 512: 14.8 / 7.9; K = 8192, N = 2048: 10.5 / 8.8; at 32 rows, K = 4096, N = 1024: 11.9 / 8.1.  From N = 4096 on the
+  // slices gain nothing (the activations are two bytes a value here, and every workgroup re-reads its slice of them).
+  // (17 to 32 rows: up to N = 1024; at 2048 the unsliced plan is level, 11.3 against 11.8 us)
+  if (!(variant & 0xffff) && !((variant >> 19) & 1) && p.m <= 32 && p.k >= 4096 && p.n >= 64 &&
+      (p.n + 31) / 32 * (p.m <= 16 ? 4 : 8) <= uint32_t(mc.compute_units)) {
+    const uint32_t cus = uint32_t(mc.compute_units), groups = (p.n + 31) / 32, chunks = (p.k + 255) / 256;
+    uint32_t s = 1;
+    while (groups * s * 2 <= cus && chunks / (s * 2) >= 2) s *= 2;
+    if (p.m <= 16 && s > 1 && chunks / (s * 2) >= 14) s *= 2;
+    if (s > 1) return MfmaPlan{true, 2, 8, s, 0.0f};  // (no estimate: the tile kernel is not weighed against it; K = 28672, N = 1024 at 32 rows: 16.9 against 18.1 us)
+  }
   // Up to 8 rows the kernel that stages the weights through LDS wins (measured at K = 4096 / N = 14336 and the
   // reverse: 15.8 against 17.1 us, 15.1-16.4 against 17.3-18.4); from 16 rows on the activations' own traffic
   // levels the two.  variant bit 18 asks for it explicitly, bit 19 for the plain kernel.
@@ -1607,7 +1623,9 @@ int launch_qmm8_t(const Q8Params& p0, uint32_t variant, const Machine& mc, hipSt
     //  8 rows 5.8 / 5.9 / 8.6 us against 8.6 / 8.8 / 9.3; K = 4096, N = 2048 at 3 / 4: 5.4 against 6.3 / 6.4; N = 4096: 8.0
     //  against 7.0, the other way round)
     const uint32_t few = 8u * uint32_t(mc.compute_units);
-    const bool few_columns = variant == 0 && ((p0.m <= 4 && p0.n <= few) || (p0.m <= 8 && 2 * p0.n <= few && p0.k <= 8192));  // (K = 16384, N = 512 at 8 rows: 17.7 against 14.4)
+    const bool few_columns = variant == 0 && ((p0.m <= 4 && p0.n <= few) || (p0.m <= 8 && 2 * p0.n <= few && p0.k <= 4096)) && (p0.m <= 2 || p0.k <= 8192);
+    // (longer rows: the staged kernel with K in slices over workgroups: K = 8192, N = 1024 at 5 to 8 rows 7.5 against
+    //  9.0 us; K = 28672, N = 1024 at 4 rows: 11.5 against 25.2)
     if ((p0.m > 2 || two_rows || ((variant >> 18) & 1)) && !few_columns && !((variant >> 17) & 1)) {
       // 3 to 8 short rows against many columns: the wave-per-column-group kernel where it pays (variant bit 23 keeps the kernels below)
       // (bits 8-15 with bits 0-7 clear ask for it whatever the size: tests, tuning)
