@@ -112,6 +112,41 @@ def test_gemm16_few_rows_k_slices(dtype, m, k, n, nt, slices):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("variant", [0, 9, 9 | 2 << 12, 9 | 3 << 12, 9 | 8 << 12])
+@pytest.mark.parametrize("m,k,n", [(1, 512, 64), (7, 1088, 200), (16, 2048, 1000), (17, 576, 72), (33, 1536, 4104), (64, 2048, 4128), (50, 4096, 520)])
+def test_gemm16_few_rows_weights_in_rows_of_n(dtype, variant, m, k, n):
+    """Up to 64 rows against weights stored [k, n] (x @ w) run on the few-row kernel that reads the weights through the
+    transposing LDS read: planned and asked for (variant 9), with K in slices over workgroups (slices that do not
+    divide the chunks of k); every row-tile count, short last workgroups; alpha, beta and a bias; a strided view of
+    the rows."""
+    import _dev
+    a = bits((torch.randn(2 * m, k, generator=gen(63)) * 0.5).to(dtype))
+    w = bits((torch.randn(k, n, generator=gen(64)) * 0.5).to(dtype))
+    want, mag = oracle.gemm16(a[::2], w, ODT[dtype], want_mag=True)
+    close(_dev.gemm16(a[::2], w, ODT[dtype], variant=variant), want, mag, dtype)
+    bias = bits(torch.randn(n, generator=gen(65)).to(dtype))
+    want2, mag2 = oracle.gemm16(a[:m], w, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, want_mag=True)
+    close(_dev.gemm16(a[:m], w, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, variant=variant), want2, mag2, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_gemm16_few_rows_weights_in_rows_of_n_infinities(dtype):
+    """Columns past n and an infinity at the matrix's start (where the loads of what lies outside go): no 0 x inf."""
+    import _dev
+    m, k, n = 5, 512, 72
+    a = (torch.randn(m, k, generator=gen(73)) * 0.5).to(dtype)
+    w = (torch.randn(k, n, generator=gen(74)) * 0.5).to(dtype)
+    a[:, 0] = 1.0
+    w[0, :] = float("inf")
+    w[0, 3] = float("-inf")
+    for variant in (9, 0, 9 | 2 << 12):
+        got = oracle.to_f32(_dev.gemm16(bits(a), bits(w), ODT[dtype], variant=variant), ODT[dtype])
+        want = np.full((m, n), np.inf, np.float32)
+        want[:, 3] = -np.inf
+        assert np.array_equal(got, want), variant
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
 def test_gemm16_few_rows_infinite_weights(dtype):
     """Rows of k that end inside a chunk of the few-row kernel, weight rows that start with an infinity: the outputs
     are the infinities float arithmetic gives (what stands in for the values past k must not meet them as 0 x inf)."""

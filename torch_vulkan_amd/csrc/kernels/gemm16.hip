@@ -238,6 +238,15 @@ int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t
     }
   }
   if ((variant & 0xff) == 7) variant = 0;
+  // The same few rows against weights stored [k, n] (x @ w): the few-row kernel that reads the weights through the
+  // transposing LDS read (variant 9 asks for it; bits 12-16: slices of K over workgroups).
+  if constexpr (!TRA && TRB) {
+    if ((variant == 0 || (variant & 0xff) == 9) && batch == 1) {
+      const int rc = launch_mma_skinny_kn<MATH>(g, mc, (variant >> 12) & 31u, stream, err, "gemmcm");
+      if (rc != -2) return rc;
+    }
+  }
+  if ((variant & 0xff) == 9) variant = 0;
   const bool direct_ok = g.k % BK == 0;
   // variant 0: planned; 1: 128x128 tiles; 2: 256x128; 3: 256x256 with direct loads; 4: 128x128 with direct loads;
   // 5: 256x256 with direct loads over 8 waves; 6: the stream kernel (mma_stream.h; else 3)

@@ -314,5 +314,154 @@ int launch_mma_skinny(const Problem& p, const Machine& mc, uint32_t forced_nt, u
   return -2;
 }
 
+// ---- The same product with the weights stored [k, n] (x @ w: rows of n, ldb bytes apart; 16-bit values).
+// A workgroup owns 64 columns and all rows of A; its 8 waves take chunks of 64 rows of k in turn.  A wave's load
+// instruction fetches 8 rows of k x 128 contiguous bytes (the workgroup's 64 columns), into registers a chunk ahead
+// and from there into the wave's own 8 KiB of LDS in the global layout, and the matrix core's weight operand (lane
+// (c, g): 8 values of k of column c) comes out of it through the transposing LDS read, two reads of 4 rows of k
+// each.  16-byte pieces are swizzled by the row of k so that neither side has bank conflicts.  K in slices over
+// workgroups as above (64 columns per workgroup are 128 workgroups at N = 8192).
+template <int MT, int WAVES, int MATH, class Problem>
+__global__ __launch_bounds__(WAVES * 64) void mma_skinny_kn(Problem p, uint32_t chunks_per_slice, uint64_t workspace) {
+  constexpr int NT = 4;
+  constexpr uint32_t KC = 64, REGION = KC * 128;
+  using V4S = short __attribute__((ext_vector_type(4)));
+  extern __shared__ __attribute__((aligned(16))) uint8_t staged[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
+  uint8_t* const mine = staged + uint32_t(wave) * REGION;
+  const uint32_t kv = p.k / 2, total = (kv + KC - 1) / KC, q_begin = blockIdx.y * chunks_per_slice;
+  const uint32_t count = (q_begin + chunks_per_slice < total ? q_begin + chunks_per_slice : total) - q_begin;  // (no slice is empty)
+  const uint32_t n0 = blockIdx.x * 64, n_end = n0 + 64 < p.n ? n0 + 64 : p.n;
+  auto swizzle = [](uint32_t row) { return ((row & 3u) << 1) | ((row >> 3) & 1u); };
+  // loads: instruction i fetches rows 8 i .. 8 i + 7 of the chunk; this lane row 8 i + lane / 8, piece lane % 8
+  const uint32_t lrow = uint32_t(lane) >> 3, piece = uint32_t(lane) & 7u;
+  const bool col_inside = n0 + 8 * piece < p.n;  // (n is a multiple of 8: a piece is inside or outside as a whole)
+  const uint64_t wsrc = p.b + uint64_t(n0 + 8 * piece) * 2;
+  uint64_t arow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const uint32_t m = uint32_t(16 * mt + c) < p.m ? 16 * mt + c : p.m - 1;
+    arow[mt] = p.a + uint64_t(m) * p.lda + 16 * g;
+  }
+  V4F acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[mt][t] = V4F{0.0f, 0.0f, 0.0f, 0.0f};
+  const U4 zero = {0, 0, 0, 0};
+  U4 wr[8];
+  auto request = [&](uint32_t q) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t k = q * KC + 8 * i + lrow;
+      // (no branch around a load: what lies past k or n is fetched from the matrix's start and replaced by zeros)
+      const bool inside = col_inside && k < kv;
+      const U4 v = ldg_stream<U4>(inside ? wsrc + uint64_t(k) * p.ldb : p.b);
+      wr[i] = inside ? v : zero;
+    }
+  };
+  const uint32_t rot = (blockIdx.x * 5u) % count;
+  auto chunk_at = [&](uint32_t i) { return q_begin + (i + rot) % count; };  // the i-th chunk this workgroup works on
+  if (uint32_t(wave) < count) request(chunk_at(wave));
+  for (uint32_t i = wave; i < count; i += WAVES) {
+    const uint32_t k0 = chunk_at(i) * KC;
+    U4 a[MT][4];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const bool inside = k0 + 32 * j + 8 * g < kv;  // (k is a multiple of 8 values)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const bool real = inside && uint32_t(16 * mt + c) < p.m;  // (rows past m are zeros, not loads)
+        a[mt][j] = real ? ldg<U4>(arow[mt] + uint64_t(k0 + 32 * j) * 2) : zero;
+        a[mt][j + 2] = zero;
+      }
+    }
+#pragma unroll
+    for (int i2 = 0; i2 < 8; ++i2) {
+      const uint32_t row = 8 * i2 + lrow;
+      *reinterpret_cast<U4*>(mine + row * 128 + ((piece ^ swizzle(row)) * 16)) = wr[i2];
+    }
+    if (i + WAVES < count) request(chunk_at(i + WAVES));
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        // (a wave's LDS operations execute in order: these reads see the writes above)
+        // lane (c, g): column 16 t + c, k = 32 j + 8 g .. + 7: two reads of 4 rows of k; in each, lane c of a group of
+        // 16 points at row + c / 4, values 4 (c % 4) .. + 3 of the tile's 16 columns, and receives column c's four
+        U4 wv;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          const uint32_t row = 32 * j + 8 * g + 4 * q + (uint32_t(c) >> 2);
+          const uint32_t at = 2 * t + ((uint32_t(c) & 3u) >> 1);
+          const V4S v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (__attribute__((address_space(3))) V4S*)(mine + row * 128 + ((at ^ swizzle(row)) * 16) + (uint32_t(c) & 1u) * 8));
+          const U2 w = __builtin_bit_cast(U2, v);
+          wv[2 * q] = w.x, wv[2 * q + 1] = w.y;
+        }
+        skinny_step<MT, NT, 0, 0, MATH>(wv, a, j, t, acc);
+      }
+    }
+  }
+  __syncthreads();
+  add_wave_tiles<MT, NT, WAVES>(acc, reinterpret_cast<V4F*>(staged), wave, lane);
+  if (wave != 0) return;
+  if (gridDim.y > 1) {
+    V4F* const out = reinterpret_cast<V4F*>(workspace) + (uint64_t(blockIdx.x) * gridDim.y + blockIdx.y) * (MT * NT * 64);
+#pragma unroll
+    for (int i = 0; i < MT * NT; ++i) out[i * 64 + lane] = acc[i / NT][i % NT];
+    return;
+  }
+  skinny_store<MT, NT>(p, n0, n_end, acc, lane);
+}
+
+template <int MT, int MATH, class Problem>
+int launch_skinny_kn_one(const Problem& p, uint32_t slices, uint64_t workspace, hipStream_t stream, std::string* err, const char* name) {
+  constexpr int WAVES = 8;
+  auto kernel = mma_skinny_kn<MT, WAVES, MATH, Problem>;
+  constexpr uint32_t stage_bytes = WAVES * 64 * 128, part_bytes = kPartSlots<MT, 4, WAVES> * MT * 4 * 1024;
+  constexpr uint32_t lds = stage_bytes > part_bytes ? stage_bytes : part_bytes;
+  static bool configured = false;  // guarded by the runtime's stream mutex
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
+      (void)hipGetLastError();
+      *err = std::string(name) + ": cannot reserve " + std::to_string(lds) + " bytes of LDS";
+      return -1;
+    }
+    configured = true;
+  }
+  const uint32_t chunks = (p.k / 2 + 63) / 64, per_slice = (chunks + slices - 1) / slices, groups = (p.n + 63) / 64;
+  slices = (chunks + per_slice - 1) / per_slice;  // (no empty slice)
+  hipLaunchKernelGGL(kernel, dim3(groups, slices), dim3(WAVES * 64), lds, stream, p, per_slice, workspace);
+  if (slices > 1) hipLaunchKernelGGL((mma_skinny_finish<MT, 4, Problem>), dim3(groups), dim3(64 * MT * 4), 0, stream, p, 64u, slices, workspace);
+  return 0;
+}
+
+// Up to 64 rows against weights stored [k, n] (16-bit values; n a multiple of 8, rows of k 16-byte aligned; 512 values
+// of k and more, 64 columns and more).  Slices of K: a power of two that brings the workgroups up to one per compute
+// unit while a wave keeps a chunk per slice; forced_slices instead (tests, tuning).  Return values as above.
+template <int MATH, class Problem>
+int launch_mma_skinny_kn(const Problem& p, const Machine& mc, uint32_t forced_slices, hipStream_t stream, std::string* err, const char* name) {
+  if (p.m > 64 || p.k < 1024 || p.n < 64 || p.n % 8) return -2;
+  const uint32_t cus = uint32_t(mc.compute_units), chunks = (p.k / 2 + 63) / 64, groups = (p.n + 63) / 64;
+  const int mt = p.m <= 16 ? 1 : p.m <= 32 ? 2 : 4;
+  uint32_t slices = 1;
+  while (groups * slices * 2 <= cus && chunks / (slices * 2) >= 8) slices *= 2;
+  if (forced_slices) slices = forced_slices;
+  while (slices > 1 && slices * 2 > chunks) --slices;
+  const uint64_t need = slices > 1 ? uint64_t(groups) * slices * mt * 4 * 1024 : 0;
+  if (need > mc.workspace_bytes) {
+    if (mc.workspace_fixed) {
+      *err = std::string(name) + ": this product's partial sums need " + std::to_string(need) + " bytes of workspace, the fixed workspace holds " +
+             std::to_string(mc.workspace_bytes);
+      return -1;
+    }
+    return -2;
+  }
+  if (mt == 1) return launch_skinny_kn_one<1, MATH>(p, slices, mc.workspace, stream, err, name);
+  if (mt == 2) return launch_skinny_kn_one<2, MATH>(p, slices, mc.workspace, stream, err, name);
+  return launch_skinny_kn_one<4, MATH>(p, slices, mc.workspace, stream, err, name);
+}
+
 }  // namespace
 }  // namespace vkt
