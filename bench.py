@@ -450,6 +450,7 @@ OTHER = {
     # (few columns against long rows, the key / value projections of a model with grouped heads: K in slices over workgroups)
     "f8_decode_m64_k28672_n1024": lambda abi, s, w: wl_fp8(abi, 64, 28672, 1024, True, s, w, decode=True),
     "mm_bf16_decode_m32_k8192_n2048": lambda abi, s, w: wl_gemm16(abi, 32, 8192, 2048, s, w, decode=True),
+    "q8_m8_k8192_n1024": lambda abi, s, w: wl_q8(abi, 8, 8192, 1024, abi.BF16, s, w, seed=1170),
     "mm_bf16_decode_nn_m8_k8192_n8192": lambda abi, s, w: wl_gemm16(abi, 8, 8192, 8192, s, w, decode=True, layout="nn"),  # (weights stored [k, n])
     "c4_fp8_8192_zero_operands": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 2, 30), max(w, 5), zero_operands=True),
 }
