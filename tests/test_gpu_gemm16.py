@@ -268,4 +268,4 @@ def test_gemm16_errors():
     with pytest.raises(abi.VktError, match="unknown kernel"):
         abi.dispatch("gemmcm_f32", [0], p)
     with pytest.raises(abi.VktError, match="unknown variant"):
-        abi.dispatch("gemmcm_bf16", [0, 0, 0, 9], p)
+        abi.dispatch("gemmcm_bf16", [0, 0, 0, 10], p)
