@@ -197,7 +197,8 @@ def test_qmm8_float32_rows_special_values():
 
 
 @pytest.mark.parametrize("variant", [0, 1 << 18, 1 << 19])
-@pytest.mark.parametrize("m,k,n", [(2, 1024, 64), (3, 2064, 200), (5, 4096, 1000), (8, 1040, 77), (13, 3072, 4100), (16, 4096, 4128), (9, 8192, 520)])
+@pytest.mark.parametrize("m,k,n", [(2, 1024, 64), (3, 2064, 200), (5, 4096, 1000), (8, 1040, 77), (13, 3072, 4100), (16, 4096, 4128), (9, 8192, 520),
+                                   (8, 8192, 1024), (5, 16400, 264), (16, 28672, 72)])  # (few columns against long rows: K in slices over workgroups)
 def test_qmm8_float32_few_rows_on_matrix_cores(variant, m, k, n):
     """2 to 16 rows of float32 activations: split into three bfloat16 planes by a launch of its own and multiplied by
     the staged matrix-core kernel (forced with bit 18, planned, and switched off with bit 19); rows of k not a multiple

@@ -112,6 +112,7 @@ __global__ __launch_bounds__(WAVES * 64) void mma_skinny(Problem p, uint32_t col
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
   uint8_t* const mine = staged + uint32_t(wave) * REGION;
   const uint32_t total = (p.k + 255) / 256, q_begin = blockIdx.y * chunks_per_slice;
+  if (q_begin >= total) return;  // (an empty slice, which the launcher does not make: the chunk count below would wrap around)
   const uint32_t count = (q_begin + chunks_per_slice < total ? q_begin + chunks_per_slice : total) - q_begin;  // (no slice is empty)
   const uint32_t n0 = blockIdx.x * cols_per_wg, n_end = n0 + cols_per_wg < p.n ? n0 + cols_per_wg : p.n;
   // loads: instruction i of tile t fetches rows 4 i .. 4 i + 3; this lane row 4 i + (lane / 16), slot lane % 16
@@ -330,6 +331,7 @@ __global__ __launch_bounds__(WAVES * 64) void mma_skinny_kn(Problem p, uint32_t 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
   uint8_t* const mine = staged + uint32_t(wave) * REGION;
   const uint32_t kv = p.k / 2, total = (kv + KC - 1) / KC, q_begin = blockIdx.y * chunks_per_slice;
+  if (q_begin >= total) return;  // (an empty slice, which the launcher does not make)
   const uint32_t count = (q_begin + chunks_per_slice < total ? q_begin + chunks_per_slice : total) - q_begin;  // (no slice is empty)
   const uint32_t n0 = blockIdx.x * 64, n_end = n0 + 64 < p.n ? n0 + 64 : p.n;
   auto swizzle = [](uint32_t row) { return ((row & 3u) << 1) | ((row >> 3) & 1u); };

@@ -544,6 +544,7 @@ __global__ __launch_bounds__(WAVES * 64) void qmm8_mfma_staged(Q8Params p, uint3
   const uint32_t total = (p.k + 255) / 256;
   const uint32_t q_begin = blockIdx.y * chunks_per_slice;
   const uint32_t q_end = q_begin + chunks_per_slice < total ? q_begin + chunks_per_slice : total;
+  if (q_begin >= total) return;  // (an empty slice, which the launchers do not make: the chunk count below would wrap around)
   // the workgroup's columns: cols_per_wg of them (at most 16 NT, a multiple of 4; 16 NT when K is sliced over workgroups)
   const uint32_t n0 = blockIdx.x * cols_per_wg, n_end = n0 + cols_per_wg < p.n ? n0 + cols_per_wg : p.n;
   // loads: instruction i of tile t fetches rows 4 i .. 4 i + 3; this lane row 4 i + (lane / 16), slot lane % 16
@@ -696,8 +697,9 @@ bool launch_staged_one(const Q8Params& p, uint32_t slices, const Machine& mc, hi
   // 448 workgroups, two for 192 of 256 units and one for the rest, and the launch lasts as long as the two take; in 28s
   // it is 512, two for each: the same bytes everywhere).  Several slices: whole tiles, which the second launch expects.
   const uint32_t cols = slices == 1 ? staged_cols(p.n, NT, uint32_t(mc.compute_units)) : 16 * NT;
-  const dim3 grid((p.n + cols - 1) / cols, slices);
   const uint32_t chunks = (p.k + 255) / 256, per_slice = (chunks + slices - 1) / slices;
+  slices = (chunks + per_slice - 1) / per_slice;  // (no empty slice: 65 chunks in 16 slices of 5 are 13 slices)
+  const dim3 grid((p.n + cols - 1) / cols, slices);
   hipLaunchKernelGGL(kernel, grid, dim3(WAVES * 64), lds, stream, p, per_slice, mc.workspace, cols);
   if (slices > 1) hipLaunchKernelGGL((qmm8_mfma_finish<T, MT, NT>), dim3(grid.x), dim3(64 * kFinishWaves<MT, NT>), 0, stream, p, slices, mc.workspace);
   return true;
@@ -1023,16 +1025,28 @@ __global__ __launch_bounds__(256) void qmm8_split_rows(Q8Params p, uint64_t plan
 inline bool launch_split_staged(const Q8Params& p0, const Machine& mc, hipStream_t stream, bool launch, float* estimate_us, std::string* err, int* rc) {
   *rc = 0;
   if (p0.m < 2 || p0.m > 16 || p0.k < 1024 || p0.n < 64 || uint64_t(p0.m) * p0.k >= (1ull << 28)) return false;
-  const uint64_t need = 3ull * p0.m * p0.k * 2;
+  const uint64_t planes_bytes = (3ull * p0.m * p0.k * 2 + 255) / 256 * 256;
   const uint32_t cus = uint32_t(mc.compute_units);
   int nt = 1;
+  uint32_t slices = 1;
   float best = 1e30f;
-  for (int t = 1; t <= 4; t *= 2) {
-    const uint32_t cols = staged_cols(p0.n, t, cus), workgroups = (p0.n + cols - 1) / cols;
-    const float cost = float((workgroups + cus - 1) / cus) * float(cols + 6 * p0.m) * float(p0.k) / 30e3f * (t == 4 && workgroups <= cus ? 1.25f : 1.0f);
-    if (cost < best) best = cost, nt = t;
+  // few columns against long rows: 32 columns per workgroup and K in slices over workgroups, as for 16-bit rows (the
+  // slices' tiles lie behind the planes in the workspace); 8 rows, K = 8192, N = 1024: 18.5 us on the one-row kernels
+  if (p0.k >= 4096 && (p0.n + 31) / 32 * 4 <= cus) {
+    const uint32_t groups = (p0.n + 31) / 32, chunks = (p0.k + 255) / 256;
+    while (groups * slices * 2 <= cus && chunks / (slices * 2) >= 2) slices *= 2;
+    if (slices > 1 && chunks / (slices * 2) >= 14) slices *= 2;
+    if (slices > 1) nt = 2, best = float(32 + 6 * p0.m) * float(p0.k) / float(slices) / 30e3f + 2.5f;  // (a third launch)
+  }
+  if (slices == 1) {
+    for (int t = 1; t <= 4; t *= 2) {
+      const uint32_t cols = staged_cols(p0.n, t, cus), workgroups = (p0.n + cols - 1) / cols;
+      const float cost = float((workgroups + cus - 1) / cus) * float(cols + 6 * p0.m) * float(p0.k) / 30e3f * (t == 4 && workgroups <= cus ? 1.25f : 1.0f);
+      if (cost < best) best = cost, nt = t;
+    }
   }
   *estimate_us = best + 6.5f;  // (what two launches in a row cost before their bytes: K = N = 1024 takes 6.3-8.1 us)
+  const uint64_t need = planes_bytes + (slices > 1 ? uint64_t((p0.n + 31) / 32) * slices * 2 * 1024 : 0);
   if (!launch) return need <= mc.workspace_bytes || mc.workspace_fixed;
   if (workspace_refused(mc, need, err)) {
     *rc = -1;
@@ -1043,10 +1057,12 @@ inline bool launch_split_staged(const Q8Params& p0, const Machine& mc, hipStream
   hipLaunchKernelGGL(qmm8_split_rows, dim3((threads + 255) / 256), dim3(256), 0, stream, p0, mc.workspace);
   Q8Params p = p0;
   p.a = mc.workspace, p.a_sm = p0.k;
+  Machine tiles = mc;  // (the slices' tiles: behind the planes)
+  tiles.workspace = mc.workspace + planes_bytes, tiles.workspace_bytes = mc.workspace_bytes - planes_bytes;
   const int waves = nt < 4 && p0.k >= 16 * 256 ? 8 : 4;
   bool ok = false;
   if (nt == 1) ok = waves == 8 ? launch_staged_one<f32_t, 1, 1, 8, 3>(p, 1, mc, stream) : launch_staged_one<f32_t, 1, 1, 4, 3>(p, 1, mc, stream);
-  else if (nt == 2) ok = waves == 8 ? launch_staged_one<f32_t, 1, 2, 8, 3>(p, 1, mc, stream) : launch_staged_one<f32_t, 1, 2, 4, 3>(p, 1, mc, stream);
+  else if (nt == 2) ok = waves == 8 ? launch_staged_one<f32_t, 1, 2, 8, 3>(p, slices, tiles, stream) : launch_staged_one<f32_t, 1, 2, 4, 3>(p, 1, mc, stream);
   else ok = launch_staged_one<f32_t, 1, 4, 4, 3>(p, 1, mc, stream);
   if (!ok) {
     *err = "qmm8: cannot reserve LDS for the staged kernel";
