@@ -113,7 +113,8 @@ def test_gemm16_few_rows_k_slices(dtype, m, k, n, nt, slices):
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
 @pytest.mark.parametrize("variant", [0, 9, 9 | 2 << 12, 9 | 3 << 12, 9 | 8 << 12])
-@pytest.mark.parametrize("m,k,n", [(1, 512, 64), (7, 1088, 200), (16, 2048, 1000), (17, 576, 72), (33, 1536, 4104), (64, 2048, 4128), (50, 4096, 520)])
+@pytest.mark.parametrize("m,k,n", [(1, 512, 64), (7, 1088, 200), (16, 2048, 1000), (17, 576, 72), (33, 1536, 4104), (64, 2048, 4128), (50, 4096, 520),
+                                   (8, 512, 14344)])  # (one slice, many columns, a short last workgroup)
 def test_gemm16_few_rows_weights_in_rows_of_n(dtype, variant, m, k, n):
     """Up to 64 rows against weights stored [k, n] (x @ w) run on the few-row kernel that reads the weights through the
     transposing LDS read: planned and asked for (variant 9), with K in slices over workgroups (slices that do not

@@ -323,7 +323,7 @@ int launch_mma_skinny(const Problem& p, const Machine& mc, uint32_t forced_nt, u
 // each.  16-byte pieces are swizzled by the row of k so that neither side has bank conflicts.  K in slices over
 // workgroups as above (64 columns per workgroup are 128 workgroups at N = 8192).
 template <int MT, int WAVES, int MATH, class Problem>
-__global__ __launch_bounds__(WAVES * 64) void mma_skinny_kn(Problem p, uint32_t chunks_per_slice, uint64_t workspace) {
+__global__ __launch_bounds__(WAVES * 64) void mma_skinny_kn(Problem p, uint32_t cols_per_wg, uint32_t chunks_per_slice, uint64_t workspace) {
   constexpr int NT = 4;
   constexpr uint32_t KC = 64, REGION = KC * 128;
   using V4S = short __attribute__((ext_vector_type(4)));
@@ -333,11 +333,12 @@ __global__ __launch_bounds__(WAVES * 64) void mma_skinny_kn(Problem p, uint32_t 
   const uint32_t kv = p.k / 2, total = (kv + KC - 1) / KC, q_begin = blockIdx.y * chunks_per_slice;
   if (q_begin >= total) return;  // (an empty slice, which the launcher does not make)
   const uint32_t count = (q_begin + chunks_per_slice < total ? q_begin + chunks_per_slice : total) - q_begin;  // (no slice is empty)
-  const uint32_t n0 = blockIdx.x * 64, n_end = n0 + 64 < p.n ? n0 + 64 : p.n;
+  // the workgroup's columns: cols_per_wg of them (a multiple of 8, 64 at most; 64 when K is sliced over workgroups)
+  const uint32_t n0 = blockIdx.x * cols_per_wg, n_end = n0 + cols_per_wg < p.n ? n0 + cols_per_wg : p.n;
   auto swizzle = [](uint32_t row) { return ((row & 3u) << 1) | ((row >> 3) & 1u); };
   // loads: instruction i fetches rows 8 i .. 8 i + 7 of the chunk; this lane row 8 i + lane / 8, piece lane % 8
   const uint32_t lrow = uint32_t(lane) >> 3, piece = uint32_t(lane) & 7u;
-  const bool col_inside = n0 + 8 * piece < p.n;  // (n is a multiple of 8: a piece is inside or outside as a whole)
+  const bool col_inside = n0 + 8 * piece < n_end;  // (n and the column count are multiples of 8: a piece is inside or outside as a whole)
   const uint64_t wsrc = p.b + uint64_t(n0 + 8 * piece) * 2;
   uint64_t arow[MT];
 #pragma unroll
@@ -418,7 +419,7 @@ __global__ __launch_bounds__(WAVES * 64) void mma_skinny_kn(Problem p, uint32_t 
 }
 
 template <int MT, int MATH, class Problem>
-int launch_skinny_kn_one(const Problem& p, uint32_t slices, uint64_t workspace, hipStream_t stream, std::string* err, const char* name) {
+int launch_skinny_kn_one(const Problem& p, uint32_t cols, uint32_t slices, uint64_t workspace, hipStream_t stream, std::string* err, const char* name) {
   constexpr int WAVES = 8;
   auto kernel = mma_skinny_kn<MT, WAVES, MATH, Problem>;
   constexpr uint32_t stage_bytes = WAVES * 64 * 128, part_bytes = kPartSlots<MT, 4, WAVES> * MT * 4 * 1024;
@@ -432,10 +433,10 @@ int launch_skinny_kn_one(const Problem& p, uint32_t slices, uint64_t workspace, 
     }
     configured = true;
   }
-  const uint32_t chunks = (p.k / 2 + 63) / 64, per_slice = (chunks + slices - 1) / slices, groups = (p.n + 63) / 64;
+  const uint32_t chunks = (p.k / 2 + 63) / 64, per_slice = (chunks + slices - 1) / slices, groups = (p.n + cols - 1) / cols;
   slices = (chunks + per_slice - 1) / per_slice;  // (no empty slice)
-  hipLaunchKernelGGL(kernel, dim3(groups, slices), dim3(WAVES * 64), lds, stream, p, per_slice, workspace);
-  if (slices > 1) hipLaunchKernelGGL((mma_skinny_finish<MT, 4, Problem>), dim3(groups), dim3(64 * MT * 4), 0, stream, p, 64u, slices, workspace);
+  hipLaunchKernelGGL(kernel, dim3(groups, slices), dim3(WAVES * 64), lds, stream, p, cols, per_slice, workspace);
+  if (slices > 1) hipLaunchKernelGGL((mma_skinny_finish<MT, 4, Problem>), dim3(groups), dim3(64 * MT * 4), 0, stream, p, cols, slices, workspace);
   return 0;
 }
 
@@ -460,9 +461,12 @@ int launch_mma_skinny_kn(const Problem& p, const Machine& mc, uint32_t forced_sl
     }
     return -2;
   }
-  if (mt == 1) return launch_skinny_kn_one<1, MATH>(p, slices, mc.workspace, stream, err, name);
-  if (mt == 2) return launch_skinny_kn_one<2, MATH>(p, slices, mc.workspace, stream, err, name);
-  return launch_skinny_kn_one<4, MATH>(p, slices, mc.workspace, stream, err, name);
+  // (64 columns whatever their count: dealt out evenly, N = 28672 in 56s, a workgroup's runs of 112 bytes straddle the
+  //  128-byte lines and share them with its neighbours': 160 us against 92)
+  const uint32_t cols = 64;
+  if (mt == 1) return launch_skinny_kn_one<1, MATH>(p, cols, slices, mc.workspace, stream, err, name);
+  if (mt == 2) return launch_skinny_kn_one<2, MATH>(p, cols, slices, mc.workspace, stream, err, name);
+  return launch_skinny_kn_one<4, MATH>(p, cols, slices, mc.workspace, stream, err, name);
 }
 
 }  // namespace
