@@ -88,4 +88,10 @@ const char* vkt_test_pool_error(void* p) { return static_cast<TestPool*>(p)->err
 // the stride bound of the stream kernel's 32-bit operand offsets (kernels/limits.h)
 int shim_mma_stream_strides_ok(uint64_t lda, uint64_t ldb) { return vkt::mma_stream_strides_ok(lda, ldb) ? 1 : 0; }
 
+// the slices of K a launcher makes for `wanted` (kernels/limits.h): slices in the low word, chunks per slice above
+uint64_t shim_k_slices(uint32_t chunks, uint32_t wanted) {
+  const vkt::KSlices s = vkt::k_slices(chunks, wanted);
+  return uint64_t(s.slices) | uint64_t(s.chunks_per_slice) << 32;
+}
+
 }  // extern "C"

@@ -190,3 +190,20 @@ def test_stream_kernel_stride_bound():
     assert not ok(limit + 1, 16) and not ok(16, limit + 1) and not ok(1 << 25, 1 << 25)
     for ld in (limit - 1, limit + 1, 1 << 24, 1 << 31):
         assert bool(ok(ld, 128)) == (255 * ld + 4096 < 1 << 32)
+
+
+def test_k_slices_leave_no_slice_empty():
+    """The launchers that cut K into slices over workgroups take the slice count from kernels/limits.h: every slice
+    they launch holds a chunk (the kernels count a slice's chunks in unsigned arithmetic), the slices cover all
+    chunks, and never more slices than asked for."""
+    L = ctypes.CDLL(os.path.join(os.path.dirname(abi.LIB_PATH), "libvkt_hosttest.so"))
+    L.shim_k_slices.argtypes = [ctypes.c_uint32, ctypes.c_uint32]
+    L.shim_k_slices.restype = ctypes.c_uint64
+    for chunks in list(range(1, 130)) + [224, 448, 1000, 65535]:
+        for wanted in list(range(0, 40)) + [64, 1 << 20]:
+            r = L.shim_k_slices(chunks, wanted)
+            slices, per = r & 0xffffffff, r >> 32
+            assert 1 <= slices <= max(wanted, 1) and per >= 1
+            assert (slices - 1) * per < chunks <= slices * per, (chunks, wanted, slices, per)
+    r = L.shim_k_slices(65, 16)
+    assert (r & 0xffffffff, r >> 32) == (13, 5)

@@ -18,6 +18,7 @@
 #include <type_traits>
 
 #include "kernels.h"
+#include "limits.h"
 #include "mma_tile.h"
 #include "wave_tiles.h"
 
@@ -231,8 +232,10 @@ int launch_skinny_one(const Problem& p, uint32_t cols, uint32_t slices, uint64_t
     }
     configured = true;
   }
-  const uint32_t chunks = (p.k + 255) / 256, per_slice = (chunks + slices - 1) / slices, groups = (p.n + cols - 1) / cols;
-  slices = (chunks + per_slice - 1) / per_slice;  // (no empty slice)
+  const uint32_t groups = (p.n + cols - 1) / cols;
+  const KSlices cut = k_slices((p.k + 255) / 256, slices);  // (no empty slice)
+  slices = cut.slices;
+  const uint32_t per_slice = cut.chunks_per_slice;
   hipLaunchKernelGGL(kernel, dim3(groups, slices), dim3(WAVES * 64), lds, stream, p, cols, per_slice, workspace);
   if (slices > 1) hipLaunchKernelGGL((mma_skinny_finish<MT, NT, Problem>), dim3(groups), dim3(64 * MT * NT), 0, stream, p, cols, slices, workspace);
   return 0;
@@ -433,8 +436,10 @@ int launch_skinny_kn_one(const Problem& p, uint32_t cols, uint32_t slices, uint6
     }
     configured = true;
   }
-  const uint32_t chunks = (p.k / 2 + 63) / 64, per_slice = (chunks + slices - 1) / slices, groups = (p.n + cols - 1) / cols;
-  slices = (chunks + per_slice - 1) / per_slice;  // (no empty slice)
+  const uint32_t groups = (p.n + cols - 1) / cols;
+  const KSlices cut = k_slices((p.k / 2 + 63) / 64, slices);  // (no empty slice)
+  slices = cut.slices;
+  const uint32_t per_slice = cut.chunks_per_slice;
   hipLaunchKernelGGL(kernel, dim3(groups, slices), dim3(WAVES * 64), lds, stream, p, cols, per_slice, workspace);
   if (slices > 1) hipLaunchKernelGGL((mma_skinny_finish<MT, 4, Problem>), dim3(groups), dim3(64 * MT * 4), 0, stream, p, cols, slices, workspace);
   return 0;

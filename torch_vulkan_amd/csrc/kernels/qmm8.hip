@@ -28,6 +28,7 @@
 #include <type_traits>
 
 #include "kernels.h"
+#include "limits.h"
 #include "wave_tiles.h"
 
 namespace vkt {
@@ -697,8 +698,9 @@ bool launch_staged_one(const Q8Params& p, uint32_t slices, const Machine& mc, hi
   // 448 workgroups, two for 192 of 256 units and one for the rest, and the launch lasts as long as the two take; in 28s
   // it is 512, two for each: the same bytes everywhere).  Several slices: whole tiles, which the second launch expects.
   const uint32_t cols = slices == 1 ? staged_cols(p.n, NT, uint32_t(mc.compute_units)) : 16 * NT;
-  const uint32_t chunks = (p.k + 255) / 256, per_slice = (chunks + slices - 1) / slices;
-  slices = (chunks + per_slice - 1) / per_slice;  // (no empty slice: 65 chunks in 16 slices of 5 are 13 slices)
+  const KSlices cut = k_slices((p.k + 255) / 256, slices);  // (no empty slice: 65 chunks in 16 slices of 5 are 13 slices)
+  slices = cut.slices;
+  const uint32_t per_slice = cut.chunks_per_slice;
   const dim3 grid((p.n + cols - 1) / cols, slices);
   hipLaunchKernelGGL(kernel, grid, dim3(WAVES * 64), lds, stream, p, per_slice, mc.workspace, cols);
   if (slices > 1) hipLaunchKernelGGL((qmm8_mfma_finish<T, MT, NT>), dim3(grid.x), dim3(64 * kFinishWaves<MT, NT>), 0, stream, p, slices, mc.workspace);
