@@ -53,6 +53,13 @@ def test_static_dispatch_few_row_products_in_slices():
         for variant in (12 | 1 << 8 | 8 << 12, 0):
             want = _dev.scaled_mm(a8, oracle.E4M3, w8, oracle.E4M3, sa, sb, True, variant=variant)
             assert np.array_equal(_dev.scaled_mm(a8, oracle.E4M3, w8, oracle.E4M3, sa, sb, True, variant=variant, static=True), want), (m, k, n)
+    # the int8 op against few columns: 16-bit rows, and float32 rows (three bfloat16 planes, the slices' tiles behind them)
+    for i, (m, k, n) in enumerate([(16, 8192, 1024), (8, 4096, 520)]):
+        a, b, s = _case(m, k, n, 350 + 10 * i)
+        assert np.array_equal(_dev.qmm8(a, oracle.BF16, b, s, static=True), _dev.qmm8(a, oracle.BF16, b, s)), (m, k, n)
+        a32 = torch.randn(m, k, generator=gen(360 + i)).numpy()
+        s32 = torch.empty(n).uniform_(0.005, 0.02, generator=gen(370 + i)).numpy()
+        assert np.array_equal(_dev.qmm8(a32, oracle.F32, b, s32, static=True), _dev.qmm8(a32, oracle.F32, b, s32)), (m, k, n)
     # more partial sums than the array holds: refused, not re-planned
     m, k, n = 64, 8192, 16384
     a = bits((torch.randn(m, k, generator=gen(340)) * 0.5).bfloat16())
