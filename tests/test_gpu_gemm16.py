@@ -148,6 +148,29 @@ def test_gemm16_few_rows_weights_in_rows_of_n_infinities(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("batch,m,k,n,layout,variant", [
+    (6, 1, 128, 520, "nt", 0), (5, 8, 128, 200, "nt", 0), (9, 16, 256, 72, "nt", 0),          # rows of k too short to share: a wave per 64 columns
+    (3, 16, 2048, 264, "nt", 0), (4, 33, 1024, 130, "nt", 0), (2, 64, 4096, 520, "nt", 7 | 2 << 8 | 4 << 12), (3, 5, 8192, 100, "nt", 0),
+    (7, 1, 1024, 128, "nn", 0), (3, 8, 4096, 128, "nn", 0), (2, 40, 576, 200, "nn", 0), (3, 16, 2048, 72, "nn", 9 | 3 << 12)])
+def test_gemm16_batched_few_rows(dtype, batch, m, k, n, layout, variant):
+    """A batch of few-row products (attention at decode: q @ k.T with rows of k of one head's length, p @ v with the
+    values in rows of n) runs on the few-row kernels, a workgroup per batch, column group and slice of K: batch strides
+    of all three matrices, a bias broadcast over rows and batches, weights shared by the batches (batch stride 0)."""
+    import _dev
+    a = bits((torch.randn(batch, m, k, generator=gen(83)) * 0.5).to(dtype))
+    w = bits((torch.randn(batch, n, k, generator=gen(84)) * 0.5).to(dtype))
+    b = w.transpose(0, 2, 1) if layout == "nt" else np.ascontiguousarray(w.transpose(0, 2, 1))
+    want, mag = oracle.gemm16(a, b, ODT[dtype], want_mag=True)
+    close(_dev.gemm16(a, b, ODT[dtype], variant=variant), want, mag, dtype)
+    bias = bits(torch.randn(n, generator=gen(85)).to(dtype))
+    want2, mag2 = oracle.gemm16(a, b, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, want_mag=True)
+    close(_dev.gemm16(a, b, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, variant=variant), want2, mag2, dtype)
+    shared = np.broadcast_to(b[:1], b.shape)
+    want3, mag3 = oracle.gemm16(a, shared, ODT[dtype], want_mag=True)
+    close(_dev.gemm16(a, shared, ODT[dtype], variant=variant), want3, mag3, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
 def test_gemm16_few_rows_infinite_weights(dtype):
     """Rows of k that end inside a chunk of the few-row kernel, weight rows that start with an infinity: the outputs
     are the infinities float arithmetic gives (what stands in for the values past k must not meet them as 0 x inf)."""

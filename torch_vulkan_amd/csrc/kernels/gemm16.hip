@@ -232,7 +232,7 @@ int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t
       if (rc != -2) return rc;
     }
     if (variant == 8) variant = 0;
-    if ((variant == 0 || (variant & 0xff) == 7) && batch == 1) {
+    if (variant == 0 || (variant & 0xff) == 7) {  // (batches too: a batch of few-row products, attention at decode)
       const int rc = launch_mma_skinny<0, 0, MATH>(g, mc, (variant >> 8) & 15u, (variant >> 12) & 31u, stream, err, "gemmcm");
       if (rc != -2) return rc;
     }
@@ -241,7 +241,7 @@ int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t
   // The same few rows against weights stored [k, n] (x @ w): the few-row kernel that reads the weights through the
   // transposing LDS read (variant 9 asks for it; bits 12-16: slices of K over workgroups).
   if constexpr (!TRA && TRB) {
-    if ((variant == 0 || (variant & 0xff) == 9) && batch == 1) {
+    if (variant == 0 || (variant & 0xff) == 9) {
       const int rc = launch_mma_skinny_kn<MATH>(g, mc, (variant >> 12) & 31u, stream, err, "gemmcm");
       if (rc != -2) return rc;
     }

@@ -76,29 +76,29 @@ __device__ __forceinline__ void skinny_step(const U4& wv, const U4 (&a)[MT][4], 
 
 // The epilogue of one 16 x 16 tile: lane (c, g) holds row row0 + c, columns col0 + 4 g .. + 3.
 template <class Problem>
-__device__ __forceinline__ void skinny_store_tile(const Problem& p, uint32_t row0, uint32_t col0, uint32_t n_end, const V4F& acc, int lane) {
+__device__ __forceinline__ void skinny_store_tile(const Problem& p, uint32_t batch, uint32_t row0, uint32_t col0, uint32_t n_end, const V4F& acc, int lane) {
   const uint32_t row = row0 + (lane & 15), col = col0 + 4 * (lane >> 4);
   if (col >= n_end || row >= p.m) return;
   const auto whole = p.whole();
-  const auto cs = p.columns(0, col, whole);
-  p.for_output_type(col + 3 < p.n, whole, [&](auto dt) { p.template store<decltype(dt)::value>(0, row, col, acc, cs, whole); });
+  const auto cs = p.columns(batch, col, whole);
+  p.for_output_type(col + 3 < p.n, whole, [&](auto dt) { p.template store<decltype(dt)::value>(batch, row, col, acc, cs, whole); });
 }
 
 // The epilogue of one workgroup's tiles: lane (c, g) holds, per tile (mt, t), row 16 mt + c, columns n0 + 16 t + 4 g .. + 3.
 template <int MT, int NT, class Problem>
-__device__ __forceinline__ void skinny_store(const Problem& p, uint32_t n0, uint32_t n_end, const V4F (&acc)[MT][NT], int lane) {
+__device__ __forceinline__ void skinny_store(const Problem& p, uint32_t batch, uint32_t n0, uint32_t n_end, const V4F (&acc)[MT][NT], int lane) {
   const int c = lane & 15, g = lane >> 4;
   const auto whole = p.whole();
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     const uint32_t col = n0 + 16 * t + 4 * g;
     if (col >= n_end) continue;
-    const auto cs = p.columns(0, col, whole);
+    const auto cs = p.columns(batch, col, whole);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const uint32_t row = 16 * mt + c;
       if (row >= p.m) continue;
-      p.for_output_type(col + 3 < p.n, whole, [&](auto dt) { p.template store<decltype(dt)::value>(0, row, col, acc[mt][t], cs, whole); });
+      p.for_output_type(col + 3 < p.n, whole, [&](auto dt) { p.template store<decltype(dt)::value>(batch, row, col, acc[mt][t], cs, whole); });
     }
   }
 }
@@ -126,14 +126,14 @@ __global__ __launch_bounds__(WAVES * 64) void mma_skinny(Problem p, uint32_t col
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const uint32_t n = n0 + 16 * t + row < n_end ? n0 + 16 * t + row : n_end - 1;  // (rows past the end: the last one again, from the caches)
-      wsrc[t][i] = p.b + uint64_t(n) * p.ldb;
+      wsrc[t][i] = p.b + uint64_t(blockIdx.z) * p.b_batch + uint64_t(n) * p.ldb;
     }
   }
   uint64_t arow[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const uint32_t m = uint32_t(16 * mt + c) < p.m ? 16 * mt + c : p.m - 1;
-    arow[mt] = p.a + uint64_t(m) * p.lda + 16 * g;
+    arow[mt] = p.a + uint64_t(blockIdx.z) * p.a_batch + uint64_t(m) * p.lda + 16 * g;
   }
   V4F acc[MT][NT];
 #pragma unroll
@@ -192,12 +192,12 @@ __global__ __launch_bounds__(WAVES * 64) void mma_skinny(Problem p, uint32_t col
   add_wave_tiles<MT, NT, WAVES>(acc, reinterpret_cast<V4F*>(staged), wave, lane);
   if (wave != 0) return;
   if (gridDim.y > 1) {
-    V4F* const out = reinterpret_cast<V4F*>(workspace) + (uint64_t(blockIdx.x) * gridDim.y + blockIdx.y) * (MT * NT * 64);
+    V4F* const out = reinterpret_cast<V4F*>(workspace) + ((uint64_t(blockIdx.z) * gridDim.x + blockIdx.x) * gridDim.y + blockIdx.y) * (MT * NT * 64);
 #pragma unroll
     for (int i = 0; i < MT * NT; ++i) out[i * 64 + lane] = acc[i / NT][i % NT];
     return;
   }
-  skinny_store<MT, NT>(p, n0, n_end, acc, lane);
+  skinny_store<MT, NT>(p, blockIdx.z, n0, n_end, acc, lane);
 }
 
 // Adds up the slices of one column group, in slice order, and runs the epilogue: a workgroup per group, a wave per
@@ -206,7 +206,7 @@ template <int MT, int NT, class Problem>
 __global__ __launch_bounds__(64 * MT * NT) void mma_skinny_finish(Problem p, uint32_t cols_per_wg, uint32_t slices, uint64_t workspace) {
   constexpr uint32_t GROUP = MT * NT * 64;  // V4F per slice of a group
   const int lane = threadIdx.x & 63, tile = threadIdx.x >> 6;
-  const V4F* const mine = reinterpret_cast<const V4F*>(workspace) + uint64_t(blockIdx.x) * slices * GROUP + tile * 64 + lane;
+  const V4F* const mine = reinterpret_cast<const V4F*>(workspace) + (uint64_t(blockIdx.z) * gridDim.x + blockIdx.x) * slices * GROUP + tile * 64 + lane;
   V4F acc = mine[0];
   uint32_t sl = 1;
   for (; sl + 4 <= slices; sl += 4) {
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(64 * MT * NT) void mma_skinny_finish(Problem p, uin
   }
   for (; sl < slices; ++sl) acc += mine[uint64_t(sl) * GROUP];
   const uint32_t n0 = blockIdx.x * cols_per_wg;
-  skinny_store_tile(p, 16 * (tile / NT), n0 + 16 * (tile % NT), n0 + cols_per_wg < p.n ? n0 + cols_per_wg : p.n, acc, lane);
+  skinny_store_tile(p, blockIdx.z, 16 * (tile / NT), n0 + 16 * (tile % NT), n0 + cols_per_wg < p.n ? n0 + cols_per_wg : p.n, acc, lane);
 }
 
 template <int MT, int NT, int WAVES, int FA, int FB, int MATH, class Problem>
@@ -236,8 +236,8 @@ int launch_skinny_one(const Problem& p, uint32_t cols, uint32_t slices, uint64_t
   const KSlices cut = k_slices((p.k + 255) / 256, slices);  // (no empty slice)
   slices = cut.slices;
   const uint32_t per_slice = cut.chunks_per_slice;
-  hipLaunchKernelGGL(kernel, dim3(groups, slices), dim3(WAVES * 64), lds, stream, p, cols, per_slice, workspace);
-  if (slices > 1) hipLaunchKernelGGL((mma_skinny_finish<MT, NT, Problem>), dim3(groups), dim3(64 * MT * NT), 0, stream, p, cols, slices, workspace);
+  hipLaunchKernelGGL(kernel, dim3(groups, slices, p.batches), dim3(WAVES * 64), lds, stream, p, cols, per_slice, workspace);
+  if (slices > 1) hipLaunchKernelGGL((mma_skinny_finish<MT, NT, Problem>), dim3(groups, 1, p.batches), dim3(64 * MT * NT), 0, stream, p, cols, slices, workspace);
   return 0;
 }
 
@@ -261,9 +261,15 @@ int launch_skinny_one(const Problem& p, uint32_t cols, uint32_t slices, uint64_t
 template <int FA, int FB, int MATH, class Problem>
 int launch_mma_skinny(const Problem& p, const Machine& mc, uint32_t forced_nt, uint32_t forced_slices, hipStream_t stream, std::string* err,
                       const char* name) {
-  if (p.m > 64 || p.k < 1024 || p.n < 64) return -2;
+  // (batches: a workgroup per batch, column group and slice; a batch of short rows, k of 256 bytes and more, is served too)
+  const uint32_t batches = p.batches;
+  if (p.m > 64 || p.n < 64 || batches == 0 || batches > 65535 || p.k < 256) return -2;
   const uint32_t cus = uint32_t(mc.compute_units), chunks = (p.k + 255) / 256;
   const int mt = p.m <= 16 ? 1 : p.m <= 32 ? 2 : 4;
+  // a batch of rows of k too short for a workgroup's waves to share (q @ k.T of a batch of attention heads: k = 128
+  // values): workgroups of one wave and 64 columns, up to 16 rows
+  if (batches > 1 && chunks < 8 && mt == 1 && !forced_nt && !forced_slices) return launch_skinny_one<1, 4, 1, FA, FB, MATH>(p, 64, 1, 0, stream, err, name);
+  if (p.k < 1024) return -2;
   auto built = [&](int t) { return !((mt == 1 && t == 4) || (mt == 4 && t == 1)); };  // (the shapes that are built)
   int nt = 2;
   uint32_t slices = 1;
@@ -273,22 +279,22 @@ int launch_mma_skinny(const Problem& p, const Machine& mc, uint32_t forced_nt, u
     return sl;
   };
   if (mt == 4 && p.m > 48 && p.n >= 4096 && p.k >= 8192) {
-    nt = 4, slices = fill((p.n + 63) / 64, cus);
+    nt = 4, slices = fill((p.n + 63) / 64 * batches, cus);
   } else if (mt == 2 && p.n >= 8192 && p.k >= 8192) {
-    nt = 4, slices = fill((p.n + 63) / 64, 2 * cus);
+    nt = 4, slices = fill((p.n + 63) / 64 * batches, 2 * cus);
   } else if (p.k >= (mt == 4 ? 2048u : 4096u)) {
-    const uint32_t groups = (p.n + 31) / 32;
+    const uint32_t groups = (p.n + 31) / 32 * batches;
     slices = fill(groups, cus);
     if (p.m <= 16 && slices > 1) {
       if (groups * slices <= cus && chunks / (slices * 2) >= 14) slices *= 2;
-      else if ((p.n + 15) / 16 >= cus) slices = 1;
+      else if ((p.n + 15) / 16 * batches >= cus) slices = 1;
     }
   }
   if (slices == 1) {
     float best = 1e30f;
     for (int t = 1; t <= 4; t *= 2) {
       if (!built(t)) continue;
-      const uint32_t cols = staged_cols(p.n, t, cus), workgroups = (p.n + cols - 1) / cols;
+      const uint32_t cols = batches == 1 ? staged_cols(p.n, t, cus) : 16u * t, workgroups = (p.n + cols - 1) / cols * batches;
       const float cost = float((workgroups + cus - 1) / cus) * float(cols + p.m) * float(p.k) * (t == 4 && workgroups <= cus ? 1.25f : 1.0f);
       if (cost < best) best = cost, nt = t;
     }
@@ -296,8 +302,8 @@ int launch_mma_skinny(const Problem& p, const Machine& mc, uint32_t forced_nt, u
   if (forced_nt && built(int(forced_nt))) nt = int(forced_nt), slices = 1;
   if (forced_slices) slices = forced_slices;
   while (slices > 1 && slices * 2 > chunks) --slices;
-  const uint32_t cols = slices == 1 ? staged_cols(p.n, nt, cus) : 16u * nt;
-  const uint64_t need = slices > 1 ? uint64_t((p.n + cols - 1) / cols) * slices * mt * nt * 1024 : 0;
+  const uint32_t cols = slices == 1 && batches == 1 ? staged_cols(p.n, nt, cus) : 16u * nt;
+  const uint64_t need = slices > 1 ? uint64_t((p.n + cols - 1) / cols) * batches * slices * mt * nt * 1024 : 0;
   if (need > mc.workspace_bytes) {
     if (mc.workspace_fixed) {
       *err = std::string(name) + ": this product's partial sums need " + std::to_string(need) + " bytes of workspace, the fixed workspace holds " +
@@ -308,7 +314,7 @@ int launch_mma_skinny(const Problem& p, const Machine& mc, uint32_t forced_nt, u
   }
   // few columns against long rows without slices: 16 waves per workgroup where half of the compute units or more would
   // have none (a workgroup's waves take the chunks of k in turn: twice the waves, half the turns)
-  if (mt == 1 && nt == 1 && slices == 1 && (p.n + cols - 1) / cols * 2 <= cus && p.k >= 32 * 256)
+  if (mt == 1 && nt == 1 && slices == 1 && (p.n + cols - 1) / cols * batches * 2 <= cus && p.k >= 32 * 256)
     return launch_skinny_one<1, 1, 16, FA, FB, MATH>(p, cols, 1, 0, stream, err, name);
 #define VKT_SKINNY_CASE(MT_, NT_, W_) \
   if (mt == MT_ && nt == NT_) return launch_skinny_one<MT_, NT_, W_, FA, FB, MATH>(p, cols, slices, mc.workspace, stream, err, name);
@@ -342,12 +348,12 @@ __global__ __launch_bounds__(WAVES * 64) void mma_skinny_kn(Problem p, uint32_t 
   // loads: instruction i fetches rows 8 i .. 8 i + 7 of the chunk; this lane row 8 i + lane / 8, piece lane % 8
   const uint32_t lrow = uint32_t(lane) >> 3, piece = uint32_t(lane) & 7u;
   const bool col_inside = n0 + 8 * piece < n_end;  // (n and the column count are multiples of 8: a piece is inside or outside as a whole)
-  const uint64_t wsrc = p.b + uint64_t(n0 + 8 * piece) * 2;
+  const uint64_t wbase = p.b + uint64_t(blockIdx.z) * p.b_batch, wsrc = wbase + uint64_t(n0 + 8 * piece) * 2;
   uint64_t arow[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const uint32_t m = uint32_t(16 * mt + c) < p.m ? 16 * mt + c : p.m - 1;
-    arow[mt] = p.a + uint64_t(m) * p.lda + 16 * g;
+    arow[mt] = p.a + uint64_t(blockIdx.z) * p.a_batch + uint64_t(m) * p.lda + 16 * g;
   }
   V4F acc[MT][NT];
 #pragma unroll
@@ -362,7 +368,7 @@ __global__ __launch_bounds__(WAVES * 64) void mma_skinny_kn(Problem p, uint32_t 
       const uint32_t k = q * KC + 8 * i + lrow;
       // (no branch around a load: what lies past k or n is fetched from the matrix's start and replaced by zeros)
       const bool inside = col_inside && k < kv;
-      const U4 v = ldg_stream<U4>(inside ? wsrc + uint64_t(k) * p.ldb : p.b);
+      const U4 v = ldg_stream<U4>(inside ? wsrc + uint64_t(k) * p.ldb : wbase);
       wr[i] = inside ? v : zero;
     }
   };
@@ -413,12 +419,12 @@ __global__ __launch_bounds__(WAVES * 64) void mma_skinny_kn(Problem p, uint32_t 
   add_wave_tiles<MT, NT, WAVES>(acc, reinterpret_cast<V4F*>(staged), wave, lane);
   if (wave != 0) return;
   if (gridDim.y > 1) {
-    V4F* const out = reinterpret_cast<V4F*>(workspace) + (uint64_t(blockIdx.x) * gridDim.y + blockIdx.y) * (MT * NT * 64);
+    V4F* const out = reinterpret_cast<V4F*>(workspace) + ((uint64_t(blockIdx.z) * gridDim.x + blockIdx.x) * gridDim.y + blockIdx.y) * (MT * NT * 64);
 #pragma unroll
     for (int i = 0; i < MT * NT; ++i) out[i * 64 + lane] = acc[i / NT][i % NT];
     return;
   }
-  skinny_store<MT, NT>(p, n0, n_end, acc, lane);
+  skinny_store<MT, NT>(p, blockIdx.z, n0, n_end, acc, lane);
 }
 
 template <int MT, int MATH, class Problem>
@@ -440,8 +446,8 @@ int launch_skinny_kn_one(const Problem& p, uint32_t cols, uint32_t slices, uint6
   const KSlices cut = k_slices((p.k / 2 + 63) / 64, slices);  // (no empty slice)
   slices = cut.slices;
   const uint32_t per_slice = cut.chunks_per_slice;
-  hipLaunchKernelGGL(kernel, dim3(groups, slices), dim3(WAVES * 64), lds, stream, p, cols, per_slice, workspace);
-  if (slices > 1) hipLaunchKernelGGL((mma_skinny_finish<MT, 4, Problem>), dim3(groups), dim3(64 * MT * 4), 0, stream, p, cols, slices, workspace);
+  hipLaunchKernelGGL(kernel, dim3(groups, slices, p.batches), dim3(WAVES * 64), lds, stream, p, cols, per_slice, workspace);
+  if (slices > 1) hipLaunchKernelGGL((mma_skinny_finish<MT, 4, Problem>), dim3(groups, 1, p.batches), dim3(64 * MT * 4), 0, stream, p, cols, slices, workspace);
   return 0;
 }
 
@@ -450,8 +456,9 @@ int launch_skinny_kn_one(const Problem& p, uint32_t cols, uint32_t slices, uint6
 // unit while a wave keeps a chunk per slice; forced_slices instead (tests, tuning).  Return values as above.
 template <int MATH, class Problem>
 int launch_mma_skinny_kn(const Problem& p, const Machine& mc, uint32_t forced_slices, hipStream_t stream, std::string* err, const char* name) {
-  if (p.m > 64 || p.k < 1024 || p.n < 64 || p.n % 8) return -2;
-  const uint32_t cus = uint32_t(mc.compute_units), chunks = (p.k / 2 + 63) / 64, groups = (p.n + 63) / 64;
+  const uint32_t batches = p.batches;
+  if (p.m > 64 || p.k < 1024 || p.n < 64 || p.n % 8 || batches == 0 || batches > 65535) return -2;
+  const uint32_t cus = uint32_t(mc.compute_units), chunks = (p.k / 2 + 63) / 64, groups = (p.n + 63) / 64 * batches;
   const int mt = p.m <= 16 ? 1 : p.m <= 32 ? 2 : 4;
   uint32_t slices = 1;
   while (groups * slices * 2 <= cus && chunks / (slices * 2) >= 8) slices *= 2;
