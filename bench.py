@@ -49,8 +49,9 @@ def _abi():
 class Launch:
     """One prebuilt vkt_dispatch call (no per-call Python allocation in the timed loop)."""
 
-    def __init__(self, abi, name, spec, params):
+    def __init__(self, abi, name, spec, params, batches=1):
         self.fn = abi.lib().vkt_dispatch
+        self.batches = batches  # (the grid's third entry: what "gemmcm_*" takes its batch count from)
         self.name = name.encode()
         self.spec = (abi.u32 * max(len(spec), 1))(*spec)
         self.nspec = len(spec)
@@ -60,7 +61,7 @@ class Launch:
         self.abi = abi
 
     def __call__(self):
-        if self.fn(self.name, self.spec, self.nspec, self.ref, self.size, 1, 1, 1) != 0:
+        if self.fn(self.name, self.spec, self.nspec, self.ref, self.size, 1, 1, self.batches) != 0:
             self.abi.check(-1)
 
 
@@ -282,6 +283,24 @@ def wl_gemm16(abi, m, k, n, steps, warmup, seed=1090, layout="nt", decode=False,
                 bytes=2 * (m * k + n * k + m * n), inputs=None, copies=1, name=f"mm bf16 M={m} K={k} N={n} ({layout}: " + {"nt": "x @ w.T, the Linear layout", "nn": "x @ w", "tn": "x.T @ w"}[layout] + ")")
 
 
+def wl_bmm16(abi, batches, m, k, n, steps, warmup, layout, seed=1180):
+    """A batch of few-row bfloat16 products, the shape of attention at decode: layout "nt": w stored [batches, n, k]
+    (q @ k.T: k the head dimension, n the cached positions); "nn": w stored [batches, k, n] (p @ v).  Priced against HBM
+    (the cached keys or values, 0.25 to 1 GiB here, do not fit the caches)."""
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(batches * m * k, generator=g).bfloat16()
+    w = torch.randn(1 << 20, generator=g).bfloat16().repeat(batches * n * k >> 20)  # (the values do not matter to the timing)
+    da, dw = abi.Buffer.from_numpy(a.view(torch.int16).numpy()), abi.Buffer.from_numpy(w.view(torch.int16).numpy())
+    out = abi.Buffer(batches * m * n * 2)
+    p = abi.GemmParams(a=da.address, b=dw.address, c=out.address, m=m, n=n, k=k, a_sb=m * k, a_sm=k, a_sk=1, b_sb=n * k, c_sb=m * n, c_sm=n,
+                       c_sn=1, alpha=int(np.float32(1).view(np.uint32)))
+    p.b_sk, p.b_sn = (1, k) if layout == "nt" else (n, 1)
+    fns = [Launch(abi, "gemmcm_bf16", [0, 0, 0, 0], p, batches=batches)]
+    return dict(kind="hbm", work=2 * batches * (n * k + m * k + m * n), flops=2 * batches * m * n * k, inputs=None,
+                name=f"bmm bf16 {batches} x (M={m} K={k} N={n}) ({layout}, decode)", **timed(abi, fns, steps, warmup))
+
+
 def wl_cast(abi, n, steps, warmup, seed=1070):
     """bfloat16 -> e4m3fn elementwise cast of n values (the float8 step in front of _scaled_mm)."""
     import torch
@@ -451,6 +470,9 @@ OTHER = {
     "f8_decode_m64_k28672_n1024": lambda abi, s, w: wl_fp8(abi, 64, 28672, 1024, True, s, w, decode=True),
     "mm_bf16_decode_m32_k8192_n2048": lambda abi, s, w: wl_gemm16(abi, 32, 8192, 2048, s, w, decode=True),
     "q8_m8_k8192_n1024": lambda abi, s, w: wl_q8(abi, 8, 8192, 1024, abi.BF16, s, w, seed=1170),
+    # (attention at decode, 32 sequences x 32 heads of 128 values, 4096 cached positions: q @ k.T and p @ v)
+    "bmm_bf16_decode_qk_b1024_k128_n4096": lambda abi, s, w: wl_bmm16(abi, 1024, 1, 128, 4096, max(s // 4, 10), w, "nt"),
+    "bmm_bf16_decode_pv_b1024_k4096_n128": lambda abi, s, w: wl_bmm16(abi, 1024, 1, 4096, 128, max(s // 4, 10), w, "nn"),
     "mm_bf16_decode_nn_m8_k8192_n8192": lambda abi, s, w: wl_gemm16(abi, 8, 8192, 8192, s, w, decode=True, layout="nn"),  # (weights stored [k, n])
     "c4_fp8_8192_zero_operands": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 2, 30), max(w, 5), zero_operands=True),
 }

@@ -180,7 +180,7 @@ typedef struct Q4CParams {
  * words.  112 bytes.  VARIANT (tests, tuning; 0: planned): 1-5 tile shapes, 6 the stream kernel, 7 the few-row kernel
  * (x @ w.T with up to 64 rows; bits 8-11: 16s of columns per workgroup, bits 12-16: slices of K over workgroups), 8 the
  * vector-unit kernel (x @ w.T, up to 4 rows), 9 the few-row kernel for weights stored [k, n] (x @ w with up to 64 rows;
- * bits 12-16: slices of K), 255 one thread per output. */
+ * bits 12-16: slices of K), 255 one thread per output.  Batches of few-row products take the few-row kernels too. */
 typedef struct GemmParams {
   uint64_t a, b, c, cin;
   uint64_t alpha, beta;
