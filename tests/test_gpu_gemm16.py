@@ -166,8 +166,9 @@ def test_gemm16_batched_few_rows(dtype, batch, m, k, n, layout, variant):
     want2, mag2 = oracle.gemm16(a, b, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, want_mag=True)
     close(_dev.gemm16(a, b, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, variant=variant), want2, mag2, dtype)
     shared = np.broadcast_to(b[:1], b.shape)
-    want3, mag3 = oracle.gemm16(a, shared, ODT[dtype], want_mag=True)
-    close(_dev.gemm16(a, shared, ODT[dtype], variant=variant), want3, mag3, dtype)
+    full = bits(torch.randn(batch, m, n, generator=gen(86)).to(dtype))  # (baddbmm: an addend of the result's shape)
+    want3, mag3 = oracle.gemm16(a, shared, ODT[dtype], cin=full, alpha=0.5, beta=-1.0, want_mag=True)
+    close(_dev.gemm16(a, shared, ODT[dtype], cin=full, alpha=0.5, beta=-1.0, variant=variant), want3, mag3, dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
