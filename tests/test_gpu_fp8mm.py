@@ -110,6 +110,19 @@ def test_scaled_mm_few_rows(fa, fb, m, k, n, out_dtype, rowwise):
         run_case(m, k, n, fa, fb, out_dtype, rowwise, bias_dtype, sr, variant=variant, seed=m + n)
 
 
+@pytest.mark.parametrize("fa,fb", [(FLOAT8[0], FLOAT8[0]), (FLOAT8[1], FLOAT8[0])])
+@pytest.mark.parametrize("m,k,n,out_dtype,rowwise", [
+    (96, 8192, 520, torch.bfloat16, True), (130, 4096, 264, torch.float32, True), (256, 16384, 128, torch.bfloat16, False),
+    (65, 4096, 200, torch.float8_e4m3fn, True), (100, 8192, 1000, torch.float16, False)])
+def test_scaled_mm_row_blocks_on_few_row_kernel(fa, fb, m, k, n, out_dtype, rowwise):
+    """65 to 256 rows against few columns (few tiles for the tile kernels, whose workgroups each walk all of K) run as
+    passes of the few-row kernel over blocks of 64 rows: a short last block, the row scales and output rows offset with
+    the block, every output size."""
+    bias_dtype = torch.bfloat16 if out_dtype == torch.bfloat16 else None
+    sr = 2.0 if out_dtype in (torch.float8_e4m3fn, torch.float8_e5m2) else None
+    run_case(m, k, n, fa, fb, out_dtype, rowwise, bias_dtype, sr, seed=m + n)
+
+
 @pytest.mark.parametrize("fa,fb", [(FLOAT8[0], FLOAT8[0]), (FLOAT8[1], FLOAT8[1])])
 @pytest.mark.parametrize("m,k,n,out_dtype,rowwise,nt,slices", [
     (5, 4096, 80, torch.bfloat16, True, 1, 2), (16, 2064, 64, torch.float8_e4m3fn, False, 2, 2), (33, 8192, 200, torch.bfloat16, True, 2, 4),

@@ -172,6 +172,26 @@ def test_gemm16_batched_few_rows(dtype, batch, m, k, n, layout, variant):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("batch,m,k,n,layout", [(1, 96, 4096, 520, "nt"), (1, 130, 4096, 264, "nn"), (1, 256, 8192, 72, "nt"), (2, 100, 2048, 128, "nn"), (3, 65, 2048, 200, "nt")])
+def test_gemm16_row_blocks_on_few_row_kernels(dtype, batch, m, k, n, layout):
+    """65 to 256 rows against few columns (few tiles for the tile kernels, whose workgroups each walk all of K) run as
+    passes of the few-row kernels over blocks of 64 rows: a short last block, both weight layouts, batches, an addend
+    of the result's shape (its rows offset with the block's) and a broadcast bias."""
+    import _dev
+    a = bits((torch.randn(batch, m, k, generator=gen(93)) * 0.5).to(dtype))
+    w = bits((torch.randn(batch, n, k, generator=gen(94)) * 0.5).to(dtype))
+    b = w.transpose(0, 2, 1) if layout == "nt" else np.ascontiguousarray(w.transpose(0, 2, 1))
+    want, mag = oracle.gemm16(a, b, ODT[dtype], want_mag=True)
+    close(_dev.gemm16(a, b, ODT[dtype]), want, mag, dtype)
+    full = bits(torch.randn(batch, m, n, generator=gen(95)).to(dtype))
+    want2, mag2 = oracle.gemm16(a, b, ODT[dtype], cin=full, alpha=0.5, beta=-1.0, want_mag=True)
+    close(_dev.gemm16(a, b, ODT[dtype], cin=full, alpha=0.5, beta=-1.0), want2, mag2, dtype)
+    bias = bits(torch.randn(n, generator=gen(96)).to(dtype))
+    want3, mag3 = oracle.gemm16(a, b, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, want_mag=True)
+    close(_dev.gemm16(a, b, ODT[dtype], cin=bias, alpha=2.0, beta=0.5), want3, mag3, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
 def test_gemm16_few_rows_infinite_weights(dtype):
     """Rows of k that end inside a chunk of the few-row kernel, weight rows that start with an infinity: the outputs
     are the infinities float arithmetic gives (what stands in for the values past k must not meet them as 0 x inf)."""

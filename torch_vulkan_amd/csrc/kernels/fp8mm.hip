@@ -364,6 +364,31 @@ int launch_formats(const F8Params& p, uint32_t variant, const Machine& mc, hipSt
   if (variant == 0 || (variant & 0xff) == 12) {  // 12: the few-row kernel where it serves (what up to 64 rows get), else as planned; bits 8-11: 16s of columns per workgroup, bits 12-16: slices of K
     const int rc = launch_skinny<FA, FB>(p, mc, (variant >> 8) & 15u, (variant >> 12) & 31u, stream, err);
     if (rc != -2) return rc;
+    // 65 to 256 rows against few tiles: the few-row kernel over blocks of 64 rows, where that many passes over the
+    // weights are estimated shorter than the tile kernel, whose workgroups each walk all of K and are a quarter of the
+    // machine at N = 8192 (us at 128 rows, tile kernel / two passes: 8192 x 8192: 73 / 56; 14336 x 4096: 123 / 54; 4096 x
+    // 4096: 40 / 27; 4096 x 14336 and 8192 x 28672 stay: 43 and 94 against 57 and 176).  A pass: ~8 us + weights at
+    // 2.95 MB/us; the 128 x 128 tile kernel: ~9 us per 1024 values of k and round of tiles.
+    if (variant == 0 && p.m > 64 && p.m <= 256 && p.k >= 1024 && p.n >= 64) {
+      const uint32_t passes = (p.m + 63) / 64, tiles = ((p.m + 127) / 128) * ((p.n + 127) / 128), cus = uint32_t(mc.compute_units);
+      const float pass_us = 8.0f + float(p.n) * float(p.k) / 2.95e6f, tile_us = float(p.k) / 1024.0f * 9.0f * float((tiles + cus - 1) / cus);
+      if (float(passes) * pass_us < 0.9f * tile_us) {
+        const uint32_t out_item = p.out_dtype == VKT_F32 ? 4 : (p.out_dtype == VKT_F16 || p.out_dtype == VKT_BF16) ? 2 : 1;
+        for (uint32_t r0 = 0; r0 < p.m; r0 += 64) {
+          F8Params q = p;
+          q.m = p.m - r0 < 64 ? p.m - r0 : 64;
+          q.a = p.a + uint64_t(r0) * p.lda;
+          q.out = p.out + uint64_t(r0) * p.ldo * out_item;
+          if (p.rowwise) q.scale_a = p.scale_a + uint64_t(r0) * 4;
+          const int rb = launch_skinny<FA, FB>(q, mc, 0, 0, stream, err);
+          if (rb != 0) {  // (-2 cannot be: the shape was checked above; a refused workspace ends the product)
+            if (rb == -2) *err = "fp8mm: the few-row kernel does not serve a block of rows";
+            return -1;
+          }
+        }
+        return 0;
+      }
+    }
     variant = 0;
   }
   // (256 x 256 tiles where they give the machine enough workgroups, else 128 x 128: the exact path from one tile per

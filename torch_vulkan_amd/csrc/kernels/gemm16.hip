@@ -247,6 +247,37 @@ int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t
     }
   }
   if ((variant & 0xff) == 9) variant = 0;
+  // 65 to 256 rows against few tiles, either weight layout: the few-row kernels over blocks of 64 rows, where that many
+  // passes over the weights are estimated shorter than the tile kernel, whose workgroups each walk all of K and are a
+  // quarter of the machine at N = 8192 (us at 128 rows, tile kernel / two passes: 8192 x 8192: 113 / 86; 14336 x 4096:
+  // 195 / 79; 4096 x 4096: 58 / 37; 4096 x 14336 and 8192 x 28672 stay).  A pass: ~8 us + weights at 3.9 MB/us; the
+  // 128 x 128 tile kernel: ~14 us per 1024 values of k and round of tiles.
+  if constexpr (!TRA) {
+    if (variant == 0 && p.m > 64 && p.m <= 256 && p.k >= 512 && p.n >= 64 && batch <= 65535) {
+      const uint32_t passes = (p.m + 63) / 64, cus = uint32_t(mc.compute_units);
+      const uint64_t tiles = uint64_t((p.m + 127) / 128) * ((p.n + 127) / 128) * batch;
+      const float pass_us = 8.0f + float(p.n) * float(p.k) * 2.0f * float(batch) / 3.9e6f;
+      const float tile_us = float(p.k) / 1024.0f * 14.0f * float((tiles + cus - 1) / cus);
+      if (float(passes) * pass_us < 0.9f * tile_us) {
+        for (uint32_t r0 = 0; r0 < p.m; r0 += 64) {
+          GemmProblem<T, TRA, TRB> q = g;
+          q.m = p.m - r0 < 64 ? p.m - r0 : 64;
+          q.a = g.a + uint64_t(r0) * g.lda;
+          q.c = g.c + uint64_t(int64_t(r0) * g.c_sm * 2);
+          if (g.cin) q.cin = g.cin + uint64_t(int64_t(r0) * g.cin_sm * 2);
+          int rb;
+          if constexpr (TRB) rb = launch_mma_skinny_kn<MATH>(q, mc, 0, stream, err, "gemmcm");
+          else rb = launch_mma_skinny<0, 0, MATH>(q, mc, 0, 0, stream, err, "gemmcm");
+          if (rb == -2 && r0 == 0) break;  // (not served: nothing is launched yet, the tile kernels take the product)
+          if (rb != 0) {
+            if (rb == -2) *err = "gemmcm: the few-row kernel does not serve a block of rows";
+            return -1;
+          }
+          if (r0 + 64 >= p.m) return 0;
+        }
+      }
+    }
+  }
   const bool direct_ok = g.k % BK == 0;
   // variant 0: planned; 1: 128x128 tiles; 2: 256x128; 3: 256x256 with direct loads; 4: 128x128 with direct loads;
   // 5: 256x256 with direct loads over 8 waves; 6: the stream kernel (mma_stream.h; else 3)
