@@ -460,6 +460,14 @@ uint64_t q8_gemm_scratch_bytes(const Q8Params& p, int dtype, const Machine& mc) 
   // (worth it where 128 x 128 tiles give every compute unit one: fewer tiles leave most of the machine idle, and the
   // row-block kernels, which split K, do better)
   if (uint64_t((p.m + 127) / 128) * ((p.n + 127) / 128) < uint64_t(mc.compute_units)) return 0;
+  // (weights whose widening does not stay in the 256 MiB last-level cache, one byte read and two written per weight:
+  // the pass costs ~0.75 us per million weights and the product ~0.0021 per million weights and row, rows rounded up
+  // to 128, against ~0.29 per pass of the 64-row tile kernel: up to 320 rows that one is ahead; K = 8192, N = 28672 at
+  // 191 / 192 rows: 203 us on it / 317 widened; K = 4096, N = 128256: 448 / 612)
+  if (uint64_t(p.n) * p.k * 3 > (256ull << 20)) {
+    const float passes = float((p.m + 63) / 64), rows = float((p.m + 127) / 128 * 128);
+    if (passes * 0.29f < 0.75f + 0.0021f * rows) return 0;
+  }
   const bool fits = (dtype == VKT_BF16 || dtype == VKT_F16) && p.m >= kQ8GemmRows && p.k % 16 == 0 && p.a % 16 == 0 && p.b % 16 == 0 &&
                     p.a_sm > 0 && p.a_sm % 8 == 0 && uint32_t(p.a_sm) >= p.k && p.a_sk == 1 && p.n > 0;
   return fits ? uint64_t(p.n) * p.k * 2 : 0;
