@@ -110,10 +110,25 @@ def test_scaled_mm_few_rows(fa, fb, m, k, n, out_dtype, rowwise):
         run_case(m, k, n, fa, fb, out_dtype, rowwise, bias_dtype, sr, variant=variant, seed=m + n)
 
 
+@pytest.mark.parametrize("fa,fb", [(FLOAT8[0], FLOAT8[0]), (FLOAT8[1], FLOAT8[0]), (FLOAT8[0], FLOAT8[1])])
+@pytest.mark.parametrize("m,k,n,out_dtype,rowwise,variant", [
+    (128, 2048, 264, torch.bfloat16, True, 14 | 2 << 8), (200, 4096, 520, torch.float32, False, 14 | 4 << 8), (70, 8192, 77, torch.float8_e4m3fn, True, 14 | 16 << 8),
+    (130, 8192, 1000, torch.bfloat16, True, 0), (96, 16384, 520, torch.float16, True, 0), (512, 4096, 1030, torch.bfloat16, False, 0),
+    (300, 14336, 2048, torch.float32, True, 0), (256, 8192, 4096, torch.float8_e5m2, True, 0)])
+def test_scaled_mm_tile_kernel_k_slices(fa, fb, m, k, n, out_dtype, rowwise, variant):
+    """65 rows and more against few tiles: the 128 x 128 tile kernel with K in slices over workgroups, the slices'
+    float32 partial sums in the workspace, added up in slice order by a second launch that runs the epilogue (scales,
+    bias, output scale, cast): asked for (variant 14) and planned; every output type, rows and columns past the last
+    whole tile, n off the vector width."""
+    bias_dtype = torch.bfloat16 if out_dtype == torch.bfloat16 else None
+    sr = 2.0 if out_dtype in (torch.float8_e4m3fn, torch.float8_e5m2) else None
+    run_case(m, k, n, fa, fb, out_dtype, rowwise, bias_dtype, sr, variant=variant, seed=m + n)
+
+
 @pytest.mark.parametrize("fa,fb", [(FLOAT8[0], FLOAT8[0]), (FLOAT8[1], FLOAT8[0])])
 @pytest.mark.parametrize("m,k,n,out_dtype,rowwise", [
-    (96, 8192, 520, torch.bfloat16, True), (130, 4096, 264, torch.float32, True), (256, 16384, 128, torch.bfloat16, False),
-    (65, 4096, 200, torch.float8_e4m3fn, True), (100, 8192, 1000, torch.float16, False)])
+    (96, 8208, 520, torch.bfloat16, True), (130, 4112, 264, torch.float32, True), (256, 16400, 128, torch.bfloat16, False),
+    (65, 4112, 200, torch.float8_e4m3fn, True), (100, 8208, 1000, torch.float16, False)])  # (k not in steps of 128 bytes: no slices of the tile kernel)
 def test_scaled_mm_row_blocks_on_few_row_kernel(fa, fb, m, k, n, out_dtype, rowwise):
     """65 to 256 rows against few columns (few tiles for the tile kernels, whose workgroups each walk all of K) run as
     passes of the few-row kernel over blocks of 64 rows: a short last block, the row scales and output rows offset with

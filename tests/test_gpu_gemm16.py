@@ -172,7 +172,28 @@ def test_gemm16_batched_few_rows(dtype, batch, m, k, n, layout, variant):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
-@pytest.mark.parametrize("batch,m,k,n,layout", [(1, 96, 4096, 520, "nt"), (1, 130, 4096, 264, "nn"), (1, 256, 8192, 72, "nt"), (2, 100, 2048, 128, "nn"), (3, 65, 2048, 200, "nt")])
+@pytest.mark.parametrize("m,k,n,variant", [(128, 1024, 264, 10 | 2 << 8), (200, 2048, 520, 10 | 4 << 8), (70, 4096, 77, 10 | 16 << 8),
+                                           (130, 4096, 1000, 0), (96, 8192, 520, 0), (512, 2048, 1030, 0), (300, 7168, 2048, 0)])
+def test_gemm16_tile_kernel_k_slices(dtype, m, k, n, variant):
+    """65 rows and more against few tiles (x @ w.T): the 128 x 128 tile kernel with K in slices over workgroups, the
+    slices' float32 partial sums in the workspace, added up in slice order by a second launch that runs the epilogue:
+    asked for (variant 10) and planned; rows and columns past the last whole tile, n off the vector width; alpha, beta,
+    a bias and an addend of the result's shape."""
+    import _dev
+    a = bits((torch.randn(m, k, generator=gen(103)) * 0.5).to(dtype))
+    w = bits((torch.randn(n, k, generator=gen(104)) * 0.5).to(dtype))
+    want, mag = oracle.gemm16(a, w.T, ODT[dtype], want_mag=True)
+    close(_dev.gemm16(a, w.T, ODT[dtype], variant=variant), want, mag, dtype)
+    bias = bits(torch.randn(n, generator=gen(105)).to(dtype))
+    want2, mag2 = oracle.gemm16(a, w.T, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, want_mag=True)
+    close(_dev.gemm16(a, w.T, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, variant=variant), want2, mag2, dtype)
+    full = bits(torch.randn(m, n, generator=gen(106)).to(dtype))
+    want3, mag3 = oracle.gemm16(a, w.T, ODT[dtype], cin=full, alpha=0.5, beta=-1.0, want_mag=True)
+    close(_dev.gemm16(a, w.T, ODT[dtype], cin=full, alpha=0.5, beta=-1.0, variant=variant), want3, mag3, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("batch,m,k,n,layout", [(1, 96, 4104, 520, "nt"), (1, 130, 4096, 264, "nn"), (1, 256, 8200, 72, "nt"), (2, 100, 2048, 128, "nn"), (3, 65, 2048, 200, "nt")])
 def test_gemm16_row_blocks_on_few_row_kernels(dtype, batch, m, k, n, layout):
     """65 to 256 rows against few columns (few tiles for the tile kernels, whose workgroups each walk all of K) run as
     passes of the few-row kernels over blocks of 64 rows: a short last block, both weight layouts, batches, an addend
@@ -313,4 +334,4 @@ def test_gemm16_errors():
     with pytest.raises(abi.VktError, match="unknown kernel"):
         abi.dispatch("gemmcm_f32", [0], p)
     with pytest.raises(abi.VktError, match="unknown variant"):
-        abi.dispatch("gemmcm_bf16", [0, 0, 0, 10], p)
+        abi.dispatch("gemmcm_bf16", [0, 0, 0, 11], p)

@@ -34,6 +34,7 @@
 #include "mma_stream.h"
 #include "mma_tile.h"
 #include "mma_skinny.h"
+#include "mma_slices.h"
 
 namespace vkt {
 namespace {
@@ -325,6 +326,20 @@ int launch_skinny(const F8Params& p0, const Machine& mc, uint32_t forced_nt, uin
   return launch_mma_skinny<FA, FB, kMathFp8>(p, mc, forced_nt, forced_slices, stream, err, "fp8mm");
 }
 
+// The 128 x 128 tile kernel with K in slices over workgroups (mma_slices.h): the float8 instruction for bfloat16 and
+// float8 outputs, exactly widened operands for float32 and float16 outputs.
+template <int FA, int FB>
+int launch_sliced(const F8Params& p0, uint32_t slices, const Machine& mc, hipStream_t stream, std::string* err) {
+  F8Problem p;
+  static_cast<F8Params&>(p) = p0;
+  if (slices < 2 || p0.k % (BK * slices) || uint64_t(slices) * p0.m * p0.n * 4 > mc.workspace_bytes) {
+    *err = "fp8mm: " + std::to_string(slices) + " slices of K do not divide its steps of 128 bytes, or their partial sums do not fit the workspace";
+    return -1;
+  }
+  if (p0.out_dtype == VKT_F32 || p0.out_dtype == VKT_F16) return launch_tile_slices<FA, FB, true, kMathFp8Wide>(p, slices, mc, stream, err, "fp8mm");
+  return launch_tile_slices<FA, FB, false, kMathFp8>(p, slices, mc, stream, err, "fp8mm");
+}
+
 template <int WAVES_M, int WAVES_N, int TM, int TN, int FA, int FB, bool MF32 = false, bool DIRECT = false, bool WIDE = false>
 int launch_tile(const F8Params& p, int compute_units, hipStream_t stream, std::string* err) {
   F8Problem problem;
@@ -364,6 +379,13 @@ int launch_formats(const F8Params& p, uint32_t variant, const Machine& mc, hipSt
   if (variant == 0 || (variant & 0xff) == 12) {  // 12: the few-row kernel where it serves (what up to 64 rows get), else as planned; bits 8-11: 16s of columns per workgroup, bits 12-16: slices of K
     const int rc = launch_skinny<FA, FB>(p, mc, (variant >> 8) & 15u, (variant >> 12) & 31u, stream, err);
     if (rc != -2) return rc;
+    // 65 rows and more against tiles that are half the machine or less: the 128 x 128 tile kernel with K in slices
+    // over workgroups (mma_slices.h; variant 14 asks for it, bits 8-12: slices)
+    if (variant == 0 && p.m > 64) {
+      const uint64_t budget = mc.workspace_bytes < VKT_STATIC_SCRATCH_BYTES ? mc.workspace_bytes : VKT_STATIC_SCRATCH_BYTES;
+      const uint32_t slices = tile_slices(p.m, p.n, p.k, uint32_t(mc.compute_units), budget);
+      if (slices >= 2 && uint64_t((p.m + 127) / 128) * ((p.n + 127) / 128) * 2 <= uint64_t(mc.compute_units)) return launch_sliced<FA, FB>(p, slices, mc, stream, err);
+    }
     // 65 to 256 rows against few tiles: the few-row kernel over blocks of 64 rows, where that many passes over the
     // weights are estimated shorter than the tile kernel, whose workgroups each walk all of K and are a quarter of the
     // machine at N = 8192 (us at 128 rows, tile kernel / two passes: 8192 x 8192: 73 / 56; 14336 x 4096: 123 / 54; 4096 x
@@ -398,6 +420,7 @@ int launch_formats(const F8Params& p, uint32_t variant, const Machine& mc, hipSt
   const uint64_t tiles256 = uint64_t((p.m + 255) / 256) * ((p.n + 255) / 256), cus = uint64_t(compute_units);
   if (variant == 0)
     variant = (p.out_dtype == VKT_F32 || p.out_dtype == VKT_F16) ? (big && tiles256 >= cus ? 6 : 7) : (big && 4 * tiles256 > cus ? 11 : 1);
+  if ((variant & 0xff) == 14) return launch_sliced<FA, FB>(p, (variant >> 8) & 31u, mc, stream, err);
   switch (variant) {
     case 6:
       if (p.k % BK == 0) return launch_tile<2, 2, 8, 8, FA, FB, true, true, true>(p, compute_units, stream, err);

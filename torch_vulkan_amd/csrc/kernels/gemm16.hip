@@ -16,6 +16,7 @@
 #include "mma_stream.h"
 #include "mma_tile.h"
 #include "mma_skinny.h"
+#include "mma_slices.h"
 
 namespace vkt {
 namespace {
@@ -247,6 +248,22 @@ int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t
     }
   }
   if ((variant & 0xff) == 9) variant = 0;
+  // 65 rows and more against tiles that are half the machine or less, both operands in rows of k: the 128 x 128 tile
+  // kernel with K in slices over workgroups (mma_slices.h; variant 10 asks for it, bits 8-12: slices)
+  if constexpr (!TRA && !TRB) {
+    if ((variant == 0 || (variant & 0xff) == 10) && batch == 1) {
+      const bool asked = (variant & 0xff) == 10;
+      const uint64_t budget = mc.workspace_bytes < VKT_STATIC_SCRATCH_BYTES ? mc.workspace_bytes : VKT_STATIC_SCRATCH_BYTES;
+      const uint32_t slices = asked ? (variant >> 8) & 31u : (p.m > 64 ? tile_slices(p.m, p.n, g.k, uint32_t(mc.compute_units), budget) : 1);
+      if (asked && (slices < 2 || g.k % (BK * slices) || uint64_t(slices) * p.m * p.n * 4 > mc.workspace_bytes)) {
+        *err = "gemmcm: " + std::to_string(slices) + " slices of K do not divide its steps of 64 values, or their partial sums do not fit the workspace";
+        return -1;
+      }
+      if (asked || (slices >= 2 && uint64_t((p.m + 127) / 128) * ((p.n + 127) / 128) * 2 <= uint64_t(mc.compute_units)))
+        return launch_tile_slices<0, 0, true, MATH>(g, slices, mc, stream, err, "gemmcm");
+    }
+  }
+  if ((variant & 0xff) == 10) variant = 0;
   // 65 to 256 rows against few tiles, either weight layout: the few-row kernels over blocks of 64 rows, where that many
   // passes over the weights are estimated shorter than the tile kernel, whose workgroups each walk all of K and are a
   // quarter of the machine at N = 8192 (us at 128 rows, tile kernel / two passes: 8192 x 8192: 113 / 86; 14336 x 4096:
