@@ -180,7 +180,9 @@ typedef struct Q4CParams {
  * words.  112 bytes.  VARIANT (tests, tuning; 0: planned): 1-5 tile shapes, 6 the stream kernel, 7 the few-row kernel
  * (x @ w.T with up to 64 rows; bits 8-11: 16s of columns per workgroup, bits 12-16: slices of K over workgroups), 8 the
  * vector-unit kernel (x @ w.T, up to 4 rows), 9 the few-row kernel for weights stored [k, n] (x @ w with up to 64 rows;
- * bits 12-16: slices of K), 255 one thread per output.  Batches of few-row products take the few-row kernels too. */
+ * bits 12-16: slices of K), 10 the 128 x 128 tile kernel with K in slices over workgroups (x @ w.T; bits 8-12: slices,
+ * which must divide k's steps of 64 values), 255 one thread per output.  Batches of few-row products take the few-row
+ * kernels too. */
 typedef struct GemmParams {
   uint64_t a, b, c, cin;
   uint64_t alpha, beta;
@@ -275,7 +277,8 @@ typedef struct MinMaxParams {
  * B: fp8, column-major, i.e. [n,k] rows ldb bytes apart.  104 bytes.  An optional entry overrides the launcher's
  * choice of kernel (tests, tuning; 0 or absent: planned): 1-9 tile shapes, 11 the stream kernel, 12 the few-row kernel
  * (up to 64 rows; bits 8-11: 16s of columns per workgroup, bits 12-16: slices of K over workgroups), 13 the vector-unit
- * kernel (up to 4 rows), 255 one thread per output. */
+ * kernel (up to 4 rows), 14 the 128 x 128 tile kernel with K in slices over workgroups (bits 8-12: slices, which must
+ * divide k's steps of 128 bytes), 255 one thread per output. */
 typedef struct F8Params {
   uint64_t a, b, scale_a, scale_b, bias, scale_result, out; /* bias / scale_result may be 0 */
   uint32_t m, n, k;
