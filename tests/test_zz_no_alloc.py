@@ -60,6 +60,17 @@ def test_static_dispatch_few_row_products_in_slices():
         a32 = torch.randn(m, k, generator=gen(360 + i)).numpy()
         s32 = torch.empty(n).uniform_(0.005, 0.02, generator=gen(370 + i)).numpy()
         assert np.array_equal(_dev.qmm8(a32, oracle.F32, b, s32, static=True), _dev.qmm8(a32, oracle.F32, b, s32)), (m, k, n)
+    # 65 rows and more against few tiles: the tile kernel with K in slices, its partial sums in the array (both entry
+    # points plan against the array's size, so their outputs are the same bits)
+    for i, (m, k, n) in enumerate([(256, 8192, 2048), (128, 4096, 1024)]):
+        a = bits((torch.randn(m, k, generator=gen(380 + i)) * 0.5).bfloat16())
+        w = bits((torch.randn(n, k, generator=gen(385 + i)) * 0.5).bfloat16())
+        assert np.array_equal(_dev.gemm16(a, w.T, oracle.BF16, static=True), _dev.gemm16(a, w.T, oracle.BF16)), (m, k, n)
+        a8 = bits((torch.randn(m, k, generator=gen(390 + i))).to(torch.float8_e4m3fn))
+        w8 = bits((torch.randn(n, k, generator=gen(395 + i))).to(torch.float8_e4m3fn))
+        sa, sb = np.full(m, 0.5, np.float32), np.full(n, 1.5, np.float32)
+        want = _dev.scaled_mm(a8, oracle.E4M3, w8, oracle.E4M3, sa, sb, True)
+        assert np.array_equal(_dev.scaled_mm(a8, oracle.E4M3, w8, oracle.E4M3, sa, sb, True, static=True), want), (m, k, n)
     # more partial sums than the array holds: refused, not re-planned
     m, k, n = 64, 8192, 16384
     a = bits((torch.randn(m, k, generator=gen(340)) * 0.5).bfloat16())
