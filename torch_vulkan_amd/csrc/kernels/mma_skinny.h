@@ -13,6 +13,9 @@
 // meet in wave 0, which runs the problem's epilogue (the tile kernels' interface: whole / columns / store).
 // (The 16x16x32 float8 instruction runs at half the rate of the 128-deep one the tile kernels use: at 64 rows the
 // matrix cores' share is ~4 us of a launch the weights hold to 12 and more.)
+// Where the column groups are too few for the machine, K is cut into slices over workgroups (gridDim.y; a second launch
+// adds the slices' tiles up in slice order); a batch of such products (gridDim.z) is a workgroup per batch, column
+// group and slice.  mma_skinny_kn below is the same product for weights stored [k, n].
 #pragma once
 #include <string>
 #include <type_traits>
@@ -103,7 +106,8 @@ __device__ __forceinline__ void skinny_store(const Problem& p, uint32_t batch, u
   }
 }
 
-// p.k, p.lda, p.ldb in bytes; k a multiple of 16, rows and bases 16-byte aligned; p.m <= 16 MT.  gridDim.y slices of K
+// p.k, p.lda, p.ldb, p.a_batch, p.b_batch in bytes; k a multiple of 16, rows and bases 16-byte aligned; p.m <= 16 MT.
+// gridDim.z = p.batches.  gridDim.y slices of K
 // (chunks_per_slice chunks of 256 bytes each), one per workgroup of the column group: with more than one, wave 0
 // leaves the workgroup's tiles in the workspace and mma_skinny_finish adds the slices up in slice order.
 template <int MT, int NT, int WAVES, int FA, int FB, int MATH, class Problem>
