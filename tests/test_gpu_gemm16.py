@@ -174,7 +174,7 @@ def test_gemm16_batched_few_rows(dtype, batch, m, k, n, layout, variant):
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
 @pytest.mark.parametrize("m,k,n,variant", [(128, 1024, 264, 10 | 2 << 8), (200, 2048, 520, 10 | 4 << 8), (70, 4096, 77, 10 | 16 << 8),
                                            (130, 4096, 520, 0), (96, 8192, 264, 0), (512, 2048, 262, 0), (300, 3584, 520, 0)])
-def test_gemm16_tile_kernel_k_slices(dtype, m, k, n, variant):
+def test_gemm16_tile_kernel_k_slices(dtype, m, k, n, variant, layout="nt"):
     """65 rows and more against few tiles (x @ w.T): the 128 x 128 tile kernel with K in slices over workgroups, the
     slices' float32 partial sums in the workspace, added up in slice order by a second launch that runs the epilogue:
     asked for (variant 10) and planned; rows and columns past the last whole tile, n off the vector width; alpha, beta,
@@ -182,14 +182,22 @@ def test_gemm16_tile_kernel_k_slices(dtype, m, k, n, variant):
     import _dev
     a = bits((torch.randn(m, k, generator=gen(103)) * 0.5).to(dtype))
     w = bits((torch.randn(n, k, generator=gen(104)) * 0.5).to(dtype))
-    want, mag = oracle.gemm16(a, w.T, ODT[dtype], want_mag=True)
-    close(_dev.gemm16(a, w.T, ODT[dtype], variant=variant), want, mag, dtype)
+    b = w.T if layout == "nt" else np.ascontiguousarray(w.T)  # ("nn": the weights stored [k, n])
+    want, mag = oracle.gemm16(a, b, ODT[dtype], want_mag=True)
+    close(_dev.gemm16(a, b, ODT[dtype], variant=variant), want, mag, dtype)
     bias = bits(torch.randn(n, generator=gen(105)).to(dtype))
-    want2, mag2 = oracle.gemm16(a, w.T, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, want_mag=True)
-    close(_dev.gemm16(a, w.T, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, variant=variant), want2, mag2, dtype)
+    want2, mag2 = oracle.gemm16(a, b, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, want_mag=True)
+    close(_dev.gemm16(a, b, ODT[dtype], cin=bias, alpha=2.0, beta=0.5, variant=variant), want2, mag2, dtype)
     full = bits(torch.randn(m, n, generator=gen(106)).to(dtype))
-    want3, mag3 = oracle.gemm16(a, w.T, ODT[dtype], cin=full, alpha=0.5, beta=-1.0, want_mag=True)
-    close(_dev.gemm16(a, w.T, ODT[dtype], cin=full, alpha=0.5, beta=-1.0, variant=variant), want3, mag3, dtype)
+    want3, mag3 = oracle.gemm16(a, b, ODT[dtype], cin=full, alpha=0.5, beta=-1.0, want_mag=True)
+    close(_dev.gemm16(a, b, ODT[dtype], cin=full, alpha=0.5, beta=-1.0, variant=variant), want3, mag3, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("m,k,n,variant", [(200, 2048, 264, 10 | 4 << 8), (130, 4096, 520, 0), (300, 3584, 72, 0)])
+def test_gemm16_tile_kernel_k_slices_weights_in_rows_of_n(dtype, m, k, n, variant):
+    """The same against weights stored [k, n] (x @ w): a slice of K begins k / slices rows down the weights."""
+    test_gemm16_tile_kernel_k_slices(dtype, m, k, n, variant, layout="nn")
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)

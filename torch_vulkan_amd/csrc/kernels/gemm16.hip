@@ -248,9 +248,9 @@ int launch_tiles(const GemmParams& p, uint32_t use_cin, uint32_t batch, uint32_t
     }
   }
   if ((variant & 0xff) == 9) variant = 0;
-  // 65 rows and more against tiles that are half the machine or less, both operands in rows of k: the 128 x 128 tile
-  // kernel with K in slices over workgroups (mma_slices.h; variant 10 asks for it, bits 8-12: slices)
-  if constexpr (!TRA && !TRB) {
+  // 65 rows and more against tiles that are half the machine or less, A in rows of k: the 128 x 128 tile kernel with K
+  // in slices over workgroups (mma_slices.h; variant 10 asks for it, bits 8-12: slices)
+  if constexpr (!TRA) {
     if ((variant == 0 || (variant & 0xff) == 10) && batch == 1) {
       const bool asked = (variant & 0xff) == 10;
       const uint64_t budget = mc.workspace_bytes < VKT_STATIC_SCRATCH_BYTES ? mc.workspace_bytes : VKT_STATIC_SCRATCH_BYTES;

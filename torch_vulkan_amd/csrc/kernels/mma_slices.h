@@ -4,9 +4,9 @@
 //
 // The tile kernel already runs batches of products; slice s of K is batch s of a product whose operands begin
 // s * (k / slices) bytes into their rows (both operands are rows of k) and whose "outputs" are float32 partial sums in
-// the workspace, [slice][m][n]: SliceProblem is that product.  A second launch adds the slices up in slice order (the
-// result does not depend on timing) and runs the real problem's epilogue on 4 consecutive columns of a row, the unit
-// every problem's store<DT>() takes.
+// the workspace, [slice][m][n]: SliceProblem is that product (weights stored [k, n]: a slice begins k / slices rows
+// down).  A second launch adds the slices up in slice order (the result does not depend on timing) and runs the real
+// problem's epilogue on 4 consecutive columns of a row, the unit every problem's store<DT>() takes.
 #pragma once
 #include <string>
 #include <type_traits>
@@ -17,12 +17,13 @@
 namespace vkt {
 namespace {
 
+template <bool TRB>
 struct SliceProblem {
-  static constexpr bool kTransA = false, kTransB = false;
+  static constexpr bool kTransA = false, kTransB = TRB;  // (TRB: the second operand stored [k, n], 16-bit values)
   static constexpr bool kRegisterEpilogue = false;
   uint64_t a, b;
   uint32_t m, n, k, lda, ldb, batches;  // (k: bytes of one slice; batches: the slices)
-  uint64_t a_batch, b_batch;            // (= k)
+  uint64_t a_batch, b_batch;            // (a slice's offset: k bytes into the rows; for [k, n] weights k / 2 rows)
   uint64_t partial;                     // float32 [batches][m][n]
   struct Whole {
     uint32_t vec_ok;
@@ -95,10 +96,12 @@ inline uint32_t tile_slices(uint32_t m, uint32_t n, uint32_t k_bytes, uint32_t c
 // (MF32: the 32 x 32 matrix-core tiles, which the widened and 16-bit forms are built on.)
 template <int FA, int FB, bool MF32, int MATH, class Problem>
 int launch_tile_slices(const Problem& p, uint32_t slices, const Machine& mc, hipStream_t stream, std::string* err, const char* name) {
-  SliceProblem sp;
+  constexpr bool TRB = Problem::kTransB;  // (k-major operands run on the tile kernel's direct-load form)
+  static_assert(!Problem::kTransA, "slices of K: the first operand in rows of k");
+  SliceProblem<TRB> sp;
   sp.a = p.a, sp.b = p.b, sp.m = p.m, sp.n = p.n, sp.k = p.k / slices, sp.lda = p.lda, sp.ldb = p.ldb, sp.batches = slices;
-  sp.a_batch = sp.k, sp.b_batch = sp.k, sp.partial = mc.workspace;
-  const int rc = launch_mma_tile<2, 2, 4, 4, FA, FB, MF32, false, MATH>(sp, mc.compute_units, stream, err, name);
+  sp.a_batch = sp.k, sp.b_batch = TRB ? uint64_t(sp.k / 2) * p.ldb : uint64_t(sp.k), sp.partial = mc.workspace;
+  const int rc = launch_mma_tile<2, 2, 4, 4, FA, FB, MF32, TRB, MATH>(sp, mc.compute_units, stream, err, name);
   if (rc != 0) return rc;
   const uint64_t threads = uint64_t(p.m) * ((p.n + 3) / 4);
   hipLaunchKernelGGL((mma_slices_finish<Problem>), dim3(uint32_t((threads + 255) / 256)), dim3(256), 0, stream, p, slices, mc.workspace);
