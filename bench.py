@@ -440,6 +440,10 @@ DECODE = {
     "q8_f32_m8_k4096_n14336": lambda abi, s, w: wl_q8(abi, 8, 4096, 14336, abi.F32, s, w, seed=1150),
     "q8_m16_k8192_n8192": lambda abi, s, w: wl_q8(abi, 16, 8192, 8192, abi.BF16, s, w, seed=1160),
     "mm_bf16_decode_m8_k8192_n8192": lambda abi, s, w: wl_gemm16(abi, 8, 8192, 8192, s, w, decode=True),
+    # (128 rows against 64 tiles of 128 x 128: the tile kernel with K in slices over workgroups)
+    "f8_decode_m128_k8192_n8192": lambda abi, s, w: wl_fp8(abi, 128, 8192, 8192, True, s, w, decode=True),
+    # (attention at decode, 32 sequences x 32 heads of 128 values, 4096 cached positions: p @ v)
+    "bmm_bf16_decode_pv_b1024_k4096_n128": lambda abi, s, w: wl_bmm16(abi, 1024, 1, 4096, 128, max(s // 4, 10), w, "nn"),
 }
 # Beside the BASELINE configurations (--all, or by name): many rows of the same operators, the steps either side of
 # the path, the planner off the Llama grid, config 4's launch on all-zero operands.
@@ -470,12 +474,9 @@ OTHER = {
     "f8_decode_m64_k28672_n1024": lambda abi, s, w: wl_fp8(abi, 64, 28672, 1024, True, s, w, decode=True),
     "mm_bf16_decode_m32_k8192_n2048": lambda abi, s, w: wl_gemm16(abi, 32, 8192, 2048, s, w, decode=True),
     "q8_m8_k8192_n1024": lambda abi, s, w: wl_q8(abi, 8, 8192, 1024, abi.BF16, s, w, seed=1170),
-    # (128 rows against 64 tiles of 128 x 128: the tile kernel with K in slices over workgroups)
-    "f8_decode_m128_k8192_n8192": lambda abi, s, w: wl_fp8(abi, 128, 8192, 8192, True, s, w, decode=True),
     "mm_bf16_decode_m128_k8192_n8192": lambda abi, s, w: wl_gemm16(abi, 128, 8192, 8192, s, w, decode=True),
-    # (attention at decode, 32 sequences x 32 heads of 128 values, 4096 cached positions: q @ k.T and p @ v)
+    # (attention at decode: q @ k.T)
     "bmm_bf16_decode_qk_b1024_k128_n4096": lambda abi, s, w: wl_bmm16(abi, 1024, 1, 128, 4096, max(s // 4, 10), w, "nt"),
-    "bmm_bf16_decode_pv_b1024_k4096_n128": lambda abi, s, w: wl_bmm16(abi, 1024, 1, 4096, 128, max(s // 4, 10), w, "nn"),
     "mm_bf16_decode_nn_m8_k8192_n8192": lambda abi, s, w: wl_gemm16(abi, 8, 8192, 8192, s, w, decode=True, layout="nn"),  # (weights stored [k, n])
     "c4_fp8_8192_zero_operands": lambda abi, s, w: wl_fp8(abi, 8192, 8192, 8192, False, max(s // 2, 30), max(w, 5), zero_operands=True),
 }
